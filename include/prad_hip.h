@@ -1,0 +1,166 @@
+/*
+ * prad_hip.h -- C ABI of libprad_hip.so: gfx950 (MI355X) implementation of
+ * ParallelReverseAutoDiff's matrix-multiply forward/backward path and the gradient kernels
+ * around it (activation backward, gradient clip, Adam).
+ *
+ * Conventions
+ *   - Every function returns an int32 status (PRAD_OK == 0, negative on failure) unless it is
+ *     documented as a plain getter.  No exception or abort crosses this boundary;
+ *     prad_last_error() returns the calling thread's last failure message.
+ *   - Matrices are dense row-major device buffers behind opaque handles (prad_buf_t).  A handle
+ *     is valid on any host thread.  The reference's jagged Matrix (one array per row) is
+ *     marshalled once with prad_buf_upload_rows and stays resident.
+ *   - All work is enqueued, in call order, on one library stream; calls may come from any
+ *     number of host threads (the reference runs Backward of different operations concurrently
+ *     on pool threads).  Downloads and prad_stream_sync wait for the stream.
+ *   - dtype: PRAD_F64 restates the PRAD (double) build, PRAD_F32 the PRADLite (float) build.
+ *
+ * Citations are to the reference tree (ameritusweb/ParallelReverseAutoDiff).
+ */
+#ifndef PRAD_HIP_H
+#define PRAD_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    PRAD_OK = 0,
+    PRAD_ERR_NOT_INITIALIZED = -1, /* CudaNotInitializedException, src/RMAD/GpuMatrixMultiplyOperation.cs:115-118 */
+    PRAD_ERR_SHAPE = -2,           /* InvalidOperationException("Input 1 columns do not match Input 2 rows"), src/RMAD/MatrixMultiplyOperation.cs:59-62 */
+    PRAD_ERR_ALLOC = -3,
+    PRAD_ERR_LAUNCH = -4,          /* InvalidOperationException("CUBLAS failure."), src/RMAD/CudaBlas.cs:251-256 */
+    PRAD_ERR_BAD_HANDLE = -5,
+    PRAD_ERR_ARG = -6,             /* ArgumentException, src/RMAD/GpuMatrixMultiplyOperation.cs:177-180 */
+    PRAD_ERR_NOT_RECTANGULAR = -7, /* InvalidOperationException("The given jagged array is not rectangular."), src/RMAD/GpuMatrixMultiplyOperation.cs:244-247 */
+    PRAD_ERR_DTYPE = -8
+};
+
+enum { PRAD_F64 = 0, PRAD_F32 = 1 };
+
+/* Activation selector for the elementwise backward kernels and the fused GEMM epilogues.
+ * `src` is what the reference operation caches: its input x or its output y. */
+enum {
+    PRAD_ACT_NONE = 0,
+    PRAD_ACT_LEAKYRELU = 1, /* src = x; src/RMAD/LeakyReLUOperation.cs:54-93 */
+    PRAD_ACT_SIGMOID = 2,   /* src = y; src/RMAD/SigmoidOperation.cs:46-84 */
+    PRAD_ACT_TANH = 3,      /* src = y; src/RMAD/TanhOperation.cs:42-79 */
+    PRAD_ACT_GELU = 4       /* src = x; src/RMAD/GELUOperation.cs:44-101 (the reference's own derivative formula) */
+};
+
+typedef struct prad_buf* prad_buf_t;
+
+/* ---- lifecycle: replaces CudaBlas.Instance.{DeviceId,Initialize,Dispose,IsInitialized},
+ *      src/RMAD/CudaBlas.cs:71-155 ------------------------------------------------------- */
+int32_t prad_init(int32_t device_id);
+int32_t prad_shutdown(void);
+int32_t prad_is_initialized(void); /* getter: 1 or 0 */
+int32_t prad_device_id(void);      /* getter: device passed to prad_init, -1 before */
+const char* prad_last_error(void); /* getter: thread-local, never NULL */
+int32_t prad_stream_sync(void);
+void* prad_stream(void);           /* getter: the library's hipStream_t, for callers that record their own events */
+
+/* ---- device-resident matrices: replace the per-call To2D / Allocate2DDenseX / CopyFromCPU /
+ *      GetAsArray2D / ToJagged of src/RMAD/GpuMatrixMultiplyOperation.cs:170-271 ----------- */
+int32_t prad_buf_alloc(int32_t dtype, int64_t rows, int64_t cols, prad_buf_t* out); /* zero-filled, like new Matrix(rows, cols) */
+int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out); /* DeepMatrix: depth contiguous slices; src/RMAD/DeepMatrix.cs:22 */
+int32_t prad_buf_wrap(int32_t dtype, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out); /* borrow caller-owned device memory */
+int32_t prad_buf_free(prad_buf_t b);
+int32_t prad_buf_shape(prad_buf_t b, int64_t* depth, int64_t* rows, int64_t* cols, int32_t* dtype);
+void* prad_buf_device_ptr(prad_buf_t b); /* getter: NULL for a bad handle */
+int32_t prad_buf_zero(prad_buf_t b);
+/* Jagged upload: row_ptrs[i] points at row i (cols elements).  row_lengths may be NULL; when given,
+ * any length != cols fails with PRAD_ERR_NOT_RECTANGULAR. For a deep buffer pass depth*rows pointers. */
+int32_t prad_buf_upload_rows(prad_buf_t b, const void* const* row_ptrs, const int64_t* row_lengths);
+int32_t prad_buf_download_rows(prad_buf_t b, void* const* row_ptrs);
+int32_t prad_buf_upload(prad_buf_t b, const void* src, int64_t ld);  /* contiguous rows, ld elements apart */
+int32_t prad_buf_download(prad_buf_t b, void* dst, int64_t ld);
+int32_t prad_buf_copy(prad_buf_t dst, prad_buf_t src);
+
+/* ---- matrix multiply: MatrixMultiplyOperation.Forward / Backward,
+ *      src/RMAD/MatrixMultiplyOperation.cs:50-80 and :83-126 (same contract as
+ *      GpuMatrixMultiplyOperation.cs:113-161 and CudaMatrixMultiplyOperation.cs:51-96) ------ */
+/* C[M x N] = A[M x K] . B[K x N] */
+int32_t prad_matmul_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t C);
+/* dA[M x K] = dC . B^T ; dB[K x N] = A^T . dC.  dA or dB may be NULL to skip that product.
+ * accumulate_dA / accumulate_dB != 0 adds into the destination instead of overwriting it
+ * (the dest += grad of OperationBase.AccumulateGradient, src/RMAD/OperationBase.cs:295-303). */
+int32_t prad_matmul_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB,
+                        int32_t accumulate_dA, int32_t accumulate_dB);
+/* Forward with the next operations of the graph fused into the product's epilogue:
+ * Z = A.B + bias (bias 1 x N, may be NULL: MatrixAddBroadcastingOperation.cs:32-54), H = act(Z).
+ * Z (may be NULL) receives the pre-activation the activation's Backward caches, H the output. */
+int32_t prad_matmul_fwd_fused(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_buf_t Z, prad_buf_t H,
+                              int32_t act, double alpha);
+/* Backward with the upstream activation's Backward fused into the dA product:
+ * dA = (dC . B^T) (.) act'(act_src), act_src shaped like dA. */
+int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB,
+                              int32_t accumulate_dB, int32_t act, prad_buf_t act_src, double alpha);
+/* General product on handles: C = op(A).op(B) (+ C when accumulate).  trans flags are 0/1.
+ * Supported: (0,0), (0,1), (1,0). */
+int32_t prad_gemm(int32_t transA, int32_t transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int32_t accumulate);
+/* Strided batched product over the slices of deep buffers (BatchMatrixMultiplyOperation and
+ * BatchGpuMatrixMultiplyOperation, src/RMAD/BatchGpuMatrixMultiplyOperation.cs:56-143).  A buffer of
+ * depth 1 is broadcast to every slice. */
+int32_t prad_gemm_batched(int32_t transA, int32_t transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int32_t accumulate);
+
+/* Raw device-pointer entry points (row-major, leading dimensions in elements, library stream). */
+int32_t prad_gemm_f64(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const double* A, int64_t lda,
+                      const double* B, int64_t ldb, double* C, int64_t ldc, int32_t accumulate);
+int32_t prad_gemm_f32(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const float* A, int64_t lda,
+                      const float* B, int64_t ldb, float* C, int64_t ldc, int32_t accumulate);
+
+/* One-shot host-pointer forms with today's call-per-operation behaviour of
+ * GpuMatrixMultiplyOperation.Forward/Backward (src/RMAD/GpuMatrixMultiplyOperation.cs:113-161):
+ * jagged rows in, jagged rows out, synchronous. */
+int32_t prad_matmul_fwd_host(int32_t dtype, const void* const* a_rows, const void* const* b_rows, void* const* c_rows,
+                             int64_t M, int64_t K, int64_t K2, int64_t N);
+int32_t prad_matmul_bwd_host(int32_t dtype, const void* const* dc_rows, const void* const* a_rows,
+                             const void* const* b_rows, void* const* da_rows, void* const* db_rows, int64_t M,
+                             int64_t K, int64_t N);
+
+/* ---- MatrixMultiplyAndSumOperation / GpuMatrixMultiplyAndSumOperation,
+ *      src/RMAD/MatrixMultiplyAndSumOperation.cs:50-89, GpuMatrixMultiplyAndSumOperation.cs:114-154 */
+/* out[0][q] = sum_ij (A . B[q])_ij ; A is M x K, B is deep (P, K, N), out is 1 x P. */
+int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out);
+/* As written in the reference: dB[q] = A^T * dOut[0][q] (deep (P, K, M)); dA = sum_q B[q]^T * dOut[0][q]
+ * (needs N == M). */
+int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_buf_t dA, prad_buf_t dB);
+
+/* ---- elementwise forward / backward (bandwidth kernels) ------------------------------------- */
+int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha);
+/* dx = dy (.) act'(src); src is x for LeakyReLU/GELU and y for Sigmoid/Tanh. */
+int32_t prad_act_bwd(int32_t act, prad_buf_t src, prad_buf_t dy, prad_buf_t dx, double alpha);
+/* HadamardProductOperation, src/RMAD/HadamardProductOperation.cs:50-118 */
+int32_t prad_hadamard_fwd(prad_buf_t a, prad_buf_t b, prad_buf_t y);
+int32_t prad_hadamard_bwd(prad_buf_t a, prad_buf_t b, prad_buf_t dy, prad_buf_t da, prad_buf_t db);
+/* dest += grad, src/RMAD/OperationBase.cs:295-303 */
+int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad);
+/* y = x + bias broadcast over rows; db[0][j] = sum_i dy[i][j]; src/RMAD/MatrixAddBroadcastingOperation.cs:32-70 */
+int32_t prad_add_broadcast_fwd(prad_buf_t x, prad_buf_t bias, prad_buf_t y);
+int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias);
+
+/* ---- GradientClipper.ClipGradients, src/RMAD/GradientClipper.cs:118-157 and :212-253 (in place) */
+int32_t prad_clip(prad_buf_t g, double clip_value, double min_value);
+/* ---- AdamOptimizer.UpdateWeightWithAdam, src/RMAD/AdamOptimizer.cs:195-239 (in place on w, m, v) */
+int32_t prad_adam(prad_buf_t w, prad_buf_t m, prad_buf_t v, prad_buf_t g, double lr, double beta1, double beta2,
+                  double eps, double t);
+/* Multi-tensor forms: one launch sequence over n tensors (the Parallel.For over layers of
+ * GradientClipper.Clip, src/RMAD/GradientClipper.cs:31-71, and AdamOptimizer.Optimize,
+ * src/RMAD/AdamOptimizer.cs:32-91). */
+int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, double min_value);
+int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
+                        double lr, double beta1, double beta2, double eps, double t);
+
+/* ---- timing helpers for harnesses: events recorded on the library stream ------------------ */
+int32_t prad_event_create(void** ev);
+int32_t prad_event_destroy(void* ev);
+int32_t prad_event_record(void* ev);
+int32_t prad_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PRAD_HIP_H */

@@ -1,0 +1,141 @@
+// Shared declarations of the prad_hip library internals (not part of the public ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// The reference's runtime rounds every multiply and add separately (no fused multiply-add), so
+// the elementwise arithmetic of this library is compiled without contraction as well.
+#pragma clang fp contract(off)
+
+namespace prad {
+
+// Activation selectors: same values as PRAD_ACT_* in include/prad_hip.h.
+enum Act : int { ACT_NONE = 0, ACT_LEAKYRELU = 1, ACT_SIGMOID = 2, ACT_TANH = 3, ACT_GELU = 4 };
+
+// ---- activation arithmetic, shared by the bandwidth kernels and the GEMM epilogues ----------
+// Formulas follow the reference operation by operation (association order included):
+//   LeakyReLU src/RMAD/LeakyReLUOperation.cs:54-93, Sigmoid src/RMAD/SigmoidOperation.cs:46-84,
+//   Tanh src/RMAD/TanhOperation.cs:42-79, GELU src/RMAD/GELUOperation.cs:86-101.
+template <typename T> struct GeluConst;
+template <> struct GeluConst<double> {
+    // sqrt(2 / pi) in double
+    static __device__ __forceinline__ double s() { return 0.79788456080286535588; }
+    static __device__ __forceinline__ double c0() { return 0.044715; }
+};
+template <> struct GeluConst<float> {
+    // PRADLite: (float)sqrt((double)(2 / (float)pi))
+    static __device__ __forceinline__ float s() { return 0.797884523868560791015625f; }
+    static __device__ __forceinline__ float c0() { return 0.044715f; }
+};
+
+__device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
+// PRADLite evaluates Math.Tanh in double and rounds once to float.
+__device__ __forceinline__ float dev_tanh(float x) { return (float)tanh((double)x); }
+__device__ __forceinline__ double dev_exp(double x) { return exp(x); }
+__device__ __forceinline__ float dev_exp(float x) { return (float)exp((double)x); }
+// pow(x, 3): correctly rounded cube.  In double the three-factor product can differ from it
+// in the last place; the float version cubes in double and rounds once, like (float)Math.Pow.
+__device__ __forceinline__ double dev_cube(double x) { return x * x * x; }
+__device__ __forceinline__ float dev_cube(float x) { double d = (double)x; return (float)(d * d * d); }
+
+template <typename T>
+__device__ __forceinline__ T act_forward(int act, T x, T alpha) {
+    switch (act) {
+        case ACT_LEAKYRELU: return x > (T)0 ? x : alpha * x;
+        case ACT_SIGMOID: return (T)1 / ((T)1 + dev_exp(-x));
+        case ACT_TANH: return dev_tanh(x);
+        case ACT_GELU: {
+            T a = (T)0.5 * ((T)1 + dev_tanh(GeluConst<T>::s() * (x + (GeluConst<T>::c0() * dev_cube(x)))));
+            return a * x;
+        }
+        default: return x;
+    }
+}
+
+// Derivative factor act'(src): src is the cached input x (LeakyReLU, GELU) or output y (Sigmoid, Tanh).
+template <typename T>
+__device__ __forceinline__ T act_derivative(int act, T s, T alpha) {
+    switch (act) {
+        case ACT_LEAKYRELU: return s > (T)0 ? (T)1 : alpha;
+        case ACT_SIGMOID: return s * ((T)1 - s);
+        case ACT_TANH: return (T)1 - s * s;
+        case ACT_GELU: {
+            T b = dev_tanh(GeluConst<T>::s() * (s + (GeluConst<T>::c0() * dev_cube(s))));
+            T omb = (T)1 - b * b;
+            T c = omb * omb;
+            T d = GeluConst<T>::s() * ((GeluConst<T>::c0() * (T)3 * (s * s)) + (T)1);
+            return ((T)0.5 * s * ((c * d) + b)) + ((T)0.5 * ((T)1 + b));
+        }
+        default: return (T)1;
+    }
+}
+
+// ---- GEMM launch description -------------------------------------------------------------
+// C[M x N] (+)= op(A)[M x K] . op(B)[K x N], all row-major with leading dimensions in elements.
+//   transA == 0: A is M x K (lda >= K);  transA == 1: A is K x M (lda >= M)
+//   transB == 0: B is K x N (ldb >= N);  transB == 1: B is N x K (ldb >= K)
+// Epilogue (applied to the finished accumulator v at (i, j), in this order):
+//   v += bias[j]                      when bias != nullptr
+//   if (Z) Z[i][j] = v                pre-activation copy
+//   v = act_forward(act_fwd, v)       when act_fwd != ACT_NONE
+//   v *= act_derivative(act_bwd, act_src[i][j])   when act_bwd != ACT_NONE
+//   C[i][j] = accumulate ? C[i][j] + v : v
+// batch > 1 runs `batch` independent products; strides are in elements (0 broadcasts).
+template <typename T>
+struct GemmArgs {
+    int transA, transB;
+    int64_t M, N, K;
+    const T* A; int64_t lda;
+    const T* B; int64_t ldb;
+    T* C; int64_t ldc;
+    int accumulate;
+    const T* bias;
+    T* Z; int64_t ldz;
+    int act_fwd;
+    int act_bwd;
+    const T* act_src; int64_t ld_act;
+    T alpha;
+    int batch;
+    int64_t strideA, strideB, strideC;
+    // When set, C is not written: each workgroup stores the sum of its finished tile to
+    // tile_sums[batch_index * tiles_per_product + tile_index] (MatrixMultiplyAndSum forward).
+    double* tile_sums;
+};
+
+// Number of 128 x 128 output tiles of one product (the tile_sums layout).
+inline int64_t gemm_tiles_per_product(int64_t M, int64_t N) { return ((M + 127) / 128) * ((N + 127) / 128); }
+
+template <typename T> hipError_t launch_gemm(const GemmArgs<T>& args, hipStream_t stream);
+
+// ---- bandwidth kernels ----------------------------------------------------------------------
+template <typename T> hipError_t launch_act_fwd(int act, const T* x, T* y, int64_t n, T alpha, hipStream_t s);
+template <typename T> hipError_t launch_act_bwd(int act, const T* src, const T* dy, T* dx, int64_t n, T alpha, hipStream_t s);
+template <typename T> hipError_t launch_hadamard_fwd(const T* a, const T* b, T* y, int64_t n, hipStream_t s);
+template <typename T> hipError_t launch_hadamard_bwd(const T* a, const T* b, const T* dy, T* da, T* db, int64_t n, hipStream_t s);
+template <typename T> hipError_t launch_accumulate(T* dest, const T* grad, int64_t n, hipStream_t s);
+template <typename T> hipError_t launch_add_broadcast_fwd(const T* x, const T* bias, T* y, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_fill_zero(T* p, int64_t n, hipStream_t s);
+
+// Descriptor of one tensor of a multi-tensor clip / Adam launch.
+template <typename T>
+struct TensorDesc {
+    T* g; T* w; T* m; T* v;
+    int64_t n;
+};
+// Clip needs device workspace of clip_workspace_bytes(sizes, ntensors) bytes.  `host_descs` is read
+// during the call only.  c1 = 1 / (1 - beta1^t), c2 = 1 / (1 - beta2^t), evaluated by the caller
+// in T like the reference does.
+size_t clip_workspace_bytes(const int64_t* n, int ntensors);
+template <typename T> hipError_t launch_clip(const TensorDesc<T>* host_descs, int ntensors, void* workspace, T clip_value,
+                                             T min_value, hipStream_t s);
+template <typename T> hipError_t launch_adam(const TensorDesc<T>* host_descs, int ntensors, T lr, T beta1, T beta2, T eps, T c1,
+                                             T c2, hipStream_t s);
+
+// MatrixMultiplyAndSum
+template <typename T> hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K,
+                                                       int64_t N, int64_t P, hipStream_t s);
+template <typename T> hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T* dB, int64_t M, int64_t K,
+                                                       int64_t N, int64_t P, hipStream_t s);
+
+}  // namespace prad

@@ -1,0 +1,304 @@
+// Dense matrix products on the gfx950 matrix cores for the three contractions of
+// MatrixMultiplyOperation (src/RMAD/MatrixMultiplyOperation.cs:50-126):
+//     forward   C  = A . B        (transA = 0, transB = 0)
+//     backward  dA = dC . B^T     (transA = 0, transB = 1)
+//     backward  dB = A^T . dC     (transA = 1, transB = 0)
+// in double (v_mfma_f64_16x16x4_f64) and float (v_mfma_f32_16x16x4_f32).  They replace the 8 x 8
+// shared-memory kernel of src/RMAD/GpuMatrixMultiplyOperation.cs:39-91 and the host-side
+// transposed copies it is fed with (:148, :154, :210-248): a transposed operand is read in its
+// stored orientation and only its placement in LDS differs.
+//
+// Shape of one workgroup: 256 threads = 4 wavefronts (2 x 2), output tile 128 x 128, each
+// wavefront owns 64 x 64 = 4 x 4 MFMA tiles of 16 x 16, so every A/B fragment read from LDS feeds
+// four MFMAs.  The reduction dimension is cut into slabs of BK (16 doubles / 32 floats = 128
+// bytes per row); slabs are double-buffered in LDS and the next slab's global loads are issued
+// before the current slab's MFMAs.
+//
+// LDS placement of an operand slab (MN = its 128 rows/columns of the output tile):
+//   stored with the reduction index contiguous ("KC": A of the forward, both operands of dA)
+//       S[mn][k], row pitch BK + pad chosen so that the 16 B of two neighbouring k of 16
+//       consecutive mn fall into distinct 16 B bank groups;
+//   stored with mn contiguous ("MC": B of the forward, both operands of dB)
+//       S[k][mn], row pitch 128 + 16.
+// An MFMA lane (mn = lane % 16, k = lane / 16) reads one element from either placement without
+// bank conflicts, so no transposed copy is ever written.
+#include "common.h"
+
+namespace prad {
+
+typedef double d4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef double d2_t __attribute__((ext_vector_type(2)));
+
+constexpr int BM = 128;
+constexpr int BN = 128;
+constexpr int LDM = 144;  // pitch of an MC slab row (128 + 16)
+constexpr int GEMM_THREADS = 256;
+constexpr int NUM_XCD = 8;
+constexpr int GROUP_M = 8;
+
+template <typename T> struct Mfma;
+template <> struct Mfma<double> {
+    typedef d4_t Acc;
+    typedef d2_t Vec;
+    static constexpr int VEC = 2;   // elements per 16-byte load
+    static constexpr int BK = 16;   // reduction slab
+    static constexpr int LDK = 18;  // pitch of a KC slab row
+    static __device__ __forceinline__ Acc run(double a, double b, Acc c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    // Row of the 16 x 16 result held in accumulator element r by lane group g = lane / 16.
+    static __device__ __forceinline__ int row(int r, int g) { return 4 * r + g; }
+};
+template <> struct Mfma<float> {
+    typedef f4_t Acc;
+    typedef f4_t Vec;
+    static constexpr int VEC = 4;
+    static constexpr int BK = 32;
+    static constexpr int LDK = 36;
+    static __device__ __forceinline__ Acc run(float a, float b, Acc c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int row(int r, int g) { return 4 * g + r; }
+};
+
+// Loads this thread's share (4 vectors) of one operand slab from global memory.
+//   KC: the operand is stored [mn][k]: 8 threads cover the 128 bytes of one row.
+//   MC: the operand is stored [k][mn]: 128 / VEC threads cover one k row.
+template <typename T, bool KC, bool EDGE>
+__device__ __forceinline__ void load_slab(typename Mfma<T>::Vec (&r)[4], const T* __restrict__ base, int64_t ld, int64_t mn0,
+                                          int64_t mn_end, int64_t k0, int64_t k_end, int tid) {
+    typedef typename Mfma<T>::Vec Vec;
+    constexpr int VEC = Mfma<T>::VEC;
+    if (KC) {
+        const int kv = tid & 7;
+        const int rowb = tid >> 3;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int64_t mn = mn0 + rowb + 32 * p;
+            const int64_t k = k0 + kv * VEC;
+            const T* g = base + mn * ld + k;
+            if (!EDGE) {
+                r[p] = *reinterpret_cast<const Vec*>(g);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) r[p][e] = (mn < mn_end && k + e < k_end) ? g[e] : (T)0;
+            }
+        }
+    } else {
+        constexpr int CV = 128 / VEC;                 // vectors per k row
+        constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
+        const int cv = tid % CV;
+        const int krow = tid / CV;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int64_t k = k0 + krow + ROWS_PER_PASS * p;
+            const int64_t mn = mn0 + cv * VEC;
+            const T* g = base + k * ld + mn;
+            if (!EDGE) {
+                r[p] = *reinterpret_cast<const Vec*>(g);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) r[p][e] = (k < k_end && mn + e < mn_end) ? g[e] : (T)0;
+            }
+        }
+    }
+}
+
+template <typename T, bool KC>
+__device__ __forceinline__ void store_slab(T* __restrict__ s, const typename Mfma<T>::Vec (&r)[4], int tid) {
+    typedef typename Mfma<T>::Vec Vec;
+    constexpr int VEC = Mfma<T>::VEC;
+    constexpr int LDK = Mfma<T>::LDK;
+    if (KC) {
+        const int kv = tid & 7;
+        const int rowb = tid >> 3;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) *reinterpret_cast<Vec*>(s + (rowb + 32 * p) * LDK + kv * VEC) = r[p];
+    } else {
+        constexpr int CV = 128 / VEC;
+        constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
+        const int cv = tid % CV;
+        const int krow = tid / CV;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) *reinterpret_cast<Vec*>(s + (krow + ROWS_PER_PASS * p) * LDM + cv * VEC) = r[p];
+    }
+}
+
+// Element (mn, k) of a slab in LDS.
+template <typename T, bool KC>
+__device__ __forceinline__ T slab_at(const T* __restrict__ s, int mn, int k) {
+    return KC ? s[mn * Mfma<T>::LDK + k] : s[k * LDM + mn];
+}
+
+// Maps the linear workgroup id to an output tile.  Hardware deals consecutive workgroup ids
+// round-robin to the 8 XCDs, each with its own L2: ids are first regrouped so that one XCD gets a
+// contiguous range of logical tiles, and logical tiles walk the output in bands of GROUP_M tile
+// rows, so the tiles resident on one XCD at a time share A row panels and B column panels.
+__device__ __forceinline__ void tile_of_workgroup(int pid, int tilesM, int tilesN, int& tm, int& tn) {
+    const int nwg = tilesM * tilesN;
+    const int per = nwg / NUM_XCD, rem = nwg % NUM_XCD;
+    const int xcd = pid % NUM_XCD, slot = pid / NUM_XCD;
+    const int lid = xcd < rem ? xcd * (per + 1) + slot : rem * (per + 1) + (xcd - rem) * per + slot;
+    const int width = GROUP_M * tilesN;
+    const int group = lid / width;
+    const int first_m = group * GROUP_M;
+    const int gsz = min(tilesM - first_m, GROUP_M);
+    const int in_group = lid % width;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+template <typename T, bool A_KC, bool B_KC, bool EDGE, bool EPI>
+__global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_kernel(const GemmArgs<T> p, const int tilesM, const int tilesN) {
+    typedef Mfma<T> MF;
+    typedef typename MF::Acc Acc;
+    typedef typename MF::Vec Vec;
+    constexpr int BK = MF::BK;
+    constexpr int SLAB = BM * MF::LDK;  // elements of one operand slab; equals BK * LDM
+    static_assert(BM * MF::LDK == BK * LDM, "both slab placements must have the same size");
+
+    __shared__ __attribute__((aligned(16))) T smem[2][2][SLAB];  // [stage][operand]
+
+    int tm, tn;
+    tile_of_workgroup(blockIdx.x, tilesM, tilesN, tm, tn);
+    const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+    const int batch = blockIdx.y;
+    const T* __restrict__ A = p.A + batch * p.strideA;
+    const T* __restrict__ B = p.B + batch * p.strideB;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 15, g = lane >> 4;
+
+    Acc acc[4][4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int y = 0; y < 4; ++y)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[x][y][r] = (T)0;
+
+    Vec ra[4], rb[4];
+    const int64_t K = p.K;
+    const int ntiles = (int)((K + BK - 1) / BK);
+
+    load_slab<T, A_KC, EDGE>(ra, A, p.lda, row0, p.M, 0, K, tid);
+    load_slab<T, B_KC, EDGE>(rb, B, p.ldb, col0, p.N, 0, K, tid);
+    store_slab<T, A_KC>(smem[0][0], ra, tid);
+    store_slab<T, B_KC>(smem[0][1], rb, tid);
+    __syncthreads();
+
+    int cur = 0;
+    for (int kt = 0; kt < ntiles; ++kt) {
+        const bool more = kt + 1 < ntiles;
+        if (more) {
+            load_slab<T, A_KC, EDGE>(ra, A, p.lda, row0, p.M, (int64_t)(kt + 1) * BK, K, tid);
+            load_slab<T, B_KC, EDGE>(rb, B, p.ldb, col0, p.N, (int64_t)(kt + 1) * BK, K, tid);
+        }
+        const T* __restrict__ sA = smem[cur][0];
+        const T* __restrict__ sB = smem[cur][1];
+#pragma unroll
+        for (int s = 0; s < BK / 4; ++s) {
+            const int k = 4 * s + g;
+            T a[4], b[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) a[x] = slab_at<T, A_KC>(sA, wm * 64 + x * 16 + li, k);
+#pragma unroll
+            for (int y = 0; y < 4; ++y) b[y] = slab_at<T, B_KC>(sB, wn * 64 + y * 16 + li, k);
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int y = 0; y < 4; ++y) acc[x][y] = MF::run(a[x], b[y], acc[x][y]);
+        }
+        if (more) {
+            store_slab<T, A_KC>(smem[cur ^ 1][0], ra, tid);
+            store_slab<T, B_KC>(smem[cur ^ 1][1], rb, tid);
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // ---- epilogue ------------------------------------------------------------------------
+    if (EPI && p.tile_sums != nullptr) {
+        // Sum of the whole tile (rows/columns past M, N hold exact zeros).
+        double s = 0.0;
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 4; ++y)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s += (double)acc[x][y][r];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
+        double* red = reinterpret_cast<double*>(&smem[0][0][0]);
+        if (lane == 0) red[wave] = s;
+        __syncthreads();
+        if (tid == 0)
+            p.tile_sums[(int64_t)batch * tilesM * tilesN + (int64_t)tm * tilesN + tn] = (red[0] + red[1]) + (red[2] + red[3]);
+        return;
+    }
+
+    T* __restrict__ C = p.C + batch * p.strideC;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int64_t i = row0 + wm * 64 + x * 16 + MF::row(r, g);
+#pragma unroll
+            for (int y = 0; y < 4; ++y) {
+                const int64_t j = col0 + wn * 64 + y * 16 + li;
+                if (EDGE && (i >= p.M || j >= p.N)) continue;
+                T v = acc[x][y][r];
+                if (EPI) {
+                    if (p.bias != nullptr) v = v + p.bias[j];
+                    if (p.Z != nullptr) p.Z[i * p.ldz + j] = v;
+                    if (p.act_fwd != ACT_NONE) v = act_forward<T>(p.act_fwd, v, p.alpha);
+                    if (p.act_bwd != ACT_NONE) v = v * act_derivative<T>(p.act_bwd, p.act_src[i * p.ld_act + j], p.alpha);
+                }
+                T* c = C + i * p.ldc + j;
+                if (p.accumulate) v = *c + v;
+                *c = v;
+            }
+        }
+    }
+}
+
+template <typename T, bool A_KC, bool B_KC>
+static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, bool epi, hipStream_t stream) {
+    const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BN - 1) / BN);
+    dim3 grid((unsigned)(tilesM * tilesN), (unsigned)a.batch, 1), block(GEMM_THREADS, 1, 1);
+    if (edge) {
+        if (epi) hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, true, true>), grid, block, 0, stream, a, tilesM, tilesN);
+        else hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, true, false>), grid, block, 0, stream, a, tilesM, tilesN);
+    } else {
+        if (epi) hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, false, true>), grid, block, 0, stream, a, tilesM, tilesN);
+        else hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, false, false>), grid, block, 0, stream, a, tilesM, tilesN);
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_gemm(const GemmArgs<T>& a, hipStream_t stream) {
+    if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return hipSuccess;
+    if (a.transA && a.transB) return hipErrorInvalidValue;
+    constexpr int VEC = Mfma<T>::VEC;
+    constexpr int BK = Mfma<T>::BK;
+    // The unguarded kernels use 16-byte loads on whole tiles.
+    const bool aligned = (a.M % BM == 0) && (a.N % BN == 0) && (a.K % BK == 0) && a.K > 0 && (a.lda % VEC == 0) &&
+                         (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
+                         (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0);
+    const bool epi = a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE ||
+                     a.tile_sums != nullptr;
+    // Grid y carries the batch; the tile count must fit the 1-D grid.
+    if ((int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN) > 0x7fffffffLL || a.batch > 65535) return hipErrorInvalidValue;
+    if (!a.transA && !a.transB) return launch_layout<T, true, false>(a, !aligned, epi, stream);
+    if (!a.transA && a.transB) return launch_layout<T, true, true>(a, !aligned, epi, stream);
+    return launch_layout<T, false, false>(a, !aligned, epi, stream);
+}
+
+template hipError_t launch_gemm<double>(const GemmArgs<double>&, hipStream_t);
+template hipError_t launch_gemm<float>(const GemmArgs<float>&, hipStream_t);
+
+}  // namespace prad

@@ -1,0 +1,132 @@
+// MatrixMultiplyAndSumOperation / GpuMatrixMultiplyAndSumOperation
+// (src/RMAD/MatrixMultiplyAndSumOperation.cs:50-89, src/RMAD/GpuMatrixMultiplyAndSumOperation.cs:114-154).
+//
+// Forward: out[0][q] = sum_ij (A . B[q])_ij.  The reference launches its tiled kernel once per
+// slice, copies every product back and sums it on the host; here all P products are one
+// strided-batched MFMA launch whose epilogue reduces each 128 x 128 tile to one double, so no
+// product is ever written to HBM; a second tiny kernel adds the tile sums of each slice.
+//
+// Backward, as the reference writes it (not the analytic gradient):
+//     dB[q] = transpose(A) * dOut[0][q]          (K x M per slice)
+//     dA    = sum_q transpose(B[q]) * dOut[0][q]  (q ascending; needs N == M)
+// Both are pure data movement: A is read once per group of slices and B exactly once.
+#include "common.h"
+
+namespace prad {
+
+template <typename T>
+__global__ void __launch_bounds__(64) sum_tiles_kernel(const double* __restrict__ tile_sums, T* __restrict__ out, int64_t tiles,
+                                                       int64_t P) {
+    const int64_t q = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (q >= P) return;
+    double s = 0.0;
+    for (int64_t t = 0; t < tiles; ++t) s += tile_sums[q * tiles + t];
+    out[q] = (T)s;
+}
+
+template <typename T>
+hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K, int64_t N, int64_t P,
+                                 hipStream_t s) {
+    if (P <= 0) return hipSuccess;
+    GemmArgs<T> g{};
+    g.transA = 0; g.transB = 0;
+    g.M = M; g.N = N; g.K = K;
+    g.A = A; g.lda = K;
+    g.B = B; g.ldb = N;
+    g.C = nullptr; g.ldc = N;
+    g.batch = (int)P;
+    g.strideA = 0; g.strideB = K * N; g.strideC = 0;
+    g.tile_sums = workspace;
+    hipError_t e = launch_gemm<T>(g, s);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((sum_tiles_kernel<T>), dim3((unsigned)((P + 63) / 64)), dim3(64), 0, s, workspace, out,
+                       gemm_tiles_per_product(M, N), P);
+    return hipGetLastError();
+}
+
+constexpr int TS = 64;       // transpose tile edge
+constexpr int Q_PER_WG = 8;  // slices written per workgroup of the dB kernel
+
+// dB[q][k][m] = A[m][k] * dOut[q]: the A tile is transposed through LDS once and scaled into
+// Q_PER_WG slices; reads walk k, writes walk m, both contiguous.
+template <typename T>
+__global__ void __launch_bounds__(256) sum_bwd_db_kernel(const T* __restrict__ A, const T* __restrict__ dOut, T* __restrict__ dB,
+                                                         int64_t M, int64_t K, int64_t P) {
+    __shared__ T tile[TS][TS + 1];
+    const int64_t m0 = (int64_t)blockIdx.x * TS, k0 = (int64_t)blockIdx.y * TS;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < TS; r += 4) {
+        const int64_t m = m0 + r, k = k0 + tx;
+        tile[r][tx] = (m < M && k < K) ? A[m * K + k] : (T)0;
+    }
+    __syncthreads();
+    const int64_t q0 = (int64_t)blockIdx.z * Q_PER_WG;
+    for (int64_t q = q0; q < q0 + Q_PER_WG && q < P; ++q) {
+        const T sc = dOut[q];
+        T* __restrict__ out = dB + q * K * M;
+        for (int r = ty; r < TS; r += 4) {
+            const int64_t k = k0 + r, m = m0 + tx;
+            if (k < K && m < M) out[k * M + m] = tile[tx][r] * sc;
+        }
+    }
+}
+
+// dA[i][j] = sum_q B[q][j][i] * dOut[q], q ascending, starting from 0 (the reference's
+// dA = dA + t).  A thread owns dA elements in the orientation B is stored in (i contiguous), keeps
+// their running sums in registers over all q, and the finished tile is transposed through LDS so
+// that the single write of dA walks j.
+template <typename T>
+__global__ void __launch_bounds__(256) sum_bwd_da_kernel(const T* __restrict__ B, const T* __restrict__ dOut, T* __restrict__ dA,
+                                                         int64_t M, int64_t K, int64_t N, int64_t P) {
+    constexpr int TJ = 16;  // rows of B (j) per workgroup; 64 columns (i)
+    __shared__ T tile[TJ][TS + 1];
+    const int64_t i0 = (int64_t)blockIdx.x * TS, j0 = (int64_t)blockIdx.y * TJ;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // ty in 0..3, rows ty, ty+4, ty+8, ty+12
+    T acc[4] = {(T)0, (T)0, (T)0, (T)0};
+    const int64_t i = i0 + tx;
+    for (int64_t q = 0; q < P; ++q) {
+        const T sc = dOut[q];
+        const T* __restrict__ Bq = B + q * K * N;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int64_t j = j0 + ty + 4 * r;
+            const T b = (i < N && j < K) ? Bq[j * N + i] : (T)0;
+            acc[r] = acc[r] + (b * sc);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) tile[ty + 4 * r][tx] = acc[r];
+    __syncthreads();
+    // write dA[i][j]: 16 consecutive j per row i
+    const int jj = threadIdx.x & 15, ib = threadIdx.x >> 4;  // ib in 0..15
+    for (int r = 0; r < TS; r += 16) {
+        const int64_t ii = i0 + ib + r, j = j0 + jj;
+        if (ii < M && j < K) dA[ii * K + j] = tile[jj][ib + r];
+    }
+}
+
+template <typename T>
+hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T* dB, int64_t M, int64_t K, int64_t N, int64_t P,
+                                 hipStream_t s) {
+    if (M <= 0 || K <= 0) return hipSuccess;
+    if (dB != nullptr && P > 0) {
+        dim3 grid((unsigned)((M + TS - 1) / TS), (unsigned)((K + TS - 1) / TS), (unsigned)((P + Q_PER_WG - 1) / Q_PER_WG));
+        hipLaunchKernelGGL((sum_bwd_db_kernel<T>), grid, dim3(256), 0, s, A, dOut, dB, M, K, P);
+    }
+    if (dA != nullptr) {
+        dim3 grid((unsigned)((M + TS - 1) / TS), (unsigned)((K + 15) / 16), 1);
+        hipLaunchKernelGGL((sum_bwd_da_kernel<T>), grid, dim3(256), 0, s, B, dOut, dA, M, K, N, P);
+    }
+    return hipGetLastError();
+}
+
+template hipError_t launch_matmul_sum_fwd<double>(const double*, const double*, double*, double*, int64_t, int64_t, int64_t,
+                                                  int64_t, hipStream_t);
+template hipError_t launch_matmul_sum_fwd<float>(const float*, const float*, float*, double*, int64_t, int64_t, int64_t, int64_t,
+                                                 hipStream_t);
+template hipError_t launch_matmul_sum_bwd<double>(const double*, const double*, const double*, double*, double*, int64_t, int64_t,
+                                                  int64_t, int64_t, hipStream_t);
+template hipError_t launch_matmul_sum_bwd<float>(const float*, const float*, const float*, float*, float*, int64_t, int64_t,
+                                                 int64_t, int64_t, hipStream_t);
+
+}  // namespace prad

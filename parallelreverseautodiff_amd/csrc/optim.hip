@@ -1,0 +1,263 @@
+// GradientClipper.ClipGradients (src/RMAD/GradientClipper.cs:118-157 with StandardizedMatrix
+// :212-253) and AdamOptimizer.UpdateWeightWithAdam (src/RMAD/AdamOptimizer.cs:195-239) as
+// multi-tensor bandwidth kernels: one launch sequence covers every (weight, gradient, m, v)
+// group of a model, replacing the Parallel.For over layers of GradientClipper.Clip (:31-71)
+// and AdamOptimizer.Optimize (:32-91) and the five temporaries per weight of the reference.
+//
+// Work is cut into chunks of CHUNK elements; chunk c of the launch belongs to the tensor whose
+// [first_chunk, first_chunk + nchunks) range contains it (binary search in the descriptor table).
+//
+// Clip statistics: the reference makes two passes (mean, then sum of squared deviations).  Here
+// each chunk produces (count, mean, M2) with a shifted two-pass over its registers, chunks are
+// merged with Chan's pairwise formula in double; this is as accurate as the two-pass form and
+// reads the gradient once.  Then one pass clamps in place.  HBM traffic: 3 element sizes per
+// element (read for statistics, read + write for the clamp).
+#include "common.h"
+
+namespace prad {
+
+constexpr int OPT_THREADS = 256;
+constexpr int OPT_CHUNK = 4096;  // elements per workgroup
+
+template <typename T>
+struct DevTensor {
+    T* g; T* w; T* m; T* v;
+    int64_t n;
+    int64_t first_chunk;  // index of this tensor's first chunk in the launch
+    int64_t nchunks;
+};
+
+constexpr int MAX_TABLE = 40;  // tensors per launch: the table travels as a kernel argument
+
+template <typename T>
+struct TensorTable {
+    DevTensor<T> t[MAX_TABLE];
+    int nt;
+};
+
+template <typename T>
+__device__ __forceinline__ int find_tensor(const DevTensor<T>* t, int nt, int64_t chunk) {
+    int lo = 0, hi = nt - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (t[mid].first_chunk <= chunk) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+struct Moments {
+    double n, mean, m2;
+};
+__device__ __forceinline__ Moments merge(const Moments& a, const Moments& b) {
+    if (b.n == 0.0) return a;
+    if (a.n == 0.0) return b;
+    Moments r;
+    r.n = a.n + b.n;
+    const double delta = b.mean - a.mean;
+    r.mean = a.mean + delta * (b.n / r.n);
+    r.m2 = a.m2 + b.m2 + delta * delta * (a.n * b.n / r.n);
+    return r;
+}
+__device__ __forceinline__ Moments shfl_down(const Moments& a, int off) {
+    Moments r;
+    r.n = __shfl_down(a.n, off, 64);
+    r.mean = __shfl_down(a.mean, off, 64);
+    r.m2 = __shfl_down(a.m2, off, 64);
+    return r;
+}
+
+// Per-chunk moments -> partial[chunk].
+template <typename T>
+__global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTable<T> tab, Moments* __restrict__ partial) {
+    const int64_t chunk = blockIdx.x;
+    const int ti = find_tensor(tab.t, tab.nt, chunk);
+    const DevTensor<T> t = tab.t[ti];
+    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
+    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
+    constexpr int PER = OPT_CHUNK / OPT_THREADS;  // 16 elements per thread
+    double x[PER];
+    int cnt = 0;
+    double sum = 0.0;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
+        if (i < end) { x[e] = (double)t.g[i]; sum += x[e]; ++cnt; } else x[e] = 0.0;
+    }
+    Moments mo;
+    mo.n = (double)cnt;
+    mo.mean = cnt > 0 ? sum / (double)cnt : 0.0;
+    mo.m2 = 0.0;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
+        if (i < end) { const double d = x[e] - mo.mean; mo.m2 += d * d; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mo = merge(mo, shfl_down(mo, off));
+    __shared__ Moments wave_part[OPT_THREADS / 64];
+    if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = mo;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Moments r = wave_part[0];
+        for (int w = 1; w < OPT_THREADS / 64; ++w) r = merge(r, wave_part[w]);
+        partial[chunk] = r;
+    }
+}
+
+// One workgroup per tensor merges its chunk moments: stats[ti] = {mean, stddev}.
+template <typename T>
+__global__ void __launch_bounds__(OPT_THREADS) clip_finalize_kernel(const TensorTable<T> tab, const Moments* __restrict__ partial,
+                                                                    double* __restrict__ stats) {
+    const int ti = blockIdx.x;
+    const int64_t c0 = tab.t[ti].first_chunk, nc = tab.t[ti].nchunks;
+    Moments mo{0.0, 0.0, 0.0};
+    for (int64_t c = threadIdx.x; c < nc; c += OPT_THREADS) mo = merge(mo, partial[c0 + c]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mo = merge(mo, shfl_down(mo, off));
+    __shared__ Moments wave_part[OPT_THREADS / 64];
+    if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = mo;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Moments r = wave_part[0];
+        for (int w = 1; w < OPT_THREADS / 64; ++w) r = merge(r, wave_part[w]);
+        stats[2 * ti] = r.mean;
+        stats[2 * ti + 1] = sqrt(r.m2 / r.n);  // population standard deviation
+    }
+}
+
+// .NET Math.Min: NaN when either argument is NaN.
+template <typename T>
+__device__ __forceinline__ T dotnet_min(T a, T b) {
+    if (a != a) return a;
+    if (b != b) return b;
+    return a < b ? a : b;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTable<T> tab, const double* __restrict__ stats,
+                                                                 T clip_value, T min_value) {
+    const int64_t chunk = blockIdx.x;
+    const int ti = find_tensor(tab.t, tab.nt, chunk);
+    const DevTensor<T> t = tab.t[ti];
+    // PRADLite keeps mean and standard deviation in float.
+    const T mean = (T)stats[2 * ti];
+    const T stddev = (T)stats[2 * ti + 1];
+    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
+    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
+    constexpr int PER = OPT_CHUNK / OPT_THREADS;
+#pragma unroll 4
+    for (int e = 0; e < PER; ++e) {
+        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
+        if (i < end) {
+            T g = t.g[i];
+            const T z = (g - mean) / stddev;
+            const T value = dotnet_min<T>(clip_value, (T)1 + (z < (T)0 ? -z : z));
+            if (g > value) g = value;
+            else if (g < -value) g = -value;
+            if (g > (T)0 && g < min_value) g = min_value;
+            else if (g < (T)0 && g > -min_value) g = -min_value;
+            t.g[i] = g;
+        }
+    }
+}
+
+// Adam: one pass over w, m, v, g (7 element sizes of HBM traffic per element).
+template <typename T>
+__global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> tab, T lr, T beta1, T beta2, T omb1, T omb2,
+                                                           T c1, T c2, T eps) {
+    const int64_t chunk = blockIdx.x;
+    const int ti = find_tensor(tab.t, tab.nt, chunk);
+    const DevTensor<T> t = tab.t[ti];
+    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
+    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
+    constexpr int PER = OPT_CHUNK / OPT_THREADS;
+    T w[PER], m[PER], v[PER], g[PER];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
+        if (i < end) { w[e] = t.w[i]; m[e] = t.m[i]; v[e] = t.v[i]; g[e] = t.g[i]; }
+    }
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
+        if (i < end) {
+            const T first = (beta1 * m[e]) + (omb1 * g[e]);
+            const T second = (beta2 * v[e]) + (omb2 * (g[e] * g[e]));
+            const T mhat = c1 * first;
+            const T vhat = c2 * second;
+            const T red = lr * mhat / (sqrt(vhat) + eps);
+            t.w[i] = w[e] - red;
+            t.m[i] = first;
+            t.v[i] = second;
+        }
+    }
+}
+
+template <typename T>
+static int64_t build_table(const TensorDesc<T>* host, int nt, TensorTable<T>& tab) {
+    int64_t chunks = 0;
+    tab.nt = nt;
+    for (int i = 0; i < nt; ++i) {
+        tab.t[i].g = host[i].g; tab.t[i].w = host[i].w; tab.t[i].m = host[i].m; tab.t[i].v = host[i].v;
+        tab.t[i].n = host[i].n;
+        tab.t[i].first_chunk = chunks;
+        tab.t[i].nchunks = (host[i].n + OPT_CHUNK - 1) / OPT_CHUNK;
+        chunks += tab.t[i].nchunks;
+    }
+    return chunks;
+}
+
+size_t clip_workspace_bytes(const int64_t* n, int nt) {
+    // Groups of MAX_TABLE tensors run one after another on the stream and reuse the space.
+    size_t worst = 0;
+    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
+        int64_t chunks = 0;
+        for (int i = g0; i < nt && i < g0 + MAX_TABLE; ++i) chunks += (n[i] + OPT_CHUNK - 1) / OPT_CHUNK;
+        const size_t need = (size_t)chunks * sizeof(Moments) + (size_t)MAX_TABLE * 16;
+        if (need > worst) worst = need;
+    }
+    return worst + 64;
+}
+
+template <typename T>
+hipError_t launch_clip(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value, hipStream_t s) {
+    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
+        const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
+        TensorTable<T> tab;
+        const int64_t chunks = build_table(host + g0, gn, tab);
+        if (chunks == 0) continue;
+        double* dstats = reinterpret_cast<double*>(workspace);
+        Moments* dpartial = reinterpret_cast<Moments*>(static_cast<char*>(workspace) + (size_t)MAX_TABLE * 16);
+        hipLaunchKernelGGL((clip_stats_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, dpartial);
+        hipLaunchKernelGGL((clip_finalize_kernel<T>), dim3((unsigned)gn), dim3(OPT_THREADS), 0, s, tab, dpartial, dstats);
+        hipLaunchKernelGGL((clip_apply_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, dstats, clip_value,
+                           min_value);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template <typename T>
+hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s) {
+    const T omb1 = (T)1 - beta1, omb2 = (T)1 - beta2;
+    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
+        const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
+        TensorTable<T> tab;
+        const int64_t chunks = build_table(host + g0, gn, tab);
+        if (chunks == 0) continue;
+        hipLaunchKernelGGL((adam_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, lr, beta1, beta2, omb1, omb2,
+                           c1, c2, eps);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template hipError_t launch_clip<double>(const TensorDesc<double>*, int, void*, double, double, hipStream_t);
+template hipError_t launch_clip<float>(const TensorDesc<float>*, int, void*, float, float, hipStream_t);
+template hipError_t launch_adam<double>(const TensorDesc<double>*, int, double, double, double, double, double, double,
+                                        hipStream_t);
+template hipError_t launch_adam<float>(const TensorDesc<float>*, int, float, float, float, float, float, float, hipStream_t);
+
+}  // namespace prad

@@ -1,0 +1,767 @@
+// C ABI of libprad_hip.so (declared in include/prad_hip.h): lifecycle, device-resident matrices,
+// and the entry points that enqueue the kernels of this library.  Replaces the per-call
+// allocate / copy / launch / copy-back sequence of src/RMAD/GpuMatrixMultiplyOperation.cs:170-202
+// and the serialise + thread-hop + cuBLAS path of src/RMAD/CudaBlas.cs:273-403.
+//
+// Threading model: one library stream; every entry point takes the context lock while it
+// validates, (re)sizes shared staging/workspace and enqueues, so calls from any number of host
+// threads are safe and execute in the order they acquired the lock.
+#include "../../include/prad_hip.h"
+#include "common.h"
+
+#include <atomic>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+using namespace prad;
+
+struct prad_buf {
+    uint32_t magic;
+    int32_t dtype;
+    int64_t depth, rows, cols;
+    void* ptr;
+    bool owned;
+};
+
+namespace {
+
+constexpr uint32_t BUF_MAGIC = 0x50524144u;  // "PRAD"
+constexpr size_t STAGING_CHUNK = (size_t)256 << 20;
+
+struct Context {
+    std::mutex mu;
+    std::atomic<bool> initialized{false};
+    int device = -1;
+    hipStream_t stream = nullptr;
+    void* pinned = nullptr;
+    size_t pinned_bytes = 0;
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
+};
+Context g_ctx;
+thread_local std::string tl_error;
+
+int32_t fail(int32_t code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    tl_error = buf;
+    return code;
+}
+
+#define HIP_TRY(expr, code)                                                                           \
+    do {                                                                                              \
+        hipError_t e_ = (expr);                                                                       \
+        if (e_ != hipSuccess) return fail((code), "%s failed: %s", #expr, hipGetErrorString(e_));     \
+    } while (0)
+
+#define REQUIRE_INIT()                                                                                \
+    do {                                                                                              \
+        if (!g_ctx.initialized.load()) return fail(PRAD_ERR_NOT_INITIALIZED, "prad_init has not been called"); \
+        hipError_t e_ = hipSetDevice(g_ctx.device);                                                   \
+        if (e_ != hipSuccess) return fail(PRAD_ERR_LAUNCH, "hipSetDevice failed: %s", hipGetErrorString(e_)); \
+    } while (0)
+
+inline bool valid(prad_buf_t b) { return b != nullptr && b->magic == BUF_MAGIC; }
+inline size_t elem_size(int32_t dtype) { return dtype == PRAD_F64 ? 8 : 4; }
+inline int64_t count(prad_buf_t b) { return b->depth * b->rows * b->cols; }
+
+#define REQUIRE_BUF(b)                                                                                \
+    do {                                                                                              \
+        if (!valid(b)) return fail(PRAD_ERR_BAD_HANDLE, "%s is not a live buffer handle", #b);        \
+    } while (0)
+
+// Lock must be held.
+int32_t ensure_pinned(size_t bytes) {
+    if (bytes <= g_ctx.pinned_bytes) return PRAD_OK;
+    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
+    g_ctx.pinned = nullptr;
+    g_ctx.pinned_bytes = 0;
+    HIP_TRY(hipHostMalloc(&g_ctx.pinned, bytes, hipHostMallocDefault), PRAD_ERR_ALLOC);
+    g_ctx.pinned_bytes = bytes;
+    return PRAD_OK;
+}
+int32_t ensure_workspace(size_t bytes) {
+    if (bytes <= g_ctx.workspace_bytes) return PRAD_OK;
+    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
+    g_ctx.workspace = nullptr;
+    g_ctx.workspace_bytes = 0;
+    bytes = (bytes + 4095) & ~(size_t)4095;
+    HIP_TRY(hipMalloc(&g_ctx.workspace, bytes), PRAD_ERR_ALLOC);
+    g_ctx.workspace_bytes = bytes;
+    return PRAD_OK;
+}
+
+int32_t same_dtype(std::initializer_list<prad_buf_t> bufs) {
+    int32_t dt = -1;
+    for (prad_buf_t b : bufs) {
+        if (b == nullptr) continue;
+        if (dt < 0) dt = b->dtype;
+        else if (b->dtype != dt) return fail(PRAD_ERR_DTYPE, "buffers of different element types in one call");
+    }
+    return PRAD_OK;
+}
+
+template <typename T>
+GemmArgs<T> plain_gemm(int transA, int transB, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B,
+                       int64_t ldb, void* C, int64_t ldc, int accumulate) {
+    GemmArgs<T> a{};
+    a.transA = transA; a.transB = transB;
+    a.M = M; a.N = N; a.K = K;
+    a.A = static_cast<const T*>(A); a.lda = lda;
+    a.B = static_cast<const T*>(B); a.ldb = ldb;
+    a.C = static_cast<T*>(C); a.ldc = ldc;
+    a.accumulate = accumulate;
+    a.batch = 1;
+    return a;
+}
+
+// Rows/columns of op(X) for a 2-D (per-slice) buffer.
+inline int64_t op_rows(prad_buf_t b, int trans) { return trans ? b->cols : b->rows; }
+inline int64_t op_cols(prad_buf_t b, int trans) { return trans ? b->rows : b->cols; }
+
+struct Epilogue {
+    prad_buf_t bias = nullptr;
+    prad_buf_t Z = nullptr;
+    int act_fwd = PRAD_ACT_NONE;
+    int act_bwd = PRAD_ACT_NONE;
+    prad_buf_t act_src = nullptr;
+    double alpha = 0.0;
+};
+
+template <typename T>
+int32_t enqueue_gemm_t(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int accumulate, const Epilogue& ep,
+                       bool batched) {
+    const int64_t M = op_rows(A, transA), K = op_cols(A, transA), N = op_cols(B, transB);
+    GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A->ptr, A->cols, B->ptr, B->cols, C->ptr, C->cols, accumulate);
+    if (ep.bias) a.bias = static_cast<const T*>(ep.bias->ptr);
+    if (ep.Z) { a.Z = static_cast<T*>(ep.Z->ptr); a.ldz = ep.Z->cols; }
+    a.act_fwd = ep.act_fwd;
+    a.act_bwd = ep.act_bwd;
+    if (ep.act_src) { a.act_src = static_cast<const T*>(ep.act_src->ptr); a.ld_act = ep.act_src->cols; }
+    a.alpha = (T)ep.alpha;
+    if (batched) {
+        a.batch = (int)C->depth;
+        a.strideA = A->depth == 1 ? 0 : A->rows * A->cols;
+        a.strideB = B->depth == 1 ? 0 : B->rows * B->cols;
+        a.strideC = C->rows * C->cols;
+    }
+    HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+// Validates shapes with the reference's messages and enqueues C = op(A).op(B).
+int32_t enqueue_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int accumulate, const Epilogue& ep,
+                     bool batched) {
+    REQUIRE_BUF(A); REQUIRE_BUF(B); REQUIRE_BUF(C);
+    if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1) || (transA && transB))
+        return fail(PRAD_ERR_ARG, "unsupported transpose combination (%d, %d)", transA, transB);
+    if (int32_t st = same_dtype({A, B, C, ep.bias, ep.Z, ep.act_src})) return st;
+    if (op_cols(A, transA) != op_rows(B, transB))
+        return fail(PRAD_ERR_SHAPE, "Input 1 columns do not match Input 2 rows");
+    if (C->rows != op_rows(A, transA) || C->cols != op_cols(B, transB))
+        return fail(PRAD_ERR_ARG, "Cannot multiply %lldx%lld matrix by %lldx%lld matrix into %lldx%lld",
+                    (long long)op_rows(A, transA), (long long)op_cols(A, transA), (long long)op_rows(B, transB),
+                    (long long)op_cols(B, transB), (long long)C->rows, (long long)C->cols);
+    if (batched) {
+        if ((A->depth != 1 && A->depth != C->depth) || (B->depth != 1 && B->depth != C->depth))
+            return fail(PRAD_ERR_SHAPE, "batched product: operand depth must be 1 or equal to the output depth");
+    } else if (A->depth != 1 || B->depth != 1 || C->depth != 1) {
+        return fail(PRAD_ERR_SHAPE, "deep buffer passed to a single product; use prad_gemm_batched");
+    }
+    if (ep.bias && (ep.bias->rows != 1 || ep.bias->cols != C->cols || ep.bias->depth != 1))
+        return fail(PRAD_ERR_ARG, "The length of the bias vector must be the same as the number of columns in the input matrix.");
+    if (ep.Z && (ep.Z->rows != C->rows || ep.Z->cols != C->cols || ep.Z->depth != C->depth))
+        return fail(PRAD_ERR_ARG, "pre-activation buffer must have the shape of the output");
+    if (ep.act_bwd != PRAD_ACT_NONE) {
+        if (!valid(ep.act_src)) return fail(PRAD_ERR_BAD_HANDLE, "act_src is not a live buffer handle");
+        if (ep.act_src->rows != C->rows || ep.act_src->cols != C->cols || ep.act_src->depth != C->depth)
+            return fail(PRAD_ERR_ARG, "act_src must have the shape of the gradient it scales");
+    }
+    if (ep.act_fwd < 0 || ep.act_fwd > PRAD_ACT_GELU || ep.act_bwd < 0 || ep.act_bwd > PRAD_ACT_GELU)
+        return fail(PRAD_ERR_ARG, "unknown activation selector");
+    if (A->dtype == PRAD_F64) return enqueue_gemm_t<double>(transA, transB, A, B, C, accumulate, ep, batched);
+    return enqueue_gemm_t<float>(transA, transB, A, B, C, accumulate, ep, batched);
+}
+
+int32_t same_shape(prad_buf_t a, prad_buf_t b, const char* what) {
+    if (a->depth != b->depth || a->rows != b->rows || a->cols != b->cols)
+        return fail(PRAD_ERR_ARG, "%s: Matrices must have the same dimensions.", what);
+    return PRAD_OK;
+}
+
+}  // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+// ---------------------------------------------------------------------------------------------
+int32_t prad_init(int32_t device_id) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (g_ctx.initialized.load()) {
+        if (device_id == g_ctx.device) return PRAD_OK;
+        return fail(PRAD_ERR_ARG, "already initialized on device %d", g_ctx.device);
+    }
+    int ndev = 0;
+    HIP_TRY(hipGetDeviceCount(&ndev), PRAD_ERR_NOT_INITIALIZED);
+    if (device_id < 0 || device_id >= ndev) return fail(PRAD_ERR_ARG, "device %d out of range (%d devices)", device_id, ndev);
+    HIP_TRY(hipSetDevice(device_id), PRAD_ERR_NOT_INITIALIZED);
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device_id), PRAD_ERR_NOT_INITIALIZED);
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(PRAD_ERR_NOT_INITIALIZED, "device %d is %s; this library is built for gfx950 only", device_id, prop.gcnArchName);
+    HIP_TRY(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking), PRAD_ERR_NOT_INITIALIZED);
+    g_ctx.device = device_id;
+    g_ctx.initialized.store(true);
+    return PRAD_OK;
+}
+
+int32_t prad_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (!g_ctx.initialized.load()) return PRAD_OK;
+    (void)hipSetDevice(g_ctx.device);
+    (void)hipStreamSynchronize(g_ctx.stream);
+    if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
+    if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
+    (void)hipStreamDestroy(g_ctx.stream);
+    g_ctx.pinned = nullptr; g_ctx.pinned_bytes = 0;
+    g_ctx.workspace = nullptr; g_ctx.workspace_bytes = 0;
+    g_ctx.stream = nullptr;
+    g_ctx.device = -1;
+    g_ctx.initialized.store(false);
+    return PRAD_OK;
+}
+
+int32_t prad_is_initialized(void) { return g_ctx.initialized.load() ? 1 : 0; }
+int32_t prad_device_id(void) { return g_ctx.device; }
+const char* prad_last_error(void) { return tl_error.c_str(); }
+void* prad_stream(void) { return g_ctx.stream; }
+
+int32_t prad_stream_sync(void) {
+    REQUIRE_INIT();
+    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out) {
+    REQUIRE_INIT();
+    if (out == nullptr) return fail(PRAD_ERR_ARG, "out is NULL");
+    *out = nullptr;
+    if (dtype != PRAD_F64 && dtype != PRAD_F32) return fail(PRAD_ERR_DTYPE, "unknown dtype %d", dtype);
+    if (depth <= 0 || rows <= 0 || cols <= 0) return fail(PRAD_ERR_ARG, "matrix dimensions must be positive");
+    const size_t bytes = (size_t)depth * rows * cols * elem_size(dtype);
+    void* p = nullptr;
+    HIP_TRY(hipMalloc(&p, bytes), PRAD_ERR_ALLOC);
+    {
+        std::lock_guard<std::mutex> lock(g_ctx.mu);
+        hipError_t e = dtype == PRAD_F64 ? launch_fill_zero<double>(static_cast<double*>(p), depth * rows * cols, g_ctx.stream)
+                                         : launch_fill_zero<float>(static_cast<float*>(p), depth * rows * cols, g_ctx.stream);
+        if (e != hipSuccess) { (void)hipFree(p); return fail(PRAD_ERR_LAUNCH, "zero fill failed: %s", hipGetErrorString(e)); }
+    }
+    prad_buf* b = new prad_buf{BUF_MAGIC, dtype, depth, rows, cols, p, true};
+    *out = b;
+    return PRAD_OK;
+}
+
+int32_t prad_buf_alloc(int32_t dtype, int64_t rows, int64_t cols, prad_buf_t* out) {
+    return prad_buf_alloc_deep(dtype, 1, rows, cols, out);
+}
+
+int32_t prad_buf_wrap(int32_t dtype, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out) {
+    REQUIRE_INIT();
+    if (out == nullptr || device_ptr == nullptr) return fail(PRAD_ERR_ARG, "NULL argument");
+    if (dtype != PRAD_F64 && dtype != PRAD_F32) return fail(PRAD_ERR_DTYPE, "unknown dtype %d", dtype);
+    if (rows <= 0 || cols <= 0) return fail(PRAD_ERR_ARG, "matrix dimensions must be positive");
+    *out = new prad_buf{BUF_MAGIC, dtype, 1, rows, cols, device_ptr, false};
+    return PRAD_OK;
+}
+
+int32_t prad_buf_free(prad_buf_t b) {
+    if (b == nullptr) return PRAD_OK;
+    REQUIRE_BUF(b);
+    if (b->owned) {
+        REQUIRE_INIT();
+        std::lock_guard<std::mutex> lock(g_ctx.mu);
+        // Work that still uses the buffer may be queued.
+        HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+        HIP_TRY(hipFree(b->ptr), PRAD_ERR_ALLOC);
+    }
+    b->magic = 0;
+    delete b;
+    return PRAD_OK;
+}
+
+int32_t prad_buf_shape(prad_buf_t b, int64_t* depth, int64_t* rows, int64_t* cols, int32_t* dtype) {
+    REQUIRE_BUF(b);
+    if (depth) *depth = b->depth;
+    if (rows) *rows = b->rows;
+    if (cols) *cols = b->cols;
+    if (dtype) *dtype = b->dtype;
+    return PRAD_OK;
+}
+
+void* prad_buf_device_ptr(prad_buf_t b) { return valid(b) ? b->ptr : nullptr; }
+
+int32_t prad_buf_zero(prad_buf_t b) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(b);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (b->dtype == PRAD_F64) HIP_TRY(launch_fill_zero<double>(static_cast<double*>(b->ptr), count(b), g_ctx.stream), PRAD_ERR_LAUNCH);
+    else HIP_TRY(launch_fill_zero<float>(static_cast<float*>(b->ptr), count(b), g_ctx.stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+int32_t prad_buf_upload_rows(prad_buf_t b, const void* const* row_ptrs, const int64_t* row_lengths) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(b);
+    if (row_ptrs == nullptr) return fail(PRAD_ERR_ARG, "row_ptrs is NULL");
+    const int64_t nrows = b->depth * b->rows;
+    if (row_lengths)
+        for (int64_t i = 0; i < nrows; ++i)
+            if (row_lengths[i] != b->cols) return fail(PRAD_ERR_NOT_RECTANGULAR, "The given jagged array is not rectangular.");
+    for (int64_t i = 0; i < nrows; ++i)
+        if (row_ptrs[i] == nullptr) return fail(PRAD_ERR_NOT_RECTANGULAR, "The given jagged array is not rectangular.");
+    const size_t row_bytes = (size_t)b->cols * elem_size(b->dtype);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int64_t rows_per_chunk = (int64_t)(STAGING_CHUNK / row_bytes);
+    if (rows_per_chunk < 1) rows_per_chunk = 1;
+    if (rows_per_chunk > nrows) rows_per_chunk = nrows;
+    if (int32_t st = ensure_pinned((size_t)rows_per_chunk * row_bytes)) return st;
+    for (int64_t r0 = 0; r0 < nrows; r0 += rows_per_chunk) {
+        const int64_t nr = nrows - r0 < rows_per_chunk ? nrows - r0 : rows_per_chunk;
+        char* stage = static_cast<char*>(g_ctx.pinned);
+        for (int64_t i = 0; i < nr; ++i) memcpy(stage + (size_t)i * row_bytes, row_ptrs[r0 + i], row_bytes);
+        HIP_TRY(hipMemcpyAsync(static_cast<char*>(b->ptr) + (size_t)r0 * row_bytes, stage, (size_t)nr * row_bytes,
+                               hipMemcpyHostToDevice, g_ctx.stream), PRAD_ERR_LAUNCH);
+        HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    }
+    return PRAD_OK;
+}
+
+int32_t prad_buf_download_rows(prad_buf_t b, void* const* row_ptrs) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(b);
+    if (row_ptrs == nullptr) return fail(PRAD_ERR_ARG, "row_ptrs is NULL");
+    const int64_t nrows = b->depth * b->rows;
+    for (int64_t i = 0; i < nrows; ++i)
+        if (row_ptrs[i] == nullptr) return fail(PRAD_ERR_NOT_RECTANGULAR, "The given jagged array is not rectangular.");
+    const size_t row_bytes = (size_t)b->cols * elem_size(b->dtype);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int64_t rows_per_chunk = (int64_t)(STAGING_CHUNK / row_bytes);
+    if (rows_per_chunk < 1) rows_per_chunk = 1;
+    if (rows_per_chunk > nrows) rows_per_chunk = nrows;
+    if (int32_t st = ensure_pinned((size_t)rows_per_chunk * row_bytes)) return st;
+    for (int64_t r0 = 0; r0 < nrows; r0 += rows_per_chunk) {
+        const int64_t nr = nrows - r0 < rows_per_chunk ? nrows - r0 : rows_per_chunk;
+        char* stage = static_cast<char*>(g_ctx.pinned);
+        HIP_TRY(hipMemcpyAsync(stage, static_cast<char*>(b->ptr) + (size_t)r0 * row_bytes, (size_t)nr * row_bytes,
+                               hipMemcpyDeviceToHost, g_ctx.stream), PRAD_ERR_LAUNCH);
+        HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+        for (int64_t i = 0; i < nr; ++i) memcpy(row_ptrs[r0 + i], stage + (size_t)i * row_bytes, row_bytes);
+    }
+    return PRAD_OK;
+}
+
+int32_t prad_buf_upload(prad_buf_t b, const void* src, int64_t ld) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(b);
+    if (src == nullptr || ld < b->cols) return fail(PRAD_ERR_ARG, "bad source pointer or leading dimension");
+    const size_t es = elem_size(b->dtype);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipMemcpy2DAsync(b->ptr, (size_t)b->cols * es, src, (size_t)ld * es, (size_t)b->cols * es,
+                             (size_t)(b->depth * b->rows), hipMemcpyHostToDevice, g_ctx.stream), PRAD_ERR_LAUNCH);
+    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+int32_t prad_buf_download(prad_buf_t b, void* dst, int64_t ld) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(b);
+    if (dst == nullptr || ld < b->cols) return fail(PRAD_ERR_ARG, "bad destination pointer or leading dimension");
+    const size_t es = elem_size(b->dtype);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipMemcpy2DAsync(dst, (size_t)ld * es, b->ptr, (size_t)b->cols * es, (size_t)b->cols * es,
+                             (size_t)(b->depth * b->rows), hipMemcpyDeviceToHost, g_ctx.stream), PRAD_ERR_LAUNCH);
+    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+int32_t prad_buf_copy(prad_buf_t dst, prad_buf_t src) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(dst); REQUIRE_BUF(src);
+    if (int32_t st = same_dtype({dst, src})) return st;
+    if (int32_t st = same_shape(dst, src, "copy")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipMemcpyAsync(dst->ptr, src->ptr, (size_t)count(src) * elem_size(src->dtype), hipMemcpyDeviceToDevice, g_ctx.stream),
+            PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+int32_t prad_gemm(int32_t transA, int32_t transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int32_t accumulate) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return enqueue_gemm(transA, transB, A, B, C, accumulate, Epilogue{}, false);
+}
+
+int32_t prad_gemm_batched(int32_t transA, int32_t transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int32_t accumulate) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return enqueue_gemm(transA, transB, A, B, C, accumulate, Epilogue{}, true);
+}
+
+int32_t prad_matmul_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t C) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return enqueue_gemm(0, 0, A, B, C, 0, Epilogue{}, false);
+}
+
+int32_t prad_matmul_fwd_fused(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_buf_t Z, prad_buf_t H, int32_t act, double alpha) {
+    REQUIRE_INIT();
+    if (bias != nullptr) REQUIRE_BUF(bias);
+    if (Z != nullptr) REQUIRE_BUF(Z);
+    Epilogue ep;
+    ep.bias = bias; ep.Z = Z; ep.act_fwd = act; ep.alpha = alpha;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return enqueue_gemm(0, 0, A, B, H, 0, ep, false);
+}
+
+static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, int32_t acc_dA,
+                                 int32_t acc_dB, const Epilogue& ep) {
+    REQUIRE_BUF(dC); REQUIRE_BUF(A); REQUIRE_BUF(B);
+    if (A->cols != B->rows) return fail(PRAD_ERR_SHAPE, "Input 1 columns do not match Input 2 rows");
+    if (dC->rows != A->rows || dC->cols != B->cols)
+        return fail(PRAD_ERR_ARG, "upstream gradient is %lldx%lld, the product is %lldx%lld", (long long)dC->rows,
+                    (long long)dC->cols, (long long)A->rows, (long long)B->cols);
+    if (dA != nullptr) {
+        if (int32_t st = enqueue_gemm(0, 1, dC, B, dA, acc_dA, ep, false)) return st;  // dA = dC . B^T
+    }
+    if (dB != nullptr) {
+        if (int32_t st = enqueue_gemm(1, 0, A, dC, dB, acc_dB, Epilogue{}, false)) return st;  // dB = A^T . dC
+    }
+    return PRAD_OK;
+}
+
+int32_t prad_matmul_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, int32_t accumulate_dA,
+                        int32_t accumulate_dB) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return matmul_bwd_locked(dC, A, B, dA, dB, accumulate_dA, accumulate_dB, Epilogue{});
+}
+
+int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, int32_t accumulate_dB,
+                              int32_t act, prad_buf_t act_src, double alpha) {
+    REQUIRE_INIT();
+    Epilogue ep;
+    ep.act_bwd = act; ep.act_src = act_src; ep.alpha = alpha;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return matmul_bwd_locked(dC, A, B, dA, dB, 0, accumulate_dB, ep);
+}
+
+#define RAW_GEMM(SFX, T)                                                                                              \
+    int32_t prad_gemm_##SFX(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const T* A, int64_t lda, \
+                            const T* B, int64_t ldb, T* C, int64_t ldc, int32_t accumulate) {                         \
+        REQUIRE_INIT();                                                                                               \
+        if (A == nullptr || B == nullptr || C == nullptr) return fail(PRAD_ERR_ARG, "NULL matrix pointer");           \
+        if (M < 0 || N < 0 || K < 0) return fail(PRAD_ERR_ARG, "negative dimension");                                 \
+        if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1) || (transA && transB))                       \
+            return fail(PRAD_ERR_ARG, "unsupported transpose combination (%d, %d)", transA, transB);                  \
+        if (lda < (transA ? M : K) || ldb < (transB ? K : N) || ldc < N) return fail(PRAD_ERR_ARG, "leading dimension too small"); \
+        GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                   \
+        std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                   \
+        HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);                                                    \
+        return PRAD_OK;                                                                                               \
+    }
+RAW_GEMM(f64, double)
+RAW_GEMM(f32, float)
+
+// ---------------------------------------------------------------------------------------------
+int32_t prad_matmul_fwd_host(int32_t dtype, const void* const* a_rows, const void* const* b_rows, void* const* c_rows, int64_t M,
+                             int64_t K, int64_t K2, int64_t N) {
+    REQUIRE_INIT();
+    if (K != K2) return fail(PRAD_ERR_SHAPE, "Input 1 columns do not match Input 2 rows");
+    prad_buf_t A = nullptr, B = nullptr, C = nullptr;
+    int32_t st = prad_buf_alloc(dtype, M, K, &A);
+    if (!st) st = prad_buf_alloc(dtype, K, N, &B);
+    if (!st) st = prad_buf_alloc(dtype, M, N, &C);
+    if (!st) st = prad_buf_upload_rows(A, a_rows, nullptr);
+    if (!st) st = prad_buf_upload_rows(B, b_rows, nullptr);
+    if (!st) st = prad_matmul_fwd(A, B, C);
+    if (!st) st = prad_buf_download_rows(C, c_rows);
+    std::string keep = tl_error;
+    prad_buf_free(A); prad_buf_free(B); prad_buf_free(C);
+    if (st) tl_error = keep;
+    return st;
+}
+
+int32_t prad_matmul_bwd_host(int32_t dtype, const void* const* dc_rows, const void* const* a_rows, const void* const* b_rows,
+                             void* const* da_rows, void* const* db_rows, int64_t M, int64_t K, int64_t N) {
+    REQUIRE_INIT();
+    prad_buf_t dC = nullptr, A = nullptr, B = nullptr, dA = nullptr, dB = nullptr;
+    int32_t st = prad_buf_alloc(dtype, M, N, &dC);
+    if (!st) st = prad_buf_alloc(dtype, M, K, &A);
+    if (!st) st = prad_buf_alloc(dtype, K, N, &B);
+    if (!st) st = prad_buf_alloc(dtype, M, K, &dA);
+    if (!st) st = prad_buf_alloc(dtype, K, N, &dB);
+    if (!st) st = prad_buf_upload_rows(dC, dc_rows, nullptr);
+    if (!st) st = prad_buf_upload_rows(A, a_rows, nullptr);
+    if (!st) st = prad_buf_upload_rows(B, b_rows, nullptr);
+    if (!st) st = prad_matmul_bwd(dC, A, B, dA, dB, 0, 0);
+    if (!st) st = prad_buf_download_rows(dA, da_rows);
+    if (!st) st = prad_buf_download_rows(dB, db_rows);
+    std::string keep = tl_error;
+    prad_buf_free(dC); prad_buf_free(A); prad_buf_free(B); prad_buf_free(dA); prad_buf_free(dB);
+    if (st) tl_error = keep;
+    return st;
+}
+
+// ---------------------------------------------------------------------------------------------
+int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(A); REQUIRE_BUF(B); REQUIRE_BUF(out);
+    if (int32_t st = same_dtype({A, B, out})) return st;
+    if (A->depth != 1) return fail(PRAD_ERR_SHAPE, "first operand must be a single matrix");
+    if (A->cols != B->rows) return fail(PRAD_ERR_SHAPE, "Matrix dimensions must be compatible for multiplication.");
+    const int64_t P = B->depth;
+    if (out->depth != 1 || out->rows != 1 || out->cols != P) return fail(PRAD_ERR_ARG, "output must be 1 x depth");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    const size_t ws = (size_t)P * gemm_tiles_per_product(A->rows, B->cols) * sizeof(double);
+    if (int32_t st = ensure_workspace(ws)) return st;
+    double* w = static_cast<double*>(g_ctx.workspace);
+    if (A->dtype == PRAD_F64)
+        HIP_TRY(launch_matmul_sum_fwd<double>(static_cast<const double*>(A->ptr), static_cast<const double*>(B->ptr),
+                                              static_cast<double*>(out->ptr), w, A->rows, A->cols, B->cols, P, g_ctx.stream),
+                PRAD_ERR_LAUNCH);
+    else
+        HIP_TRY(launch_matmul_sum_fwd<float>(static_cast<const float*>(A->ptr), static_cast<const float*>(B->ptr),
+                                             static_cast<float*>(out->ptr), w, A->rows, A->cols, B->cols, P, g_ctx.stream),
+                PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_buf_t dA, prad_buf_t dB) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(A); REQUIRE_BUF(B); REQUIRE_BUF(dOut);
+    if (dA != nullptr) REQUIRE_BUF(dA);
+    if (dB != nullptr) REQUIRE_BUF(dB);
+    if (int32_t st = same_dtype({A, B, dOut, dA, dB})) return st;
+    const int64_t M = A->rows, K = A->cols, N = B->cols, P = B->depth;
+    if (A->depth != 1 || B->rows != K) return fail(PRAD_ERR_SHAPE, "Matrix dimensions must be compatible for multiplication.");
+    if (dOut->depth != 1 || dOut->rows != 1 || dOut->cols != P) return fail(PRAD_ERR_ARG, "upstream gradient must be 1 x depth");
+    if (dA != nullptr) {
+        if (N != M) return fail(PRAD_ERR_SHAPE, "transpose(B[q]) must have the shape of A (the reference adds them elementwise)");
+        if (dA->depth != 1 || dA->rows != M || dA->cols != K) return fail(PRAD_ERR_ARG, "dA must have the shape of A");
+    }
+    if (dB != nullptr && (dB->depth != P || dB->rows != K || dB->cols != M))
+        return fail(PRAD_ERR_ARG, "dB must be depth x cols(A) x rows(A)");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (A->dtype == PRAD_F64)
+        HIP_TRY(launch_matmul_sum_bwd<double>(static_cast<const double*>(A->ptr), static_cast<const double*>(B->ptr),
+                                              static_cast<const double*>(dOut->ptr), dA ? static_cast<double*>(dA->ptr) : nullptr,
+                                              dB ? static_cast<double*>(dB->ptr) : nullptr, M, K, N, P, g_ctx.stream),
+                PRAD_ERR_LAUNCH);
+    else
+        HIP_TRY(launch_matmul_sum_bwd<float>(static_cast<const float*>(A->ptr), static_cast<const float*>(B->ptr),
+                                             static_cast<const float*>(dOut->ptr), dA ? static_cast<float*>(dA->ptr) : nullptr,
+                                             dB ? static_cast<float*>(dB->ptr) : nullptr, M, K, N, P, g_ctx.stream),
+                PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+#define DISPATCH(b, call64, call32)                                  \
+    do {                                                             \
+        if ((b)->dtype == PRAD_F64) HIP_TRY(call64, PRAD_ERR_LAUNCH); \
+        else HIP_TRY(call32, PRAD_ERR_LAUNCH);                       \
+    } while (0)
+#define D(b) static_cast<double*>((b)->ptr)
+#define F(b) static_cast<float*>((b)->ptr)
+
+int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(y);
+    if (act < PRAD_ACT_LEAKYRELU || act > PRAD_ACT_GELU) return fail(PRAD_ERR_ARG, "unknown activation selector");
+    if (int32_t st = same_dtype({x, y})) return st;
+    if (int32_t st = same_shape(x, y, "activation")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_act_fwd<double>(act, D(x), D(y), count(x), alpha, g_ctx.stream),
+             launch_act_fwd<float>(act, F(x), F(y), count(x), (float)alpha, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_act_bwd(int32_t act, prad_buf_t src, prad_buf_t dy, prad_buf_t dx, double alpha) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(src); REQUIRE_BUF(dy); REQUIRE_BUF(dx);
+    if (act < PRAD_ACT_LEAKYRELU || act > PRAD_ACT_GELU) return fail(PRAD_ERR_ARG, "unknown activation selector");
+    if (int32_t st = same_dtype({src, dy, dx})) return st;
+    if (int32_t st = same_shape(src, dy, "activation backward")) return st;
+    if (int32_t st = same_shape(src, dx, "activation backward")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(src, launch_act_bwd<double>(act, D(src), D(dy), D(dx), count(src), alpha, g_ctx.stream),
+             launch_act_bwd<float>(act, F(src), F(dy), F(dx), count(src), (float)alpha, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_hadamard_fwd(prad_buf_t a, prad_buf_t b, prad_buf_t y) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(a); REQUIRE_BUF(b); REQUIRE_BUF(y);
+    if (int32_t st = same_dtype({a, b, y})) return st;
+    if (int32_t st = same_shape(a, b, "Hadamard product")) return st;
+    if (int32_t st = same_shape(a, y, "Hadamard product")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(a, launch_hadamard_fwd<double>(D(a), D(b), D(y), count(a), g_ctx.stream),
+             launch_hadamard_fwd<float>(F(a), F(b), F(y), count(a), g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_hadamard_bwd(prad_buf_t a, prad_buf_t b, prad_buf_t dy, prad_buf_t da, prad_buf_t db) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(a); REQUIRE_BUF(b); REQUIRE_BUF(dy); REQUIRE_BUF(da); REQUIRE_BUF(db);
+    if (int32_t st = same_dtype({a, b, dy, da, db})) return st;
+    for (prad_buf_t o : {b, dy, da, db})
+        if (int32_t st = same_shape(a, o, "Hadamard product")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(a, launch_hadamard_bwd<double>(D(a), D(b), D(dy), D(da), D(db), count(a), g_ctx.stream),
+             launch_hadamard_bwd<float>(F(a), F(b), F(dy), F(da), F(db), count(a), g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(dest); REQUIRE_BUF(grad);
+    if (int32_t st = same_dtype({dest, grad})) return st;
+    if (int32_t st = same_shape(dest, grad, "accumulate")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(dest, launch_accumulate<double>(D(dest), D(grad), count(dest), g_ctx.stream),
+             launch_accumulate<float>(F(dest), F(grad), count(dest), g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_add_broadcast_fwd(prad_buf_t x, prad_buf_t bias, prad_buf_t y) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(bias); REQUIRE_BUF(y);
+    if (int32_t st = same_dtype({x, bias, y})) return st;
+    if (bias->cols != x->cols || bias->rows != 1 || bias->depth != 1)
+        return fail(PRAD_ERR_ARG, "The length of the bias vector must be the same as the number of columns in the input matrix.");
+    if (int32_t st = same_shape(x, y, "add broadcasting")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_add_broadcast_fwd<double>(D(x), D(bias), D(y), x->depth * x->rows, x->cols, g_ctx.stream),
+             launch_add_broadcast_fwd<float>(F(x), F(bias), F(y), x->depth * x->rows, x->cols, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(dy); REQUIRE_BUF(dbias);
+    if (int32_t st = same_dtype({dy, dbias})) return st;
+    if (dbias->cols != dy->cols || dbias->rows != 1 || dbias->depth != 1 || dy->depth != 1)
+        return fail(PRAD_ERR_ARG, "bias gradient must be 1 x cols");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(dy, launch_colsum<double>(D(dy), D(dbias), dy->rows, dy->cols, g_ctx.stream),
+             launch_colsum<float>(F(dy), F(dbias), dy->rows, dy->cols, g_ctx.stream));
+    return PRAD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, double min_value) {
+    REQUIRE_INIT();
+    if (n < 0 || (n > 0 && g == nullptr)) return fail(PRAD_ERR_ARG, "bad tensor list");
+    if (n == 0) return PRAD_OK;
+    for (int i = 0; i < n; ++i) {
+        REQUIRE_BUF(g[i]);
+        if (g[i]->dtype != g[0]->dtype) return fail(PRAD_ERR_DTYPE, "buffers of different element types in one call");
+    }
+    std::vector<int64_t> sizes((size_t)n);
+    for (int i = 0; i < n; ++i) sizes[i] = count(g[i]);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (int32_t st = ensure_workspace(clip_workspace_bytes(sizes.data(), n))) return st;
+    if (g[0]->dtype == PRAD_F64) {
+        std::vector<TensorDesc<double>> d((size_t)n);
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<double>{D(g[i]), nullptr, nullptr, nullptr, sizes[i]};
+        HIP_TRY(launch_clip<double>(d.data(), n, g_ctx.workspace, clip_value, min_value, g_ctx.stream), PRAD_ERR_LAUNCH);
+    } else {
+        std::vector<TensorDesc<float>> d((size_t)n);
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<float>{F(g[i]), nullptr, nullptr, nullptr, sizes[i]};
+        HIP_TRY(launch_clip<float>(d.data(), n, g_ctx.workspace, (float)clip_value, (float)min_value, g_ctx.stream), PRAD_ERR_LAUNCH);
+    }
+    return PRAD_OK;
+}
+
+int32_t prad_clip(prad_buf_t g, double clip_value, double min_value) { return prad_clip_multi(&g, 1, clip_value, min_value); }
+
+int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n, double lr,
+                        double beta1, double beta2, double eps, double t) {
+    REQUIRE_INIT();
+    if (n < 0 || (n > 0 && (w == nullptr || m == nullptr || v == nullptr || g == nullptr))) return fail(PRAD_ERR_ARG, "bad tensor list");
+    if (n == 0) return PRAD_OK;
+    for (int i = 0; i < n; ++i) {
+        REQUIRE_BUF(w[i]); REQUIRE_BUF(m[i]); REQUIRE_BUF(v[i]); REQUIRE_BUF(g[i]);
+        for (prad_buf_t o : {w[i], m[i], v[i], g[i]})
+            if (o->dtype != w[0]->dtype) return fail(PRAD_ERR_DTYPE, "buffers of different element types in one call");
+        for (prad_buf_t o : {m[i], v[i], g[i]})
+            if (int32_t st = same_shape(w[i], o, "Adam")) return st;
+    }
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (w[0]->dtype == PRAD_F64) {
+        // 1 / (1 - Math.Pow(beta, AdamIteration)), src/RMAD/AdamOptimizer.cs:204-207
+        const double c1 = 1 / (1 - std::pow(beta1, t)), c2 = 1 / (1 - std::pow(beta2, t));
+        std::vector<TensorDesc<double>> d((size_t)n);
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<double>{D(g[i]), D(w[i]), D(m[i]), D(v[i]), count(w[i])};
+        HIP_TRY(launch_adam<double>(d.data(), n, lr, beta1, beta2, eps, c1, c2, g_ctx.stream), PRAD_ERR_LAUNCH);
+    } else {
+        // PRADLite: every parameter is a float and PradMath.Pow(float, float) is (float)Math.Pow.
+        const float b1 = (float)beta1, b2 = (float)beta2, tf = (float)t;
+        const float c1 = 1 / (1 - (float)std::pow((double)b1, (double)tf));
+        const float c2 = 1 / (1 - (float)std::pow((double)b2, (double)tf));
+        std::vector<TensorDesc<float>> d((size_t)n);
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<float>{F(g[i]), F(w[i]), F(m[i]), F(v[i]), count(w[i])};
+        HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, g_ctx.stream), PRAD_ERR_LAUNCH);
+    }
+    return PRAD_OK;
+}
+
+int32_t prad_adam(prad_buf_t w, prad_buf_t m, prad_buf_t v, prad_buf_t g, double lr, double beta1, double beta2, double eps,
+                  double t) {
+    return prad_adam_multi(&w, &m, &v, &g, 1, lr, beta1, beta2, eps, t);
+}
+
+// ---------------------------------------------------------------------------------------------
+int32_t prad_event_create(void** ev) {
+    REQUIRE_INIT();
+    if (ev == nullptr) return fail(PRAD_ERR_ARG, "ev is NULL");
+    hipEvent_t e;
+    HIP_TRY(hipEventCreate(&e), PRAD_ERR_ALLOC);
+    *ev = e;
+    return PRAD_OK;
+}
+int32_t prad_event_destroy(void* ev) {
+    REQUIRE_INIT();
+    HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(ev)), PRAD_ERR_ARG);
+    return PRAD_OK;
+}
+int32_t prad_event_record(void* ev) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(ev), g_ctx.stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+int32_t prad_event_elapsed_ms(void* start, void* stop, float* ms) {
+    REQUIRE_INIT();
+    if (ms == nullptr) return fail(PRAD_ERR_ARG, "ms is NULL");
+    HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)), PRAD_ERR_LAUNCH);
+    HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+}  // extern "C"
+#pragma GCC visibility pop
