@@ -1,0 +1,363 @@
+"""Parity of the HIP matrix-multiply path with the CPU oracle, through the operation classes and
+the C ABI.  Bar: bit-exact where the arithmetic is exact (small integers), otherwise
+max |x - ref| / max(|ref|, 1e-3 rms) <= 1e-12 (double) / 1e-5 (float); the reduction order of the
+MFMA kernels differs from the reference's k-ascending loop, which is what the tolerance is for."""
+import ctypes
+import json
+import math
+import os
+import threading
+
+import numpy as np
+import pytest
+
+from conftest import assert_parity, dot_bound
+from parallelreverseautodiff_amd import _lib, seeded
+from parallelreverseautodiff_amd.exceptions import ArgumentException, InvalidOperationException
+from parallelreverseautodiff_amd.matrix import DeepMatrix, DeviceBuffer, Matrix
+from parallelreverseautodiff_amd.operations import (BatchGpuMatrixMultiplyOperation, CudaMatrixMultiplyOperation,
+                                                   GpuMatrixMultiplyOperation, MatrixMultiplyOperation, accumulate_gradient)
+
+pytestmark = pytest.mark.gpu
+DTYPES = [np.float64, np.float32]
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+SHAPES = [  # M, K, N: tile-aligned, ragged in every dimension, degenerate vectors, MLP layers
+    (128, 128, 128), (256, 64, 384), (1, 1, 1), (1, 7, 1), (5, 3, 2), (127, 129, 130), (129, 17, 3), (257, 33, 65),
+    (64, 784, 256), (64, 256, 128), (64, 128, 10), (100, 100, 1), (1, 100, 100), (384, 512, 256), (130, 260, 390),
+]
+
+
+def inputs(dtype, M, K, N, seed=seeded.DEFAULT_SEED):
+    return (seeded.uniform(seed, 1, (M, K), -1, 1, dtype), seeded.uniform(seed, 2, (K, N), -1, 1, dtype),
+            seeded.normal(seed, 3, (M, N), 1.0, dtype))
+
+
+def check_against_oracle(oracle, dtype, got, A, B, dC, threads=8, what=""):
+    """Compares (C, dA, dB) with the oracle: relative error bar plus the per-entry rounding bound."""
+    C, dA, dB = got
+    rC = oracle.matmul_fwd(A, B, threads=threads)
+    rdA, rdB = oracle.matmul_bwd(dC, A, B, threads=threads)
+    assert_parity(C, rC, dtype, "C " + what, bound=dot_bound(A, B, dtype))
+    assert_parity(dA, rdA, dtype, "dA " + what, bound=dot_bound(dC, B.T, dtype))
+    assert_parity(dB, rdB, dtype, "dB " + what, bound=dot_bound(A.T, dC, dtype))
+
+
+def run_op(cls, A, B, dC):
+    op = cls.Instantiate(None)
+    mA, mB = Matrix.from_numpy(A), Matrix.from_numpy(B)
+    C = op.Forward(mA, mB)
+    assert op.GetOutput() is C and (C.Rows, C.Cols) == (A.shape[0], B.shape[1])
+    res = op.Backward(Matrix.from_numpy(dC))
+    assert res.HasMultipleInputs and len(res.Results) == 2
+    return C.to_numpy(), res.Item1.to_numpy(), res.Item2.to_numpy()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", SHAPES)
+def test_forward_backward_matches_oracle(gpu, oracle, dtype, shape):
+    M, K, N = shape
+    A, B, dC = inputs(dtype, M, K, N)
+    check_against_oracle(oracle, dtype, run_op(GpuMatrixMultiplyOperation, A, B, dC), A, B, dC, what=str(shape))
+
+
+@pytest.mark.parametrize("cls", [MatrixMultiplyOperation, GpuMatrixMultiplyOperation, CudaMatrixMultiplyOperation])
+def test_all_operation_names_share_the_path(gpu, oracle, cls):
+    A, B, dC = inputs(np.float64, 70, 90, 50)
+    C, dA, dB = run_op(cls, A, B, dC)
+    assert_parity(C, oracle.matmul_fwd(A, B), np.float64)
+    rdA, rdB = oracle.matmul_bwd(dC, A, B)
+    assert_parity(dA, rdA, np.float64)
+    assert_parity(dB, rdB, np.float64)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [512, 1024])
+def test_square_sizes_of_the_benchmark(gpu, oracle, dtype, n):
+    A, B, dC = inputs(dtype, n, n, n)
+    check_against_oracle(oracle, dtype, run_op(GpuMatrixMultiplyOperation, A, B, dC), A, B, dC, threads=16, what=str(n))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_exact_integer_products_are_bit_exact(gpu, oracle, dtype):
+    rng = np.random.default_rng(3)
+    A = rng.integers(-8, 9, (200, 150)).astype(dtype)
+    B = rng.integers(-8, 9, (150, 140)).astype(dtype)
+    dC = rng.integers(-8, 9, (200, 140)).astype(dtype)
+    C, dA, dB = run_op(GpuMatrixMultiplyOperation, A, B, dC)
+    rdA, rdB = oracle.matmul_bwd(dC, A, B)
+    assert np.array_equal(C, oracle.matmul_fwd(A, B))
+    assert np.array_equal(dA, rdA) and np.array_equal(dB, rdB)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_identity_and_ones(gpu, dtype):
+    B = seeded.uniform(9, 1, (200, 130), -1, 1, dtype)
+    C, _, _ = run_op(GpuMatrixMultiplyOperation, np.eye(200, dtype=dtype), B, np.zeros((200, 130), dtype))
+    assert np.array_equal(C, B)
+    C, _, _ = run_op(GpuMatrixMultiplyOperation, np.ones((131, 777), dtype), np.ones((777, 5), dtype), np.zeros((131, 5), dtype))
+    assert np.array_equal(C, np.full((131, 5), 777, dtype))
+
+
+def test_reference_gpu_vs_cpu_contract(gpu, oracle):
+    """test/ParallelReverseAutoDiff.Test/GpuMatrixMultiplyOperationTest.cs:24-53: A 1000x1000 Xavier, B and the
+    upstream gradient 1000x1 Xavier; GPU and CPU results equal after rounding to 10 decimals."""
+    A = seeded.xavier(31, 1, 1000, 1000)
+    B = seeded.xavier(31, 2, 1000, 1)
+    dC = seeded.xavier(31, 3, 1000, 1)
+    C, dA, dB = run_op(GpuMatrixMultiplyOperation, A, B, dC)
+    rC = oracle.matmul_fwd(A, B, threads=8)
+    rdA, rdB = oracle.matmul_bwd(dC, A, B, threads=8)
+    for got, ref in ((C, rC), (dA, rdA), (dB, rdB)):
+        assert np.max(np.abs(got - ref)) < 5e-11
+        assert_parity(got, ref, np.float64)
+
+
+def test_golden_small_cases(gpu):
+    golden = json.load(open(os.path.join(HERE, "golden", "golden.json")))
+    for name in ("tiny_f64", "tiny_f32"):
+        case = golden["matmul"][name]
+        dtype = np.dtype(case["dtype"])
+        A, B, dC = inputs(dtype, case["M"], case["K"], case["N"])
+        C, dA, dB = run_op(GpuMatrixMultiplyOperation, A, B, dC)
+        for got, key in ((C, "C"), (dA, "dA"), (dB, "dB")):
+            want = np.array([float.fromhex(h) for h in case[key]["hex"]], dtype).reshape(case[key]["shape"])
+            assert_parity(got, want, dtype, "%s %s" % (name, key))  # K = 6: no room for reordering error
+
+
+@pytest.mark.parametrize("n", [2048, 4096])
+def test_full_size_properties_fp64(gpu, n):
+    """At sizes the oracle cannot finish in seconds: sampled entries against exactly rounded dot products,
+    and the adjoint identity <dA, A> = <dB, B> = <dC, C>."""
+    A, B, dC = inputs(np.float64, n, n, n)
+    C, dA, dB = run_op(GpuMatrixMultiplyOperation, A, B, dC)
+    rng = np.random.default_rng(n)
+    scale_c = math.sqrt(n / 3.0)
+    for _ in range(48):
+        i, j = int(rng.integers(n)), int(rng.integers(n))
+        assert abs(C[i, j] - math.fsum(A[i, :] * B[:, j])) <= 1e-12 * scale_c
+        assert abs(dA[i, j] - math.fsum(dC[i, :] * B[j, :])) <= 1e-12 * math.sqrt(n)
+        assert abs(dB[i, j] - math.fsum(A[:, i] * dC[:, j])) <= 1e-12 * math.sqrt(n)
+    lhs = float(np.sum(dC * C))
+    assert abs(float(np.sum(dA * A)) - lhs) <= 1e-11 * abs(lhs)
+    assert abs(float(np.sum(dB * B)) - lhs) <= 1e-11 * abs(lhs)
+
+
+def test_full_size_properties_fp32(gpu):
+    n = 2048
+    A, B, dC = inputs(np.float32, n, n, n)
+    C, dA, dB = run_op(GpuMatrixMultiplyOperation, A, B, dC)
+    rng = np.random.default_rng(5)
+    A64, B64, G64 = A.astype(np.float64), B.astype(np.float64), dC.astype(np.float64)
+    for _ in range(48):
+        i, j = int(rng.integers(n)), int(rng.integers(n))
+        assert abs(C[i, j] - math.fsum(A64[i, :] * B64[:, j])) <= 1e-5 * math.sqrt(n / 3.0)
+        assert abs(dA[i, j] - math.fsum(G64[i, :] * B64[j, :])) <= 1e-5 * math.sqrt(n)
+        assert abs(dB[i, j] - math.fsum(A64[:, i] * G64[:, j])) <= 1e-5 * math.sqrt(n)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_accumulating_backward(gpu, oracle, dtype):
+    """dW += A^T.dC written by the product's own epilogue equals OperationBase.AccumulateGradient after Backward."""
+    lib = _lib.load()
+    A, B, dC = inputs(dtype, 96, 200, 72)
+    dest0 = seeded.normal(4, 9, (200, 72), 1.0, dtype)
+    mA, mB, mG, dest = (Matrix.from_numpy(x) for x in (A, B, dC, dest0))
+    from parallelreverseautodiff_amd.exceptions import check
+    check(lib.prad_matmul_bwd(mG.device().handle, mA.device().handle, mB.device().handle, None, dest.device().handle, 0, 1))
+    dest._device_written()
+    _, rdB = oracle.matmul_bwd(dC, A, B)
+    assert_parity(dest.to_numpy(), oracle.accumulate(dest0, rdB), dtype)
+    # the separate accumulate kernel gives the same
+    d2 = Matrix.from_numpy(dest0)
+    accumulate_gradient(d2, Matrix.from_numpy(rdB))
+    assert np.array_equal(d2.to_numpy(), oracle.accumulate(dest0, rdB))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act", ["leakyrelu", "sigmoid", "tanh", "gelu"])
+def test_fused_epilogues(gpu, oracle, dtype, act):
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    code = {"leakyrelu": _lib.ACT_LEAKYRELU, "sigmoid": _lib.ACT_SIGMOID, "tanh": _lib.ACT_TANH, "gelu": _lib.ACT_GELU}[act]
+    alpha = 0.01
+    M, K, N = 70, 150, 130
+    A, B, _ = inputs(dtype, M, K, N)
+    bias = seeded.normal(6, 4, (1, N), 0.5, dtype)
+    mA, mB, mb = Matrix.from_numpy(A), Matrix.from_numpy(B), Matrix.from_numpy(bias)
+    Z, H = DeviceBuffer.alloc(dtype, M, N), DeviceBuffer.alloc(dtype, M, N)
+    check(lib.prad_matmul_fwd_fused(mA.device().handle, mB.device().handle, mb.device().handle, Z.handle, H.handle, code, alpha))
+    rZ = oracle.add_broadcast_fwd(oracle.matmul_fwd(A, B), bias)
+    fwd = {"leakyrelu": lambda z: oracle.leakyrelu_fwd(z, alpha), "sigmoid": oracle.sigmoid_fwd, "tanh": oracle.tanh_fwd,
+           "gelu": oracle.gelu_fwd}[act]
+    gZ = Z.download()
+    assert_parity(gZ, rZ, dtype, "Z")
+    # the activation is checked on the GPU's own pre-activation, so that only the activation is compared
+    assert_parity(H.download(), fwd(gZ), dtype, "H")
+    # backward: dA = (dC . B^T) (.) act'(src), src shaped like A
+    dC = seeded.normal(6, 5, (M, N), 1.0, dtype)
+    src = seeded.normal(6, 6, (M, K), 1.0, dtype)
+    if act in ("sigmoid", "tanh"):
+        src = fwd(src)  # these cache their output
+    mG, mS = Matrix.from_numpy(dC), Matrix.from_numpy(src)
+    dA, dB = DeviceBuffer.alloc(dtype, M, K), DeviceBuffer.alloc(dtype, K, N)
+    check(lib.prad_matmul_bwd_fused(mG.device().handle, mA.device().handle, mB.device().handle, dA.handle, dB.handle, 0, code,
+                                    mS.device().handle, alpha))
+    rdA, rdB = oracle.matmul_bwd(dC, A, B)
+    bwd = {"leakyrelu": lambda s, g: oracle.leakyrelu_bwd(s, g, alpha), "sigmoid": oracle.sigmoid_bwd, "tanh": oracle.tanh_bwd,
+           "gelu": oracle.gelu_bwd}[act]
+    assert_parity(dA.download(), bwd(src, rdA), dtype, "fused dA")
+    assert_parity(dB.download(), rdB, dtype, "dB", bound=dot_bound(A.T, dC, dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batched_products(gpu, oracle, dtype):
+    depth, M, K, N = 5, 40, 70, 30
+    A = seeded.uniform(8, 1, (depth, M, K), -1, 1, dtype)
+    B = seeded.uniform(8, 2, (depth, K, N), -1, 1, dtype)
+    dC = seeded.normal(8, 3, (depth, M, N), 1.0, dtype)
+    op = BatchGpuMatrixMultiplyOperation.Instantiate(None)
+    out = op.Forward(DeepMatrix.from_numpy(A), DeepMatrix.from_numpy(B))
+    res = op.Backward(DeepMatrix.from_numpy(dC))
+    assert out.Depth == depth and len(res) == depth
+    for i in range(depth):
+        assert_parity(out[i].to_numpy(), oracle.matmul_fwd(A[i], B[i]), dtype, bound=dot_bound(A[i], B[i], dtype))
+        rdA, rdB = oracle.matmul_bwd(dC[i], A[i], B[i])
+        assert_parity(res[i].Item1.to_numpy(), rdA, dtype, bound=dot_bound(dC[i], B[i].T, dtype))
+        assert_parity(res[i].Item2.to_numpy(), rdB, dtype, bound=dot_bound(A[i].T, dC[i], dtype))
+    # (DeepMatrix, Matrix) overload: the single matrix is shared by every sample
+    op2 = BatchGpuMatrixMultiplyOperation.Instantiate(None)
+    out2 = op2.Forward(DeepMatrix.from_numpy(A), Matrix.from_numpy(B[0]))
+    for i in range(depth):
+        assert_parity(out2[i].to_numpy(), oracle.matmul_fwd(A[i], B[0]), dtype, bound=dot_bound(A[i], B[0], dtype))
+    op3 = BatchGpuMatrixMultiplyOperation.Instantiate(None)
+    out3 = op3.Forward(Matrix.from_numpy(A[1]), DeepMatrix.from_numpy(B))
+    for i in range(depth):
+        assert_parity(out3[i].to_numpy(), oracle.matmul_fwd(A[1], B[i]), dtype, bound=dot_bound(A[1], B[i], dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_one_shot_host_entry_points(gpu, oracle, dtype):
+    """Jagged rows in, jagged rows out, one call per operation (today's GpuMatrixMultiplyOperation behaviour)."""
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    M, K, N = 37, 53, 29
+    A, B, dC = inputs(dtype, M, K, N)
+    code = _lib.PRAD_F64 if dtype == np.float64 else _lib.PRAD_F32
+
+    def jag(a):
+        rows = [np.array(a[i]) for i in range(a.shape[0])]
+        return rows, (ctypes.c_void_p * len(rows))(*[r.ctypes.data for r in rows])
+
+    ra, pa = jag(A); rb, pb = jag(B); rg, pg = jag(dC)
+    rc, pc = jag(np.zeros((M, N), dtype)); rda, pda = jag(np.zeros((M, K), dtype)); rdb, pdb = jag(np.zeros((K, N), dtype))
+    check(lib.prad_matmul_fwd_host(code, pa, pb, pc, M, K, K, N))
+    check(lib.prad_matmul_bwd_host(code, pg, pa, pb, pda, pdb, M, K, N))
+    assert_parity(np.stack(rc), oracle.matmul_fwd(A, B), dtype, bound=dot_bound(A, B, dtype))
+    rdA, rdB = oracle.matmul_bwd(dC, A, B)
+    assert_parity(np.stack(rda), rdA, dtype, bound=dot_bound(dC, B.T, dtype))
+    assert_parity(np.stack(rdb), rdB, dtype, bound=dot_bound(A.T, dC, dtype))
+    assert lib.prad_matmul_fwd_host(code, pa, pb, pc, M, K, K + 1, N) == _lib.PRAD_ERR_SHAPE
+
+
+def test_error_behaviour(gpu):
+    op = GpuMatrixMultiplyOperation.Instantiate(None)
+    with pytest.raises(InvalidOperationException, match="Input 1 columns do not match Input 2 rows"):
+        op.Forward(Matrix(3, 4), Matrix(5, 2))
+    lib = _lib.load()
+    a, b, c = DeviceBuffer.alloc(np.float64, 3, 4), DeviceBuffer.alloc(np.float64, 5, 2), DeviceBuffer.alloc(np.float64, 3, 2)
+    assert lib.prad_matmul_fwd(a.handle, b.handle, c.handle) == _lib.PRAD_ERR_SHAPE
+    assert b"Input 1 columns do not match Input 2 rows" in lib.prad_last_error()
+    b2, cbad = DeviceBuffer.alloc(np.float64, 4, 2), DeviceBuffer.alloc(np.float64, 2, 2)
+    assert lib.prad_matmul_fwd(a.handle, b2.handle, cbad.handle) == _lib.PRAD_ERR_ARG
+    f = DeviceBuffer.alloc(np.float32, 4, 2)
+    assert lib.prad_matmul_fwd(a.handle, f.handle, c.handle) == _lib.PRAD_ERR_DTYPE
+    assert lib.prad_matmul_fwd(a.handle, None, c.handle) == _lib.PRAD_ERR_BAD_HANDLE
+    assert lib.prad_gemm(1, 1, a.handle, b2.handle, c.handle, 0) == _lib.PRAD_ERR_ARG
+    # jagged upload with a short row
+    m = Matrix([np.zeros(4), np.zeros(3)])
+    with pytest.raises(InvalidOperationException, match="not rectangular"):
+        m.device()
+    rows = [np.zeros(4), np.zeros(4)]
+    ptrs = (ctypes.c_void_p * 2)(*[r.ctypes.data for r in rows])
+    lens = (ctypes.c_int64 * 2)(4, 3)
+    d = DeviceBuffer.alloc(np.float64, 2, 4)
+    assert lib.prad_buf_upload_rows(d.handle, ptrs, lens) == _lib.PRAD_ERR_NOT_RECTANGULAR
+    h = ctypes.c_void_p()
+    assert lib.prad_buf_alloc(7, 2, 2, ctypes.byref(h)) == _lib.PRAD_ERR_DTYPE
+    assert lib.prad_buf_alloc(_lib.PRAD_F64, 0, 2, ctypes.byref(h)) == _lib.PRAD_ERR_ARG
+
+
+def test_residency_protocol(gpu, oracle):
+    """Weights are marshalled once; a host-side in-place edit is seen by the next operation; outputs are
+    downloaded only when the host reads them."""
+    A, B, _ = inputs(np.float64, 20, 30, 10)
+    mA, mB = Matrix.from_numpy(A), Matrix.from_numpy(B)
+    op = GpuMatrixMultiplyOperation.Instantiate(None)
+    C1 = op.Forward(mA, mB)
+    assert mB._dev_valid and not C1._host_valid
+    assert_parity(C1.to_numpy(), oracle.matmul_fwd(A, B), np.float64)
+    assert not C1._host_valid  # to_numpy does not materialise rows
+    mB[0][0] += 1.0  # host mutation through the live row, as Adam does in the reference
+    assert not mB._dev_valid
+    B2 = B.copy(); B2[0, 0] += 1.0
+    C2 = op.Forward(mA, mB)
+    assert_parity(C2.to_numpy(), oracle.matmul_fwd(A, B2), np.float64)
+    row = C2[3]  # jagged host access downloads
+    assert C2._host_valid and np.array_equal(row, C2.to_numpy()[3])
+
+
+def test_store_restore_intermediates(gpu, oracle):
+    op = GpuMatrixMultiplyOperation.Instantiate(None)
+    A1, B1, dC = inputs(np.float64, 12, 9, 7, seed=1)
+    A2, B2, _ = inputs(np.float64, 12, 9, 7, seed=2)
+    op.Forward(Matrix.from_numpy(A1), Matrix.from_numpy(B1)); op.Store("s1")
+    op.Forward(Matrix.from_numpy(A2), Matrix.from_numpy(B2)); op.Store("s2")
+    op.Restore("s1")
+    rdA, rdB = oracle.matmul_bwd(dC, A1, B1)
+    res = op.Backward(Matrix.from_numpy(dC))
+    assert_parity(res.Item1.to_numpy(), rdA, np.float64)
+    assert_parity(res.Item2.to_numpy(), rdB, np.float64)
+
+
+def test_concurrent_backward_from_pool_threads(gpu, oracle):
+    """The reference's visitor runs Backward of different operations on pool threads at the same time
+    (src/RMAD/OperationNeuralNetworkVisitor.cs:303-306)."""
+    cases = []
+    for s in range(6):
+        A, B, dC = inputs(np.float64, 60 + s, 80, 50 - s, seed=100 + s)
+        op = GpuMatrixMultiplyOperation.Instantiate(None)
+        op.Forward(Matrix.from_numpy(A), Matrix.from_numpy(B))
+        cases.append((op, A, B, dC))
+    results = [None] * len(cases)
+    errors = []
+
+    def work(i):
+        try:
+            for _ in range(5):
+                results[i] = cases[i][0].Backward(Matrix.from_numpy(cases[i][3]))
+        except Exception as exc:  # pragma: no cover
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(cases))]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    assert not errors
+    for (op, A, B, dC), res in zip(cases, results):
+        rdA, rdB = oracle.matmul_bwd(dC, A, B)
+        assert_parity(res.Item1.to_numpy(), rdA, np.float64)
+        assert_parity(res.Item2.to_numpy(), rdB, np.float64)
+
+
+def test_raw_pointer_entry_point_with_leading_dimensions(gpu, oracle):
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    M, K, N, lda, ldb, ldc = 50, 40, 30, 47, 33, 36
+    A = seeded.uniform(2, 1, (M, lda), -1, 1); B = seeded.uniform(2, 2, (K, ldb), -1, 1)
+    dA_, dB_, dC_ = DeviceBuffer.alloc(np.float64, M, lda), DeviceBuffer.alloc(np.float64, K, ldb), DeviceBuffer.alloc(np.float64, M, ldc)
+    dA_.upload(A); dB_.upload(B)
+    check(lib.prad_gemm_f64(0, 0, M, N, K, dA_.ptr, lda, dB_.ptr, ldb, dC_.ptr, ldc, 0))
+    got = dC_.download()
+    assert_parity(got[:, :N], oracle.matmul_fwd(np.ascontiguousarray(A[:, :K]), np.ascontiguousarray(B[:, :N])), np.float64)
+    assert not got[:, N:].any()  # padding columns untouched
+    assert lib.prad_gemm_f64(0, 0, M, N, K, dA_.ptr, K - 1, dB_.ptr, ldb, dC_.ptr, ldc, 0) == _lib.PRAD_ERR_ARG

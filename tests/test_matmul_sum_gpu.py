@@ -1,0 +1,70 @@
+"""Parity of MatrixMultiplyAndSum forward/backward with the oracle (reference semantics as written)."""
+import numpy as np
+import pytest
+
+from conftest import TOL, assert_parity
+from parallelreverseautodiff_amd import seeded
+from parallelreverseautodiff_amd.exceptions import InvalidOperationException
+from parallelreverseautodiff_amd.matrix import DeepMatrix, Matrix
+from parallelreverseautodiff_amd.operations import GpuMatrixMultiplyAndSumOperation, MatrixMultiplyAndSumOperation
+
+pytestmark = pytest.mark.gpu
+DTYPES = [np.float64, np.float32]
+
+
+def check_forward(out, A, B, ref, dtype):
+    """out[q] is a sum of M*N products of mixed sign; the error that matters is relative to the magnitude
+    of what is summed (sum_ij |(A.B[q])_ij|), for the oracle's sequential sums as much as for the GPU's."""
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    exact = np.array([[np.sum(A64 @ B64[q]) for q in range(B.shape[0])]])
+    scale = np.array([[np.sum(np.abs(A64 @ B64[q])) for q in range(B.shape[0])]])
+    tol = TOL[np.dtype(dtype)]
+    assert np.all(np.abs(out - exact) <= tol * scale)
+    assert np.all(np.abs(out - ref) <= 2 * tol * scale)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(6, 9, 3), (64, 96, 5), (130, 70, 4), (128, 256, 8)])
+def test_forward_backward(gpu, oracle, dtype, shape):
+    M, K, P = shape
+    A = seeded.normal(81, 1, (M, K), 1.0, dtype)
+    B = seeded.normal(81, 2, (P, K, M), 1.0, dtype)
+    dOut = seeded.normal(81, 3, (1, P), 1.0, dtype)
+    op = GpuMatrixMultiplyAndSumOperation.Instantiate(None)
+    out = op.Forward(Matrix.from_numpy(A), DeepMatrix.from_numpy(B))
+    assert (out.Rows, out.Cols) == (1, P)
+    check_forward(out.to_numpy(), A, B, oracle.matmul_sum_fwd(A, B, threads=8), dtype)
+    res = op.Backward(Matrix.from_numpy(dOut))
+    assert res.HasMultipleInputs and len(res.Results) == 1 + P
+    rdA, rdB = oracle.matmul_sum_bwd(A, B, dOut)
+    assert np.array_equal(res.Item1.to_numpy(), rdA)  # same products, same q-ascending sums: bit exact
+    for q in range(P):
+        assert np.array_equal(res.Results[1 + q].to_numpy(), rdB[q])
+
+
+def test_benchmark_configuration_shape_fp32(gpu, oracle):
+    """A 512x768, 32 slices of 768x512 (N(0, 0.02)), upstream gradient N(0, 1)."""
+    M, K, P = 512, 768, 32
+    A = seeded.normal(82, 1, (M, K), 0.02, np.float32)
+    B = seeded.normal(82, 2, (P, K, M), 0.02, np.float32)
+    dOut = seeded.normal(82, 3, (1, P), 1.0, np.float32)
+    op = GpuMatrixMultiplyAndSumOperation.Instantiate(None)
+    out = op.Forward(Matrix.from_numpy(A), DeepMatrix.from_numpy(B)).to_numpy()
+    check_forward(out, A, B, oracle.matmul_sum_fwd(A, B, threads=16), np.float32)
+    res = op.Backward(Matrix.from_numpy(dOut))
+    rdA, rdB = oracle.matmul_sum_bwd(A, B, dOut)
+    assert np.array_equal(res.Item1.to_numpy(), rdA)
+    for q in (0, 13, 31):
+        assert np.array_equal(res.Results[1 + q].to_numpy(), rdB[q])
+
+
+def test_ones_closed_form_and_cpu_name(gpu):
+    op = MatrixMultiplyAndSumOperation.Instantiate(None)
+    out = op.Forward(Matrix.from_numpy(np.ones((4, 5))), DeepMatrix.from_numpy(np.ones((2, 5, 4)))).to_numpy()
+    assert np.array_equal(out, np.full((1, 2), 80.0))
+
+
+def test_shape_errors(gpu):
+    op = GpuMatrixMultiplyAndSumOperation.Instantiate(None)
+    with pytest.raises(InvalidOperationException, match="compatible for multiplication"):
+        op.Forward(Matrix(4, 5), DeepMatrix(2, 6, 4))

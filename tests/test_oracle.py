@@ -1,0 +1,283 @@
+"""Pins the CPU oracle (oracle/prad_oracle.cpp) without running the reference.
+
+The reference holds no golden vectors for this path (its only numeric test compares its own GPU
+and CPU operations, test/ParallelReverseAutoDiff.Test/GpuMatrixMultiplyOperationTest.cs:24-53),
+so every oracle function is checked against facts the mathematics fixes, chosen so that a dropped
+term, a wrong sign or index, or a transposed operand fails at least one of them:
+
+  matmul_fwd / matmul_bwd   exact integer products vs numpy int64; identity; all-ones; non-square
+                            shapes (a transposed operand changes the shape or the values);
+                            bit-for-bit agreement with an independent numpy statement of the same
+                            k-ascending, unfused accumulation; adjoint identity; exact rational
+                            brute force on a tiny case
+  matmul_fwd_tiled8         bit-for-bit vs numpy blocked-by-8 sums
+  matmul_sum_fwd / bwd      ones closed form; numpy expression of the written formulas
+  activations               known values (LeakyReLU'(0) = alpha, GELU'(0) = 0.5, GELU'(10) = 6.0 which
+                            separates the reference's formula from the analytic derivative 1.0),
+                            central differences for the true derivatives, numpy mirrors
+  clip                      constant / one-element matrices unchanged (NaN path of Math.Min),
+                            tiny magnitudes floored, outlier clamped to min(clip, 1 + |z|)
+  adam                      closed form at t = 1 with zero moments; ReverseAdamUpdate round trip
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from parallelreverseautodiff_amd import seeded
+
+DTYPES = [np.float64, np.float32]
+
+
+def seq_matmul(A, B):
+    """Independent statement of the reference loop: C[i][j] += A[i][k]*B[k][j], k ascending, no FMA."""
+    C = np.zeros((A.shape[0], B.shape[1]), dtype=A.dtype)
+    for k in range(A.shape[1]):
+        C = C + A[:, k:k + 1] * B[k:k + 1, :]  # one rounded multiply, one rounded add, in A's dtype
+    return C
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_matmul_exact_integers(oracle, dtype):
+    rng = np.random.default_rng(7)
+    A = rng.integers(-8, 9, (13, 29)).astype(dtype)
+    B = rng.integers(-8, 9, (29, 7)).astype(dtype)
+    dC = rng.integers(-8, 9, (13, 7)).astype(dtype)
+    Ai, Bi, Gi = A.astype(np.int64), B.astype(np.int64), dC.astype(np.int64)
+    assert np.array_equal(oracle.matmul_fwd(A, B).astype(np.int64), Ai @ Bi)
+    dA, dB = oracle.matmul_bwd(dC, A, B)
+    assert dA.shape == A.shape and dB.shape == B.shape
+    assert np.array_equal(dA.astype(np.int64), Gi @ Bi.T)
+    assert np.array_equal(dB.astype(np.int64), Ai.T @ Gi)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_matmul_identity_and_ones(oracle, dtype):
+    B = seeded.uniform(1, 1, (17, 9), -1, 1, dtype)
+    assert np.array_equal(oracle.matmul_fwd(np.eye(17, dtype=dtype), B), B)
+    ones = oracle.matmul_fwd(np.ones((5, 300), dtype), np.ones((300, 4), dtype))
+    assert np.array_equal(ones, np.full((5, 4), 300, dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(3, 5, 4), (33, 70, 19), (64, 257, 31)])
+def test_matmul_bitwise_vs_numpy_sequential(oracle, dtype, shape):
+    M, K, N = shape
+    A = seeded.uniform(2, 1, (M, K), -1, 1, dtype)
+    B = seeded.uniform(2, 2, (K, N), -1, 1, dtype)
+    dC = seeded.normal(2, 3, (M, N), 1.0, dtype)
+    assert np.array_equal(oracle.matmul_fwd(A, B), seq_matmul(A, B))
+    dA, dB = oracle.matmul_bwd(dC, A, B)
+    # Backward is the same loop on transposed operands (same k order), so it must agree bit for bit.
+    assert np.array_equal(dA, seq_matmul(dC, np.ascontiguousarray(B.T)))
+    assert np.array_equal(dB, seq_matmul(np.ascontiguousarray(A.T), dC))
+    assert np.array_equal(dA, oracle.matmul_fwd(dC, np.ascontiguousarray(B.T)))
+    assert np.array_equal(dB, oracle.matmul_fwd(np.ascontiguousarray(A.T), dC))
+
+
+def test_matmul_threads_do_not_change_results(oracle):
+    A = seeded.uniform(3, 1, (37, 41), -1, 1)
+    B = seeded.uniform(3, 2, (41, 23), -1, 1)
+    assert np.array_equal(oracle.matmul_fwd(A, B, threads=1), oracle.matmul_fwd(A, B, threads=5))
+
+
+def test_matmul_exact_rational_brute_force(oracle):
+    A = seeded.uniform(4, 1, (4, 6), -1, 1)
+    B = seeded.uniform(4, 2, (6, 3), -1, 1)
+    C = oracle.matmul_fwd(A, B)
+    for i in range(4):
+        for j in range(3):
+            exact = sum(Fraction(float(A[i, k])) * Fraction(float(B[k, j])) for k in range(6))
+            scale = sum(abs(float(A[i, k]) * float(B[k, j])) for k in range(6))
+            assert abs(Fraction(float(C[i, j])) - exact) <= Fraction(6 * 2.0 ** -52) * Fraction(scale)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_matmul_adjoint_identity(oracle, dtype):
+    A = seeded.uniform(5, 1, (31, 45), -1, 1, dtype)
+    B = seeded.uniform(5, 2, (45, 27), -1, 1, dtype)
+    dC = seeded.normal(5, 3, (31, 27), 1.0, dtype)
+    C = oracle.matmul_fwd(A, B).astype(np.float64)
+    dA, dB = (x.astype(np.float64) for x in oracle.matmul_bwd(dC, A, B))
+    lhs = float(np.sum(dC.astype(np.float64) * C))
+    tol = 1e-12 if dtype == np.float64 else 1e-4
+    assert abs(float(np.sum(dA * A)) - lhs) <= tol * abs(lhs)
+    assert abs(float(np.sum(dB * B)) - lhs) <= tol * abs(lhs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_matmul_tiled8_order(oracle, dtype):
+    M, K, N = 9, 43, 6
+    A = seeded.uniform(6, 1, (M, K), -1, 1, dtype)
+    B = seeded.uniform(6, 2, (K, N), -1, 1, dtype)
+    total = np.zeros((M, N), dtype)
+    for k0 in range(0, K, 8):
+        s = np.zeros((M, N), dtype)
+        for k in range(k0, min(k0 + 8, K)):
+            s = s + A[:, k:k + 1] * B[k:k + 1, :]
+        total = total + s
+    assert np.array_equal(oracle.matmul_fwd(A, B, tiled8=True), total)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_matmul_sum(oracle, dtype):
+    M, K, P = 6, 9, 3
+    A = seeded.normal(7, 1, (M, K), 1.0, dtype)
+    B = seeded.normal(7, 2, (P, K, M), 1.0, dtype)
+    out = oracle.matmul_sum_fwd(A, B)
+    assert out.shape == (1, P)
+    ref = np.array([[np.sum(A.astype(np.float64) @ B[q].astype(np.float64)) for q in range(P)]])
+    assert np.allclose(out, ref, rtol=1e-12 if dtype == np.float64 else 2e-5, atol=1e-12 if dtype == np.float64 else 1e-5)
+    ones = oracle.matmul_sum_fwd(np.ones((4, 5), dtype), np.ones((2, 5, 4), dtype))
+    assert np.array_equal(ones, np.full((1, 2), 4 * 4 * 5, dtype))
+    dOut = seeded.normal(7, 3, (1, P), 1.0, dtype)
+    dA, dB = oracle.matmul_sum_bwd(A, B, dOut)
+    assert dA.shape == (M, K) and dB.shape == (P, K, M)
+    for q in range(P):
+        assert np.array_equal(dB[q], A.T * dOut[0, q])
+    acc = np.zeros((M, K), dtype)
+    for q in range(P):
+        acc = acc + B[q].T * dOut[0, q]
+    assert np.array_equal(dA, acc)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_activation_known_values(oracle, dtype):
+    a = dtype(0.01)
+    x = np.array([-2.0, 0.0, 3.0], dtype)
+    one = np.ones(3, dtype)
+    assert np.array_equal(oracle.leakyrelu_fwd(x, a), np.array([a * dtype(-2.0), 0.0, 3.0], dtype))
+    assert np.array_equal(oracle.leakyrelu_bwd(x, one, a), np.array([a, a, 1.0], dtype))  # x == 0 takes alpha
+    y = oracle.sigmoid_fwd(np.zeros(1, dtype))
+    assert y[0] == dtype(0.5)
+    assert oracle.sigmoid_bwd(y, np.full(1, 2.0, dtype))[0] == dtype(0.5)  # 2 * 0.5 * 0.5
+    assert oracle.tanh_bwd(np.array([0.5], dtype), np.array([4.0], dtype))[0] == dtype(3.0)
+    g = oracle.gelu_bwd(np.array([0.0, 10.0], dtype), np.ones(2, dtype))
+    assert g[0] == dtype(0.5)
+    assert g[1] == dtype(6.0)  # reference formula: 0.5*10*(0 + 1) + 0.5*2; the analytic derivative is 1.0
+
+
+def test_activation_numpy_mirrors(oracle):
+    x = seeded.normal(8, 1, (257,), 2.0)
+    dy = seeded.normal(8, 2, (257,), 1.0)
+    s = np.sqrt(2 / np.pi)
+    inner = s * (x + 0.044715 * x ** 3)
+    # 1 + tanh cancels for negative x, so last-ulp differences of tanh are amplified
+    assert np.allclose(oracle.gelu_fwd(x), 0.5 * (1 + np.tanh(inner)) * x, rtol=1e-11, atol=1e-15)
+    b = np.tanh(inner)
+    ref = 0.5 * x * ((1 - b * b) ** 2 * (s * (0.044715 * 3 * x * x + 1)) + b) + 0.5 * (1 + b)
+    assert np.allclose(oracle.gelu_bwd(x, dy), dy * ref, rtol=1e-11, atol=1e-15)
+    assert np.allclose(oracle.sigmoid_fwd(x), 1 / (1 + np.exp(-x)), rtol=1e-15)
+    assert np.allclose(oracle.tanh_fwd(x), np.tanh(x), rtol=1e-15)
+    a, b2 = x, dy
+    assert np.array_equal(oracle.hadamard_fwd(a, b2), a * b2)
+    da, db = oracle.hadamard_bwd(a, b2, x)
+    assert np.array_equal(da, x * b2) and np.array_equal(db, x * a)
+    assert np.array_equal(oracle.accumulate(a, b2), a + b2)
+
+
+def test_true_derivatives_by_central_difference(oracle):
+    """Sigmoid, Tanh and LeakyReLU backward are true derivatives (GELU's is not, by design)."""
+    x = seeded.uniform(9, 1, (64,), 0.1, 2.0) * np.where(seeded.u01(9, 2, 64) > 0.5, 1, -1)
+    h = 1e-6
+    one = np.ones_like(x)
+    for fwd, bwd in ((oracle.sigmoid_fwd, lambda: oracle.sigmoid_bwd(oracle.sigmoid_fwd(x), one)),
+                     (oracle.tanh_fwd, lambda: oracle.tanh_bwd(oracle.tanh_fwd(x), one)),
+                     (lambda z: oracle.leakyrelu_fwd(z, 0.01), lambda: oracle.leakyrelu_bwd(x, one, 0.01))):
+        num = (fwd(x + h) - fwd(x - h)) / (2 * h)
+        assert np.allclose(bwd(), num, rtol=1e-6, atol=1e-8)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_clip_edge_cases(oracle, dtype):
+    const = np.full((3, 4), 7.5, dtype)
+    assert np.array_equal(oracle.clip(const, 4.0, 1e-16), const)  # sigma == 0 -> NaN limit -> no comparison fires
+    single = np.array([[123.0]], dtype)
+    assert np.array_equal(oracle.clip(single, 4.0, 1e-16), single)
+    minv = 1e-16 if dtype == np.float64 else 1e-8
+    g = np.array([[1e-20, -1e-20, 0.0, 0.5, -0.5, 0.25]], dtype)
+    out = oracle.clip(g, 4.0, minv)
+    assert out[0, 0] == dtype(minv) and out[0, 1] == dtype(-minv) and out[0, 2] == 0
+    assert out[0, 3] == dtype(0.5) and out[0, 4] == dtype(-0.5)
+
+
+def test_clip_outlier_and_mirror(oracle):
+    g = seeded.normal(10, 1, (40, 25), 1.0)
+    g[3, 7] = 100.0
+    g[9, 1] = -3.9
+    out = oracle.clip(g, 4.0, 1e-16)
+    mean = g.sum() / g.size
+    std = np.sqrt(((g - mean) ** 2).sum() / g.size)
+    z = (g - mean) / std
+    lim = np.minimum(4.0, 1 + np.abs(z))
+    ref = np.clip(g, -lim, lim)
+    assert out[3, 7] == 4.0
+    assert np.allclose(out, ref, rtol=1e-13, atol=0)
+    # entries inside their own limit are untouched bit for bit
+    inside = np.abs(g) <= lim * (1 - 1e-9)
+    assert np.array_equal(out[inside], g[inside])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_adam_closed_form_and_round_trip(oracle, dtype):
+    n = 101
+    w0 = seeded.uniform(11, 1, (n,), -1, 1, dtype)
+    g = seeded.normal(11, 2, (n,), 1.0, dtype)
+    zeros = np.zeros(n, dtype)
+    lr, b1, b2, eps = 1e-3, 0.9, 0.999, 1e-8
+    w1, m1, v1 = oracle.adam(w0, zeros, zeros, g, lr, b1, b2, eps, 1.0)
+    # t = 1, m = v = 0: m_hat = g, v_hat = g^2  =>  w -= lr * g / (|g| + eps)
+    g64 = g.astype(np.float64)
+    rtol = 1e-12 if dtype == np.float64 else 1e-5
+    assert np.allclose(w1, w0.astype(np.float64) - lr * g64 / (np.abs(g64) + eps), rtol=rtol, atol=rtol * 1e-3)
+    # 1 - beta is evaluated in the build's own precision (1 - 0.999f is 1.0000467e-3)
+    omb1, omb2 = float(dtype(1) - dtype(b1)), float(dtype(1) - dtype(b2))
+    assert np.allclose(m1, omb1 * g64, rtol=rtol) and np.allclose(v1, omb2 * g64 * g64, rtol=rtol)
+    # a second step, then ReverseAdamUpdate (src/RMAD/AdamOptimizer.cs:158-193) must return to step one
+    w2, m2, v2 = oracle.adam(w1, m1, v1, g, lr, b1, b2, eps, 2.0)
+    wr, mr, vr = oracle.adam(w2, m2, v2, g, lr, b1, b2, eps, 2.0, reverse=True)
+    rt = 1e-11 if dtype == np.float64 else 2e-4
+    assert np.allclose(wr, w1, rtol=rt, atol=rt) and np.allclose(mr, m1, rtol=rt, atol=rt * 1e-3)
+    assert np.allclose(vr, v1, rtol=1e-8 if dtype == np.float64 else 2e-2, atol=rt * 1e-3)
+
+
+def test_adam_numpy_mirror_bitwise(oracle):
+    n = 77
+    w = seeded.uniform(12, 1, (n,), -1, 1)
+    m = seeded.normal(12, 2, (n,), 0.1)
+    v = np.abs(seeded.normal(12, 3, (n,), 0.01))
+    g = seeded.normal(12, 4, (n,), 1.0)
+    lr, b1, b2, eps, t = 1e-3, 0.9, 0.999, 1e-8, 5.0
+    w1, m1, v1 = oracle.adam(w, m, v, g, lr, b1, b2, eps, t)
+    fm = (b1 * m) + ((1 - b1) * g)
+    sm = (b2 * v) + ((1 - b2) * (g * g))
+    mh = (1 / (1 - np.power(b1, t))) * fm
+    vh = (1 / (1 - np.power(b2, t))) * sm
+    assert np.array_equal(m1, fm) and np.array_equal(v1, sm)
+    assert np.array_equal(w1, w - (lr * mh / (np.sqrt(vh) + eps)))
+
+
+def test_mlp_adjacent_ops(oracle):
+    x = seeded.normal(13, 1, (6, 5), 1.0)
+    b = seeded.normal(13, 2, (1, 5), 1.0)
+    assert np.array_equal(oracle.add_broadcast_fwd(x, b), x + b)
+    assert np.allclose(oracle.add_broadcast_bwd_bias(x), x.sum(axis=0, keepdims=True), rtol=1e-14)
+    p = oracle.softmax_fwd(x)
+    assert np.allclose(p.sum(axis=1), 1.0, rtol=1e-14)
+    e = np.exp(x - x.max(axis=1, keepdims=True))
+    assert np.allclose(p, e / e.sum(axis=1, keepdims=True), rtol=1e-14)
+    dy = seeded.normal(13, 3, (6, 5), 1.0)
+    jac = oracle.softmax_bwd(p, dy)
+    ref = p * (dy - (dy * p).sum(axis=1, keepdims=True))
+    assert np.allclose(jac, ref, rtol=1e-12, atol=1e-15)
+    t = seeded.one_hot_labels(13, 4, 6, 5)
+    assert np.isclose(oracle.cce_fwd(p, t), -np.sum(t * np.log(p + 1e-15)) / 6, rtol=1e-14)
+    assert np.allclose(oracle.cce_bwd(p, t), -(1 / 6) * t / (p + 1e-15), rtol=1e-15)
+
+
+def test_generator_matches_c_copy(oracle):
+    u = seeded.u01(seeded.DEFAULT_SEED, 3, 50)
+    for i in (0, 1, 17, 49):
+        assert u[i] == oracle.u01(seeded.DEFAULT_SEED, 3, i)
+    assert np.array_equal(seeded.uniform(5, 1, (4, 4)), seeded.uniform(5, 1, (16,)).reshape(4, 4))
+    assert 0.0 <= u.min() and u.max() < 1.0
