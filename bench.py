@@ -1,0 +1,210 @@
+"""Benchmark of the matrix-multiply forward+backward path on one MI355X.
+
+One step = MatrixMultiplyOperation forward (C = A.B) plus backward (dA = dC.B^T, dB = A^T.dC) on
+device-resident square double matrices, N = 4096 by default: three launches of the MFMA product
+kernel, 6 N^3 floating-point operations.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--n N] [--dtype f64|f32] [--no-cpu]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3}  # MI355X dense matrix-core peaks
+METRIC = "fp64/fp32 matmul fwd+bwd TFLOP/s (% MFMA peak); MLP train steps/sec"
+
+
+def gpu_leg(n, dtype_name, steps, warmup):
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = int(os.environ.get("LOCAL_RANK", "0"))
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    A = seeded.uniform(seeded.DEFAULT_SEED, 1, (n, n), -1, 1, dtype)
+    B = seeded.uniform(seeded.DEFAULT_SEED, 2, (n, n), -1, 1, dtype)
+    dC = seeded.normal(seeded.DEFAULT_SEED, 3, (n, n), 1.0, dtype)
+    bufs = {k: DeviceBuffer.alloc(dtype, n, n) for k in ("A", "B", "C", "dC", "dA", "dB")}
+    bufs["A"].upload(A); bufs["B"].upload(B); bufs["dC"].upload(dC)
+    h = {k: v.handle for k, v in bufs.items()}
+
+    def step():
+        check(lib.prad_matmul_fwd(h["A"], h["B"], h["C"]))
+        check(lib.prad_matmul_bwd(h["dC"], h["A"], h["B"], h["dA"], h["dB"], 0, 0))
+
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.prad_event_create(ctypes.byref(e0)))
+    check(lib.prad_event_create(ctypes.byref(e1)))
+    for _ in range(warmup):
+        step()
+    check(lib.prad_stream_sync())
+    t0 = time.perf_counter()
+    check(lib.prad_event_record(e0))  # events are recorded on the stream the kernels run on
+    for _ in range(steps):
+        step()
+    check(lib.prad_event_record(e1))
+    check(lib.prad_stream_sync())
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = ctypes.c_float()
+    check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    # spot check of the timed buffers: a few entries against exactly rounded dot products
+    import math
+    C = bufs["C"].download()
+    rng = np.random.default_rng(0)
+    worst = 0.0
+    for _ in range(8):
+        i, j = int(rng.integers(n)), int(rng.integers(n))
+        exact = math.fsum(A[i, :].astype(np.float64) * B[:, j].astype(np.float64))
+        worst = max(worst, abs(float(C[i, j]) - exact) / math.sqrt(n / 3.0))
+    tol = 1e-12 if dtype_name == "f64" else 1e-5
+    if not worst <= tol:
+        raise SystemExit("benchmark output failed its spot check: %.3e" % worst)
+    return float(ms.value), wall_ms, worst
+
+
+def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
+    """Times each bandwidth kernel on n_elems elements (default 64 Mi: beyond the 256 MB last-level cache).
+    Algorithmic bytes per element, s = element size: activation backward 3s (read src, dy; write dx),
+    Hadamard backward 5s, accumulate 3s, copy 2s, clip 3s (read for statistics; read + write), Adam 7s."""
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = 0
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    es = np.dtype(dtype).itemsize
+    rows, cols = n_elems // 4096, 4096
+    n = rows * cols
+    host = [seeded.normal(7, t, (rows, cols), 1.0, dtype) for t in range(3)]
+    host[2] = np.abs(host[2])
+    b = [DeviceBuffer.alloc(dtype, rows, cols) for _ in range(5)]
+    for i in range(3):
+        b[i].upload(host[i])
+    h = [x.handle for x in b]
+    cases = {
+        "copy": (2, lambda: lib.prad_buf_copy(h[3], h[0])),
+        "leakyrelu_bwd": (3, lambda: lib.prad_act_bwd(_lib.ACT_LEAKYRELU, h[0], h[1], h[3], 0.01)),
+        "sigmoid_bwd": (3, lambda: lib.prad_act_bwd(_lib.ACT_SIGMOID, h[0], h[1], h[3], 0.0)),
+        "tanh_bwd": (3, lambda: lib.prad_act_bwd(_lib.ACT_TANH, h[0], h[1], h[3], 0.0)),
+        "gelu_bwd": (3, lambda: lib.prad_act_bwd(_lib.ACT_GELU, h[0], h[1], h[3], 0.0)),
+        "hadamard_bwd": (5, lambda: lib.prad_hadamard_bwd(h[0], h[1], h[2], h[3], h[4])),
+        "accumulate": (3, lambda: lib.prad_accumulate(h[3], h[1])),
+        "clip": (3, lambda: lib.prad_clip(h[1], 4.0, 1e-16 if dtype_name == "f64" else 1e-8)),
+        "adam": (7, lambda: lib.prad_adam(h[0], h[3], h[2], h[1], 1e-3, 0.9, 0.999, 1e-8, 1.0)),
+    }
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.prad_event_create(ctypes.byref(e0)))
+    check(lib.prad_event_create(ctypes.byref(e1)))
+    out = {}
+    for name, (factor, fn) in cases.items():
+        if only and name not in only:
+            continue
+        for _ in range(warmup):
+            check(fn())
+        check(lib.prad_stream_sync())
+        check(lib.prad_event_record(e0))
+        for _ in range(steps):
+            check(fn())
+        check(lib.prad_event_record(e1))
+        ms = ctypes.c_float()
+        check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        per = ms.value / steps
+        gbs = factor * es * n / (per * 1e-3) / 1e9
+        out[name] = {"ms": per, "GB/s": gbs, "frac_of_8TBps": gbs / 8000.0, "bytes_per_element": factor * es}
+    return out, n
+
+
+def cpu_leg(budget_s=40.0):
+    """Times the CPU restatement of the reference's Parallel.For path (jagged rows, row-parallel scalar
+    i-j-k loops) on this host: a bounded sample of the same workload at a smaller N."""
+    from oracle import oracle
+    threads = min(16, oracle.hardware_threads() or 1)
+    n = 1024
+    secs = oracle.time_matmul_fwdbwd(n, np.float64, threads=threads, iters=1)
+    for bigger in (2048, 4096):  # each doubling costs 8x the work and misses cache more often
+        if secs * 9.0 > budget_s:
+            break
+        n = bigger
+        secs = oracle.time_matmul_fwdbwd(n, np.float64, threads=threads, iters=1)
+    flops = 6.0 * n ** 3
+    return {"value": flops / secs / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "fp64 MatrixMultiplyOperation forward+backward at N=%d (%.1f GFLOP, 1 pass, %.2f s), "
+                      "C++ restatement of the reference's Parallel.For loops on jagged rows, -O2, no FMA" % (n, flops / 1e9, secs)}
+
+
+def load_traffic(n, dtype_name):
+    """HBM bytes per launch measured with rocprofv3 --pmc (recorded under profiles/), or None."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get("gemm_%s_n%d" % (dtype_name, n), {}).get("bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--n", type=int, default=4096)
+    ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--mode", choices=["gemm", "bandwidth"], default="gemm",
+                    help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels")
+    ap.add_argument("--elems", type=int, default=64 * 1024 * 1024, help="elements per tensor in bandwidth mode")
+    ap.add_argument("--only", default="", help="bandwidth mode: comma-separated kernel names")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py measures one GPU: this path has no multi-GPU part (--gpus 1 only)")
+    if args.mode == "bandwidth":
+        res, n = bandwidth_leg(args.elems, args.dtype, args.steps, args.warmup, [x for x in args.only.split(",") if x])
+        best = max(res.values(), key=lambda r: r["GB/s"])
+        print(json.dumps({"metric": "fused gradient kernels GB/s (% of 8 TB/s HBM)", "unit": "GB/s", "value": best["GB/s"],
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
+                          "higher_is_better": True, "config": {"workload": "elementwise/clip/Adam kernels on %d elements" % n},
+                          "kernels": res}))
+        return
+
+    ms, wall_ms, spot = gpu_leg(args.n, args.dtype, args.steps, args.warmup)
+    flops_per_step = 6.0 * args.n ** 3
+    ms_per_step = ms / args.steps
+    tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[args.dtype]
+    # dominant kernel: the MFMA product kernel, three launches per step of 2 N^3 flop each
+    launch_ms = ms / (3 * args.steps)
+    achieved = 2.0 * args.n ** 3 / (launch_ms * 1e-3) / 1e12
+    line = {
+        "metric": METRIC, "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[1]: single MatrixMultiplyOperation forward+backward, %s, square M=N=K=%d, "
+                               "A,B~U[-1,1], dC~N(0,1), seed %d, device-resident" % (args.dtype, args.n, 20240611),
+                   "flop_per_step": flops_per_step, "launches_per_step": 3},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
+                     "traffic": load_traffic(args.n, args.dtype), "kernel": "prad::gemm_kernel<%s> (NN, NT, TN instantiations)" %
+                     ("double" if args.dtype == "f64" else "float"), "launch_ms": launch_ms},
+        "wall_ms_per_step": wall_ms / args.steps, "spot_check_error": spot,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_leg()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

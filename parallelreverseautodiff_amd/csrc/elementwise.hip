@@ -131,6 +131,9 @@ template <typename T> struct HadBwd {  // in: a, b, dy ; out: da, db
         out[1] = in[2] * in[0];
     }
 };
+template <typename T> struct Copy {
+    __device__ __forceinline__ void apply(const T (&in)[1], T (&out)[1]) const { out[0] = in[0]; }
+};
 template <typename T> struct Accum {  // in: dest, grad ; out: dest
     __device__ __forceinline__ void apply(const T (&in)[2], T (&out)[1]) const { out[0] = in[0] + in[1]; }
 };
@@ -171,6 +174,12 @@ template <typename T>
 hipError_t launch_accumulate(T* dest, const T* grad, int64_t n, hipStream_t s) {
     StreamPtrs<T, 2, 1> p{{dest, grad}, {dest}};
     return launch_stream(p, n, Accum<T>{}, s);
+}
+
+template <typename T>
+hipError_t launch_copy(T* dst, const T* src, int64_t n, hipStream_t s) {
+    StreamPtrs<T, 1, 1> p{{src}, {dst}};
+    return launch_stream(p, n, Copy<T>{}, s);
 }
 
 // ---- zero fill (a kernel, so it can be recorded into a captured graph) --------------------
@@ -229,6 +238,7 @@ hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, hipStre
     template hipError_t launch_hadamard_fwd<T>(const T*, const T*, T*, int64_t, hipStream_t);                      \
     template hipError_t launch_hadamard_bwd<T>(const T*, const T*, const T*, T*, T*, int64_t, hipStream_t);        \
     template hipError_t launch_accumulate<T>(T*, const T*, int64_t, hipStream_t);                                  \
+    template hipError_t launch_copy<T>(T*, const T*, int64_t, hipStream_t);                                        \
     template hipError_t launch_add_broadcast_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);        \
     template hipError_t launch_colsum<T>(const T*, T*, int64_t, int64_t, hipStream_t);                             \
     template hipError_t launch_fill_zero<T>(T*, int64_t, hipStream_t);

@@ -402,8 +402,14 @@ int32_t prad_buf_copy(prad_buf_t dst, prad_buf_t src) {
     if (int32_t st = same_dtype({dst, src})) return st;
     if (int32_t st = same_shape(dst, src, "copy")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    HIP_TRY(hipMemcpyAsync(dst->ptr, src->ptr, (size_t)count(src) * elem_size(src->dtype), hipMemcpyDeviceToDevice, g_ctx.stream),
-            PRAD_ERR_LAUNCH);
+    // A kernel rather than hipMemcpyAsync: it can be recorded into a captured graph and shows up in
+    // kernel traces as a plain copy of known size.
+    if (src->dtype == PRAD_F64)
+        HIP_TRY(launch_copy<double>(static_cast<double*>(dst->ptr), static_cast<const double*>(src->ptr), count(src), g_ctx.stream),
+                PRAD_ERR_LAUNCH);
+    else
+        HIP_TRY(launch_copy<float>(static_cast<float*>(dst->ptr), static_cast<const float*>(src->ptr), count(src), g_ctx.stream),
+                PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
 
