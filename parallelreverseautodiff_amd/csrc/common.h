@@ -33,10 +33,38 @@ __device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
 __device__ __forceinline__ float dev_tanh(float x) { return (float)tanh((double)x); }
 __device__ __forceinline__ double dev_exp(double x) { return exp(x); }
 __device__ __forceinline__ float dev_exp(float x) { return (float)exp((double)x); }
-// pow(x, 3): correctly rounded cube.  In double the three-factor product can differ from it
-// in the last place; the float version cubes in double and rounds once, like (float)Math.Pow.
-__device__ __forceinline__ double dev_cube(double x) { return x * x * x; }
-__device__ __forceinline__ float dev_cube(float x) { double d = (double)x; return (float)(d * d * d); }
+// tanh for the GELU kernels, which would otherwise be bound by the math library's tanh instead of
+// by memory: tanh|u| = (1 - t) / (1 + t) with t = exp(-2|u|); below 0.01 the difference 1 - t cancels,
+// so a Taylor polynomial (next term ~1e-22 relative) takes over.  Relative error ~1e-15 in double.
+__device__ __forceinline__ double gelu_tanh(double u) {
+    const double a = fabs(u);
+    double r;
+    if (a < 0.01) {
+        const double a2 = a * a;
+        r = a * (1.0 + a2 * (-1.0 / 3.0 + a2 * (2.0 / 15.0 + a2 * (-17.0 / 315.0 + a2 * (62.0 / 2835.0)))));
+    } else {
+        const double t = exp(-2.0 * a);
+        r = (1.0 - t) / (1.0 + t);
+    }
+    return copysign(r, u);
+}
+// PRADLite rounds a double tanh to float; evaluating in float is within 2e-7 of it, far inside the
+// 1e-5 parity bar, and keeps the kernel memory-bound.
+__device__ __forceinline__ float gelu_tanh(float u) {
+    const float a = fabsf(u);
+    float r;
+    if (a < 0.01f) {
+        const float a2 = a * a;
+        r = a * (1.0f + a2 * (-1.0f / 3.0f + a2 * (2.0f / 15.0f)));
+    } else {
+        const float t = __expf(-2.0f * a);
+        r = (1.0f - t) / (1.0f + t);
+    }
+    return copysignf(r, u);
+}
+// x^3 (the reference's pow(x, 3) is correctly rounded; the product is within one ulp of it).
+__device__ __forceinline__ float gelu_cube(float x) { return x * x * x; }
+__device__ __forceinline__ double gelu_cube(double x) { return x * x * x; }
 
 template <typename T>
 __device__ __forceinline__ T act_forward(int act, T x, T alpha) {
@@ -45,7 +73,7 @@ __device__ __forceinline__ T act_forward(int act, T x, T alpha) {
         case ACT_SIGMOID: return (T)1 / ((T)1 + dev_exp(-x));
         case ACT_TANH: return dev_tanh(x);
         case ACT_GELU: {
-            T a = (T)0.5 * ((T)1 + dev_tanh(GeluConst<T>::s() * (x + (GeluConst<T>::c0() * dev_cube(x)))));
+            T a = (T)0.5 * ((T)1 + gelu_tanh(GeluConst<T>::s() * (x + (GeluConst<T>::c0() * gelu_cube(x)))));
             return a * x;
         }
         default: return x;
@@ -60,7 +88,7 @@ __device__ __forceinline__ T act_derivative(int act, T s, T alpha) {
         case ACT_SIGMOID: return s * ((T)1 - s);
         case ACT_TANH: return (T)1 - s * s;
         case ACT_GELU: {
-            T b = dev_tanh(GeluConst<T>::s() * (s + (GeluConst<T>::c0() * dev_cube(s))));
+            T b = gelu_tanh(GeluConst<T>::s() * (s + (GeluConst<T>::c0() * gelu_cube(s))));
             T omb = (T)1 - b * b;
             T c = omb * omb;
             T d = GeluConst<T>::s() * ((GeluConst<T>::c0() * (T)3 * (s * s)) + (T)1);

@@ -8,21 +8,27 @@
 // transposed copies it is fed with (:148, :154, :210-248): a transposed operand is read in its
 // stored orientation and only its placement in LDS differs.
 //
-// Shape of one workgroup: 256 threads = 4 wavefronts (2 x 2), output tile 128 x 128, each
-// wavefront owns 64 x 64 = 4 x 4 MFMA tiles of 16 x 16, so every A/B fragment read from LDS feeds
-// four MFMAs.  The reduction dimension is cut into slabs of BK (16 doubles / 32 floats = 128
-// bytes per row); slabs are double-buffered in LDS and the next slab's global loads are issued
-// before the current slab's MFMAs.
+// Shape of one workgroup: 256 threads = 4 wavefronts (2 x 2).  The output tile is 32*WTM x 32*WTN:
+// each wavefront owns WTM x WTN MFMA tiles of 16 x 16, so an A fragment read from LDS feeds WTN MFMAs
+// and a B fragment WTM.  128 x 128 (WTM = WTN = 4) is the steady-state shape; the smaller tiles exist
+// so that products with few 128 x 128 tiles still put work on all 256 compute units.  The reduction
+// dimension is cut into slabs of BK (16 doubles / 32 floats = 128 bytes per row); slabs are
+// double-buffered in LDS and the next slab's global loads are issued before the current slab's MFMAs.
 //
-// LDS placement of an operand slab (MN = its 128 rows/columns of the output tile):
+// LDS placement of an operand slab (MN = its rows/columns of the output tile):
 //   stored with the reduction index contiguous ("KC": A of the forward, both operands of dA)
-//       S[mn][k], row pitch BK + pad chosen so that the 16 B of two neighbouring k of 16
-//       consecutive mn fall into distinct 16 B bank groups;
+//       S[mn][k], row pitch BK + pad (144 bytes) chosen so that the 16 bytes of two neighbouring k
+//       of 16 consecutive mn fall into distinct 16-byte bank groups (an XOR-swizzled unpadded
+//       layout was measured too: same speed in double, 6 % slower in float because the compiler
+//       can no longer merge neighbouring LDS reads);
 //   stored with mn contiguous ("MC": B of the forward, both operands of dB)
-//       S[k][mn], row pitch 128 + 16.
+//       S[k][mn], row pitch MN + 16 elements.
 // An MFMA lane (mn = lane % 16, k = lane / 16) reads one element from either placement without
 // bank conflicts, so no transposed copy is ever written.
 #include "common.h"
+
+#include <cstdlib>
+#include <cstring>
 
 namespace prad {
 
@@ -30,9 +36,6 @@ typedef double d4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef double d2_t __attribute__((ext_vector_type(2)));
 
-constexpr int BM = 128;
-constexpr int BN = 128;
-constexpr int LDM = 144;  // pitch of an MC slab row (128 + 16)
 constexpr int GEMM_THREADS = 256;
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 8;
@@ -62,11 +65,17 @@ template <> struct Mfma<float> {
     static __device__ __forceinline__ int row(int r, int g) { return 4 * g + r; }
 };
 
-// Loads this thread's share (4 vectors) of one operand slab from global memory.
+// Offset (in elements) of element (mn, k) of a KC slab.
+template <typename T>
+__device__ __forceinline__ int kc_offset(int mn, int k) {
+    return mn * Mfma<T>::LDK + k;
+}
+
+// Loads this thread's share (NV vectors) of one operand slab (MN = 32*NV rows/columns x BK) from global memory.
 //   KC: the operand is stored [mn][k]: 8 threads cover the 128 bytes of one row.
-//   MC: the operand is stored [k][mn]: 128 / VEC threads cover one k row.
-template <typename T, bool KC, bool EDGE>
-__device__ __forceinline__ void load_slab(typename Mfma<T>::Vec (&r)[4], const T* __restrict__ base, int64_t ld, int64_t mn0,
+//   MC: the operand is stored [k][mn]: MN / VEC threads cover one k row.
+template <typename T, int NV, bool KC, bool EDGE>
+__device__ __forceinline__ void load_slab(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ base, int64_t ld, int64_t mn0,
                                           int64_t mn_end, int64_t k0, int64_t k_end, int tid) {
     typedef typename Mfma<T>::Vec Vec;
     constexpr int VEC = Mfma<T>::VEC;
@@ -74,7 +83,7 @@ __device__ __forceinline__ void load_slab(typename Mfma<T>::Vec (&r)[4], const T
         const int kv = tid & 7;
         const int rowb = tid >> 3;
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
+        for (int p = 0; p < NV; ++p) {
             const int64_t mn = mn0 + rowb + 32 * p;
             const int64_t k = k0 + kv * VEC;
             const T* g = base + mn * ld + k;
@@ -86,12 +95,12 @@ __device__ __forceinline__ void load_slab(typename Mfma<T>::Vec (&r)[4], const T
             }
         }
     } else {
-        constexpr int CV = 128 / VEC;                 // vectors per k row
+        constexpr int CV = 32 * NV / VEC;             // vectors per k row
         constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
         const int cv = tid % CV;
         const int krow = tid / CV;
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
+        for (int p = 0; p < NV; ++p) {
             const int64_t k = k0 + krow + ROWS_PER_PASS * p;
             const int64_t mn = mn0 + cv * VEC;
             const T* g = base + k * ld + mn;
@@ -105,31 +114,58 @@ __device__ __forceinline__ void load_slab(typename Mfma<T>::Vec (&r)[4], const T
     }
 }
 
-template <typename T, bool KC>
-__device__ __forceinline__ void store_slab(T* __restrict__ s, const typename Mfma<T>::Vec (&r)[4], int tid) {
+template <typename T, int NV, bool KC>
+__device__ __forceinline__ void store_slab(T* __restrict__ s, const typename Mfma<T>::Vec (&r)[NV], int tid) {
     typedef typename Mfma<T>::Vec Vec;
     constexpr int VEC = Mfma<T>::VEC;
-    constexpr int LDK = Mfma<T>::LDK;
     if (KC) {
         const int kv = tid & 7;
         const int rowb = tid >> 3;
 #pragma unroll
-        for (int p = 0; p < 4; ++p) *reinterpret_cast<Vec*>(s + (rowb + 32 * p) * LDK + kv * VEC) = r[p];
+        for (int p = 0; p < NV; ++p) *reinterpret_cast<Vec*>(s + kc_offset<T>(rowb + 32 * p, kv * VEC)) = r[p];
     } else {
-        constexpr int CV = 128 / VEC;
+        constexpr int LDM = 32 * NV + 16;  // pitch of an MC slab row
+        constexpr int CV = 32 * NV / VEC;
         constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
         const int cv = tid % CV;
         const int krow = tid / CV;
 #pragma unroll
-        for (int p = 0; p < 4; ++p) *reinterpret_cast<Vec*>(s + (krow + ROWS_PER_PASS * p) * LDM + cv * VEC) = r[p];
+        for (int p = 0; p < NV; ++p) *reinterpret_cast<Vec*>(s + (krow + ROWS_PER_PASS * p) * LDM + cv * VEC) = r[p];
     }
 }
 
-// Element (mn, k) of a slab in LDS.
-template <typename T, bool KC>
-__device__ __forceinline__ T slab_at(const T* __restrict__ s, int mn, int k) {
-    return KC ? s[mn * Mfma<T>::LDK + k] : s[k * LDM + mn];
+// Unguarded loads of one slab, addressed as a wavefront-uniform base (scalar registers, advanced slab
+// by slab) plus a per-thread 32-bit element offset that never changes: the loads take the
+// scalar-base form and the two prefetch register sets share one set of offsets.
+template <typename T, int NV, bool KC>
+__device__ __forceinline__ void slab_offsets(unsigned (&off)[NV], int64_t ld, int tid) {
+    constexpr int VEC = Mfma<T>::VEC;
+    if (KC) {
+#pragma unroll
+        for (int p = 0; p < NV; ++p) off[p] = (unsigned)(((tid >> 3) + 32 * p) * ld + (tid & 7) * VEC);
+    } else {
+        constexpr int CV = 32 * NV / VEC;
+        constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
+#pragma unroll
+        for (int p = 0; p < NV; ++p) off[p] = (unsigned)((tid / CV + ROWS_PER_PASS * p) * ld + (tid % CV) * VEC);
+    }
 }
+template <typename T, int NV>
+__device__ __forceinline__ void load_slab_fast(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ ubase,
+                                               const unsigned (&off)[NV]) {
+    typedef typename Mfma<T>::Vec Vec;
+#pragma unroll
+    for (int p = 0; p < NV; ++p) r[p] = *reinterpret_cast<const Vec*>(ubase + off[p]);
+}
+
+// Element (mn, k) of a slab in LDS.
+template <typename T, int NV, bool KC>
+__device__ __forceinline__ T slab_at(const T* __restrict__ s, int mn, int k) {
+    return KC ? s[kc_offset<T>(mn, k)] : s[k * (32 * NV + 16) + mn];
+}
+
+template <typename T, int NV, bool KC>
+constexpr int slab_elems() { return KC ? 32 * NV * Mfma<T>::LDK : Mfma<T>::BK * (32 * NV + 16); }
 
 // Maps the linear workgroup id to an output tile.  Hardware deals consecutive workgroup ids
 // round-robin to the 8 XCDs, each with its own L2: ids are first regrouped so that one XCD gets a
@@ -149,16 +185,20 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tilesM, int tiles
     tn = in_group / gsz;
 }
 
-template <typename T, bool A_KC, bool B_KC, bool EDGE, bool EPI>
-__global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_kernel(const GemmArgs<T> p, const int tilesM, const int tilesN) {
+constexpr int min_blocks(int wtm, int wtn) { return wtm * wtn >= 16 ? 2 : wtm * wtn >= 8 ? 3 : 4; }
+
+template <typename T, int WTM, int WTN, bool A_KC, bool B_KC, bool EDGE, bool EPI>
+__global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WTM, WTN)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
+                                                                                  const int tilesN) {
     typedef Mfma<T> MF;
     typedef typename MF::Acc Acc;
     typedef typename MF::Vec Vec;
     constexpr int BK = MF::BK;
-    constexpr int SLAB = BM * MF::LDK;  // elements of one operand slab; equals BK * LDM
-    static_assert(BM * MF::LDK == BK * LDM, "both slab placements must have the same size");
+    constexpr int BM = 32 * WTM, BN = 32 * WTN;  // output tile
+    constexpr int WSM = 16 * WTM, WSN = 16 * WTN;  // one wavefront's share
+    constexpr int SA = slab_elems<T, WTM, A_KC>(), SB = slab_elems<T, WTN, B_KC>();
 
-    __shared__ __attribute__((aligned(16))) T smem[2][2][SLAB];  // [stage][operand]
+    __shared__ __attribute__((aligned(16))) T smem[2][SA + SB];  // [stage][A slab | B slab]
 
     int tm, tn;
     tile_of_workgroup(blockIdx.x, tilesM, tilesN, tm, tn);
@@ -172,52 +212,103 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_kernel(const GemmArgs<T>
     const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 15, g = lane >> 4;
 
-    Acc acc[4][4];
+    Acc acc[WTM][WTN];
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
+    for (int x = 0; x < WTM; ++x)
 #pragma unroll
-        for (int y = 0; y < 4; ++y)
+        for (int y = 0; y < WTN; ++y)
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[x][y][r] = (T)0;
 
-    Vec ra[4], rb[4];
     const int64_t K = p.K;
     const int ntiles = (int)((K + BK - 1) / BK);
 
-    load_slab<T, A_KC, EDGE>(ra, A, p.lda, row0, p.M, 0, K, tid);
-    load_slab<T, B_KC, EDGE>(rb, B, p.ldb, col0, p.N, 0, K, tid);
-    store_slab<T, A_KC>(smem[0][0], ra, tid);
-    store_slab<T, B_KC>(smem[0][1], rb, tid);
-    __syncthreads();
-
-    int cur = 0;
-    for (int kt = 0; kt < ntiles; ++kt) {
-        const bool more = kt + 1 < ntiles;
-        if (more) {
-            load_slab<T, A_KC, EDGE>(ra, A, p.lda, row0, p.M, (int64_t)(kt + 1) * BK, K, tid);
-            load_slab<T, B_KC, EDGE>(rb, B, p.ldb, col0, p.N, (int64_t)(kt + 1) * BK, K, tid);
-        }
-        const T* __restrict__ sA = smem[cur][0];
-        const T* __restrict__ sB = smem[cur][1];
+    // One slab of MFMAs from the LDS stage at `st`.
+    auto compute = [&](const T* __restrict__ st) {
+        const T* __restrict__ sA = st;
+        const T* __restrict__ sB = st + SA;
 #pragma unroll
         for (int s = 0; s < BK / 4; ++s) {
             const int k = 4 * s + g;
-            T a[4], b[4];
+            T a[WTM], b[WTN];
 #pragma unroll
-            for (int x = 0; x < 4; ++x) a[x] = slab_at<T, A_KC>(sA, wm * 64 + x * 16 + li, k);
+            for (int x = 0; x < WTM; ++x) a[x] = slab_at<T, WTM, A_KC>(sA, wm * WSM + x * 16 + li, k);
 #pragma unroll
-            for (int y = 0; y < 4; ++y) b[y] = slab_at<T, B_KC>(sB, wn * 64 + y * 16 + li, k);
+            for (int y = 0; y < WTN; ++y) b[y] = slab_at<T, WTN, B_KC>(sB, wn * WSN + y * 16 + li, k);
 #pragma unroll
-            for (int x = 0; x < 4; ++x)
+            for (int x = 0; x < WTM; ++x)
 #pragma unroll
-                for (int y = 0; y < 4; ++y) acc[x][y] = MF::run(a[x], b[y], acc[x][y]);
+                for (int y = 0; y < WTN; ++y) acc[x][y] = MF::run(a[x], b[y], acc[x][y]);
         }
-        if (more) {
-            store_slab<T, A_KC>(smem[cur ^ 1][0], ra, tid);
-            store_slab<T, B_KC>(smem[cur ^ 1][1], rb, tid);
+    };
+
+    if (!EDGE) {
+        // Two register sets: while slab t is multiplied out of LDS, slab t+1 waits in one set and the loads
+        // of slab t+2 are issued into the other, so a global load has two slabs of MFMAs to arrive
+        // (measured +5 % at N = 4096 over a prefetch distance of one slab).  The loop is unrolled by two so
+        // that the sets are named statically.
+        Vec ra0[WTM], rb0[WTN], ra1[WTM], rb1[WTN];
+        unsigned offa[WTM], offb[WTN];
+        slab_offsets<T, WTM, A_KC>(offa, p.lda, tid);
+        slab_offsets<T, WTN, B_KC>(offb, p.ldb, tid);
+        // uniform bases of slab 0 and their per-slab strides
+        const T* __restrict__ ua = A + (A_KC ? row0 * p.lda : row0);
+        const T* __restrict__ ub = B + (B_KC ? col0 * p.ldb : col0);
+        const int64_t stepa = A_KC ? (int64_t)BK : (int64_t)BK * p.lda;
+        const int64_t stepb = B_KC ? (int64_t)BK : (int64_t)BK * p.ldb;
+        load_slab_fast<T, WTM>(ra0, ua, offa);
+        load_slab_fast<T, WTN>(rb0, ub, offb);
+        if (ntiles > 1) {
+            load_slab_fast<T, WTM>(ra1, ua + stepa, offa);
+            load_slab_fast<T, WTN>(rb1, ub + stepb, offb);
         }
+        store_slab<T, WTM, A_KC>(smem[0], ra0, tid);
+        store_slab<T, WTN, B_KC>(smem[0] + SA, rb0, tid);
         __syncthreads();
-        cur ^= 1;
+        for (int kt = 0; kt + 1 < ntiles; kt += 2) {
+            // LDS stage 0 holds slab kt, set 1 holds slab kt+1 (in flight), set 0 is free.
+            if (kt + 2 < ntiles) {
+                load_slab_fast<T, WTM>(ra0, ua + (kt + 2) * stepa, offa);
+                load_slab_fast<T, WTN>(rb0, ub + (kt + 2) * stepb, offb);
+            }
+            compute(smem[0]);
+            store_slab<T, WTM, A_KC>(smem[1], ra1, tid);
+            store_slab<T, WTN, B_KC>(smem[1] + SA, rb1, tid);
+            __syncthreads();
+            if (kt + 3 < ntiles) {
+                load_slab_fast<T, WTM>(ra1, ua + (kt + 3) * stepa, offa);
+                load_slab_fast<T, WTN>(rb1, ub + (kt + 3) * stepb, offb);
+            }
+            compute(smem[1]);
+            if (kt + 2 < ntiles) {
+                store_slab<T, WTM, A_KC>(smem[0], ra0, tid);
+                store_slab<T, WTN, B_KC>(smem[0] + SA, rb0, tid);
+            }
+            __syncthreads();
+        }
+        if (ntiles & 1) compute(smem[0]);  // an odd last slab was staged into stage 0
+    } else {
+        Vec ra[WTM], rb[WTN];
+        load_slab<T, WTM, A_KC, true>(ra, A, p.lda, row0, p.M, 0, K, tid);
+        load_slab<T, WTN, B_KC, true>(rb, B, p.ldb, col0, p.N, 0, K, tid);
+        store_slab<T, WTM, A_KC>(smem[0], ra, tid);
+        store_slab<T, WTN, B_KC>(smem[0] + SA, rb, tid);
+        __syncthreads();
+        int cur = 0;
+        for (int kt = 0; kt < ntiles; ++kt) {
+            const bool more = kt + 1 < ntiles;
+            if (more) {
+                load_slab<T, WTM, A_KC, true>(ra, A, p.lda, row0, p.M, (int64_t)(kt + 1) * BK, K, tid);
+                load_slab<T, WTN, B_KC, true>(rb, B, p.ldb, col0, p.N, (int64_t)(kt + 1) * BK, K, tid);
+            }
+            compute(smem[cur]);
+            if (more) {
+                store_slab<T, WTM, A_KC>(smem[cur ^ 1], ra, tid);
+                store_slab<T, WTN, B_KC>(smem[cur ^ 1] + SA, rb, tid);
+            }
+            __syncthreads();
+            cur ^= 1;
+        }
     }
 
     // ---- epilogue ------------------------------------------------------------------------
@@ -225,14 +316,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_kernel(const GemmArgs<T>
         // Sum of the whole tile (rows/columns past M, N hold exact zeros).
         double s = 0.0;
 #pragma unroll
-        for (int x = 0; x < 4; ++x)
+        for (int x = 0; x < WTM; ++x)
 #pragma unroll
-            for (int y = 0; y < 4; ++y)
+            for (int y = 0; y < WTN; ++y)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) s += (double)acc[x][y][r];
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
-        double* red = reinterpret_cast<double*>(&smem[0][0][0]);
+        double* red = reinterpret_cast<double*>(&smem[0][0]);
         if (lane == 0) red[wave] = s;
         __syncthreads();
         if (tid == 0)
@@ -242,13 +333,13 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_kernel(const GemmArgs<T>
 
     T* __restrict__ C = p.C + batch * p.strideC;
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
+    for (int x = 0; x < WTM; ++x) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int64_t i = row0 + wm * 64 + x * 16 + MF::row(r, g);
+            const int64_t i = row0 + wm * WSM + x * 16 + MF::row(r, g);
 #pragma unroll
-            for (int y = 0; y < 4; ++y) {
-                const int64_t j = col0 + wn * 64 + y * 16 + li;
+            for (int y = 0; y < WTN; ++y) {
+                const int64_t j = col0 + wn * WSN + y * 16 + li;
                 if (EDGE && (i >= p.M || j >= p.N)) continue;
                 T v = acc[x][y][r];
                 if (EPI) {
@@ -265,37 +356,74 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_kernel(const GemmArgs<T>
     }
 }
 
-template <typename T, bool A_KC, bool B_KC>
+template <typename T, int WTM, int WTN, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, bool epi, hipStream_t stream) {
+    constexpr int BM = 32 * WTM, BN = 32 * WTN;
     const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BN - 1) / BN);
     dim3 grid((unsigned)(tilesM * tilesN), (unsigned)a.batch, 1), block(GEMM_THREADS, 1, 1);
     if (edge) {
-        if (epi) hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, true, true>), grid, block, 0, stream, a, tilesM, tilesN);
-        else hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, true, false>), grid, block, 0, stream, a, tilesM, tilesN);
+        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, true, true>), grid, block, 0, stream, a, tilesM, tilesN);
+        else hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, true, false>), grid, block, 0, stream, a, tilesM, tilesN);
     } else {
-        if (epi) hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, false, true>), grid, block, 0, stream, a, tilesM, tilesN);
-        else hipLaunchKernelGGL((gemm_kernel<T, A_KC, B_KC, false, false>), grid, block, 0, stream, a, tilesM, tilesN);
+        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, false, true>), grid, block, 0, stream, a, tilesM, tilesN);
+        else hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, false, false>), grid, block, 0, stream, a, tilesM, tilesN);
     }
     return hipGetLastError();
+}
+
+template <typename T, int WTM, int WTN>
+static hipError_t launch_tile(const GemmArgs<T>& a, bool epi, hipStream_t stream) {
+    constexpr int VEC = Mfma<T>::VEC;
+    constexpr int BK = Mfma<T>::BK;
+    constexpr int BM = 32 * WTM, BN = 32 * WTN;
+    // The unguarded kernels use 16-byte loads on whole tiles.
+    const bool aligned = (a.M % BM == 0) && (a.N % BN == 0) && (a.K % BK == 0) && a.K > 0 && (a.lda % VEC == 0) &&
+                         (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
+                         (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
+                         // per-thread element offsets inside one tile's slab are kept in 32 bits
+                         (a.lda < (1 << 23)) && (a.ldb < (1 << 23));
+    // Grid y carries the batch; the tile count must fit the 1-D grid.
+    if ((int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN) > 0x7fffffffLL || a.batch > 65535) return hipErrorInvalidValue;
+    if (!a.transA && !a.transB) return launch_layout<T, WTM, WTN, true, false>(a, !aligned, epi, stream);
+    if (!a.transA && a.transB) return launch_layout<T, WTM, WTN, true, true>(a, !aligned, epi, stream);
+    return launch_layout<T, WTM, WTN, false, false>(a, !aligned, epi, stream);
+}
+
+enum TileShape { TILE_128x128, TILE_64x64, TILE_32x32 };
+
+// Output tile for a product: the largest tile that still yields one workgroup per compute unit, so
+// that small products are spread over the whole chip (measured in double: N = 1024 runs 2.6x faster
+// on 64 x 64 tiles than on 128 x 128, N = 512 4.8x faster on 32 x 32; a 128 x 64 tile was measured at
+// N = 2048 and 4096 and was never faster than 128 x 128).  PRAD_GEMM_TILE=128x128|64x64|32x32 in the
+// environment overrides the choice (a tuning aid).
+static TileShape choose_tile(int64_t M, int64_t N, int batch, bool tile_sums) {
+    if (tile_sums) return TILE_128x128;  // the tile_sums layout is defined on 128 x 128 tiles
+    static const int forced = []() {
+        const char* e = getenv("PRAD_GEMM_TILE");
+        if (!e) return -1;
+        if (!strcmp(e, "128x128")) return (int)TILE_128x128;
+        if (!strcmp(e, "64x64")) return (int)TILE_64x64;
+        if (!strcmp(e, "32x32")) return (int)TILE_32x32;
+        return -1;
+    }();
+    if (forced >= 0) return (TileShape)forced;
+    auto tiles = [&](int64_t em, int64_t en) { return ((M + em - 1) / em) * ((N + en - 1) / en) * batch; };
+    if (tiles(128, 128) >= 256) return TILE_128x128;
+    if (tiles(64, 64) >= 256) return TILE_64x64;
+    return TILE_32x32;
 }
 
 template <typename T>
 hipError_t launch_gemm(const GemmArgs<T>& a, hipStream_t stream) {
     if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return hipSuccess;
     if (a.transA && a.transB) return hipErrorInvalidValue;
-    constexpr int VEC = Mfma<T>::VEC;
-    constexpr int BK = Mfma<T>::BK;
-    // The unguarded kernels use 16-byte loads on whole tiles.
-    const bool aligned = (a.M % BM == 0) && (a.N % BN == 0) && (a.K % BK == 0) && a.K > 0 && (a.lda % VEC == 0) &&
-                         (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
-                         (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0);
     const bool epi = a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE ||
                      a.tile_sums != nullptr;
-    // Grid y carries the batch; the tile count must fit the 1-D grid.
-    if ((int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN) > 0x7fffffffLL || a.batch > 65535) return hipErrorInvalidValue;
-    if (!a.transA && !a.transB) return launch_layout<T, true, false>(a, !aligned, epi, stream);
-    if (!a.transA && a.transB) return launch_layout<T, true, true>(a, !aligned, epi, stream);
-    return launch_layout<T, false, false>(a, !aligned, epi, stream);
+    switch (choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr)) {
+        case TILE_128x128: return launch_tile<T, 4, 4>(a, epi, stream);
+        case TILE_64x64: return launch_tile<T, 2, 2>(a, epi, stream);
+        default: return launch_tile<T, 1, 1>(a, epi, stream);
+    }
 }
 
 template hipError_t launch_gemm<double>(const GemmArgs<double>&, hipStream_t);

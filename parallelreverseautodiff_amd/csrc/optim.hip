@@ -66,9 +66,25 @@ __device__ __forceinline__ Moments shfl_down(const Moments& a, int off) {
     return r;
 }
 
+// A chunk is processed with 16-byte vector accesses when it is full and its tensor's pointers are
+// 16-byte aligned (chunks start at multiples of 4096 elements); partial last chunks and borrowed,
+// unaligned buffers take the scalar path.
+template <typename T> struct OptVec;
+template <> struct OptVec<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
+template <> struct OptVec<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
+
+template <typename T>
+__device__ __forceinline__ bool vector_chunk(const void* a, const void* b, const void* c, const void* d, int64_t begin, int64_t end) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c) |
+                           reinterpret_cast<uintptr_t>(d);
+    return (end - begin == OPT_CHUNK) && (bits % 16 == 0);
+}
+
 // Per-chunk moments -> partial[chunk].
 template <typename T>
 __global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTable<T> tab, Moments* __restrict__ partial) {
+    typedef typename OptVec<T>::type V;
+    constexpr int VN = OptVec<T>::N;
     const int64_t chunk = blockIdx.x;
     const int ti = find_tensor(tab.t, tab.nt, chunk);
     const DevTensor<T> t = tab.t[ti];
@@ -78,19 +94,36 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTab
     double x[PER];
     int cnt = 0;
     double sum = 0.0;
+    if (vector_chunk<T>(t.g, nullptr, nullptr, nullptr, begin, end)) {
+        const V* __restrict__ gv = reinterpret_cast<const V*>(t.g + begin);
+        V v[PER / VN];
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
-        if (i < end) { x[e] = (double)t.g[i]; sum += x[e]; ++cnt; } else x[e] = 0.0;
+        for (int e = 0; e < PER / VN; ++e) v[e] = __builtin_nontemporal_load(gv + e * OPT_THREADS + threadIdx.x);
+#pragma unroll
+        for (int e = 0; e < PER / VN; ++e)
+#pragma unroll
+            for (int c = 0; c < VN; ++c) { x[e * VN + c] = (double)v[e][c]; sum += x[e * VN + c]; }
+        cnt = PER;
+    } else {
+#pragma unroll
+        for (int e = 0; e < PER; ++e) {
+            const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
+            if (i < end) { x[e] = (double)t.g[i]; sum += x[e]; ++cnt; } else x[e] = 0.0;
+        }
     }
     Moments mo;
     mo.n = (double)cnt;
     mo.mean = cnt > 0 ? sum / (double)cnt : 0.0;
     mo.m2 = 0.0;
+    if (cnt == PER) {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
-        if (i < end) { const double d = x[e] - mo.mean; mo.m2 += d * d; }
+        for (int e = 0; e < PER; ++e) { const double d = x[e] - mo.mean; mo.m2 += d * d; }
+    } else {
+#pragma unroll
+        for (int e = 0; e < PER; ++e) {
+            const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
+            if (i < end) { const double d = x[e] - mo.mean; mo.m2 += d * d; }
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mo = merge(mo, shfl_down(mo, off));
@@ -145,19 +178,34 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTab
     const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
     const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
     constexpr int PER = OPT_CHUNK / OPT_THREADS;
+    auto clamp = [&](T g) -> T {
+        const T z = (g - mean) / stddev;
+        const T value = dotnet_min<T>(clip_value, (T)1 + (z < (T)0 ? -z : z));
+        if (g > value) g = value;
+        else if (g < -value) g = -value;
+        if (g > (T)0 && g < min_value) g = min_value;
+        else if (g < (T)0 && g > -min_value) g = -min_value;
+        return g;
+    };
+    if (vector_chunk<T>(t.g, nullptr, nullptr, nullptr, begin, end)) {
+        typedef typename OptVec<T>::type V;
+        constexpr int VN = OptVec<T>::N;
+        V* __restrict__ gv = reinterpret_cast<V*>(t.g + begin);
+        V v[PER / VN];
+#pragma unroll
+        for (int e = 0; e < PER / VN; ++e) v[e] = __builtin_nontemporal_load(gv + e * OPT_THREADS + threadIdx.x);
+#pragma unroll
+        for (int e = 0; e < PER / VN; ++e) {
+#pragma unroll
+            for (int c = 0; c < VN; ++c) v[e][c] = clamp(v[e][c]);
+            __builtin_nontemporal_store(v[e], gv + e * OPT_THREADS + threadIdx.x);
+        }
+        return;
+    }
 #pragma unroll 4
     for (int e = 0; e < PER; ++e) {
         const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
-        if (i < end) {
-            T g = t.g[i];
-            const T z = (g - mean) / stddev;
-            const T value = dotnet_min<T>(clip_value, (T)1 + (z < (T)0 ? -z : z));
-            if (g > value) g = value;
-            else if (g < -value) g = -value;
-            if (g > (T)0 && g < min_value) g = min_value;
-            else if (g < (T)0 && g > -min_value) g = -min_value;
-            t.g[i] = g;
-        }
+        if (i < end) t.g[i] = clamp(t.g[i]);
     }
 }
 
@@ -171,24 +219,58 @@ __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> 
     const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
     const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
     constexpr int PER = OPT_CHUNK / OPT_THREADS;
-    T w[PER], m[PER], v[PER], g[PER];
+    auto update = [&](T& w, T& m, T& v, T g) {
+        const T first = (beta1 * m) + (omb1 * g);
+        const T second = (beta2 * v) + (omb2 * (g * g));
+        const T mhat = c1 * first;
+        const T vhat = c2 * second;
+        const T red = lr * mhat / (sqrt(vhat) + eps);
+        w = w - red;
+        m = first;
+        v = second;
+    };
+    if (vector_chunk<T>(t.w, t.m, t.v, t.g, begin, end)) {
+        typedef typename OptVec<T>::type V;
+        constexpr int VN = OptVec<T>::N;
+        constexpr int HALF = PER / VN / 2;  // two passes keep the register footprint moderate
+        V* __restrict__ wv = reinterpret_cast<V*>(t.w + begin);
+        V* __restrict__ mv = reinterpret_cast<V*>(t.m + begin);
+        V* __restrict__ vv = reinterpret_cast<V*>(t.v + begin);
+        const V* __restrict__ gv = reinterpret_cast<const V*>(t.g + begin);
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-        const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
-        if (i < end) { w[e] = t.w[i]; m[e] = t.m[i]; v[e] = t.v[i]; g[e] = t.g[i]; }
+        for (int h = 0; h < 2; ++h) {
+            V w[HALF], m[HALF], v[HALF], g[HALF];
+#pragma unroll
+            for (int e = 0; e < HALF; ++e) {
+                const int iv = (h * HALF + e) * OPT_THREADS + threadIdx.x;
+                w[e] = __builtin_nontemporal_load(wv + iv);
+                m[e] = __builtin_nontemporal_load(mv + iv);
+                v[e] = __builtin_nontemporal_load(vv + iv);
+                g[e] = __builtin_nontemporal_load(gv + iv);
+            }
+#pragma unroll
+            for (int e = 0; e < HALF; ++e) {
+                const int iv = (h * HALF + e) * OPT_THREADS + threadIdx.x;
+#pragma unroll
+                for (int c = 0; c < VN; ++c) {
+                    T wi = w[e][c], mi = m[e][c], vi = v[e][c];
+                    update(wi, mi, vi, g[e][c]);
+                    w[e][c] = wi; m[e][c] = mi; v[e][c] = vi;
+                }
+                __builtin_nontemporal_store(w[e], wv + iv);
+                __builtin_nontemporal_store(m[e], mv + iv);
+                __builtin_nontemporal_store(v[e], vv + iv);
+            }
+        }
+        return;
     }
-#pragma unroll
+#pragma unroll 4
     for (int e = 0; e < PER; ++e) {
         const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
         if (i < end) {
-            const T first = (beta1 * m[e]) + (omb1 * g[e]);
-            const T second = (beta2 * v[e]) + (omb2 * (g[e] * g[e]));
-            const T mhat = c1 * first;
-            const T vhat = c2 * second;
-            const T red = lr * mhat / (sqrt(vhat) + eps);
-            t.w[i] = w[e] - red;
-            t.m[i] = first;
-            t.v[i] = second;
+            T wi = t.w[i], mi = t.m[i], vi = t.v[i];
+            update(wi, mi, vi, t.g[i]);
+            t.w[i] = wi; t.m[i] = mi; t.v[i] = vi;
         }
     }
 }
