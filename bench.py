@@ -129,6 +129,97 @@ def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
     return out, n
 
 
+def mlp_leg(dtype_name, steps, warmup, with_cpu):
+    """Feed-forward training step of configs[0]: batch 64, 784-256-128-10, LeakyReLU(0.01), softmax
+    cross-entropy, clip, Adam.  Timed launch by launch and as one recorded launch sequence."""
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.feedforward import FeedForwardNetwork
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = 0
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    net = FeedForwardNetwork(dtype=dtype)
+    X = seeded.uniform(seeded.DEFAULT_SEED, 1, (64, 784), 0.0, 1.0, dtype)
+    T = seeded.one_hot_labels(seeded.DEFAULT_SEED, 2, 64, 10, dtype)
+    net.set_batch(X, T)
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.prad_event_create(ctypes.byref(e0)))
+    check(lib.prad_event_create(ctypes.byref(e1)))
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        check(lib.prad_stream_sync())
+        t0 = time.perf_counter()
+        check(lib.prad_event_record(e0))
+        for _ in range(steps):
+            fn()
+        check(lib.prad_event_record(e1))
+        check(lib.prad_stream_sync())
+        wall = time.perf_counter() - t0
+        ms = ctypes.c_float()
+        check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        return ms.value / steps, wall * 1e3 / steps
+
+    eager_ms, eager_wall = timed(net.step)
+    net.record(adam_iteration=float(net.iteration + 1))
+    graph_ms, graph_wall = timed(net.replay)
+    loss = float(net.loss.download()[0, 0])
+    net.release()
+    out = {"eager_ms_per_step": eager_ms, "eager_wall_ms_per_step": eager_wall, "recorded_ms_per_step": graph_ms,
+           "recorded_wall_ms_per_step": graph_wall, "loss_after": loss, "flop_per_step": net.flops_per_step(),
+           "parameters": net.parameter_count()}
+    if with_cpu:
+        out["cpu"] = mlp_cpu_leg(net.host_W, X, T, net.params, dtype)
+    return out
+
+
+def mlp_cpu_leg(W0, X, T, params, dtype, budget_s=15.0):
+    """The same step composed from the oracle's restatements of the reference operations, on the host."""
+    from oracle import oracle
+    threads = min(16, oracle.hardware_threads() or 1)
+    alpha = dtype(params.LeakyReLUAlpha)
+    W = [w.copy() for w in W0]
+    b = [np.zeros((1, w.shape[1]), dtype) for w in W]
+    m = [np.zeros_like(x) for x in W + b]
+    v = [np.zeros_like(x) for x in W + b]
+    L = len(W)
+
+    def step(t):
+        nonlocal W, b, m, v
+        a, Z, H = X, [], []
+        for l in range(L):
+            z = oracle.add_broadcast_fwd(oracle.matmul_fwd(a, W[l], threads=threads), b[l])
+            Z.append(z)
+            a = z if l == L - 1 else oracle.leakyrelu_fwd(z, alpha)
+            H.append(a)
+        P = oracle.softmax_fwd(Z[-1])
+        oracle.cce_fwd(P, T)
+        dz = oracle.softmax_bwd(P, oracle.cce_bwd(P, T))
+        dW, db = [None] * L, [None] * L
+        for l in range(L - 1, -1, -1):
+            db[l] = oracle.add_broadcast_bwd_bias(dz)
+            dA, dW[l] = oracle.matmul_bwd(dz, X if l == 0 else H[l - 1], W[l], threads=threads)
+            if l > 0:
+                dz = oracle.leakyrelu_bwd(Z[l - 1], dA, alpha)
+        grads = [oracle.clip(g, params.ClipValue, params.MinimumClipValue) for g in dW + db]
+        new = [oracle.adam(w, mm, vv, g, params.LearningRate, params.AdamBeta1, params.AdamBeta2, params.AdamEpsilon, float(t))
+               for w, mm, vv, g in zip(W + b, m, v, grads)]
+        W, b = [n[0] for n in new[:L]], [n[0] for n in new[L:]]
+        m, v = [n[1] for n in new], [n[2] for n in new]
+
+    step(1)
+    n, t0 = 0, time.perf_counter()
+    while n < 200 and time.perf_counter() - t0 < budget_s:
+        step(n + 2)
+        n += 1
+    secs = (time.perf_counter() - t0) / n
+    return {"steps_per_s": 1.0 / secs, "ms_per_step": secs * 1e3, "cores": threads, "steps_timed": n, "kind": "port"}
+
+
 def cpu_leg(budget_s=40.0):
     """Times the CPU restatement of the reference's Parallel.For path (jagged rows, row-parallel scalar
     i-j-k loops) on this host: a bounded sample of the same workload at a smaller N."""
@@ -165,13 +256,23 @@ def main():
     ap.add_argument("--n", type=int, default=4096)
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["gemm", "bandwidth"], default="gemm",
-                    help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels")
+    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp"], default="gemm",
+                    help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
+                         "mlp: the feed-forward training step of configs[0]")
     ap.add_argument("--elems", type=int, default=64 * 1024 * 1024, help="elements per tensor in bandwidth mode")
     ap.add_argument("--only", default="", help="bandwidth mode: comma-separated kernel names")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: this path has no multi-GPU part (--gpus 1 only)")
+    if args.mode == "mlp":
+        res = mlp_leg(args.dtype, args.steps, args.warmup, not args.no_cpu)
+        print(json.dumps({"metric": "MLP train steps/sec", "unit": "steps/s", "value": 1e3 / res["recorded_ms_per_step"],
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
+                          "higher_is_better": True, "ms_per_step": res["recorded_ms_per_step"],
+                          "config": {"workload": "configs[0]: 3-layer MLP 784-256-128-10, batch 64, LeakyReLU(0.01), softmax "
+                                                 "cross-entropy, clip(4), Adam(lr 1e-3): forward + backward + update"},
+                          "detail": res}))
+        return
     if args.mode == "bandwidth":
         res, n = bandwidth_leg(args.elems, args.dtype, args.steps, args.warmup, [x for x in args.only.split(",") if x])
         best = max(res.values(), key=lambda r: r["GB/s"])

@@ -142,6 +142,26 @@ int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad);
 int32_t prad_add_broadcast_fwd(prad_buf_t x, prad_buf_t bias, prad_buf_t y);
 int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias);
 
+/* ---- operations that close a training step on the device ------------------------------------ */
+/* Row-wise softmax, src/RMAD/SoftmaxOperation.cs:45-110 (backward: dx = J^T . dy per row). */
+int32_t prad_softmax_fwd(prad_buf_t x, prad_buf_t y);
+int32_t prad_softmax_bwd(prad_buf_t y, prad_buf_t dy, prad_buf_t dx);
+/* Categorical cross-entropy, src/RMAD/Loss/CategoricalCrossEntropyLossOperation.cs:37-86:
+ * loss (1 x 1) = sum(-t * log(p + 1e-15)) / rows ; dp = -(1/rows) * t / (p + 1e-15). */
+int32_t prad_cce_fwd(prad_buf_t p, prad_buf_t target, prad_buf_t loss);
+int32_t prad_cce_bwd(prad_buf_t p, prad_buf_t target, prad_buf_t dp);
+
+/* ---- replay of a fixed launch sequence: everything enqueued by this thread between begin and end
+ *      is recorded instead of executed and can then be launched as one submission.  The forward loop
+ *      of the reference walks the same operation list every step
+ *      (examples/feedforward/FeedForwardNeuralNetworkExample/FeedForwardNeuralNetwork.cs:212-303);
+ *      a recorded step replaces ~20 launches by one.  Only entry points that neither allocate nor
+ *      copy to or from the host may be recorded. */
+int32_t prad_graph_begin(void);
+int32_t prad_graph_end(void** graph);
+int32_t prad_graph_launch(void* graph);
+int32_t prad_graph_destroy(void* graph);
+
 /* ---- GradientClipper.ClipGradients, src/RMAD/GradientClipper.cs:118-157 and :212-253 (in place) */
 int32_t prad_clip(prad_buf_t g, double clip_value, double min_value);
 /* ---- AdamOptimizer.UpdateWeightWithAdam, src/RMAD/AdamOptimizer.cs:195-239 (in place on w, m, v) */

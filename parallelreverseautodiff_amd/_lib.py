@@ -71,6 +71,14 @@ SIGNATURES = {
     "prad_accumulate": (_i32, [_vp, _vp]),
     "prad_add_broadcast_fwd": (_i32, [_vp, _vp, _vp]),
     "prad_add_broadcast_bwd_bias": (_i32, [_vp, _vp]),
+    "prad_softmax_fwd": (_i32, [_vp, _vp]),
+    "prad_softmax_bwd": (_i32, [_vp, _vp, _vp]),
+    "prad_cce_fwd": (_i32, [_vp, _vp, _vp]),
+    "prad_cce_bwd": (_i32, [_vp, _vp, _vp]),
+    "prad_graph_begin": (_i32, []),
+    "prad_graph_end": (_i32, [_vpp]),
+    "prad_graph_launch": (_i32, [_vp]),
+    "prad_graph_destroy": (_i32, [_vp]),
     "prad_clip": (_i32, [_vp, _f64, _f64]),
     "prad_adam": (_i32, [_vp, _vp, _vp, _vp, _f64, _f64, _f64, _f64, _f64]),
     "prad_clip_multi": (_i32, [_vpp, _i32, _f64, _f64]),

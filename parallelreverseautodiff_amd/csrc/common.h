@@ -161,6 +161,12 @@ template <typename T> hipError_t launch_clip(const TensorDesc<T>* host_descs, in
 template <typename T> hipError_t launch_adam(const TensorDesc<T>* host_descs, int ntensors, T lr, T beta1, T beta2, T eps, T c1,
                                              T c2, hipStream_t s);
 
+// softmax / categorical cross-entropy (csrc/loss.hip)
+template <typename T> hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_cce_fwd(const T* p, const T* t, T* loss, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t cols, hipStream_t s);
+
 // MatrixMultiplyAndSum
 template <typename T> hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K,
                                                        int64_t N, int64_t P, hipStream_t s);

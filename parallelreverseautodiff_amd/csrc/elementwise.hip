@@ -214,21 +214,34 @@ hipError_t launch_add_broadcast_fwd(const T* x, const T* bias, T* y, int64_t row
     return hipGetLastError();
 }
 
-// ---- bias gradient: db[j] = sum_i dy[i][j], rows ascending, accumulated in double and rounded
-// once (LINQ Sum over Column(j), which for float accumulates in double).  One thread per column;
-// neighbouring threads read neighbouring columns, so every row is one coalesced read.
+// ---- bias gradient: db[j] = sum_i dy[i][j], accumulated in double and rounded once (LINQ Sum over
+// Column(j), which for float accumulates in double).  A workgroup owns 64 columns; its four
+// wavefronts take rows i = w, w+4, w+8, ... with four independent loads in flight each, and the four
+// partial sums are added in wavefront order, so the result does not depend on timing.  Neighbouring
+// lanes read neighbouring columns: every row is one coalesced read.
 template <typename T>
-__global__ void __launch_bounds__(64) colsum_kernel(const T* __restrict__ dy, T* __restrict__ db, int64_t rows, int64_t cols) {
-    const int64_t j = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (j >= cols) return;
-    double acc = 0.0;
-    for (int64_t i = 0; i < rows; ++i) acc += (double)dy[i * cols + j];
-    db[j] = (T)acc;
+__global__ void __launch_bounds__(256) colsum_kernel(const T* __restrict__ dy, T* __restrict__ db, int64_t rows, int64_t cols) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int64_t j = (int64_t)blockIdx.x * 64 + lane;
+    double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
+    if (j < cols) {
+        int64_t i = w;
+        for (; i + 12 < rows; i += 16) {
+            const double a = (double)dy[i * cols + j], b = (double)dy[(i + 4) * cols + j];
+            const double c = (double)dy[(i + 8) * cols + j], d = (double)dy[(i + 12) * cols + j];
+            acc0 += a; acc1 += b; acc2 += c; acc3 += d;
+        }
+        for (; i < rows; i += 4) acc0 += (double)dy[i * cols + j];
+    }
+    __shared__ double part[4][64];
+    part[w][lane] = (acc0 + acc1) + (acc2 + acc3);
+    __syncthreads();
+    if (w == 0 && j < cols) db[j] = (T)((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]));
 }
 template <typename T>
 hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, hipStream_t s) {
     if (cols <= 0) return hipSuccess;
-    hipLaunchKernelGGL((colsum_kernel<T>), dim3((unsigned)((cols + 63) / 64)), dim3(64), 0, s, dy, db, rows, cols);
+    hipLaunchKernelGGL((colsum_kernel<T>), dim3((unsigned)((cols + 63) / 64)), dim3(256), 0, s, dy, db, rows, cols);
     return hipGetLastError();
 }
 

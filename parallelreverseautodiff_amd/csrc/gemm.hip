@@ -8,16 +8,16 @@
 // transposed copies it is fed with (:148, :154, :210-248): a transposed operand is read in its
 // stored orientation and only its placement in LDS differs.
 //
-// Shape of one workgroup: 256 threads = 4 wavefronts (2 x 2).  The output tile is 32*WTM x 32*WTN:
-// each wavefront owns WTM x WTN MFMA tiles of 16 x 16, so an A fragment read from LDS feeds WTN MFMAs
-// and a B fragment WTM.  128 x 128 (WTM = WTN = 4) is the steady-state shape; the smaller tiles exist
-// so that products with few 128 x 128 tiles still put work on all 256 compute units.  The reduction
-// dimension is cut into slabs of BK (16 doubles / 32 floats = 128 bytes per row); slabs are
-// double-buffered in LDS and the next slab's global loads are issued before the current slab's MFMAs.
+// Shape of one workgroup: 256 threads = 4 wavefronts (2 x 2).  The output tile is 32*WT x 32*WT:
+// each wavefront owns WT x WT MFMA tiles of 16 x 16, so a fragment read from LDS feeds WT MFMAs.
+// 128 x 128 (WT = 4) is the steady-state shape; the 64 and 32 tiles exist so that products with few
+// 128 x 128 tiles still put work on all 256 compute units.  The reduction dimension is cut into
+// slabs of 16 KiB per operand (BK = 16 doubles for the 128 tile, 64 for the 32 tile); slabs are
+// double-buffered in LDS and global loads run two slabs ahead of the MFMAs.
 //
 // LDS placement of an operand slab (MN = its rows/columns of the output tile):
 //   stored with the reduction index contiguous ("KC": A of the forward, both operands of dA)
-//       S[mn][k], row pitch BK + pad (144 bytes) chosen so that the 16 bytes of two neighbouring k
+//       S[mn][k], row pitch BK elements + 16 bytes, chosen so that the 16 bytes of two neighbouring k
 //       of 16 consecutive mn fall into distinct 16-byte bank groups (an XOR-swizzled unpadded
 //       layout was measured too: same speed in double, 6 % slower in float because the compiler
 //       can no longer merge neighbouring LDS reads);
@@ -39,14 +39,15 @@ typedef double d2_t __attribute__((ext_vector_type(2)));
 constexpr int GEMM_THREADS = 256;
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 8;
+constexpr int NV = 4;  // 16-byte vectors per thread per operand slab, for every tile shape
 
 template <typename T> struct Mfma;
 template <> struct Mfma<double> {
     typedef d4_t Acc;
     typedef d2_t Vec;
-    static constexpr int VEC = 2;   // elements per 16-byte load
-    static constexpr int BK = 16;   // reduction slab
-    static constexpr int LDK = 18;  // pitch of a KC slab row
+    static constexpr int VEC = 2;           // elements per 16-byte load
+    static constexpr int SLAB_ELEMS = 2048; // elements of one operand slab: MN x BK, 16 KiB
+    static constexpr int KPAD = 2;          // padding of a KC slab row (16 bytes)
     static __device__ __forceinline__ Acc run(double a, double b, Acc c) {
         return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
     }
@@ -57,100 +58,72 @@ template <> struct Mfma<float> {
     typedef f4_t Acc;
     typedef f4_t Vec;
     static constexpr int VEC = 4;
-    static constexpr int BK = 32;
-    static constexpr int LDK = 36;
+    static constexpr int SLAB_ELEMS = 4096;
+    static constexpr int KPAD = 4;
     static __device__ __forceinline__ Acc run(float a, float b, Acc c) {
         return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ int row(int r, int g) { return 4 * g + r; }
 };
 
-// Offset (in elements) of element (mn, k) of a KC slab.
-template <typename T>
-__device__ __forceinline__ int kc_offset(int mn, int k) {
-    return mn * Mfma<T>::LDK + k;
-}
+// Geometry of one operand slab for an output tile edge MN = 32 * WT: MN rows/columns by BK of the
+// reduction dimension, always 16 KiB, so BK = 16, 32, 64 doubles (32, 64, 128 floats) for the
+// 128, 64, 32 tiles: the small tiles, which run with one wavefront per SIMD and cannot hide a
+// global-memory round trip behind another workgroup, make four times fewer of them.
+template <typename T, int WT>
+struct Slab {
+    static constexpr int MN = 32 * WT;
+    static constexpr int BK = Mfma<T>::SLAB_ELEMS / MN;
+    static constexpr int LDK = BK + Mfma<T>::KPAD;  // pitch of a KC row: 16 bytes past a multiple of 128/256/512 bytes
+    static constexpr int LDM = MN + 16;             // pitch of an MC row
+    static constexpr int TPR_KC = BK / Mfma<T>::VEC;        // threads covering one KC row
+    static constexpr int ROWS_KC = GEMM_THREADS / TPR_KC;   // KC rows per pass
+    static constexpr int TPR_MC = MN / Mfma<T>::VEC;        // threads covering one MC row
+    static constexpr int ROWS_MC = GEMM_THREADS / TPR_MC;   // MC rows (k) per pass
+    static_assert(MN / ROWS_KC == NV && BK / ROWS_MC == NV, "four vectors per thread per slab");
+    template <bool KC> static constexpr int elems() { return KC ? MN * LDK : BK * LDM; }
+};
 
-// Loads this thread's share (NV vectors) of one operand slab (MN = 32*NV rows/columns x BK) from global memory.
-//   KC: the operand is stored [mn][k]: 8 threads cover the 128 bytes of one row.
-//   MC: the operand is stored [k][mn]: MN / VEC threads cover one k row.
-template <typename T, int NV, bool KC, bool EDGE>
-__device__ __forceinline__ void load_slab(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ base, int64_t ld, int64_t mn0,
-                                          int64_t mn_end, int64_t k0, int64_t k_end, int tid) {
-    typedef typename Mfma<T>::Vec Vec;
+// Guarded loads of this thread's share of one operand slab (shapes that are not whole tiles or not
+// 16-byte aligned).  KC: the operand is stored [mn][k]; MC: it is stored [k][mn].
+template <typename T, int WT, bool KC>
+__device__ __forceinline__ void load_slab_guarded(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ base, int64_t ld,
+                                                  int64_t mn0, int64_t mn_end, int64_t k0, int64_t k_end, int tid) {
+    typedef Slab<T, WT> S;
     constexpr int VEC = Mfma<T>::VEC;
-    if (KC) {
-        const int kv = tid & 7;
-        const int rowb = tid >> 3;
 #pragma unroll
-        for (int p = 0; p < NV; ++p) {
-            const int64_t mn = mn0 + rowb + 32 * p;
-            const int64_t k = k0 + kv * VEC;
-            const T* g = base + mn * ld + k;
-            if (!EDGE) {
-                r[p] = *reinterpret_cast<const Vec*>(g);
-            } else {
+    for (int p = 0; p < NV; ++p) {
+        int64_t mn, k;
+        const T* g;
+        if (KC) {
+            mn = mn0 + tid / S::TPR_KC + S::ROWS_KC * p;
+            k = k0 + (tid % S::TPR_KC) * VEC;
+            g = base + mn * ld + k;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) r[p][e] = (mn < mn_end && k + e < k_end) ? g[e] : (T)0;
-            }
+            for (int e = 0; e < VEC; ++e) r[p][e] = (mn < mn_end && k + e < k_end) ? g[e] : (T)0;
+        } else {
+            k = k0 + tid / S::TPR_MC + S::ROWS_MC * p;
+            mn = mn0 + (tid % S::TPR_MC) * VEC;
+            g = base + k * ld + mn;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[p][e] = (k < k_end && mn + e < mn_end) ? g[e] : (T)0;
         }
-    } else {
-        constexpr int CV = 32 * NV / VEC;             // vectors per k row
-        constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
-        const int cv = tid % CV;
-        const int krow = tid / CV;
-#pragma unroll
-        for (int p = 0; p < NV; ++p) {
-            const int64_t k = k0 + krow + ROWS_PER_PASS * p;
-            const int64_t mn = mn0 + cv * VEC;
-            const T* g = base + k * ld + mn;
-            if (!EDGE) {
-                r[p] = *reinterpret_cast<const Vec*>(g);
-            } else {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) r[p][e] = (k < k_end && mn + e < mn_end) ? g[e] : (T)0;
-            }
-        }
-    }
-}
-
-template <typename T, int NV, bool KC>
-__device__ __forceinline__ void store_slab(T* __restrict__ s, const typename Mfma<T>::Vec (&r)[NV], int tid) {
-    typedef typename Mfma<T>::Vec Vec;
-    constexpr int VEC = Mfma<T>::VEC;
-    if (KC) {
-        const int kv = tid & 7;
-        const int rowb = tid >> 3;
-#pragma unroll
-        for (int p = 0; p < NV; ++p) *reinterpret_cast<Vec*>(s + kc_offset<T>(rowb + 32 * p, kv * VEC)) = r[p];
-    } else {
-        constexpr int LDM = 32 * NV + 16;  // pitch of an MC slab row
-        constexpr int CV = 32 * NV / VEC;
-        constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
-        const int cv = tid % CV;
-        const int krow = tid / CV;
-#pragma unroll
-        for (int p = 0; p < NV; ++p) *reinterpret_cast<Vec*>(s + (krow + ROWS_PER_PASS * p) * LDM + cv * VEC) = r[p];
     }
 }
 
 // Unguarded loads of one slab, addressed as a wavefront-uniform base (scalar registers, advanced slab
 // by slab) plus a per-thread 32-bit element offset that never changes: the loads take the
 // scalar-base form and the two prefetch register sets share one set of offsets.
-template <typename T, int NV, bool KC>
+template <typename T, int WT, bool KC>
 __device__ __forceinline__ void slab_offsets(unsigned (&off)[NV], int64_t ld, int tid) {
+    typedef Slab<T, WT> S;
     constexpr int VEC = Mfma<T>::VEC;
-    if (KC) {
 #pragma unroll
-        for (int p = 0; p < NV; ++p) off[p] = (unsigned)(((tid >> 3) + 32 * p) * ld + (tid & 7) * VEC);
-    } else {
-        constexpr int CV = 32 * NV / VEC;
-        constexpr int ROWS_PER_PASS = GEMM_THREADS / CV;
-#pragma unroll
-        for (int p = 0; p < NV; ++p) off[p] = (unsigned)((tid / CV + ROWS_PER_PASS * p) * ld + (tid % CV) * VEC);
-    }
+    for (int p = 0; p < NV; ++p)
+        off[p] = KC ? (unsigned)((tid / S::TPR_KC + S::ROWS_KC * p) * ld + (tid % S::TPR_KC) * VEC)
+                    : (unsigned)((tid / S::TPR_MC + S::ROWS_MC * p) * ld + (tid % S::TPR_MC) * VEC);
 }
-template <typename T, int NV>
+template <typename T>
 __device__ __forceinline__ void load_slab_fast(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ ubase,
                                                const unsigned (&off)[NV]) {
     typedef typename Mfma<T>::Vec Vec;
@@ -158,14 +131,23 @@ __device__ __forceinline__ void load_slab_fast(typename Mfma<T>::Vec (&r)[NV], c
     for (int p = 0; p < NV; ++p) r[p] = *reinterpret_cast<const Vec*>(ubase + off[p]);
 }
 
-// Element (mn, k) of a slab in LDS.
-template <typename T, int NV, bool KC>
-__device__ __forceinline__ T slab_at(const T* __restrict__ s, int mn, int k) {
-    return KC ? s[kc_offset<T>(mn, k)] : s[k * (32 * NV + 16) + mn];
+template <typename T, int WT, bool KC>
+__device__ __forceinline__ void store_slab(T* __restrict__ s, const typename Mfma<T>::Vec (&r)[NV], int tid) {
+    typedef Slab<T, WT> S;
+    typedef typename Mfma<T>::Vec Vec;
+    constexpr int VEC = Mfma<T>::VEC;
+#pragma unroll
+    for (int p = 0; p < NV; ++p) {
+        if (KC) *reinterpret_cast<Vec*>(s + (tid / S::TPR_KC + S::ROWS_KC * p) * S::LDK + (tid % S::TPR_KC) * VEC) = r[p];
+        else *reinterpret_cast<Vec*>(s + (tid / S::TPR_MC + S::ROWS_MC * p) * S::LDM + (tid % S::TPR_MC) * VEC) = r[p];
+    }
 }
 
-template <typename T, int NV, bool KC>
-constexpr int slab_elems() { return KC ? 32 * NV * Mfma<T>::LDK : Mfma<T>::BK * (32 * NV + 16); }
+// Element (mn, k) of a slab in LDS.
+template <typename T, int WT, bool KC>
+__device__ __forceinline__ T slab_at(const T* __restrict__ s, int mn, int k) {
+    return KC ? s[mn * Slab<T, WT>::LDK + k] : s[k * Slab<T, WT>::LDM + mn];
+}
 
 // Maps the linear workgroup id to an output tile.  Hardware deals consecutive workgroup ids
 // round-robin to the 8 XCDs, each with its own L2: ids are first regrouped so that one XCD gets a
@@ -185,18 +167,20 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tilesM, int tiles
     tn = in_group / gsz;
 }
 
-constexpr int min_blocks(int wtm, int wtn) { return wtm * wtn >= 16 ? 2 : wtm * wtn >= 8 ? 3 : 4; }
+constexpr int min_blocks(int wt) { return wt >= 4 ? 2 : 4; }
 
-template <typename T, int WTM, int WTN, bool A_KC, bool B_KC, bool EDGE, bool EPI>
-__global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WTM, WTN)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
-                                                                                  const int tilesN) {
+template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, bool EPI>
+__global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
+                                                                            const int tilesN) {
     typedef Mfma<T> MF;
+    typedef Slab<T, WT> S;
     typedef typename MF::Acc Acc;
     typedef typename MF::Vec Vec;
-    constexpr int BK = MF::BK;
-    constexpr int BM = 32 * WTM, BN = 32 * WTN;  // output tile
-    constexpr int WSM = 16 * WTM, WSN = 16 * WTN;  // one wavefront's share
-    constexpr int SA = slab_elems<T, WTM, A_KC>(), SB = slab_elems<T, WTN, B_KC>();
+    constexpr int BK = S::BK;
+    constexpr int BM = 32 * WT, BN = 32 * WT;  // output tile
+    constexpr int WS = 16 * WT;                // edge of one wavefront's share
+    constexpr int WTM = WT, WTN = WT;
+    constexpr int SA = S::template elems<A_KC>(), SB = S::template elems<B_KC>();
 
     __shared__ __attribute__((aligned(16))) T smem[2][SA + SB];  // [stage][A slab | B slab]
 
@@ -232,9 +216,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WTM, WTN)) gemm_kerne
             const int k = 4 * s + g;
             T a[WTM], b[WTN];
 #pragma unroll
-            for (int x = 0; x < WTM; ++x) a[x] = slab_at<T, WTM, A_KC>(sA, wm * WSM + x * 16 + li, k);
+            for (int x = 0; x < WTM; ++x) a[x] = slab_at<T, WT, A_KC>(sA, wm * WS + x * 16 + li, k);
 #pragma unroll
-            for (int y = 0; y < WTN; ++y) b[y] = slab_at<T, WTN, B_KC>(sB, wn * WSN + y * 16 + li, k);
+            for (int y = 0; y < WTN; ++y) b[y] = slab_at<T, WT, B_KC>(sB, wn * WS + y * 16 + li, k);
 #pragma unroll
             for (int x = 0; x < WTM; ++x)
 #pragma unroll
@@ -247,64 +231,64 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WTM, WTN)) gemm_kerne
         // of slab t+2 are issued into the other, so a global load has two slabs of MFMAs to arrive
         // (measured +5 % at N = 4096 over a prefetch distance of one slab).  The loop is unrolled by two so
         // that the sets are named statically.
-        Vec ra0[WTM], rb0[WTN], ra1[WTM], rb1[WTN];
-        unsigned offa[WTM], offb[WTN];
-        slab_offsets<T, WTM, A_KC>(offa, p.lda, tid);
-        slab_offsets<T, WTN, B_KC>(offb, p.ldb, tid);
+        Vec ra0[NV], rb0[NV], ra1[NV], rb1[NV];
+        unsigned offa[NV], offb[NV];
+        slab_offsets<T, WT, A_KC>(offa, p.lda, tid);
+        slab_offsets<T, WT, B_KC>(offb, p.ldb, tid);
         // uniform bases of slab 0 and their per-slab strides
         const T* __restrict__ ua = A + (A_KC ? row0 * p.lda : row0);
         const T* __restrict__ ub = B + (B_KC ? col0 * p.ldb : col0);
         const int64_t stepa = A_KC ? (int64_t)BK : (int64_t)BK * p.lda;
         const int64_t stepb = B_KC ? (int64_t)BK : (int64_t)BK * p.ldb;
-        load_slab_fast<T, WTM>(ra0, ua, offa);
-        load_slab_fast<T, WTN>(rb0, ub, offb);
+        load_slab_fast<T>(ra0, ua, offa);
+        load_slab_fast<T>(rb0, ub, offb);
         if (ntiles > 1) {
-            load_slab_fast<T, WTM>(ra1, ua + stepa, offa);
-            load_slab_fast<T, WTN>(rb1, ub + stepb, offb);
+            load_slab_fast<T>(ra1, ua + stepa, offa);
+            load_slab_fast<T>(rb1, ub + stepb, offb);
         }
-        store_slab<T, WTM, A_KC>(smem[0], ra0, tid);
-        store_slab<T, WTN, B_KC>(smem[0] + SA, rb0, tid);
+        store_slab<T, WT, A_KC>(smem[0], ra0, tid);
+        store_slab<T, WT, B_KC>(smem[0] + SA, rb0, tid);
         __syncthreads();
         for (int kt = 0; kt + 1 < ntiles; kt += 2) {
             // LDS stage 0 holds slab kt, set 1 holds slab kt+1 (in flight), set 0 is free.
             if (kt + 2 < ntiles) {
-                load_slab_fast<T, WTM>(ra0, ua + (kt + 2) * stepa, offa);
-                load_slab_fast<T, WTN>(rb0, ub + (kt + 2) * stepb, offb);
+                load_slab_fast<T>(ra0, ua + (kt + 2) * stepa, offa);
+                load_slab_fast<T>(rb0, ub + (kt + 2) * stepb, offb);
             }
             compute(smem[0]);
-            store_slab<T, WTM, A_KC>(smem[1], ra1, tid);
-            store_slab<T, WTN, B_KC>(smem[1] + SA, rb1, tid);
+            store_slab<T, WT, A_KC>(smem[1], ra1, tid);
+            store_slab<T, WT, B_KC>(smem[1] + SA, rb1, tid);
             __syncthreads();
             if (kt + 3 < ntiles) {
-                load_slab_fast<T, WTM>(ra1, ua + (kt + 3) * stepa, offa);
-                load_slab_fast<T, WTN>(rb1, ub + (kt + 3) * stepb, offb);
+                load_slab_fast<T>(ra1, ua + (kt + 3) * stepa, offa);
+                load_slab_fast<T>(rb1, ub + (kt + 3) * stepb, offb);
             }
             compute(smem[1]);
             if (kt + 2 < ntiles) {
-                store_slab<T, WTM, A_KC>(smem[0], ra0, tid);
-                store_slab<T, WTN, B_KC>(smem[0] + SA, rb0, tid);
+                store_slab<T, WT, A_KC>(smem[0], ra0, tid);
+                store_slab<T, WT, B_KC>(smem[0] + SA, rb0, tid);
             }
             __syncthreads();
         }
         if (ntiles & 1) compute(smem[0]);  // an odd last slab was staged into stage 0
     } else {
-        Vec ra[WTM], rb[WTN];
-        load_slab<T, WTM, A_KC, true>(ra, A, p.lda, row0, p.M, 0, K, tid);
-        load_slab<T, WTN, B_KC, true>(rb, B, p.ldb, col0, p.N, 0, K, tid);
-        store_slab<T, WTM, A_KC>(smem[0], ra, tid);
-        store_slab<T, WTN, B_KC>(smem[0] + SA, rb, tid);
+        Vec ra[NV], rb[NV];
+        load_slab_guarded<T, WT, A_KC>(ra, A, p.lda, row0, p.M, 0, K, tid);
+        load_slab_guarded<T, WT, B_KC>(rb, B, p.ldb, col0, p.N, 0, K, tid);
+        store_slab<T, WT, A_KC>(smem[0], ra, tid);
+        store_slab<T, WT, B_KC>(smem[0] + SA, rb, tid);
         __syncthreads();
         int cur = 0;
         for (int kt = 0; kt < ntiles; ++kt) {
             const bool more = kt + 1 < ntiles;
             if (more) {
-                load_slab<T, WTM, A_KC, true>(ra, A, p.lda, row0, p.M, (int64_t)(kt + 1) * BK, K, tid);
-                load_slab<T, WTN, B_KC, true>(rb, B, p.ldb, col0, p.N, (int64_t)(kt + 1) * BK, K, tid);
+                load_slab_guarded<T, WT, A_KC>(ra, A, p.lda, row0, p.M, (int64_t)(kt + 1) * BK, K, tid);
+                load_slab_guarded<T, WT, B_KC>(rb, B, p.ldb, col0, p.N, (int64_t)(kt + 1) * BK, K, tid);
             }
             compute(smem[cur]);
             if (more) {
-                store_slab<T, WTM, A_KC>(smem[cur ^ 1], ra, tid);
-                store_slab<T, WTN, B_KC>(smem[cur ^ 1] + SA, rb, tid);
+                store_slab<T, WT, A_KC>(smem[cur ^ 1], ra, tid);
+                store_slab<T, WT, B_KC>(smem[cur ^ 1] + SA, rb, tid);
             }
             __syncthreads();
             cur ^= 1;
@@ -336,10 +320,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WTM, WTN)) gemm_kerne
     for (int x = 0; x < WTM; ++x) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int64_t i = row0 + wm * WSM + x * 16 + MF::row(r, g);
+            const int64_t i = row0 + wm * WS + x * 16 + MF::row(r, g);
 #pragma unroll
             for (int y = 0; y < WTN; ++y) {
-                const int64_t j = col0 + wn * WSN + y * 16 + li;
+                const int64_t j = col0 + wn * WS + y * 16 + li;
                 if (EDGE && (i >= p.M || j >= p.N)) continue;
                 T v = acc[x][y][r];
                 if (EPI) {
@@ -356,37 +340,37 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WTM, WTN)) gemm_kerne
     }
 }
 
-template <typename T, int WTM, int WTN, bool A_KC, bool B_KC>
+template <typename T, int WT, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, bool epi, hipStream_t stream) {
-    constexpr int BM = 32 * WTM, BN = 32 * WTN;
-    const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BN - 1) / BN);
+    constexpr int BM = 32 * WT;
+    const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BM - 1) / BM);
     dim3 grid((unsigned)(tilesM * tilesN), (unsigned)a.batch, 1), block(GEMM_THREADS, 1, 1);
     if (edge) {
-        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, true, true>), grid, block, 0, stream, a, tilesM, tilesN);
-        else hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, true, false>), grid, block, 0, stream, a, tilesM, tilesN);
+        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, true, true>), grid, block, 0, stream, a, tilesM, tilesN);
+        else hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, true, false>), grid, block, 0, stream, a, tilesM, tilesN);
     } else {
-        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, false, true>), grid, block, 0, stream, a, tilesM, tilesN);
-        else hipLaunchKernelGGL((gemm_kernel<T, WTM, WTN, A_KC, B_KC, false, false>), grid, block, 0, stream, a, tilesM, tilesN);
+        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, false, true>), grid, block, 0, stream, a, tilesM, tilesN);
+        else hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, false, false>), grid, block, 0, stream, a, tilesM, tilesN);
     }
     return hipGetLastError();
 }
 
-template <typename T, int WTM, int WTN>
+template <typename T, int WT>
 static hipError_t launch_tile(const GemmArgs<T>& a, bool epi, hipStream_t stream) {
     constexpr int VEC = Mfma<T>::VEC;
-    constexpr int BK = Mfma<T>::BK;
-    constexpr int BM = 32 * WTM, BN = 32 * WTN;
+    constexpr int BK = Slab<T, WT>::BK;
+    constexpr int BM = 32 * WT;
     // The unguarded kernels use 16-byte loads on whole tiles.
-    const bool aligned = (a.M % BM == 0) && (a.N % BN == 0) && (a.K % BK == 0) && a.K > 0 && (a.lda % VEC == 0) &&
+    const bool aligned = (a.M % BM == 0) && (a.N % BM == 0) && (a.K % BK == 0) && a.K > 0 && (a.lda % VEC == 0) &&
                          (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
                          // per-thread element offsets inside one tile's slab are kept in 32 bits
                          (a.lda < (1 << 23)) && (a.ldb < (1 << 23));
     // Grid y carries the batch; the tile count must fit the 1-D grid.
-    if ((int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN) > 0x7fffffffLL || a.batch > 65535) return hipErrorInvalidValue;
-    if (!a.transA && !a.transB) return launch_layout<T, WTM, WTN, true, false>(a, !aligned, epi, stream);
-    if (!a.transA && a.transB) return launch_layout<T, WTM, WTN, true, true>(a, !aligned, epi, stream);
-    return launch_layout<T, WTM, WTN, false, false>(a, !aligned, epi, stream);
+    if ((int64_t)((a.M + BM - 1) / BM) * ((a.N + BM - 1) / BM) > 0x7fffffffLL || a.batch > 65535) return hipErrorInvalidValue;
+    if (!a.transA && !a.transB) return launch_layout<T, WT, true, false>(a, !aligned, epi, stream);
+    if (!a.transA && a.transB) return launch_layout<T, WT, true, true>(a, !aligned, epi, stream);
+    return launch_layout<T, WT, false, false>(a, !aligned, epi, stream);
 }
 
 enum TileShape { TILE_128x128, TILE_64x64, TILE_32x32 };
@@ -420,9 +404,9 @@ hipError_t launch_gemm(const GemmArgs<T>& a, hipStream_t stream) {
     const bool epi = a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE ||
                      a.tile_sums != nullptr;
     switch (choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr)) {
-        case TILE_128x128: return launch_tile<T, 4, 4>(a, epi, stream);
-        case TILE_64x64: return launch_tile<T, 2, 2>(a, epi, stream);
-        default: return launch_tile<T, 1, 1>(a, epi, stream);
+        case TILE_128x128: return launch_tile<T, 4>(a, epi, stream);
+        case TILE_64x64: return launch_tile<T, 2>(a, epi, stream);
+        default: return launch_tile<T, 1>(a, epi, stream);
     }
 }
 

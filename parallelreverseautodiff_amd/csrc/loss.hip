@@ -1,0 +1,115 @@
+// Operations that close the loop of a training step around the matrix products, so that a whole
+// forward + backward + update stays on the device: row-wise softmax
+// (src/RMAD/SoftmaxOperation.cs:45-110) and the categorical cross-entropy loss
+// (src/RMAD/Loss/CategoricalCrossEntropyLossOperation.cs:37-86).  They are tiny (batch x classes)
+// and latency-bound: one wavefront per row, no LDS.
+#include "common.h"
+
+namespace prad {
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_max(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmax(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// y[i][j] = exp(x[i][j] - max_i) / sum_j exp(x[i][j] - max_i)
+template <typename T>
+__global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols) {
+    const int64_t i = blockIdx.x;
+    const T* __restrict__ xr = x + i * cols;
+    T* __restrict__ yr = y + i * cols;
+    double mx = -INFINITY;
+    for (int64_t j = threadIdx.x; j < cols; j += 64) mx = fmax(mx, (double)xr[j]);
+    const T m = (T)wave_max(mx);
+    double sum = 0.0;
+    for (int64_t j = threadIdx.x; j < cols; j += 64) {
+        const T e = dev_exp(xr[j] - m);
+        yr[j] = e;
+        sum += (double)e;
+    }
+    const T s = (T)wave_sum(sum);
+    for (int64_t j = threadIdx.x; j < cols; j += 64) yr[j] = yr[j] / s;
+}
+
+// The reference multiplies dy with the explicit Jacobian row by row (O(cols^2)):
+//   dx[j] = dy[j]*y[j]*(1-y[j]) - sum_{k != j} dy[k]*y[j]*y[k]  =  y[j] * (dy[j] - sum_k dy[k]*y[k]).
+template <typename T>
+__global__ void __launch_bounds__(64) softmax_bwd_kernel(const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx,
+                                                         int64_t rows, int64_t cols) {
+    const int64_t i = blockIdx.x;
+    const T* __restrict__ yr = y + i * cols;
+    const T* __restrict__ gr = dy + i * cols;
+    double dot = 0.0;
+    for (int64_t j = threadIdx.x; j < cols; j += 64) dot += (double)gr[j] * (double)yr[j];
+    dot = wave_sum(dot);
+    for (int64_t j = threadIdx.x; j < cols; j += 64) dx[i * cols + j] = (T)((double)yr[j] * ((double)gr[j] - dot));
+}
+
+// loss[0] = (sum_ij -t*log(p + 1e-15)) / rows ; one workgroup.
+template <typename T>
+__global__ void __launch_bounds__(256) cce_fwd_kernel(const T* __restrict__ p, const T* __restrict__ t, T* __restrict__ loss,
+                                                      int64_t rows, int64_t cols) {
+    const int64_t n = rows * cols;
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += 256) {
+        const T term = -t[i] * (T)log((double)(p[i] + (T)1e-15));
+        s += (double)term;
+    }
+    s = wave_sum(s);
+    __shared__ double part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) loss[0] = (T)((part[0] + part[1]) + (part[2] + part[3])) / (T)rows;
+}
+
+// dp = -(1/rows) * t / (p + 1e-15)
+template <typename T>
+__global__ void __launch_bounds__(256) cce_bwd_kernel(const T* __restrict__ p, const T* __restrict__ t, T* __restrict__ dp,
+                                                      int64_t rows, int64_t cols) {
+    const int64_t n = rows * cols;
+    const T scale = (T)1 / (T)rows;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        dp[i] = -scale * t[i] / (p[i] + (T)1e-15);
+}
+
+template <typename T>
+hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL((softmax_fwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, x, y, rows, cols);
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, y, dy, dx, rows, cols);
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t launch_cce_fwd(const T* p, const T* t, T* loss, int64_t rows, int64_t cols, hipStream_t s) {
+    hipLaunchKernelGGL((cce_fwd_kernel<T>), dim3(1), dim3(256), 0, s, p, t, loss, rows, cols);
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t cols, hipStream_t s) {
+    int64_t blocks = (rows * cols + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL((cce_bwd_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, p, t, dp, rows, cols);
+    return hipGetLastError();
+}
+
+#define INSTANTIATE(T)                                                                              \
+    template hipError_t launch_softmax_fwd<T>(const T*, T*, int64_t, int64_t, hipStream_t);         \
+    template hipError_t launch_softmax_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t); \
+    template hipError_t launch_cce_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
+    template hipError_t launch_cce_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);
+INSTANTIATE(double)
+INSTANTIATE(float)
+
+}  // namespace prad

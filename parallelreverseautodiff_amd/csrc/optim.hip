@@ -58,6 +58,16 @@ __device__ __forceinline__ Moments merge(const Moments& a, const Moments& b) {
     r.m2 = a.m2 + b.m2 + delta * delta * (a.n * b.n / r.n);
     return r;
 }
+// Merge of two groups of equal size (no division): used inside full chunks, where every lane and
+// every wavefront holds the same number of elements.
+__device__ __forceinline__ Moments merge_equal(const Moments& a, const Moments& b) {
+    Moments r;
+    const double delta = b.mean - a.mean;
+    r.n = a.n + a.n;
+    r.mean = a.mean + 0.5 * delta;
+    r.m2 = a.m2 + b.m2 + delta * delta * (0.5 * a.n);
+    return r;
+}
 __device__ __forceinline__ Moments shfl_down(const Moments& a, int off) {
     Moments r;
     r.n = __shfl_down(a.n, off, 64);
@@ -125,8 +135,14 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTab
             if (i < end) { const double d = x[e] - mo.mean; mo.m2 += d * d; }
         }
     }
+    const bool full = end - begin == OPT_CHUNK;  // uniform over the workgroup
+    if (full) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mo = merge(mo, shfl_down(mo, off));
+        for (int off = 32; off > 0; off >>= 1) mo = merge_equal(mo, shfl_down(mo, off));
+    } else {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mo = merge(mo, shfl_down(mo, off));
+    }
     __shared__ Moments wave_part[OPT_THREADS / 64];
     if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = mo;
     __syncthreads();
@@ -144,7 +160,17 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_finalize_kernel(const Tensor
     const int ti = blockIdx.x;
     const int64_t c0 = tab.t[ti].first_chunk, nc = tab.t[ti].nchunks;
     Moments mo{0.0, 0.0, 0.0};
-    for (int64_t c = threadIdx.x; c < nc; c += OPT_THREADS) mo = merge(mo, partial[c0 + c]);
+    // Eight independent loads in flight per lane before the (serial) merges.
+    for (int64_t c = threadIdx.x; c < nc; c += OPT_THREADS * 8) {
+        Moments part[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int64_t idx = c + (int64_t)u * OPT_THREADS;
+            part[u] = idx < nc ? partial[c0 + idx] : Moments{0.0, 0.0, 0.0};
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) mo = merge(mo, part[u]);
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mo = merge(mo, shfl_down(mo, off));
     __shared__ Moments wave_part[OPT_THREADS / 64];

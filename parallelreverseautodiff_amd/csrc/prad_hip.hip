@@ -679,6 +679,97 @@ int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias) {
 }
 
 // ---------------------------------------------------------------------------------------------
+int32_t prad_softmax_fwd(prad_buf_t x, prad_buf_t y) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(y);
+    if (int32_t st = same_dtype({x, y})) return st;
+    if (int32_t st = same_shape(x, y, "softmax")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_softmax_fwd<double>(D(x), D(y), x->depth * x->rows, x->cols, g_ctx.stream),
+             launch_softmax_fwd<float>(F(x), F(y), x->depth * x->rows, x->cols, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_softmax_bwd(prad_buf_t y, prad_buf_t dy, prad_buf_t dx) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(y); REQUIRE_BUF(dy); REQUIRE_BUF(dx);
+    if (int32_t st = same_dtype({y, dy, dx})) return st;
+    if (int32_t st = same_shape(y, dy, "softmax backward")) return st;
+    if (int32_t st = same_shape(y, dx, "softmax backward")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(y, launch_softmax_bwd<double>(D(y), D(dy), D(dx), y->depth * y->rows, y->cols, g_ctx.stream),
+             launch_softmax_bwd<float>(F(y), F(dy), F(dx), y->depth * y->rows, y->cols, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_cce_fwd(prad_buf_t p, prad_buf_t target, prad_buf_t loss) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(p); REQUIRE_BUF(target); REQUIRE_BUF(loss);
+    if (int32_t st = same_dtype({p, target, loss})) return st;
+    if (p->depth != 1 || p->rows != target->rows || p->cols != target->cols || target->depth != 1)
+        return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
+    if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(p, launch_cce_fwd<double>(D(p), D(target), D(loss), p->rows, p->cols, g_ctx.stream),
+             launch_cce_fwd<float>(F(p), F(target), F(loss), p->rows, p->cols, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_cce_bwd(prad_buf_t p, prad_buf_t target, prad_buf_t dp) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(p); REQUIRE_BUF(target); REQUIRE_BUF(dp);
+    if (int32_t st = same_dtype({p, target, dp})) return st;
+    if (p->depth != 1 || p->rows != target->rows || p->cols != target->cols || target->depth != 1)
+        return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
+    if (int32_t st = same_shape(p, dp, "cross-entropy backward")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(p, launch_cce_bwd<double>(D(p), D(target), D(dp), p->rows, p->cols, g_ctx.stream),
+             launch_cce_bwd<float>(F(p), F(target), F(dp), p->rows, p->cols, g_ctx.stream));
+    return PRAD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Recording holds the context lock's place in line only per call: other threads must not enqueue
+// while a recording is open (their work would be recorded too), which the caller guarantees.
+int32_t prad_graph_begin(void) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipStreamBeginCapture(g_ctx.stream, hipStreamCaptureModeThreadLocal), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+int32_t prad_graph_end(void** graph) {
+    REQUIRE_INIT();
+    if (graph == nullptr) return fail(PRAD_ERR_ARG, "graph is NULL");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    hipGraph_t g = nullptr;
+    HIP_TRY(hipStreamEndCapture(g_ctx.stream, &g), PRAD_ERR_LAUNCH);
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return fail(PRAD_ERR_LAUNCH, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    *graph = exec;
+    return PRAD_OK;
+}
+
+int32_t prad_graph_launch(void* graph) {
+    REQUIRE_INIT();
+    if (graph == nullptr) return fail(PRAD_ERR_ARG, "graph is NULL");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), g_ctx.stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+int32_t prad_graph_destroy(void* graph) {
+    REQUIRE_INIT();
+    if (graph == nullptr) return PRAD_OK;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)), PRAD_ERR_ARG);
+    return PRAD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
 int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, double min_value) {
     REQUIRE_INIT();
     if (n < 0 || (n > 0 && g == nullptr)) return fail(PRAD_ERR_ARG, "bad tensor list");

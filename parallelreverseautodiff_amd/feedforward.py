@@ -1,0 +1,130 @@
+"""Device-resident training step of the feed-forward configuration: the call sequence the reference's
+training loop makes (forward walk over the operation list, loss, backward visitor with gradient
+accumulation, clip, Adam: examples/feedforward/FeedForwardNeuralNetworkExample/FeedForwardNeuralNetwork.cs:212-358)
+replayed on pre-allocated device buffers, either launch by launch or as one recorded submission.
+
+Network: X (batch x n0) -> [MatrixMultiply(W_l) -> MatrixAddBroadcasting(b_l) -> LeakyReLU] x (L-1)
+         -> MatrixMultiply(W_L) -> MatrixAddBroadcasting(b_L) -> Softmax -> CategoricalCrossEntropy.
+Per layer the product, the bias add and the activation are one launch (fused epilogue), and the
+activation's Backward is the epilogue of the next layer's dA product.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib, seeded
+from .exceptions import check
+from .matrix import DeviceBuffer
+from .operations import _ensure_initialized, handle_array
+from .optim import NeuralNetworkParameters
+
+
+class FeedForwardNetwork:
+    def __init__(self, sizes=(784, 256, 128, 10), batch=64, dtype=np.float64, seed=seeded.DEFAULT_SEED, parameters=None):
+        _ensure_initialized()
+        self.lib = _lib.load()
+        self.dtype = np.dtype(dtype)
+        self.sizes, self.batch = tuple(sizes), batch
+        self.params = parameters or NeuralNetworkParameters(lite=self.dtype == np.float32)
+        L = len(sizes) - 1
+        alloc = lambda r, c: DeviceBuffer.alloc(self.dtype, r, c)
+        # weights Xavier-uniform, biases zero (Matrix.InitializeXavier, src/RMAD/Matrix.cs:1037-1046)
+        self.host_W = [seeded.xavier(seed, 10 + l, sizes[l], sizes[l + 1], self.dtype) for l in range(L)]
+        self.W = [alloc(sizes[l], sizes[l + 1]) for l in range(L)]
+        self.b = [alloc(1, sizes[l + 1]) for l in range(L)]
+        for w, h in zip(self.W, self.host_W):
+            w.upload(h)
+        self.dW = [alloc(sizes[l], sizes[l + 1]) for l in range(L)]
+        self.db = [alloc(1, sizes[l + 1]) for l in range(L)]
+        self.mW = [alloc(sizes[l], sizes[l + 1]) for l in range(L)]
+        self.vW = [alloc(sizes[l], sizes[l + 1]) for l in range(L)]
+        self.mb = [alloc(1, sizes[l + 1]) for l in range(L)]
+        self.vb = [alloc(1, sizes[l + 1]) for l in range(L)]
+        self.X = alloc(batch, sizes[0])
+        self.T = alloc(batch, sizes[-1])
+        self.Z = [alloc(batch, sizes[l + 1]) for l in range(L)]      # pre-activations (what LeakyReLU caches)
+        self.H = [alloc(batch, sizes[l + 1]) for l in range(L - 1)]  # activations
+        self.P = alloc(batch, sizes[-1])                             # softmax output
+        self.loss = alloc(1, 1)
+        self.dP = alloc(batch, sizes[-1])
+        self.dZ = [alloc(batch, sizes[l + 1]) for l in range(L)]
+        self.dX = alloc(batch, sizes[0])
+        self.iteration = 0
+        self._graph = None
+        self._weights = self.W + self.b
+        self._grads = self.dW + self.db
+        self._m = self.mW + self.mb
+        self._v = self.vW + self.vb
+
+    def set_batch(self, X, T):
+        self.X.upload(X)
+        self.T.upload(T)
+
+    # ---- one step, launch by launch ------------------------------------------------------------
+    def _enqueue_forward_backward(self):
+        lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
+        a = self.X
+        for l in range(L):
+            last = l == L - 1
+            out = self.Z[l] if last else self.H[l]
+            z = None if last else self.Z[l].handle
+            check(lib.prad_matmul_fwd_fused(a.handle, self.W[l].handle, self.b[l].handle, z, out.handle,
+                                            _lib.ACT_NONE if last else _lib.ACT_LEAKYRELU, alpha))
+            a = out
+        check(lib.prad_softmax_fwd(self.Z[-1].handle, self.P.handle))
+        check(lib.prad_cce_fwd(self.P.handle, self.T.handle, self.loss.handle))
+        check(lib.prad_cce_bwd(self.P.handle, self.T.handle, self.dP.handle))
+        check(lib.prad_softmax_bwd(self.P.handle, self.dP.handle, self.dZ[-1].handle))
+        for l in range(L - 1, -1, -1):
+            inp = self.X if l == 0 else self.H[l - 1]
+            check(lib.prad_add_broadcast_bwd_bias(self.dZ[l].handle, self.db[l].handle))
+            if l == 0:
+                # MatrixMultiplyOperation.Backward always forms both gradients, also for the input
+                check(lib.prad_matmul_bwd(self.dZ[0].handle, inp.handle, self.W[0].handle, self.dX.handle, self.dW[0].handle, 0, 0))
+            else:
+                check(lib.prad_matmul_bwd_fused(self.dZ[l].handle, inp.handle, self.W[l].handle, self.dZ[l - 1].handle,
+                                                self.dW[l].handle, 0, _lib.ACT_LEAKYRELU, self.Z[l - 1].handle, alpha))
+
+    def _enqueue_update(self, t):
+        p = self.params
+        n = len(self._grads)
+        check(self.lib.prad_clip_multi(handle_array(self._grads), n, float(p.ClipValue), float(p.MinimumClipValue)))
+        check(self.lib.prad_adam_multi(handle_array(self._weights), handle_array(self._m), handle_array(self._v),
+                                       handle_array(self._grads), n, float(p.LearningRate), float(p.AdamBeta1),
+                                       float(p.AdamBeta2), float(p.AdamEpsilon), float(t)))
+
+    def step(self):
+        """Forward, loss, backward, clip, Adam (AdamIteration = step number, as the reference's caller sets it)."""
+        self.iteration += 1
+        self._enqueue_forward_backward()
+        self._enqueue_update(self.iteration)
+
+    # ---- one step as a recorded launch sequence ------------------------------------------------
+    def record(self, adam_iteration=1.0):
+        """Records one step with a fixed AdamIteration (the bias-correction factors are launch arguments);
+        one eager step must have run before so that shared workspace is already sized."""
+        lib = self.lib
+        check(lib.prad_graph_begin())
+        try:
+            self._enqueue_forward_backward()
+            self._enqueue_update(adam_iteration)
+        finally:
+            g = ctypes.c_void_p()
+            check(lib.prad_graph_end(ctypes.byref(g)))
+        self._graph = g
+        return g
+
+    def replay(self):
+        check(self.lib.prad_graph_launch(self._graph))
+
+    def release(self):
+        if self._graph is not None:
+            check(self.lib.prad_graph_destroy(self._graph))
+            self._graph = None
+
+    def flops_per_step(self):
+        fwd = sum(2.0 * self.batch * self.sizes[l] * self.sizes[l + 1] for l in range(len(self.W)))
+        return 3.0 * fwd
+
+    def parameter_count(self):
+        return sum(self.sizes[l] * self.sizes[l + 1] + self.sizes[l + 1] for l in range(len(self.W)))

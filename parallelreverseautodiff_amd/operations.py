@@ -462,3 +462,55 @@ def accumulate_gradient(dest, grad):
 def handle_array(buffers):
     """ctypes array of prad_buf_t for the multi-tensor entry points."""
     return (ctypes.c_void_p * len(buffers))(*[b.handle.value for b in buffers])
+
+
+class SoftmaxOperation(Operation):
+    """Row-wise softmax (src/RMAD/SoftmaxOperation.cs:45-110)."""
+
+    @staticmethod
+    def Instantiate(net):
+        return SoftmaxOperation()
+
+    def Forward(self, input):
+        _ensure_initialized()
+        out = DeviceBuffer.alloc(input.dtype, input.Rows, input.Cols)
+        check(_lib.load().prad_softmax_fwd(input.device().handle, out.handle))
+        self.Output = Matrix._from_device(out)
+        return self.Output
+
+    def Backward(self, dLdOutput):
+        _ensure_initialized()
+        y = self.Output
+        dx = DeviceBuffer.alloc(y.dtype, y.Rows, y.Cols)
+        check(_lib.load().prad_softmax_bwd(y.device().handle, dLdOutput.device().handle, dx.handle))
+        return BackwardResultBuilder().AddInputGradient(Matrix._from_device(dx)).Build()
+
+
+class CategoricalCrossEntropyLossOperation(Operation):
+    """loss = sum(-t log(p + 1e-15)) / rows (src/RMAD/Loss/CategoricalCrossEntropyLossOperation.cs:37-86)."""
+
+    def __init__(self):
+        super().__init__()
+        self.target = None
+
+    @staticmethod
+    def Instantiate(net):
+        return CategoricalCrossEntropyLossOperation()
+
+    def Forward(self, output, target):
+        _ensure_initialized()
+        if target is None:
+            raise ArgumentException("target")
+        if output.Rows != target.Rows or output.Cols != target.Cols:
+            raise ArgumentException("Output and target matrices must have the same dimensions.")
+        self.target = target
+        loss = DeviceBuffer.alloc(output.dtype, 1, 1)
+        check(_lib.load().prad_cce_fwd(output.device().handle, target.device().handle, loss.handle))
+        self.Output = Matrix._from_device(loss)
+        return self.Output
+
+    def Backward(self, output):
+        _ensure_initialized()
+        dp = DeviceBuffer.alloc(output.dtype, output.Rows, output.Cols)
+        check(_lib.load().prad_cce_bwd(output.device().handle, self.target.device().handle, dp.handle))
+        return BackwardResultBuilder().AddInputGradient(Matrix._from_device(dp)).Build()

@@ -80,7 +80,8 @@ def test_add_broadcast_and_bias_gradient(gpu, oracle, dtype):
     g = Matrix.from_numpy(dy)
     res = op.Backward(g)
     assert res.Item1 is g and not res.HasMultipleInputs  # dOutput is passed through, not copied
-    assert np.array_equal(res.Item2.to_numpy(), oracle.add_broadcast_bwd_bias(dy))
+    # the column sum is taken by four wavefronts and combined, not row by row: same value within rounding
+    assert_parity(res.Item2.to_numpy(), oracle.add_broadcast_bwd_bias(dy), dtype, "bias gradient")
 
 
 def test_large_vector_tail_and_size(gpu, oracle):
