@@ -205,7 +205,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
             for (int r = 0; r < 4; ++r) acc[x][y][r] = (T)0;
 
     const int64_t K = p.K;
-    const int ntiles = (int)((K + BK - 1) / BK);
+    // Unguarded kernels run the whole slabs with vector loads and finish a ragged end of K (784 = 12 x 64 + 16)
+    // with one guarded slab; guarded kernels treat every slab alike.
+    const int ntiles = EDGE ? (int)((K + BK - 1) / BK) : (int)(K / BK);
 
     // One slab of MFMAs from the LDS stage at `st`.
     auto compute = [&](const T* __restrict__ st) {
@@ -240,14 +242,18 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         const T* __restrict__ ub = B + (B_KC ? col0 * p.ldb : col0);
         const int64_t stepa = A_KC ? (int64_t)BK : (int64_t)BK * p.lda;
         const int64_t stepb = B_KC ? (int64_t)BK : (int64_t)BK * p.ldb;
-        load_slab_fast<T>(ra0, ua, offa);
-        load_slab_fast<T>(rb0, ub, offb);
+        if (ntiles > 0) {
+            load_slab_fast<T>(ra0, ua, offa);
+            load_slab_fast<T>(rb0, ub, offb);
+        }
         if (ntiles > 1) {
             load_slab_fast<T>(ra1, ua + stepa, offa);
             load_slab_fast<T>(rb1, ub + stepb, offb);
         }
-        store_slab<T, WT, A_KC>(smem[0], ra0, tid);
-        store_slab<T, WT, B_KC>(smem[0] + SA, rb0, tid);
+        if (ntiles > 0) {
+            store_slab<T, WT, A_KC>(smem[0], ra0, tid);
+            store_slab<T, WT, B_KC>(smem[0] + SA, rb0, tid);
+        }
         __syncthreads();
         for (int kt = 0; kt + 1 < ntiles; kt += 2) {
             // LDS stage 0 holds slab kt, set 1 holds slab kt+1 (in flight), set 0 is free.
@@ -271,6 +277,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
             __syncthreads();
         }
         if (ntiles & 1) compute(smem[0]);  // an odd last slab was staged into stage 0
+        if ((int64_t)ntiles * BK < K) {    // ragged end of K: one guarded slab through stage 1
+            load_slab_guarded<T, WT, A_KC>(ra1, A, p.lda, row0, p.M, (int64_t)ntiles * BK, K, tid);
+            load_slab_guarded<T, WT, B_KC>(rb1, B, p.ldb, col0, p.N, (int64_t)ntiles * BK, K, tid);
+            store_slab<T, WT, A_KC>(smem[1], ra1, tid);
+            store_slab<T, WT, B_KC>(smem[1] + SA, rb1, tid);
+            __syncthreads();
+            compute(smem[1]);
+        }
     } else {
         Vec ra[NV], rb[NV];
         load_slab_guarded<T, WT, A_KC>(ra, A, p.lda, row0, p.M, 0, K, tid);
@@ -358,10 +372,9 @@ static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, bool epi, hipSt
 template <typename T, int WT>
 static hipError_t launch_tile(const GemmArgs<T>& a, bool epi, hipStream_t stream) {
     constexpr int VEC = Mfma<T>::VEC;
-    constexpr int BK = Slab<T, WT>::BK;
     constexpr int BM = 32 * WT;
-    // The unguarded kernels use 16-byte loads on whole tiles.
-    const bool aligned = (a.M % BM == 0) && (a.N % BM == 0) && (a.K % BK == 0) && a.K > 0 && (a.lda % VEC == 0) &&
+    // The unguarded kernels use 16-byte loads on whole tiles (any K: a ragged end is handled inside).
+    const bool aligned = (a.M % BM == 0) && (a.N % BM == 0) && a.K > 0 && (a.lda % VEC == 0) &&
                          (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
                          // per-thread element offsets inside one tile's slab are kept in 32 bits

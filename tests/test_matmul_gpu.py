@@ -25,6 +25,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SHAPES = [  # M, K, N: tile-aligned, ragged in every dimension, degenerate vectors, MLP layers
     (128, 128, 128), (256, 64, 384), (1, 1, 1), (1, 7, 1), (5, 3, 2), (127, 129, 130), (129, 17, 3), (257, 33, 65),
     (64, 784, 256), (64, 256, 128), (64, 128, 10), (100, 100, 1), (1, 100, 100), (384, 512, 256), (130, 260, 390),
+    # whole tiles with a ragged reduction: one slab plus a tail, a tail only, an odd number of slabs
+    (128, 70, 64), (64, 40, 32), (256, 200, 256), (512, 1000, 512), (2048, 24, 2048),
 ]
 
 
