@@ -129,6 +129,51 @@ def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
     return out, n
 
 
+def matmul_sum_leg(dtype_name, steps, warmup):
+    """configs[2]: MatrixMultiplyAndSum, A 512x768, 32 slices of 768x512, forward (MFMA, 12.88 GFLOP) and the
+    reference's backward (data movement: read A and B once, write dA and dB once = 103.8 MB in float)."""
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = 0
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    M, K, P = 512, 768, 32
+    A = DeviceBuffer.alloc(dtype, M, K); B = DeviceBuffer.alloc(dtype, K, M, depth=P)
+    out = DeviceBuffer.alloc(dtype, 1, P); dOut = DeviceBuffer.alloc(dtype, 1, P)
+    dA = DeviceBuffer.alloc(dtype, M, K); dB = DeviceBuffer.alloc(dtype, K, M, depth=P)
+    A.upload(seeded.normal(seeded.DEFAULT_SEED, 1, (M, K), 0.02, dtype))
+    B.upload(seeded.normal(seeded.DEFAULT_SEED, 2, (P, K, M), 0.02, dtype))
+    dOut.upload(seeded.normal(seeded.DEFAULT_SEED, 3, (1, P), 1.0, dtype))
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.prad_event_create(ctypes.byref(e0)))
+    check(lib.prad_event_create(ctypes.byref(e1)))
+
+    def timed(fn):
+        for _ in range(warmup):
+            check(fn())
+        check(lib.prad_stream_sync())
+        check(lib.prad_event_record(e0))
+        for _ in range(steps):
+            check(fn())
+        check(lib.prad_event_record(e1))
+        ms = ctypes.c_float()
+        check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        return ms.value / steps
+
+    fwd_ms = timed(lambda: lib.prad_matmul_sum_fwd(A.handle, B.handle, out.handle))
+    bwd_ms = timed(lambda: lib.prad_matmul_sum_bwd(A.handle, B.handle, dOut.handle, dA.handle, dB.handle))
+    es = np.dtype(dtype).itemsize
+    flops = 2.0 * M * K * M * P
+    bytes_bwd = 2.0 * (M * K + P * K * M) * es
+    return {"fwd_ms": fwd_ms, "fwd_TFLOPs": flops / (fwd_ms * 1e-3) / 1e12, "fwd_frac_of_mfma_peak": flops / (fwd_ms * 1e-3) / 1e12 / PEAK_TFLOPS[dtype_name],
+            "bwd_ms": bwd_ms, "bwd_GBps": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "bwd_frac_of_8TBps": bytes_bwd / (bwd_ms * 1e-3) / 8e12,
+            "fwd_flop": flops, "bwd_bytes": bytes_bwd}
+
+
 def mlp_leg(dtype_name, steps, warmup, with_cpu):
     """Feed-forward training step of configs[0]: batch 64, 784-256-128-10, LeakyReLU(0.01), softmax
     cross-entropy, clip, Adam.  Timed launch by launch and as one recorded launch sequence."""
@@ -256,7 +301,7 @@ def main():
     ap.add_argument("--n", type=int, default=4096)
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp"], default="gemm",
+    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum"], default="gemm",
                     help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
                          "mlp: the feed-forward training step of configs[0]")
     ap.add_argument("--elems", type=int, default=64 * 1024 * 1024, help="elements per tensor in bandwidth mode")
@@ -264,6 +309,15 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: this path has no multi-GPU part (--gpus 1 only)")
+    if args.mode == "matmul_sum":
+        res = matmul_sum_leg(args.dtype, args.steps, args.warmup)
+        print(json.dumps({"metric": "MatrixMultiplyAndSum forward TFLOP/s, backward GB/s", "unit": "TFLOP/s", "value": res["fwd_TFLOPs"],
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
+                          "higher_is_better": True, "ms_per_step": res["fwd_ms"] + res["bwd_ms"],
+                          "config": {"workload": "configs[2]: GpuMatrixMultiplyAndSumOperation, A 512x768 ~N(0,0.02), 32 slices 768x512, "
+                                                 "reference semantics (out 1x32; backward as written)"},
+                          "detail": res}))
+        return
     if args.mode == "mlp":
         res = mlp_leg(args.dtype, args.steps, args.warmup, not args.no_cpu)
         print(json.dumps({"metric": "MLP train steps/sec", "unit": "steps/s", "value": 1e3 / res["recorded_ms_per_step"],

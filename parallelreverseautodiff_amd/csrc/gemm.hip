@@ -167,9 +167,14 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tilesM, int tiles
     tn = in_group / gsz;
 }
 
-constexpr int min_blocks(int wt) { return wt >= 4 ? 2 : 4; }
+constexpr int min_blocks(int) { return 2; }
 
-template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, bool EPI>
+// Epilogue kinds (template argument EPI).
+constexpr int EPI_PLAIN = 0;      // store (or accumulate into) C
+constexpr int EPI_ELEMENTWISE = 1;  // bias / pre-activation copy / activation forward / upstream activation backward
+constexpr int EPI_TILE_SUM = 2;   // reduce the tile to one double (MatrixMultiplyAndSum forward)
+
+template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI>
 __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
                                                                             const int tilesN) {
     typedef Mfma<T> MF;
@@ -310,7 +315,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     }
 
     // ---- epilogue ------------------------------------------------------------------------
-    if (EPI && p.tile_sums != nullptr) {
+    if (EPI == EPI_TILE_SUM) {
         // Sum of the whole tile (rows/columns past M, N hold exact zeros).
         double s = 0.0;
 #pragma unroll
@@ -321,6 +326,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
                 for (int r = 0; r < 4; ++r) s += (double)acc[x][y][r];
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
+        __syncthreads();  // every wavefront is done with the slab stages
         double* red = reinterpret_cast<double*>(&smem[0][0]);
         if (lane == 0) red[wave] = s;
         __syncthreads();
@@ -330,6 +336,40 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     }
 
     T* __restrict__ C = p.C + batch * p.strideC;
+    if (EPI == EPI_ELEMENTWISE) {
+        // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
+        // row-major: the elementwise arithmetic (which includes exp/tanh code) then sits in one runtime loop
+        // instead of being inlined into 64 unrolled stores, and every global access covers whole rows.
+        constexpr int LDW = WS + 4;
+        __syncthreads();  // every wavefront is done with the slab stages
+        T* __restrict__ stage = &smem[0][0] + wave * (16 * LDW);
+#pragma unroll
+        for (int x = 0; x < WTM; ++x) {
+#pragma unroll
+            for (int y = 0; y < WTN; ++y)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) stage[MF::row(r, g) * LDW + y * 16 + li] = acc[x][y][r];
+            __syncthreads();
+#pragma unroll 1
+            for (int idx = lane; idx < 16 * WS; idx += 64) {
+                const int rr = idx / WS, c = idx % WS;
+                const int64_t i = row0 + wm * WS + x * 16 + rr;
+                const int64_t j = col0 + wn * WS + c;
+                if (EDGE && (i >= p.M || j >= p.N)) continue;
+                T v = stage[rr * LDW + c];
+                if (p.bias != nullptr) v = v + p.bias[j];
+                if (p.Z != nullptr) p.Z[i * p.ldz + j] = v;
+                if (p.act_fwd != ACT_NONE) v = act_forward<T>(p.act_fwd, v, p.alpha);
+                if (p.act_bwd != ACT_NONE) v = v * act_derivative<T>(p.act_bwd, p.act_src[i * p.ld_act + j], p.alpha);
+                T* c_out = C + i * p.ldc + j;
+                if (p.accumulate) v = *c_out + v;
+                *c_out = v;
+            }
+            __syncthreads();
+        }
+        return;
+    }
+
 #pragma unroll
     for (int x = 0; x < WTM; ++x) {
 #pragma unroll
@@ -340,12 +380,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
                 const int64_t j = col0 + wn * WS + y * 16 + li;
                 if (EDGE && (i >= p.M || j >= p.N)) continue;
                 T v = acc[x][y][r];
-                if (EPI) {
-                    if (p.bias != nullptr) v = v + p.bias[j];
-                    if (p.Z != nullptr) p.Z[i * p.ldz + j] = v;
-                    if (p.act_fwd != ACT_NONE) v = act_forward<T>(p.act_fwd, v, p.alpha);
-                    if (p.act_bwd != ACT_NONE) v = v * act_derivative<T>(p.act_bwd, p.act_src[i * p.ld_act + j], p.alpha);
-                }
                 T* c = C + i * p.ldc + j;
                 if (p.accumulate) v = *c + v;
                 *c = v;
@@ -355,22 +389,27 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
 }
 
 template <typename T, int WT, bool A_KC, bool B_KC>
-static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, bool epi, hipStream_t stream) {
+static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStream_t stream) {
     constexpr int BM = 32 * WT;
     const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BM - 1) / BM);
     dim3 grid((unsigned)(tilesM * tilesN), (unsigned)a.batch, 1), block(GEMM_THREADS, 1, 1);
+#define PRAD_LAUNCH(EDGE_, EPI_) \
+    hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, EDGE_, EPI_>), grid, block, 0, stream, a, tilesM, tilesN)
     if (edge) {
-        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, true, true>), grid, block, 0, stream, a, tilesM, tilesN);
-        else hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, true, false>), grid, block, 0, stream, a, tilesM, tilesN);
+        if (epi == EPI_PLAIN) PRAD_LAUNCH(true, EPI_PLAIN);
+        else if (epi == EPI_ELEMENTWISE) PRAD_LAUNCH(true, EPI_ELEMENTWISE);
+        else PRAD_LAUNCH(true, EPI_TILE_SUM);
     } else {
-        if (epi) hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, false, true>), grid, block, 0, stream, a, tilesM, tilesN);
-        else hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, false, false>), grid, block, 0, stream, a, tilesM, tilesN);
+        if (epi == EPI_PLAIN) PRAD_LAUNCH(false, EPI_PLAIN);
+        else if (epi == EPI_ELEMENTWISE) PRAD_LAUNCH(false, EPI_ELEMENTWISE);
+        else PRAD_LAUNCH(false, EPI_TILE_SUM);
     }
+#undef PRAD_LAUNCH
     return hipGetLastError();
 }
 
 template <typename T, int WT>
-static hipError_t launch_tile(const GemmArgs<T>& a, bool epi, hipStream_t stream) {
+static hipError_t launch_tile(const GemmArgs<T>& a, int epi, hipStream_t stream) {
     constexpr int VEC = Mfma<T>::VEC;
     constexpr int BM = 32 * WT;
     // The unguarded kernels use 16-byte loads on whole tiles (any K: a ragged end is handled inside).
@@ -414,8 +453,9 @@ template <typename T>
 hipError_t launch_gemm(const GemmArgs<T>& a, hipStream_t stream) {
     if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return hipSuccess;
     if (a.transA && a.transB) return hipErrorInvalidValue;
-    const bool epi = a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE ||
-                     a.tile_sums != nullptr;
+    const int epi = a.tile_sums != nullptr ? EPI_TILE_SUM
+                    : (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) ? EPI_ELEMENTWISE
+                                                                                                             : EPI_PLAIN;
     switch (choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr)) {
         case TILE_128x128: return launch_tile<T, 4>(a, epi, stream);
         case TILE_64x64: return launch_tile<T, 2>(a, epi, stream);
