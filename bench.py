@@ -174,6 +174,55 @@ def matmul_sum_leg(dtype_name, steps, warmup):
             "fwd_flop": flops, "bwd_bytes": bytes_bwd}
 
 
+def lstm_leg(dtype_name, steps, warmup, with_cpu):
+    """configs[3]: one LSTM layer, input 256, hidden 512, batch 128, 64 time steps, fused 4-gate weight,
+    MSE on the hidden states, backprop through time, clip, Adam."""
+    from parallelreverseautodiff_amd import _lib
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.lstm import LSTMLayer
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = 0
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    layer = LSTMLayer(dtype=dtype)
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.prad_event_create(ctypes.byref(e0)))
+    check(lib.prad_event_create(ctypes.byref(e1)))
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        check(lib.prad_stream_sync())
+        check(lib.prad_event_record(e0))
+        for _ in range(steps):
+            fn()
+        check(lib.prad_event_record(e1))
+        check(lib.prad_stream_sync())
+        ms = ctypes.c_float()
+        check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        return ms.value / steps
+
+    eager_ms = timed(layer.step)
+    layer.record(adam_iteration=float(layer.iteration + 1))
+    rec_ms = timed(layer.replay)
+    layer.release()
+    flops = layer.flops_per_step()
+    out = {"eager_ms_per_step": eager_ms, "recorded_ms_per_step": rec_ms, "flop_per_step": flops,
+           "TFLOPs": flops / (rec_ms * 1e-3) / 1e12, "loss_after": float(layer.loss.download()[0, 0])}
+    if with_cpu:
+        from oracle import compose, oracle
+        threads = min(16, oracle.hardware_threads() or 1)
+        I, H, B, T = layer.input_dim, layer.hidden, layer.batch, layer.steps
+        t0 = time.perf_counter()
+        compose.lstm_forward_backward(layer.host_W, np.zeros((1, 4 * H), dtype), layer.host_X, layer.host_Y, I, H, B, T, threads=threads)
+        secs = time.perf_counter() - t0
+        out["cpu"] = {"steps_per_s": 1.0 / secs, "ms_per_step": secs * 1e3, "cores": threads, "steps_timed": 1, "kind": "port",
+                      "note": "forward + backward only (no clip/Adam), node-by-node composition of the oracle's operations"}
+    return out
+
+
 def mlp_leg(dtype_name, steps, warmup, with_cpu):
     """Feed-forward training step of configs[0]: batch 64, 784-256-128-10, LeakyReLU(0.01), softmax
     cross-entropy, clip, Adam.  Timed launch by launch and as one recorded launch sequence."""
@@ -301,7 +350,7 @@ def main():
     ap.add_argument("--n", type=int, default=4096)
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum"], default="gemm",
+    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum", "lstm"], default="gemm",
                     help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
                          "mlp: the feed-forward training step of configs[0]")
     ap.add_argument("--elems", type=int, default=64 * 1024 * 1024, help="elements per tensor in bandwidth mode")
@@ -309,6 +358,15 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: this path has no multi-GPU part (--gpus 1 only)")
+    if args.mode == "lstm":
+        res = lstm_leg(args.dtype, args.steps, args.warmup, not args.no_cpu)
+        print(json.dumps({"metric": "LSTM train steps/sec", "unit": "steps/s", "value": 1e3 / res["recorded_ms_per_step"],
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
+                          "higher_is_better": True, "ms_per_step": res["recorded_ms_per_step"],
+                          "config": {"workload": "configs[3]: LSTM layer 256->512, batch 128, 64 steps, fused 4-gate weight, MSE, "
+                                                 "BPTT, clip, Adam"},
+                          "detail": res}))
+        return
     if args.mode == "matmul_sum":
         res = matmul_sum_leg(args.dtype, args.steps, args.warmup)
         print(json.dumps({"metric": "MatrixMultiplyAndSum forward TFLOP/s, backward GB/s", "unit": "TFLOP/s", "value": res["fwd_TFLOPs"],

@@ -151,6 +151,25 @@ int32_t prad_softmax_bwd(prad_buf_t y, prad_buf_t dy, prad_buf_t dx);
 int32_t prad_cce_fwd(prad_buf_t p, prad_buf_t target, prad_buf_t loss);
 int32_t prad_cce_bwd(prad_buf_t p, prad_buf_t target, prad_buf_t dp);
 
+/* Mean squared error, src/RMAD/Loss/MeanSquaredErrorLossOperation.cs:
+ * loss (1 x 1) = sum((y - t)^2) / (rows*cols) ; dy = (2 / (rows*cols)) * (y - t). */
+int32_t prad_mse_fwd(prad_buf_t y, prad_buf_t target, prad_buf_t loss);
+int32_t prad_mse_bwd(prad_buf_t y, prad_buf_t target, prad_buf_t dy);
+/* One LSTM time step's pointwise part, fused.  The reference builds it from separate nodes: three
+ * SigmoidOperation and two TanhOperation forward (src/RMAD/SigmoidOperation.cs:46-62, TanhOperation.cs:42-57),
+ * three HadamardProductOperation (HadamardProductOperation.cs:50-81) and a MatrixAddOperation (MatrixAddOperation.cs:29-45).
+ * G (rows x 4*hidden, gate blocks [i|f|g|o]) holds the pre-activations and is overwritten with the activated
+ * gates; c = f.c_prev + i.g ; tanh_c = tanh(c) ; h = o.tanh_c. */
+int32_t prad_lstm_cell_fwd(prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_buf_t tanh_c, prad_buf_t h);
+/* Backward of the same nodes (their Backward methods, same files): dh = dh_a + dh_b (dh_b may be NULL),
+ * dc_in (may be NULL) is the cell-state gradient arriving from the next step; writes dG (rows x 4*hidden,
+ * gradient of the pre-activations) and dc_prev. */
+int32_t prad_lstm_cell_bwd(prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_c, prad_buf_t dh_a, prad_buf_t dh_b,
+                           prad_buf_t dc_in, prad_buf_t dG, prad_buf_t dc_prev);
+/* Borrowed view of rows [row0, row0 + rows) of a 2-D buffer (a block of a fused weight, a time step of a
+ * stacked sequence).  The view must be freed before its parent. */
+int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out);
+
 /* ---- replay of a fixed launch sequence: everything enqueued by this thread between begin and end
  *      is recorded instead of executed and can then be launched as one submission.  The forward loop
  *      of the reference walks the same operation list every step

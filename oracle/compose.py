@@ -1,0 +1,49 @@
+"""Compositions of the oracle's per-operation restatements into whole training steps, node by node as the
+reference's graph would run them.  TEST INFRASTRUCTURE ONLY (same rule as oracle.py): used by tests and by
+the benchmark's cpu_baseline leg."""
+import numpy as np
+
+from . import oracle
+
+
+def lstm_forward_backward(W, b, X, Y, I, H, B, T, threads=8):
+    """One LSTM layer over T steps with MSE on the stacked hidden states: returns loss, hidden states, dW, db, dX."""
+    dt = W.dtype
+    h, c = np.zeros((B, H), dt), np.zeros((B, H), dt)
+    cache = []
+    hs = []
+    for t in range(T):
+        xh = np.ascontiguousarray(np.concatenate([X[t * B:(t + 1) * B], h], axis=1))
+        G = oracle.add_broadcast_fwd(oracle.matmul_fwd(xh, W, threads=threads), b)
+        i_, f_ = oracle.sigmoid_fwd(np.ascontiguousarray(G[:, :H])), oracle.sigmoid_fwd(np.ascontiguousarray(G[:, H:2 * H]))
+        g_, o_ = oracle.tanh_fwd(np.ascontiguousarray(G[:, 2 * H:3 * H])), oracle.sigmoid_fwd(np.ascontiguousarray(G[:, 3 * H:]))
+        c_new = oracle.hadamard_fwd(f_, c) + oracle.hadamard_fwd(i_, g_)
+        tc = oracle.tanh_fwd(c_new)
+        h_new = oracle.hadamard_fwd(o_, tc)
+        cache.append((xh, i_, f_, g_, o_, c, tc))
+        h, c = h_new, c_new
+        hs.append(h)
+    Hout = np.concatenate(hs, axis=0)
+    loss = oracle.mse_fwd(Hout, Y)
+    dH = oracle.mse_bwd(Hout, Y)
+    dW, db = np.zeros_like(W), np.zeros_like(b)
+    dh_rec, dc_next = None, None
+    dX = np.zeros_like(X)
+    for t in range(T - 1, -1, -1):
+        xh, i_, f_, g_, o_, c_prev, tc = cache[t]
+        dh = dH[t * B:(t + 1) * B] if dh_rec is None else dH[t * B:(t + 1) * B] + dh_rec
+        d_o, d_tc = oracle.hadamard_bwd(o_, tc, dh)          # h = o . tanh(c)
+        dc = oracle.tanh_bwd(tc, d_tc)
+        if dc_next is not None:
+            dc = dc + dc_next
+        d_f, dc_prev = oracle.hadamard_bwd(f_, c_prev, dc)   # f . c_prev
+        d_i, d_g = oracle.hadamard_bwd(i_, g_, dc)           # i . g
+        dG = np.concatenate([oracle.sigmoid_bwd(i_, d_i), oracle.sigmoid_bwd(f_, d_f), oracle.tanh_bwd(g_, d_g),
+                             oracle.sigmoid_bwd(o_, d_o)], axis=1)
+        dG = np.ascontiguousarray(dG)
+        db = db + oracle.add_broadcast_bwd_bias(dG)
+        dxh, dWt = oracle.matmul_bwd(dG, xh, W, threads=threads)
+        dW = dW + dWt                                        # OperationBase.AccumulateGradient over the time steps
+        dX[t * B:(t + 1) * B] = dxh[:, :I]
+        dh_rec, dc_next = np.ascontiguousarray(dxh[:, I:]), dc_prev
+    return loss, Hout, dW, db, dX

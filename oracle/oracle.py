@@ -35,6 +35,8 @@ def load():
                 ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
         _lib.oracle_cce_fwd_f64.restype = ctypes.c_double
         _lib.oracle_cce_fwd_f32.restype = ctypes.c_float
+        _lib.oracle_mse_fwd_f64.restype = ctypes.c_double
+        _lib.oracle_mse_fwd_f32.restype = ctypes.c_float
     return _lib
 
 
@@ -238,6 +240,20 @@ def cce_bwd(p, t):
     dp = np.empty_like(p)
     _fn("cce_bwd", dt)(_p(p), _p(t), _p(dp), p.shape[0], p.shape[1])
     return dp
+
+
+def mse_fwd(y, t):
+    dt = y.dtype
+    y, t = _c(y, dt), _c(t, dt)
+    return float(_fn("mse_fwd", dt)(_p(y), _p(t), y.shape[0], y.shape[1]))
+
+
+def mse_bwd(y, t):
+    dt = y.dtype
+    y, t = _c(y, dt), _c(t, dt)
+    dy = np.empty_like(y)
+    _fn("mse_bwd", dt)(_p(y), _p(t), _p(dy), y.shape[0], y.shape[1])
+    return dy
 
 
 def time_matmul_fwdbwd(n, dtype=np.float64, threads=1, iters=1):

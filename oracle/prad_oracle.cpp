@@ -372,6 +372,18 @@ template <class T> void cce_bwd(const T* p, const T* t, T* dp, int rows, int col
     for (int64_t i = 0; i < (int64_t)rows * cols; ++i) dp[i] = -((T)1.0 / rows) * t[i] / (p[i] + (T)1e-15);
 }
 
+// MeanSquaredErrorLossOperation (src/RMAD/Loss/MeanSquaredErrorLossOperation.cs): LINQ sum of diff*diff over all
+// elements, divided by rows*cols; gradient (2/(rows*cols)) * (y - t).
+template <class T> T mse_fwd(const T* y, const T* t, int rows, int cols) {
+    std::vector<T> terms((size_t)rows * cols);
+    for (size_t i = 0; i < terms.size(); ++i) { T d = y[i] - t[i]; terms[i] = d * d; }
+    return linq_sum(terms.data(), (int)terms.size()) / (rows * cols);
+}
+template <class T> void mse_bwd(const T* y, const T* t, T* dy, int rows, int cols) {
+    const T scale = (T)2 / (rows * cols);
+    for (int64_t i = 0; i < (int64_t)rows * cols; ++i) dy[i] = scale * (y[i] - t[i]);
+}
+
 // ---------------------------------------------------------------------------------------
 // Seeded fill used only by the timing entry point: SplitMix64 of (seed, tensor, index).
 // ---------------------------------------------------------------------------------------
@@ -490,6 +502,8 @@ double time_matmul_fwdbwd(int N, int threads, int iters, double* checksum) {
     }                                                                                                          \
     EXPORT T oracle_cce_fwd_##SFX(const T* p, const T* t, int rows, int cols) { return cce_fwd<T>(p, t, rows, cols); } \
     EXPORT void oracle_cce_bwd_##SFX(const T* p, const T* t, T* dp, int rows, int cols) { cce_bwd<T>(p, t, dp, rows, cols); } \
+    EXPORT T oracle_mse_fwd_##SFX(const T* y, const T* t, int rows, int cols) { return mse_fwd<T>(y, t, rows, cols); } \
+    EXPORT void oracle_mse_bwd_##SFX(const T* y, const T* t, T* dy, int rows, int cols) { mse_bwd<T>(y, t, dy, rows, cols); } \
     EXPORT double oracle_time_matmul_fwdbwd_##SFX(int N, int threads, int iters, double* checksum) {           \
         return time_matmul_fwdbwd<T>(N, threads, iters, checksum);                                             \
     }

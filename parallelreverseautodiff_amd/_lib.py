@@ -75,6 +75,11 @@ SIGNATURES = {
     "prad_softmax_bwd": (_i32, [_vp, _vp, _vp]),
     "prad_cce_fwd": (_i32, [_vp, _vp, _vp]),
     "prad_cce_bwd": (_i32, [_vp, _vp, _vp]),
+    "prad_mse_fwd": (_i32, [_vp, _vp, _vp]),
+    "prad_mse_bwd": (_i32, [_vp, _vp, _vp]),
+    "prad_lstm_cell_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp]),
+    "prad_lstm_cell_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "prad_buf_view_rows": (_i32, [_vp, _i64, _i64, _vpp]),
     "prad_graph_begin": (_i32, []),
     "prad_graph_end": (_i32, [_vpp]),
     "prad_graph_launch": (_i32, [_vp]),

@@ -167,6 +167,16 @@ template <typename T> hipError_t launch_softmax_bwd(const T* y, const T* dy, T* 
 template <typename T> hipError_t launch_cce_fwd(const T* p, const T* t, T* loss, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t cols, hipStream_t s);
 
+size_t mse_workspace_bytes();
+template <typename T> hipError_t launch_mse_fwd(const T* y, const T* t, T* loss, double* workspace, int64_t n, hipStream_t s);
+template <typename T> hipError_t launch_mse_bwd(const T* y, const T* t, T* dy, int64_t n, hipStream_t s);
+
+// LSTM cell (csrc/lstm.hip)
+template <typename T> hipError_t launch_lstm_cell_fwd(T* G, const T* c_prev, T* c, T* tanh_c, T* h, int64_t rows, int64_t hidden,
+                                                      hipStream_t s);
+template <typename T> hipError_t launch_lstm_cell_bwd(const T* gates, const T* c_prev, const T* tanh_c, const T* dh_a, const T* dh_b,
+                                                      const T* dc_in, T* dG, T* dc_prev, int64_t rows, int64_t hidden, hipStream_t s);
+
 // MatrixMultiplyAndSum
 template <typename T> hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K,
                                                        int64_t N, int64_t P, hipStream_t s);

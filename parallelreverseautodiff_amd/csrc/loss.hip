@@ -78,6 +78,55 @@ __global__ void __launch_bounds__(256) cce_bwd_kernel(const T* __restrict__ p, c
         dp[i] = -scale * t[i] / (p[i] + (T)1e-15);
 }
 
+// MeanSquaredErrorLossOperation (src/RMAD/Loss/MeanSquaredErrorLossOperation.cs): loss = sum (y - t)^2 / (rows*cols),
+// dy = (2 / (rows*cols)) * (y - t).  The sum is taken in two levels (per workgroup, then by one thread).
+template <typename T>
+__global__ void __launch_bounds__(256) mse_partial_kernel(const T* __restrict__ y, const T* __restrict__ t, double* __restrict__ part,
+                                                          int64_t n) {
+    double s = 0.0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const T d = y[i] - t[i];
+        s += (double)(d * d);
+    }
+    s = wave_sum(s);
+    __shared__ double w[4];
+    if ((threadIdx.x & 63) == 0) w[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) part[blockIdx.x] = (w[0] + w[1]) + (w[2] + w[3]);
+}
+template <typename T>
+__global__ void __launch_bounds__(64) mse_final_kernel(const double* __restrict__ part, int nparts, T* __restrict__ loss, int64_t n) {
+    double s = 0.0;
+    for (int i = threadIdx.x; i < nparts; i += 64) s += part[i];
+    s = wave_sum(s);
+    if (threadIdx.x == 0) loss[0] = (T)s / (T)n;
+}
+template <typename T>
+__global__ void __launch_bounds__(256) mse_bwd_kernel(const T* __restrict__ y, const T* __restrict__ t, T* __restrict__ dy, int64_t n) {
+    const T scale = (T)2 / (T)n;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dy[i] = scale * (y[i] - t[i]);
+}
+
+constexpr int MSE_PARTS = 1024;
+size_t mse_workspace_bytes() { return MSE_PARTS * sizeof(double); }
+template <typename T>
+hipError_t launch_mse_fwd(const T* y, const T* t, T* loss, double* workspace, int64_t n, hipStream_t s) {
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > MSE_PARTS) blocks = MSE_PARTS;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL((mse_partial_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, n);
+    hipLaunchKernelGGL((mse_final_kernel<T>), dim3(1), dim3(64), 0, s, workspace, (int)blocks, loss, n);
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t launch_mse_bwd(const T* y, const T* t, T* dy, int64_t n, hipStream_t s) {
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL((mse_bwd_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, dy, n);
+    return hipGetLastError();
+}
+
 template <typename T>
 hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
@@ -108,7 +157,9 @@ hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t c
     template hipError_t launch_softmax_fwd<T>(const T*, T*, int64_t, int64_t, hipStream_t);         \
     template hipError_t launch_softmax_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t); \
     template hipError_t launch_cce_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
-    template hipError_t launch_cce_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);
+    template hipError_t launch_cce_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
+    template hipError_t launch_mse_fwd<T>(const T*, const T*, T*, double*, int64_t, hipStream_t);   \
+    template hipError_t launch_mse_bwd<T>(const T*, const T*, T*, int64_t, hipStream_t);
 INSTANTIATE(double)
 INSTANTIATE(float)
 

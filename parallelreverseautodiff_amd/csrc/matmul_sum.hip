@@ -45,7 +45,7 @@ hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspa
 }
 
 constexpr int TS = 64;       // transpose tile edge
-constexpr int Q_PER_WG = 8;  // slices written per workgroup of the dB kernel
+constexpr int Q_PER_WG = 2;  // slices written per workgroup of the dB kernel
 
 // dB[q][k][m] = A[m][k] * dOut[q]: the A tile is transposed through LDS once and scaled into
 // Q_PER_WG slices; reads walk k, writes walk m, both contiguous.
@@ -84,7 +84,27 @@ __global__ void __launch_bounds__(256) sum_bwd_da_kernel(const T* __restrict__ B
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // ty in 0..3, rows ty, ty+4, ty+8, ty+12
     T acc[4] = {(T)0, (T)0, (T)0, (T)0};
     const int64_t i = i0 + tx;
-    for (int64_t q = 0; q < P; ++q) {
+    // Loads of four slices are issued before their (ordered) additions, to keep 16 reads in flight per lane.
+    int64_t q = 0;
+    for (; q + 4 <= P; q += 4) {
+        T b[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const T* __restrict__ Bq = B + (q + u) * K * N;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t j = j0 + ty + 4 * r;
+                b[u][r] = (i < N && j < K) ? Bq[j * N + i] : (T)0;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const T sc = dOut[q + u];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] = acc[r] + (b[u][r] * sc);
+        }
+    }
+    for (; q < P; ++q) {
         const T sc = dOut[q];
         const T* __restrict__ Bq = B + q * K * N;
 #pragma unroll

@@ -728,6 +728,82 @@ int32_t prad_cce_bwd(prad_buf_t p, prad_buf_t target, prad_buf_t dp) {
     return PRAD_OK;
 }
 
+int32_t prad_mse_fwd(prad_buf_t y, prad_buf_t target, prad_buf_t loss) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(y); REQUIRE_BUF(target); REQUIRE_BUF(loss);
+    if (int32_t st = same_dtype({y, target, loss})) return st;
+    if (y->depth != target->depth || y->rows != target->rows || y->cols != target->cols)
+        return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
+    if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (int32_t st = ensure_workspace(mse_workspace_bytes())) return st;
+    double* w = static_cast<double*>(g_ctx.workspace);
+    DISPATCH(y, launch_mse_fwd<double>(D(y), D(target), D(loss), w, count(y), g_ctx.stream),
+             launch_mse_fwd<float>(F(y), F(target), F(loss), w, count(y), g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_mse_bwd(prad_buf_t y, prad_buf_t target, prad_buf_t dy) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(y); REQUIRE_BUF(target); REQUIRE_BUF(dy);
+    if (int32_t st = same_dtype({y, target, dy})) return st;
+    if (y->depth != target->depth || y->rows != target->rows || y->cols != target->cols)
+        return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
+    if (int32_t st = same_shape(y, dy, "mean squared error backward")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(y, launch_mse_bwd<double>(D(y), D(target), D(dy), count(y), g_ctx.stream),
+             launch_mse_bwd<float>(F(y), F(target), F(dy), count(y), g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_lstm_cell_fwd(prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_buf_t tanh_c, prad_buf_t h) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(G); REQUIRE_BUF(c_prev); REQUIRE_BUF(c); REQUIRE_BUF(tanh_c); REQUIRE_BUF(h);
+    if (int32_t st = same_dtype({G, c_prev, c, tanh_c, h})) return st;
+    const int64_t rows = c->rows, hidden = c->cols;
+    if (G->depth != 1 || c->depth != 1 || G->rows != rows || G->cols != 4 * hidden)
+        return fail(PRAD_ERR_ARG, "gate pre-activations must be rows x 4*hidden");
+    for (prad_buf_t o : {c_prev, tanh_c, h})
+        if (int32_t st = same_shape(c, o, "LSTM cell")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(c, launch_lstm_cell_fwd<double>(D(G), D(c_prev), D(c), D(tanh_c), D(h), rows, hidden, g_ctx.stream),
+             launch_lstm_cell_fwd<float>(F(G), F(c_prev), F(c), F(tanh_c), F(h), rows, hidden, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_lstm_cell_bwd(prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_c, prad_buf_t dh_a, prad_buf_t dh_b, prad_buf_t dc_in,
+                           prad_buf_t dG, prad_buf_t dc_prev) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(gates); REQUIRE_BUF(c_prev); REQUIRE_BUF(tanh_c); REQUIRE_BUF(dh_a); REQUIRE_BUF(dG); REQUIRE_BUF(dc_prev);
+    if (dh_b != nullptr) REQUIRE_BUF(dh_b);
+    if (dc_in != nullptr) REQUIRE_BUF(dc_in);
+    if (int32_t st = same_dtype({gates, c_prev, tanh_c, dh_a, dh_b, dc_in, dG, dc_prev})) return st;
+    const int64_t rows = c_prev->rows, hidden = c_prev->cols;
+    if (gates->rows != rows || gates->cols != 4 * hidden || c_prev->depth != 1 || gates->depth != 1)
+        return fail(PRAD_ERR_ARG, "gates must be rows x 4*hidden");
+    if (int32_t st = same_shape(gates, dG, "LSTM cell backward")) return st;
+    for (prad_buf_t o : {tanh_c, dh_a, dh_b, dc_in, dc_prev})
+        if (o != nullptr)
+            if (int32_t st = same_shape(c_prev, o, "LSTM cell backward")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(c_prev,
+             launch_lstm_cell_bwd<double>(D(gates), D(c_prev), D(tanh_c), D(dh_a), dh_b ? D(dh_b) : nullptr, dc_in ? D(dc_in) : nullptr,
+                                          D(dG), D(dc_prev), rows, hidden, g_ctx.stream),
+             launch_lstm_cell_bwd<float>(F(gates), F(c_prev), F(tanh_c), F(dh_a), dh_b ? F(dh_b) : nullptr, dc_in ? F(dc_in) : nullptr,
+                                         F(dG), F(dc_prev), rows, hidden, g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(parent);
+    if (out == nullptr) return fail(PRAD_ERR_ARG, "out is NULL");
+    if (parent->depth != 1 || row0 < 0 || rows <= 0 || row0 + rows > parent->rows) return fail(PRAD_ERR_ARG, "row range outside the buffer");
+    char* base = static_cast<char*>(parent->ptr) + (size_t)row0 * parent->cols * elem_size(parent->dtype);
+    *out = new prad_buf{BUF_MAGIC, parent->dtype, 1, rows, parent->cols, base, false};
+    return PRAD_OK;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Recording holds the context lock's place in line only per call: other threads must not enqueue
 // while a recording is open (their work would be recorded too), which the caller guarantees.

@@ -67,6 +67,12 @@ class DeviceBuffer:
         check(lib.prad_buf_wrap(_dtype_code(self.dtype), self.rows, self.cols, ctypes.c_void_p(base + off), ctypes.byref(h)))
         return DeviceBuffer(h, self.dtype, 1, self.rows, self.cols, parent=self)
 
+    def view_rows(self, row0, rows):
+        """A borrowed view of rows [row0, row0 + rows) of a 2-D buffer."""
+        h = ctypes.c_void_p()
+        check(_lib.load().prad_buf_view_rows(self.handle, row0, rows, ctypes.byref(h)))
+        return DeviceBuffer(h, self.dtype, 1, rows, self.cols, parent=self)
+
     @property
     def ptr(self):
         return _lib.load().prad_buf_device_ptr(self.handle)
