@@ -128,7 +128,17 @@ struct GemmArgs {
     // When set, C is not written: each workgroup stores the sum of its finished tile to
     // tile_sums[batch_index * tiles_per_product + tile_index] (MatrixMultiplyAndSum forward).
     double* tile_sums;
+    // Scratch for products that are split along K (see gemm_split_factor): split_ws holds
+    // split_factor * batch * M * N elements.  Filled in by the caller; nullptr disables splitting.
+    T* split_ws;
+    // Set by launch_gemm for the kernels: K range per split (0 = not split).
+    int64_t ksplit;
 };
+
+// How many ways launch_gemm splits the reduction of a product whose output has too few tiles to occupy
+// the chip (1 = not split).  A split product writes its partial results to GemmArgs::split_ws and a
+// second kernel adds them in split order and applies the epilogue.
+int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size);
 
 // Number of 128 x 128 output tiles of one product (the tile_sums layout).
 inline int64_t gemm_tiles_per_product(int64_t M, int64_t N) { return ((M + 127) / 128) * ((N + 127) / 128); }
@@ -143,7 +153,8 @@ template <typename T> hipError_t launch_hadamard_bwd(const T* a, const T* b, con
 template <typename T> hipError_t launch_accumulate(T* dest, const T* grad, int64_t n, hipStream_t s);
 template <typename T> hipError_t launch_copy(T* dst, const T* src, int64_t n, hipStream_t s);
 template <typename T> hipError_t launch_add_broadcast_fwd(const T* x, const T* bias, T* y, int64_t rows, int64_t cols, hipStream_t s);
-template <typename T> hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, hipStream_t s);
+int colsum_chunks(int64_t rows);
+template <typename T> hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double* workspace, hipStream_t s);
 template <typename T> hipError_t launch_fill_zero(T* p, int64_t n, hipStream_t s);
 
 // Descriptor of one tensor of a multi-tensor clip / Adam launch.

@@ -218,30 +218,54 @@ hipError_t launch_add_broadcast_fwd(const T* x, const T* bias, T* y, int64_t row
 // Column(j), which for float accumulates in double).  A workgroup owns 64 columns; its four
 // wavefronts take rows i = w, w+4, w+8, ... with four independent loads in flight each, and the four
 // partial sums are added in wavefront order, so the result does not depend on timing.  Neighbouring
-// lanes read neighbouring columns: every row is one coalesced read.
-template <typename T>
-__global__ void __launch_bounds__(256) colsum_kernel(const T* __restrict__ dy, T* __restrict__ db, int64_t rows, int64_t cols) {
+// lanes read neighbouring columns: every row is one coalesced read.  Tall matrices (a whole sequence of
+// gate gradients) are cut into up to 64 row chunks whose partial sums a second kernel adds in chunk order.
+// Rows [blockIdx.y * rows_per_chunk, ...) of 64 columns; out is db itself (one chunk) or a row of partial sums.
+template <typename T, typename OUT>
+__global__ void __launch_bounds__(256) colsum_kernel(const T* __restrict__ dy, OUT* __restrict__ out, int64_t rows, int64_t cols,
+                                                     int64_t rows_per_chunk) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int64_t j = (int64_t)blockIdx.x * 64 + lane;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk;
+    const int64_t r1 = min(rows, r0 + rows_per_chunk);
     double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
     if (j < cols) {
-        int64_t i = w;
-        for (; i + 12 < rows; i += 16) {
+        int64_t i = r0 + w;
+        for (; i + 12 < r1; i += 16) {
             const double a = (double)dy[i * cols + j], b = (double)dy[(i + 4) * cols + j];
             const double c = (double)dy[(i + 8) * cols + j], d = (double)dy[(i + 12) * cols + j];
             acc0 += a; acc1 += b; acc2 += c; acc3 += d;
         }
-        for (; i < rows; i += 4) acc0 += (double)dy[i * cols + j];
+        for (; i < r1; i += 4) acc0 += (double)dy[i * cols + j];
     }
     __shared__ double part[4][64];
     part[w][lane] = (acc0 + acc1) + (acc2 + acc3);
     __syncthreads();
-    if (w == 0 && j < cols) db[j] = (T)((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]));
+    if (w == 0 && j < cols)
+        out[(int64_t)blockIdx.y * cols + j] = (OUT)((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]));
 }
 template <typename T>
-hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, hipStream_t s) {
+__global__ void __launch_bounds__(64) colsum_final_kernel(const double* __restrict__ partial, T* __restrict__ db, int chunks, int64_t cols) {
+    const int64_t j = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (j >= cols) return;
+    double s = 0.0;
+    for (int c = 0; c < chunks; ++c) s += partial[(int64_t)c * cols + j];
+    db[j] = (T)s;
+}
+int colsum_chunks(int64_t rows) { return rows >= 2048 ? (int)((rows + 255) / 256 > 64 ? 64 : (rows + 255) / 256) : 1; }
+// workspace: colsum_chunks(rows) * cols doubles when colsum_chunks(rows) > 1.
+template <typename T>
+hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double* workspace, hipStream_t s) {
     if (cols <= 0) return hipSuccess;
-    hipLaunchKernelGGL((colsum_kernel<T>), dim3((unsigned)((cols + 63) / 64)), dim3(256), 0, s, dy, db, rows, cols);
+    const int chunks = workspace != nullptr ? colsum_chunks(rows) : 1;
+    const unsigned gx = (unsigned)((cols + 63) / 64);
+    if (chunks == 1) {
+        hipLaunchKernelGGL((colsum_kernel<T, T>), dim3(gx, 1), dim3(256), 0, s, dy, db, rows, cols, rows);
+    } else {
+        const int64_t per = (rows + chunks - 1) / chunks;
+        hipLaunchKernelGGL((colsum_kernel<T, double>), dim3(gx, (unsigned)chunks), dim3(256), 0, s, dy, workspace, rows, cols, per);
+        hipLaunchKernelGGL((colsum_final_kernel<T>), dim3(gx), dim3(64), 0, s, workspace, db, chunks, cols);
+    }
     return hipGetLastError();
 }
 
@@ -253,7 +277,7 @@ hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, hipStre
     template hipError_t launch_accumulate<T>(T*, const T*, int64_t, hipStream_t);                                  \
     template hipError_t launch_copy<T>(T*, const T*, int64_t, hipStream_t);                                        \
     template hipError_t launch_add_broadcast_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);        \
-    template hipError_t launch_colsum<T>(const T*, T*, int64_t, int64_t, hipStream_t);                             \
+    template hipError_t launch_colsum<T>(const T*, T*, int64_t, int64_t, double*, hipStream_t);                             \
     template hipError_t launch_fill_zero<T>(T*, int64_t, hipStream_t);
 INSTANTIATE(double)
 INSTANTIATE(float)

@@ -195,6 +195,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     const int batch = blockIdx.y;
     const T* __restrict__ A = p.A + batch * p.strideA;
     const T* __restrict__ B = p.B + batch * p.strideB;
+    // A product split along K: this workgroup reduces [kb, kb + K) and writes its own M x N partial result.
+    int64_t K = p.K;
+    if (p.ksplit > 0) {
+        const int64_t kb = (int64_t)blockIdx.z * p.ksplit;
+        K = min(p.ksplit, p.K - kb);
+        A += A_KC ? kb : kb * p.lda;
+        B += B_KC ? kb : kb * p.ldb;
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -209,7 +217,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[x][y][r] = (T)0;
 
-    const int64_t K = p.K;
     // Unguarded kernels run the whole slabs with vector loads and finish a ragged end of K (784 = 12 x 64 + 16)
     // with one guarded slab; guarded kernels treat every slab alike.
     const int ntiles = EDGE ? (int)((K + BK - 1) / BK) : (int)(K / BK);
@@ -335,7 +342,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         return;
     }
 
-    T* __restrict__ C = p.C + batch * p.strideC;
+    T* __restrict__ C = p.C + batch * p.strideC + (p.ksplit > 0 ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
         // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
         // row-major: the elementwise arithmetic (which includes exp/tanh code) then sits in one runtime loop
@@ -392,7 +399,8 @@ template <typename T, int WT, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStream_t stream) {
     constexpr int BM = 32 * WT;
     const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BM - 1) / BM);
-    dim3 grid((unsigned)(tilesM * tilesN), (unsigned)a.batch, 1), block(GEMM_THREADS, 1, 1);
+    const unsigned splits = a.ksplit > 0 ? (unsigned)((a.K + a.ksplit - 1) / a.ksplit) : 1u;
+    dim3 grid((unsigned)(tilesM * tilesN), (unsigned)a.batch, splits), block(GEMM_THREADS, 1, 1);
 #define PRAD_LAUNCH(EDGE_, EPI_) \
     hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, EDGE_, EPI_>), grid, block, 0, stream, a, tilesM, tilesN)
     if (edge) {
@@ -449,13 +457,61 @@ static TileShape choose_tile(int64_t M, int64_t N, int batch, bool tile_sums) {
     return TILE_32x32;
 }
 
+int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
+    const int64_t tiles = ((M + 31) / 32) * ((N + 31) / 32) * batch;  // the smallest tile is what such products get
+    if (tiles >= 192) return 1;
+    const int64_t bk = (elem_size == 8 ? Slab<double, 1>::BK : Slab<float, 1>::BK);
+    int64_t s = 384 / tiles;
+    if (s > 8) s = 8;
+    if (s > K / (2 * bk)) s = K / (2 * bk);  // at least two slabs per split
+    if (s < 2) return 1;
+    const int64_t ksplit = ((K + s - 1) / s + bk - 1) / bk * bk;
+    return (int)((K + ksplit - 1) / ksplit);
+}
+
+// Adds the partial results of a split product in split order and applies the epilogue.
 template <typename T>
-hipError_t launch_gemm(const GemmArgs<T>& a, hipStream_t stream) {
-    if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return hipSuccess;
-    if (a.transA && a.transB) return hipErrorInvalidValue;
+__global__ void __launch_bounds__(256) split_reduce_kernel(const GemmArgs<T> p, const T* __restrict__ ws, int splits) {
+    const int64_t mn = p.M * p.N, total = mn * p.batch;
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        const int64_t b = idx / mn, e = idx % mn, i = e / p.N, j = e % p.N;
+        T v = ws[idx];
+        for (int z = 1; z < splits; ++z) v = v + ws[(int64_t)z * total + idx];
+        if (p.bias != nullptr) v = v + p.bias[j];
+        if (p.Z != nullptr) p.Z[i * p.ldz + j] = v;
+        if (p.act_fwd != ACT_NONE) v = act_forward<T>(p.act_fwd, v, p.alpha);
+        if (p.act_bwd != ACT_NONE) v = v * act_derivative<T>(p.act_bwd, p.act_src[i * p.ld_act + j], p.alpha);
+        T* c = p.C + b * p.strideC + i * p.ldc + j;
+        if (p.accumulate) v = *c + v;
+        *c = v;
+    }
+}
+
+template <typename T>
+hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
+    if (a_in.M <= 0 || a_in.N <= 0 || a_in.batch <= 0) return hipSuccess;
+    if (a_in.transA && a_in.transB) return hipErrorInvalidValue;
+    GemmArgs<T> a = a_in;
+    a.ksplit = 0;
     const int epi = a.tile_sums != nullptr ? EPI_TILE_SUM
                     : (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) ? EPI_ELEMENTWISE
                                                                                                              : EPI_PLAIN;
+    const int splits = (a.split_ws != nullptr && epi != EPI_TILE_SUM) ? gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T)) : 1;
+    if (splits > 1) {
+        constexpr int64_t bk = Slab<T, 1>::BK;
+        GemmArgs<T> part = a;
+        part.ksplit = ((a.K + splits - 1) / splits + bk - 1) / bk * bk;
+        part.C = a.split_ws; part.ldc = a.N; part.strideC = a.M * a.N;  // split z, batch b at ((z * batch) + b) * M * N
+        part.accumulate = 0;
+        part.bias = nullptr; part.Z = nullptr; part.act_fwd = ACT_NONE; part.act_bwd = ACT_NONE; part.act_src = nullptr;
+        hipError_t e = launch_tile<T, 1>(part, EPI_PLAIN, stream);
+        if (e != hipSuccess) return e;
+        const int64_t total = a.M * a.N * a.batch;
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL((split_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, a, a.split_ws, splits);
+        return hipGetLastError();
+    }
     switch (choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr)) {
         case TILE_128x128: return launch_tile<T, 4>(a, epi, stream);
         case TILE_64x64: return launch_tile<T, 2>(a, epi, stream);

@@ -125,6 +125,16 @@ GemmArgs<T> plain_gemm(int transA, int transB, int64_t M, int64_t N, int64_t K, 
     return a;
 }
 
+// Products split along K need room for their partial results; the shared workspace is grown here (lock held).
+template <typename T>
+int32_t attach_split_workspace(GemmArgs<T>& a) {
+    const int splits = gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T));
+    if (splits <= 1) return PRAD_OK;
+    if (int32_t st = ensure_workspace((size_t)splits * a.batch * a.M * a.N * sizeof(T))) return st;
+    a.split_ws = static_cast<T*>(g_ctx.workspace);
+    return PRAD_OK;
+}
+
 // Rows/columns of op(X) for a 2-D (per-slice) buffer.
 inline int64_t op_rows(prad_buf_t b, int trans) { return trans ? b->cols : b->rows; }
 inline int64_t op_cols(prad_buf_t b, int trans) { return trans ? b->rows : b->cols; }
@@ -155,6 +165,7 @@ int32_t enqueue_gemm_t(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_
         a.strideB = B->depth == 1 ? 0 : B->rows * B->cols;
         a.strideC = C->rows * C->cols;
     }
+    if (int32_t st = attach_split_workspace(a)) return st;
     HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -485,6 +496,7 @@ int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_bu
         if (lda < (transA ? M : K) || ldb < (transB ? K : N) || ldc < N) return fail(PRAD_ERR_ARG, "leading dimension too small"); \
         GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                   \
         std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                   \
+        if (int32_t st = attach_split_workspace(a)) return st;                                                        \
         HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);                                                    \
         return PRAD_OK;                                                                                               \
     }
@@ -673,8 +685,13 @@ int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias) {
     if (dbias->cols != dy->cols || dbias->rows != 1 || dbias->depth != 1 || dy->depth != 1)
         return fail(PRAD_ERR_ARG, "bias gradient must be 1 x cols");
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(dy, launch_colsum<double>(D(dy), D(dbias), dy->rows, dy->cols, g_ctx.stream),
-             launch_colsum<float>(F(dy), F(dbias), dy->rows, dy->cols, g_ctx.stream));
+    double* ws = nullptr;
+    if (colsum_chunks(dy->rows) > 1) {
+        if (int32_t st = ensure_workspace((size_t)colsum_chunks(dy->rows) * dy->cols * sizeof(double))) return st;
+        ws = static_cast<double*>(g_ctx.workspace);
+    }
+    DISPATCH(dy, launch_colsum<double>(D(dy), D(dbias), dy->rows, dy->cols, ws, g_ctx.stream),
+             launch_colsum<float>(F(dy), F(dbias), dy->rows, dy->cols, ws, g_ctx.stream));
     return PRAD_OK;
 }
 

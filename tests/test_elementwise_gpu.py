@@ -94,3 +94,11 @@ def test_large_vector_tail_and_size(gpu, oracle):
     dx = op.Backward(Matrix.from_numpy(dy)).Item1.to_numpy()
     assert_parity(y, oracle.sigmoid_fwd(x), np.float32)
     assert_parity(dx, oracle.sigmoid_bwd(y, dy), np.float32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bias_gradient_of_a_tall_matrix(gpu, oracle, dtype):
+    """Enough rows for the chunked column sum (a whole sequence of gate gradients)."""
+    dy = seeded.normal(43, 1, (5000, 130), 1.0, dtype)
+    res = MatrixAddBroadcastingOperation.Instantiate(None).Backward(Matrix.from_numpy(dy))
+    assert_parity(res.Item2.to_numpy(), oracle.add_broadcast_bwd_bias(dy), dtype, "bias gradient")
