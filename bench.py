@@ -223,6 +223,55 @@ def lstm_leg(dtype_name, steps, warmup, with_cpu):
     return out
 
 
+def swin_leg(dtype_name, steps, warmup, with_cpu):
+    """configs[4]: Swin-style windowed self-attention block, batch 16, 56x56 tokens in 7x7 windows, embed 96, 3 heads,
+    MLP x4 with GELU (GELUOperation's own derivative), MSE, full backward, clip, Adam."""
+    from parallelreverseautodiff_amd import _lib
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.swin import SwinBlock
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = 0
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    blk = SwinBlock(dtype=dtype)
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.prad_event_create(ctypes.byref(e0)))
+    check(lib.prad_event_create(ctypes.byref(e1)))
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        check(lib.prad_stream_sync())
+        check(lib.prad_event_record(e0))
+        for _ in range(steps):
+            fn()
+        check(lib.prad_event_record(e1))
+        check(lib.prad_stream_sync())
+        ms = ctypes.c_float()
+        check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        return ms.value / steps
+
+    eager_ms = timed(blk.step)
+    blk.record(adam_iteration=float(blk.iteration + 1))
+    rec_ms = timed(blk.replay)
+    blk.release()
+    flops = blk.flops_per_step()
+    out = {"eager_ms_per_step": eager_ms, "recorded_ms_per_step": rec_ms, "flop_per_step": flops,
+           "TFLOPs": flops / (rec_ms * 1e-3) / 1e12, "loss_after": float(blk.loss.download()[0, 0])}
+    if with_cpu:
+        from oracle import compose, oracle
+        threads = min(16, oracle.hardware_threads() or 1)
+        t0 = time.perf_counter()
+        compose.swin_block_forward_backward({k: blk.host[k] for k in blk.names}, blk.host["X"], blk.host["T"], blk.nw, blk.wt,
+                                            blk.heads, threads=threads)
+        secs = time.perf_counter() - t0
+        out["cpu"] = {"steps_per_s": 1.0 / secs, "ms_per_step": secs * 1e3, "cores": threads, "steps_timed": 1, "kind": "port",
+                      "note": "forward + backward only, node-by-node composition of the oracle's operations (per-window loop in Python)"}
+    return out
+
+
 def mlp_leg(dtype_name, steps, warmup, with_cpu):
     """Feed-forward training step of configs[0]: batch 64, 784-256-128-10, LeakyReLU(0.01), softmax
     cross-entropy, clip, Adam.  Timed launch by launch and as one recorded launch sequence."""
@@ -350,7 +399,7 @@ def main():
     ap.add_argument("--n", type=int, default=4096)
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum", "lstm"], default="gemm",
+    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum", "lstm", "swin"], default="gemm",
                     help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
                          "mlp: the feed-forward training step of configs[0]")
     ap.add_argument("--elems", type=int, default=64 * 1024 * 1024, help="elements per tensor in bandwidth mode")
@@ -358,6 +407,15 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: this path has no multi-GPU part (--gpus 1 only)")
+    if args.mode == "swin":
+        res = swin_leg(args.dtype, args.steps, args.warmup, not args.no_cpu)
+        print(json.dumps({"metric": "Swin block train steps/sec", "unit": "steps/s", "value": 1e3 / res["recorded_ms_per_step"],
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
+                          "higher_is_better": True, "ms_per_step": res["recorded_ms_per_step"],
+                          "config": {"workload": "configs[4]: windowed self-attention block, 16 x 56x56 tokens, 7x7 windows, embed 96, "
+                                                 "3 heads, MLP x4 GELU, MSE, full backward, clip, Adam"},
+                          "detail": res}))
+        return
     if args.mode == "lstm":
         res = lstm_leg(args.dtype, args.steps, args.warmup, not args.no_cpu)
         print(json.dumps({"metric": "LSTM train steps/sec", "unit": "steps/s", "value": 1e3 / res["recorded_ms_per_step"],

@@ -112,6 +112,17 @@ int32_t prad_gemm_f64(int32_t transA, int32_t transB, int64_t M, int64_t N, int6
 int32_t prad_gemm_f32(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const float* A, int64_t lda,
                       const float* B, int64_t ldb, float* C, int64_t ldc, int32_t accumulate);
 
+/* Strided batched product on raw device pointers: `batch` products, operand b at base + b * stride (elements;
+ * stride 0 shares an operand).  This is the form the per-window, per-head products of an attention block
+ * take, and the one a batched Tensor.MatrixMultiply (src/PRAD/Tensor.cs:572-608, which rejects more than
+ * two dimensions today) would bind. */
+int32_t prad_gemm_strided_batched_f64(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const double* A,
+                                      int64_t lda, int64_t strideA, const double* B, int64_t ldb, int64_t strideB, double* C,
+                                      int64_t ldc, int64_t strideC, int32_t batch, int32_t accumulate);
+int32_t prad_gemm_strided_batched_f32(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const float* A,
+                                      int64_t lda, int64_t strideA, const float* B, int64_t ldb, int64_t strideB, float* C,
+                                      int64_t ldc, int64_t strideC, int32_t batch, int32_t accumulate);
+
 /* One-shot host-pointer forms with today's call-per-operation behaviour of
  * GpuMatrixMultiplyOperation.Forward/Backward (src/RMAD/GpuMatrixMultiplyOperation.cs:113-161):
  * jagged rows in, jagged rows out, synchronous. */
@@ -136,6 +147,8 @@ int32_t prad_act_bwd(int32_t act, prad_buf_t src, prad_buf_t dy, prad_buf_t dx, 
 /* HadamardProductOperation, src/RMAD/HadamardProductOperation.cs:50-118 */
 int32_t prad_hadamard_fwd(prad_buf_t a, prad_buf_t b, prad_buf_t y);
 int32_t prad_hadamard_bwd(prad_buf_t a, prad_buf_t b, prad_buf_t dy, prad_buf_t da, prad_buf_t db);
+/* y = x * scalar, MatrixMultiplyScalarOperation.Forward and (with dy for x) Backward, src/RMAD/MatrixMultiplyScalarOperation.cs */
+int32_t prad_scale(prad_buf_t x, prad_buf_t y, double scalar);
 /* dest += grad, src/RMAD/OperationBase.cs:295-303 */
 int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad);
 /* y = x + bias broadcast over rows; db[0][j] = sum_i dy[i][j]; src/RMAD/MatrixAddBroadcastingOperation.cs:32-70 */

@@ -152,6 +152,7 @@ template <typename T> hipError_t launch_hadamard_fwd(const T* a, const T* b, T* 
 template <typename T> hipError_t launch_hadamard_bwd(const T* a, const T* b, const T* dy, T* da, T* db, int64_t n, hipStream_t s);
 template <typename T> hipError_t launch_accumulate(T* dest, const T* grad, int64_t n, hipStream_t s);
 template <typename T> hipError_t launch_copy(T* dst, const T* src, int64_t n, hipStream_t s);
+template <typename T> hipError_t launch_scale(T* y, const T* x, int64_t n, T alpha, hipStream_t s);
 template <typename T> hipError_t launch_add_broadcast_fwd(const T* x, const T* bias, T* y, int64_t rows, int64_t cols, hipStream_t s);
 int colsum_chunks(int64_t rows);
 template <typename T> hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double* workspace, hipStream_t s);

@@ -131,6 +131,10 @@ template <typename T> struct HadBwd {  // in: a, b, dy ; out: da, db
         out[1] = in[2] * in[0];
     }
 };
+template <typename T> struct Scale {
+    T alpha;
+    __device__ __forceinline__ void apply(const T (&in)[1], T (&out)[1]) const { out[0] = in[0] * alpha; }
+};
 template <typename T> struct Copy {
     __device__ __forceinline__ void apply(const T (&in)[1], T (&out)[1]) const { out[0] = in[0]; }
 };
@@ -174,6 +178,13 @@ template <typename T>
 hipError_t launch_accumulate(T* dest, const T* grad, int64_t n, hipStream_t s) {
     StreamPtrs<T, 2, 1> p{{dest, grad}, {dest}};
     return launch_stream(p, n, Accum<T>{}, s);
+}
+
+// MatrixMultiplyScalarOperation (src/RMAD/MatrixMultiplyScalarOperation.cs): y = x * scalar, both directions.
+template <typename T>
+hipError_t launch_scale(T* y, const T* x, int64_t n, T alpha, hipStream_t s) {
+    StreamPtrs<T, 1, 1> p{{x}, {y}};
+    return launch_stream(p, n, Scale<T>{alpha}, s);
 }
 
 template <typename T>
@@ -276,6 +287,7 @@ hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double*
     template hipError_t launch_hadamard_bwd<T>(const T*, const T*, const T*, T*, T*, int64_t, hipStream_t);        \
     template hipError_t launch_accumulate<T>(T*, const T*, int64_t, hipStream_t);                                  \
     template hipError_t launch_copy<T>(T*, const T*, int64_t, hipStream_t);                                        \
+    template hipError_t launch_scale<T>(T*, const T*, int64_t, T, hipStream_t);                                    \
     template hipError_t launch_add_broadcast_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);        \
     template hipError_t launch_colsum<T>(const T*, T*, int64_t, int64_t, double*, hipStream_t);                             \
     template hipError_t launch_fill_zero<T>(T*, int64_t, hipStream_t);

@@ -503,6 +503,28 @@ int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_bu
 RAW_GEMM(f64, double)
 RAW_GEMM(f32, float)
 
+#define RAW_BATCHED_GEMM(SFX, T)                                                                                       \
+    int32_t prad_gemm_strided_batched_##SFX(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const T* A, \
+                                            int64_t lda, int64_t strideA, const T* B, int64_t ldb, int64_t strideB, T* C, \
+                                            int64_t ldc, int64_t strideC, int32_t batch, int32_t accumulate) {         \
+        REQUIRE_INIT();                                                                                                \
+        if (A == nullptr || B == nullptr || C == nullptr) return fail(PRAD_ERR_ARG, "NULL matrix pointer");            \
+        if (M < 0 || N < 0 || K < 0 || batch < 0 || strideA < 0 || strideB < 0 || strideC < 0)                         \
+            return fail(PRAD_ERR_ARG, "negative dimension");                                                           \
+        if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1) || (transA && transB))                        \
+            return fail(PRAD_ERR_ARG, "unsupported transpose combination (%d, %d)", transA, transB);                   \
+        if (lda < (transA ? M : K) || ldb < (transB ? K : N) || ldc < N) return fail(PRAD_ERR_ARG, "leading dimension too small"); \
+        if (batch > 1 && strideC < (M - 1) * ldc + N) return fail(PRAD_ERR_ARG, "outputs of different products overlap"); \
+        if (batch > 65535) return fail(PRAD_ERR_ARG, "at most 65535 products per call");                               \
+        GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                    \
+        a.batch = batch; a.strideA = strideA; a.strideB = strideB; a.strideC = strideC;                                \
+        std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                    \
+        HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);                                                     \
+        return PRAD_OK;                                                                                                \
+    }
+RAW_BATCHED_GEMM(f64, double)
+RAW_BATCHED_GEMM(f32, float)
+
 // ---------------------------------------------------------------------------------------------
 int32_t prad_matmul_fwd_host(int32_t dtype, const void* const* a_rows, const void* const* b_rows, void* const* c_rows, int64_t M,
                              int64_t K, int64_t K2, int64_t N) {
@@ -651,6 +673,17 @@ int32_t prad_hadamard_bwd(prad_buf_t a, prad_buf_t b, prad_buf_t dy, prad_buf_t 
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     DISPATCH(a, launch_hadamard_bwd<double>(D(a), D(b), D(dy), D(da), D(db), count(a), g_ctx.stream),
              launch_hadamard_bwd<float>(F(a), F(b), F(dy), F(da), F(db), count(a), g_ctx.stream));
+    return PRAD_OK;
+}
+
+int32_t prad_scale(prad_buf_t x, prad_buf_t y, double scalar) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(y);
+    if (int32_t st = same_dtype({x, y})) return st;
+    if (int32_t st = same_shape(x, y, "multiply by scalar")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_scale<double>(D(y), D(x), count(x), scalar, g_ctx.stream),
+             launch_scale<float>(F(y), F(x), count(x), (float)scalar, g_ctx.stream));
     return PRAD_OK;
 }
 

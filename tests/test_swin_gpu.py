@@ -1,0 +1,60 @@
+"""Windowed self-attention block step against the oracle's node-by-node composition (reduced sizes; the
+strided-batched entry point is also checked on its own)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import assert_parity
+from oracle import compose
+from parallelreverseautodiff_amd import _lib, seeded
+from parallelreverseautodiff_amd.matrix import DeviceBuffer
+from parallelreverseautodiff_amd.swin import SwinBlock
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype,cfg", [(np.float64, (1, 14, 32, 2)), (np.float32, (1, 14, 32, 2)), (np.float32, (2, 28, 96, 3))])
+def test_swin_block_matches_node_by_node_oracle(gpu, oracle, dtype, cfg):
+    images, side, embed, heads = cfg
+    blk = SwinBlock(images=images, side=side, embed=embed, heads=heads, dtype=dtype)
+    blk.step(update=False)
+    params = {k: blk.host[k] for k in blk.names}
+    loss, Y2, g, dX = compose.swin_block_forward_backward(params, blk.host["X"], blk.host["T"], blk.nw, blk.wt, heads)
+    tol = 1e-12 if dtype == np.float64 else 1e-5
+    assert abs(float(blk.loss.download()[0, 0]) - loss) <= tol * abs(loss)
+    assert_parity(blk.Y2.download(), Y2, dtype, "block output")
+    for k in blk.names:
+        assert_parity(blk.g[k].download(), g[k], dtype, "gradient of " + k)
+    assert_parity(blk.dX.download(), dX, dtype, "dX")
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_strided_batched_products_on_column_blocks(gpu, oracle, dtype):
+    """49 x 32 blocks taken out of a wide matrix by leading dimension and stride, all three orientations."""
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    fn = lib.prad_gemm_strided_batched_f64 if dtype == np.float64 else lib.prad_gemm_strided_batched_f32
+    nb, m, k, ld = 7, 49, 32, 96
+    A = seeded.normal(9, 1, (nb * m, ld), 1.0, dtype)
+    B = seeded.normal(9, 2, (nb * m, ld), 1.0, dtype)
+    dA, dB = DeviceBuffer.alloc(dtype, nb * m, ld), DeviceBuffer.alloc(dtype, nb * m, ld)
+    dA.upload(A); dB.upload(B)
+    es = np.dtype(dtype).itemsize
+    S = DeviceBuffer.alloc(dtype, nb * m, m)
+    check(fn(0, 1, m, m, k, ctypes.c_void_p(dA.ptr + 32 * es), ld, m * ld, ctypes.c_void_p(dB.ptr + 64 * es), ld, m * ld,
+             ctypes.c_void_p(S.ptr), m, m * m, nb, 0))
+    got = S.download()
+    for b in range(nb):
+        a_blk = np.ascontiguousarray(A[b * m:(b + 1) * m, 32:64]); b_blk = np.ascontiguousarray(B[b * m:(b + 1) * m, 64:96])
+        assert_parity(got[b * m:(b + 1) * m], oracle.matmul_fwd(a_blk, np.ascontiguousarray(b_blk.T)), dtype, "Q.K^T")
+    O = DeviceBuffer.alloc(dtype, nb * m, ld)
+    check(fn(1, 0, m, k, m, ctypes.c_void_p(S.ptr), m, m * m, ctypes.c_void_p(dB.ptr), ld, m * ld, ctypes.c_void_p(O.ptr + 32 * es),
+             ld, m * ld, nb, 0))
+    out = O.download()
+    for b in range(nb):
+        ref = oracle.matmul_fwd(np.ascontiguousarray(got[b * m:(b + 1) * m].T), np.ascontiguousarray(B[b * m:(b + 1) * m, 0:32]))
+        assert_parity(out[b * m:(b + 1) * m, 32:64], ref, dtype, "S^T.B")
+    assert not out[:, :32].any() and not out[:, 64:].any()  # neighbouring column blocks untouched
+    assert fn(0, 0, m, k, m, ctypes.c_void_p(S.ptr), m, m * m, ctypes.c_void_p(dB.ptr), ld, m * ld, ctypes.c_void_p(O.ptr), ld, 10, nb, 0) \
+        == _lib.PRAD_ERR_ARG  # overlapping outputs
