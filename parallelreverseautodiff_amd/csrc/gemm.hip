@@ -451,18 +451,27 @@ static TileShape choose_tile(int64_t M, int64_t N, int batch, bool tile_sums) {
         return -1;
     }();
     if (forced >= 0) return (TileShape)forced;
-    auto tiles = [&](int64_t em, int64_t en) { return ((M + em - 1) / em) * ((N + en - 1) / en) * batch; };
-    if (tiles(128, 128) >= 256) return TILE_128x128;
-    if (tiles(64, 64) >= 256) return TILE_64x64;
-    return TILE_32x32;
+    // Work actually multiplied when the output is padded to whole tiles of edge e.
+    auto padded = [&](int64_t e) { return ((M + e - 1) / e * e) * ((N + e - 1) / e * e); };
+    auto tiles = [&](int64_t e) { return ((M + e - 1) / e) * ((N + e - 1) / e) * batch; };
+    const int64_t least = padded(32) < padded(64) ? (padded(32) < padded(128) ? padded(32) : padded(128))
+                                                  : (padded(64) < padded(128) ? padded(64) : padded(128));
+    // A tile is admissible unless padding makes it multiply more than twice the best choice's work (a 49 x 49
+    // product must not run on a 128 x 128 tile, but a 96-wide output is still faster on it: measured);
+    // among the admissible ones take the largest that still gives 256 workgroups.
+    auto ok = [&](int64_t e) { return padded(e) <= 2 * least; };
+    if (ok(128) && tiles(128) >= 256) return TILE_128x128;
+    if (ok(64) && tiles(64) >= 256) return TILE_64x64;
+    if (ok(32)) return TILE_32x32;
+    return ok(64) ? TILE_64x64 : TILE_128x128;
 }
 
 int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
     const int64_t tiles = ((M + 31) / 32) * ((N + 31) / 32) * batch;  // the smallest tile is what such products get
     if (tiles >= 192) return 1;
     const int64_t bk = (elem_size == 8 ? Slab<double, 1>::BK : Slab<float, 1>::BK);
-    int64_t s = 384 / tiles;
-    if (s > 8) s = 8;
+    int64_t s = 512 / tiles;
+    if (s > 32) s = 32;
     if (s > K / (2 * bk)) s = K / (2 * bk);  // at least two slabs per split
     if (s < 2) return 1;
     const int64_t ksplit = ((K + s - 1) / s + bk - 1) / bk * bk;
