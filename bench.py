@@ -272,6 +272,36 @@ def swin_leg(dtype_name, steps, warmup, with_cpu):
     return out
 
 
+def oneshot_leg(n, dtype_name, steps):
+    """The call-per-operation entry points (jagged host rows in, jagged host rows out, like today's
+    GpuMatrixMultiplyOperation): marshalling, PCIe both ways and allocation are inside the timed region."""
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = 0
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    code = _lib.PRAD_F64 if dtype_name == "f64" else _lib.PRAD_F32
+
+    def jag(a):
+        rows = [np.array(a[i]) for i in range(a.shape[0])]
+        return rows, (ctypes.c_void_p * len(rows))(*[r.ctypes.data for r in rows])
+
+    A, pa = jag(seeded.uniform(1, 1, (n, n), -1, 1, dtype)); B, pb = jag(seeded.uniform(1, 2, (n, n), -1, 1, dtype))
+    G, pg = jag(seeded.normal(1, 3, (n, n), 1.0, dtype))
+    C, pc = jag(np.zeros((n, n), dtype)); dA, pda = jag(np.zeros((n, n), dtype)); dB, pdb = jag(np.zeros((n, n), dtype))
+    check(lib.prad_matmul_fwd_host(code, pa, pb, pc, n, n, n, n))
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        check(lib.prad_matmul_fwd_host(code, pa, pb, pc, n, n, n, n))
+        check(lib.prad_matmul_bwd_host(code, pg, pa, pb, pda, pdb, n, n, n))
+    secs = (time.perf_counter() - t0) / steps
+    return {"n": n, "ms_per_step": secs * 1e3, "TFLOPs": 6.0 * n ** 3 / secs / 1e12,
+            "host_bytes_per_step": 8 * n * n * np.dtype(dtype).itemsize}
+
+
 def mlp_leg(dtype_name, steps, warmup, with_cpu):
     """Feed-forward training step of configs[0]: batch 64, 784-256-128-10, LeakyReLU(0.01), softmax
     cross-entropy, clip, Adam.  Timed launch by launch and as one recorded launch sequence."""
@@ -399,7 +429,7 @@ def main():
     ap.add_argument("--n", type=int, default=4096)
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum", "lstm", "swin"], default="gemm",
+    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum", "lstm", "swin", "oneshot"], default="gemm",
                     help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
                          "mlp: the feed-forward training step of configs[0]")
     ap.add_argument("--elems", type=int, default=64 * 1024 * 1024, help="elements per tensor in bandwidth mode")
@@ -407,6 +437,13 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: this path has no multi-GPU part (--gpus 1 only)")
+    if args.mode == "oneshot":
+        res = oneshot_leg(args.n, args.dtype, args.steps)
+        print(json.dumps({"metric": "one-shot host-pointer matmul fwd+bwd TFLOP/s (PCIe and marshalling inclusive)", "unit": "TFLOP/s",
+                          "value": res["TFLOPs"], "n_gpus": 1, "steps": args.steps, "warmup": 1, "dtype": args.dtype, "data": "synthetic",
+                          "higher_is_better": True, "ms_per_step": res["ms_per_step"],
+                          "config": {"workload": "prad_matmul_fwd_host + prad_matmul_bwd_host, N=%d, jagged rows" % args.n}, "detail": res}))
+        return
     if args.mode == "swin":
         res = swin_leg(args.dtype, args.steps, args.warmup, not args.no_cpu)
         print(json.dumps({"metric": "Swin block train steps/sec", "unit": "steps/s", "value": 1e3 / res["recorded_ms_per_step"],
