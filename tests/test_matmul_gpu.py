@@ -1,6 +1,7 @@
 """Parity of the HIP matrix-multiply path with the CPU oracle, through the operation classes and
 the C ABI.  Bar: bit-exact where the arithmetic is exact (small integers), otherwise
-max |x - ref| / max(|ref|, 1e-3 rms) <= 1e-12 (double) / 1e-5 (float); the reduction order of the
+max |x - ref| / max(|ref|, rms(ref)) <= 1e-12 (double) / 1e-5 (float) and every entry of a product
+within the order-independent rounding bound 8*sqrt(K)*eps*(|A|.|B|)_ij; the reduction order of the
 MFMA kernels differs from the reference's k-ascending loop, which is what the tolerance is for."""
 import ctypes
 import json
