@@ -98,6 +98,13 @@ int32_t prad_matmul_fwd_fused(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_
  * dA = (dC . B^T) (.) act'(act_src), act_src shaped like dA. */
 int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB,
                               int32_t accumulate_dB, int32_t act, prad_buf_t act_src, double alpha);
+/* Backward of the pair MatrixMultiply -> MatrixAddBroadcasting (a layer's Z = A.B + bias) for the
+ * upstream gradient dC of Z: dB = A^T . dC, dbias = column sums of dC
+ * (src/RMAD/MatrixAddBroadcastingOperation.cs:57-70), dA = (dC . B^T) (.) act'(act_src) with
+ * act = PRAD_ACT_NONE for a plain dA.  dA, dB, dbias may each be NULL.  The column sum shares the
+ * launch of the dB product (both read dC only), so the pair costs two launches. */
+int32_t prad_matmul_bias_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, prad_buf_t dbias,
+                             int32_t accumulate_dB, int32_t act, prad_buf_t act_src, double alpha);
 /* General product on handles: C = op(A).op(B) (+ C when accumulate).  trans flags are 0/1.
  * Supported: (0,0), (0,1), (1,0). */
 int32_t prad_gemm(int32_t transA, int32_t transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int32_t accumulate);
@@ -186,13 +193,31 @@ int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_b
 /* ---- replay of a fixed launch sequence: everything enqueued by this thread between begin and end
  *      is recorded instead of executed and can then be launched as one submission.  The forward loop
  *      of the reference walks the same operation list every step
- *      (examples/feedforward/FeedForwardNeuralNetworkExample/FeedForwardNeuralNetwork.cs:212-303);
+ *      (examples/feedforward/ParallelReverseAutoDiff.FeedForwardExample/FeedForwardNeuralNetwork.cs:212-303);
  *      a recorded step replaces ~20 launches by one.  Only entry points that neither allocate nor
  *      copy to or from the host may be recorded. */
 int32_t prad_graph_begin(void);
 int32_t prad_graph_end(void** graph);
 int32_t prad_graph_launch(void* graph);
 int32_t prad_graph_destroy(void* graph);
+
+/* ---- branches: the reference's backward visitor runs Backward of operations that do not depend on
+ *      each other on pool threads (src/RMAD/OperationNeuralNetworkVisitor.cs:303-306).  Here such
+ *      operations are enqueued on different branches and may execute side by side; in a recording they
+ *      become parallel paths.  prad_fork(n) makes branches 1..n-1 start after everything enqueued on
+ *      branch 0 so far (it may be called again to hand later results of branch 0 to the open branches,
+ *      each branch keeps its own order); prad_branch(i) selects the branch that following calls enqueue
+ *      on (0 = the library stream); prad_join() makes branch 0 wait for all open branches, closes them
+ *      and selects branch 0.  The selection is library-wide: one thread submits while branches are open. */
+#define PRAD_MAX_BRANCHES 4
+int32_t prad_fork(int32_t branches);
+int32_t prad_branch(int32_t index);
+int32_t prad_join(void);
+/* Softmax.Forward (p), CategoricalCrossEntropy.Forward (loss, may be NULL) and .Backward (dp) and
+ * Softmax.Backward (dx) of one batch; same arithmetic as prad_softmax_fwd + prad_cce_fwd + prad_cce_bwd +
+ * prad_softmax_bwd (src/RMAD/SoftmaxOperation.cs:45-110,
+ * src/RMAD/Loss/CategoricalCrossEntropyLossOperation.cs:37-86), in one launch. */
+int32_t prad_softmax_cce(prad_buf_t x, prad_buf_t target, prad_buf_t p, prad_buf_t loss, prad_buf_t dp, prad_buf_t dx);
 
 /* ---- GradientClipper.ClipGradients, src/RMAD/GradientClipper.cs:118-157 and :212-253 (in place) */
 int32_t prad_clip(prad_buf_t g, double clip_value, double min_value);
@@ -205,6 +230,14 @@ int32_t prad_adam(prad_buf_t w, prad_buf_t m, prad_buf_t v, prad_buf_t g, double
 int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, double min_value);
 int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
                         double lr, double beta1, double beta2, double eps, double t);
+/* GradientClipper.Clip immediately followed by AdamOptimizer.Optimize over the same tensors, as every
+ * training loop of the reference calls them
+ * (examples/feedforward/ParallelReverseAutoDiff.FeedForwardExample/FeedForwardNeuralNetwork.cs:287-303): the clamping
+ * pass and the update share one pass over the data.  Results (clamped g, w, m, v) are those of
+ * prad_clip_multi followed by prad_adam_multi. */
+int32_t prad_clip_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
+                             double clip_value, double min_value, double lr, double beta1, double beta2, double eps,
+                             double t);
 
 /* ---- timing helpers for harnesses: events recorded on the library stream ------------------ */
 int32_t prad_event_create(void** ev);

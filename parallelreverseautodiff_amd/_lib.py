@@ -56,6 +56,7 @@ SIGNATURES = {
     "prad_matmul_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32]),
     "prad_matmul_fwd_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _f64]),
     "prad_matmul_bwd_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp, _f64]),
+    "prad_matmul_bias_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp, _f64]),
     "prad_gemm": (_i32, [_i32, _i32, _vp, _vp, _vp, _i32]),
     "prad_gemm_batched": (_i32, [_i32, _i32, _vp, _vp, _vp, _i32]),
     "prad_gemm_f64": (_i32, [_i32, _i32, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i32]),
@@ -83,6 +84,10 @@ SIGNATURES = {
     "prad_lstm_cell_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp]),
     "prad_lstm_cell_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_buf_view_rows": (_i32, [_vp, _i64, _i64, _vpp]),
+    "prad_fork": (_i32, [_i32]),
+    "prad_branch": (_i32, [_i32]),
+    "prad_join": (_i32, []),
+    "prad_softmax_cce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_graph_begin": (_i32, []),
     "prad_graph_end": (_i32, [_vpp]),
     "prad_graph_launch": (_i32, [_vp]),
@@ -91,6 +96,7 @@ SIGNATURES = {
     "prad_adam": (_i32, [_vp, _vp, _vp, _vp, _f64, _f64, _f64, _f64, _f64]),
     "prad_clip_multi": (_i32, [_vpp, _i32, _f64, _f64]),
     "prad_adam_multi": (_i32, [_vpp, _vpp, _vpp, _vpp, _i32, _f64, _f64, _f64, _f64, _f64]),
+    "prad_clip_adam_multi": (_i32, [_vpp, _vpp, _vpp, _vpp, _i32, _f64, _f64, _f64, _f64, _f64, _f64, _f64]),
     "prad_event_create": (_i32, [_vpp]),
     "prad_event_destroy": (_i32, [_vp]),
     "prad_event_record": (_i32, [_vp]),

@@ -133,7 +133,37 @@ struct GemmArgs {
     T* split_ws;
     // Set by launch_gemm for the kernels: K range per split (0 = not split).
     int64_t ksplit;
+    // A column sum that rides along with the product's launch (the bias gradient of
+    // MatrixAddBroadcasting next to the weight gradient, both functions of the same upstream
+    // gradient): colsum_dst[j] = sum_i colsum_src[i][j] over colsum_rows x colsum_cols, taken by extra
+    // workgroups appended to the grid.  nullptr = none.  Only for colsum_rows below COLSUM_CHUNK_ROWS.
+    const T* colsum_src;
+    T* colsum_dst;
+    int64_t colsum_rows, colsum_cols;
 };
+
+// Column sums of 64 columns [64 * bx, ...) over rows [r0, r1) by one workgroup of 256 threads (four
+// wavefronts take every fourth row, four accumulators each); part is 4 x 64 doubles of LDS.
+template <typename T, typename OUT>
+__device__ __forceinline__ void colsum_block(const T* __restrict__ dy, OUT* __restrict__ out, int64_t cols, int64_t r0, int64_t r1,
+                                             int64_t bx, double* part) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int64_t j = bx * 64 + lane;
+    double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
+    if (j < cols) {
+        int64_t i = r0 + w;
+        for (; i + 12 < r1; i += 16) {
+            const double a = (double)dy[i * cols + j], b = (double)dy[(i + 4) * cols + j];
+            const double c = (double)dy[(i + 8) * cols + j], d = (double)dy[(i + 12) * cols + j];
+            acc0 += a; acc1 += b; acc2 += c; acc3 += d;
+        }
+        for (; i < r1; i += 4) acc0 += (double)dy[i * cols + j];
+    }
+    part[w * 64 + lane] = (acc0 + acc1) + (acc2 + acc3);
+    __syncthreads();
+    if (w == 0 && j < cols) out[j] = (OUT)((part[lane] + part[64 + lane]) + (part[128 + lane] + part[192 + lane]));
+}
+constexpr int64_t COLSUM_CHUNK_ROWS = 2048;  // taller matrices are summed in row chunks by two launches
 
 // How many ways launch_gemm splits the reduction of a product whose output has too few tiles to occupy
 // the chip (1 = not split).  A split product writes its partial results to GemmArgs::split_ws and a
@@ -172,10 +202,13 @@ template <typename T> hipError_t launch_clip(const TensorDesc<T>* host_descs, in
                                              T min_value, hipStream_t s);
 template <typename T> hipError_t launch_adam(const TensorDesc<T>* host_descs, int ntensors, T lr, T beta1, T beta2, T eps, T c1,
                                              T c2, hipStream_t s);
+template <typename T> hipError_t launch_clip_adam(const TensorDesc<T>* host_descs, int ntensors, void* workspace, T clip_value,
+                                                  T min_value, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s);
 
 // softmax / categorical cross-entropy (csrc/loss.hip)
 template <typename T> hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_softmax_cce(const T* x, const T* t, T* y, T* dy, T* dx, T* loss, unsigned* counter, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_cce_fwd(const T* p, const T* t, T* loss, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t cols, hipStream_t s);
 

@@ -235,25 +235,10 @@ hipError_t launch_add_broadcast_fwd(const T* x, const T* bias, T* y, int64_t row
 template <typename T, typename OUT>
 __global__ void __launch_bounds__(256) colsum_kernel(const T* __restrict__ dy, OUT* __restrict__ out, int64_t rows, int64_t cols,
                                                      int64_t rows_per_chunk) {
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int64_t j = (int64_t)blockIdx.x * 64 + lane;
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk;
     const int64_t r1 = min(rows, r0 + rows_per_chunk);
-    double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
-    if (j < cols) {
-        int64_t i = r0 + w;
-        for (; i + 12 < r1; i += 16) {
-            const double a = (double)dy[i * cols + j], b = (double)dy[(i + 4) * cols + j];
-            const double c = (double)dy[(i + 8) * cols + j], d = (double)dy[(i + 12) * cols + j];
-            acc0 += a; acc1 += b; acc2 += c; acc3 += d;
-        }
-        for (; i < r1; i += 4) acc0 += (double)dy[i * cols + j];
-    }
-    __shared__ double part[4][64];
-    part[w][lane] = (acc0 + acc1) + (acc2 + acc3);
-    __syncthreads();
-    if (w == 0 && j < cols)
-        out[(int64_t)blockIdx.y * cols + j] = (OUT)((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]));
+    __shared__ double part[4 * 64];
+    colsum_block<T, OUT>(dy, out + (int64_t)blockIdx.y * cols, cols, r0, r1, blockIdx.x, part);
 }
 template <typename T>
 __global__ void __launch_bounds__(64) colsum_final_kernel(const double* __restrict__ partial, T* __restrict__ db, int chunks, int64_t cols) {
@@ -263,7 +248,7 @@ __global__ void __launch_bounds__(64) colsum_final_kernel(const double* __restri
     for (int c = 0; c < chunks; ++c) s += partial[(int64_t)c * cols + j];
     db[j] = (T)s;
 }
-int colsum_chunks(int64_t rows) { return rows >= 2048 ? (int)((rows + 255) / 256 > 64 ? 64 : (rows + 255) / 256) : 1; }
+int colsum_chunks(int64_t rows) { return rows >= COLSUM_CHUNK_ROWS ? (int)((rows + 255) / 256 > 64 ? 64 : (rows + 255) / 256) : 1; }
 // workspace: colsum_chunks(rows) * cols doubles when colsum_chunks(rows) > 1.
 template <typename T>
 hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double* workspace, hipStream_t s) {

@@ -189,6 +189,13 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
 
     __shared__ __attribute__((aligned(16))) T smem[2][SA + SB];  // [stage][A slab | B slab]
 
+    // Workgroups beyond the tiles carry a column sum that rides along with this launch.
+    if (blockIdx.x >= (unsigned)(tilesM * tilesN)) {
+        if (blockIdx.y == 0 && blockIdx.z == 0)
+            colsum_block<T, T>(p.colsum_src, p.colsum_dst, p.colsum_cols, 0, p.colsum_rows, blockIdx.x - tilesM * tilesN,
+                               reinterpret_cast<double*>(&smem[0][0]));
+        return;
+    }
     int tm, tn;
     tile_of_workgroup(blockIdx.x, tilesM, tilesN, tm, tn);
     const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
@@ -400,7 +407,8 @@ static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStr
     constexpr int BM = 32 * WT;
     const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BM - 1) / BM);
     const unsigned splits = a.ksplit > 0 ? (unsigned)((a.K + a.ksplit - 1) / a.ksplit) : 1u;
-    dim3 grid((unsigned)(tilesM * tilesN), (unsigned)a.batch, splits), block(GEMM_THREADS, 1, 1);
+    const unsigned riders = a.colsum_dst != nullptr ? (unsigned)((a.colsum_cols + 63) / 64) : 0u;
+    dim3 grid((unsigned)(tilesM * tilesN) + riders, (unsigned)a.batch, splits), block(GEMM_THREADS, 1, 1);
 #define PRAD_LAUNCH(EDGE_, EPI_) \
     hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, EDGE_, EPI_>), grid, block, 0, stream, a, tilesM, tilesN)
     if (edge) {
@@ -466,10 +474,23 @@ static TileShape choose_tile(int64_t M, int64_t N, int batch, bool tile_sums) {
     return ok(64) ? TILE_64x64 : TILE_128x128;
 }
 
+// Splitting K buys parallelism for products with few output tiles, at the price of a second launch
+// (the reduce) and a round trip of the partial results through memory: it pays only when the
+// unsplit K loop is long.  PRAD_GEMM_SPLIT_MIN_SLABS overrides the threshold (tuning aid).
+static int split_min_slabs() {
+    static const int v = [] {
+        const char* e = getenv("PRAD_GEMM_SPLIT_MIN_SLABS");
+        const int x = e ? atoi(e) : 0;
+        return x > 0 ? x : 6;
+    }();
+    return v;
+}
+
 int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
     const int64_t tiles = ((M + 31) / 32) * ((N + 31) / 32) * batch;  // the smallest tile is what such products get
     if (tiles >= 192) return 1;
     const int64_t bk = (elem_size == 8 ? Slab<double, 1>::BK : Slab<float, 1>::BK);
+    if ((K + bk - 1) / bk < split_min_slabs()) return 1;
     int64_t s = 512 / tiles;
     if (s > 32) s = 32;
     if (s > K / (2 * bk)) s = K / (2 * bk);  // at least two slabs per split

@@ -78,6 +78,71 @@ __global__ void __launch_bounds__(256) cce_bwd_kernel(const T* __restrict__ p, c
         dp[i] = -scale * t[i] / (p[i] + (T)1e-15);
 }
 
+// Softmax.Forward, CategoricalCrossEntropy.Backward and Softmax.Backward of one row by one wavefront
+// (same arithmetic, statement by statement, as the three kernels above).
+template <typename T>
+__device__ __forceinline__ void softmax_cce_row(const T* __restrict__ xr, const T* __restrict__ tr, T* __restrict__ yr,
+                                                T* __restrict__ gr, T* __restrict__ dxr, int64_t rows, int64_t cols, int lane) {
+    double mx = -INFINITY;
+    for (int64_t j = lane; j < cols; j += 64) mx = fmax(mx, (double)xr[j]);
+    const T m = (T)wave_max(mx);
+    double sum = 0.0;
+    for (int64_t j = lane; j < cols; j += 64) {
+        const T e = dev_exp(xr[j] - m);
+        yr[j] = e;
+        sum += (double)e;
+    }
+    const T s = (T)wave_sum(sum);
+    const T scale = (T)1 / (T)rows;
+    double dot = 0.0;
+    for (int64_t j = lane; j < cols; j += 64) {
+        const T p = yr[j] / s;
+        const T g = -scale * tr[j] / (p + (T)1e-15);
+        yr[j] = p;
+        gr[j] = g;
+        dot += (double)g * (double)p;
+    }
+    dot = wave_sum(dot);
+    for (int64_t j = lane; j < cols; j += 64) dxr[j] = (T)((double)yr[j] * ((double)gr[j] - dot));
+}
+
+// One wavefront per row, four rows per workgroup.  When the loss value is wanted, the workgroup that
+// finishes last (a counter in device memory tells) forms it from the finished p exactly as cce_fwd_kernel
+// does, so the whole loss stage of a step is one launch; it leaves the counter at zero for the next launch.
+template <typename T>
+__global__ void __launch_bounds__(256) softmax_cce_kernel(const T* __restrict__ x, const T* __restrict__ t, T* __restrict__ y,
+                                                          T* __restrict__ dy, T* __restrict__ dx, T* __restrict__ loss,
+                                                          unsigned* __restrict__ counter, int64_t rows, int64_t cols) {
+    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i < rows) {
+        const int64_t o = i * cols;
+        softmax_cce_row<T>(x + o, t + o, y + o, dy + o, dx + o, rows, cols, threadIdx.x & 63);
+    }
+    if (loss == nullptr) return;
+    __shared__ int last;
+    __threadfence();  // this workgroup's p is visible device-wide before its arrival is counted
+    __syncthreads();
+    if (threadIdx.x == 0) last = atomicAdd(counter, 1u) == gridDim.x - 1 ? 1 : 0;
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    const volatile T* p = y;  // written by other workgroups: read past this compute unit's cache
+    const int64_t n = rows * cols;
+    double s = 0.0;
+    for (int64_t e = threadIdx.x; e < n; e += 256) {
+        const T term = -t[e] * (T)log((double)(p[e] + (T)1e-15));
+        s += (double)term;
+    }
+    s = wave_sum(s);
+    __shared__ double part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        loss[0] = (T)((part[0] + part[1]) + (part[2] + part[3])) / (T)rows;
+        *counter = 0u;
+    }
+}
+
 // MeanSquaredErrorLossOperation (src/RMAD/Loss/MeanSquaredErrorLossOperation.cs): loss = sum (y - t)^2 / (rows*cols),
 // dy = (2 / (rows*cols)) * (y - t).  The sum is taken in two levels (per workgroup, then by one thread).
 template <typename T>
@@ -139,6 +204,16 @@ hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int6
     hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, y, dy, dx, rows, cols);
     return hipGetLastError();
 }
+// counter: one unsigned in device memory that is zero between launches (not shared with a launch that may
+// run at the same time).
+template <typename T>
+hipError_t launch_softmax_cce(const T* x, const T* t, T* y, T* dy, T* dx, T* loss, unsigned* counter, int64_t rows, int64_t cols,
+                              hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL((softmax_cce_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, x, t, y, dy, dx, loss, counter, rows,
+                       cols);
+    return hipGetLastError();
+}
 template <typename T>
 hipError_t launch_cce_fwd(const T* p, const T* t, T* loss, int64_t rows, int64_t cols, hipStream_t s) {
     hipLaunchKernelGGL((cce_fwd_kernel<T>), dim3(1), dim3(256), 0, s, p, t, loss, rows, cols);
@@ -156,6 +231,7 @@ hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t c
 #define INSTANTIATE(T)                                                                              \
     template hipError_t launch_softmax_fwd<T>(const T*, T*, int64_t, int64_t, hipStream_t);         \
     template hipError_t launch_softmax_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t); \
+    template hipError_t launch_softmax_cce<T>(const T*, const T*, T*, T*, T*, T*, unsigned*, int64_t, int64_t, hipStream_t); \
     template hipError_t launch_cce_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
     template hipError_t launch_cce_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
     template hipError_t launch_mse_fwd<T>(const T*, const T*, T*, double*, int64_t, hipStream_t);   \

@@ -153,12 +153,10 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTab
     }
 }
 
-// One workgroup per tensor merges its chunk moments: stats[ti] = {mean, stddev}.
-template <typename T>
-__global__ void __launch_bounds__(OPT_THREADS) clip_finalize_kernel(const TensorTable<T> tab, const Moments* __restrict__ partial,
-                                                                    double* __restrict__ stats) {
-    const int ti = blockIdx.x;
-    const int64_t c0 = tab.t[ti].first_chunk, nc = tab.t[ti].nchunks;
+// The whole workgroup merges the chunk moments [c0, c0 + nc) of one tensor; the result (mean,
+// population standard deviation) is valid in thread 0.  Contains a barrier.
+__device__ __forceinline__ void merge_tensor_chunks(const Moments* __restrict__ partial, int64_t c0, int64_t nc, double& mean,
+                                                    double& stddev) {
     Moments mo{0.0, 0.0, 0.0};
     // Eight independent loads in flight per lane before the (serial) merges.
     for (int64_t c = threadIdx.x; c < nc; c += OPT_THREADS * 8) {
@@ -176,12 +174,48 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_finalize_kernel(const Tensor
     __shared__ Moments wave_part[OPT_THREADS / 64];
     if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = mo;
     __syncthreads();
+    mean = 0.0; stddev = 0.0;
     if (threadIdx.x == 0) {
         Moments r = wave_part[0];
         for (int w = 1; w < OPT_THREADS / 64; ++w) r = merge(r, wave_part[w]);
-        stats[2 * ti] = r.mean;
-        stats[2 * ti + 1] = sqrt(r.m2 / r.n);  // population standard deviation
+        mean = r.mean;
+        stddev = sqrt(r.m2 / r.n);  // population standard deviation
     }
+}
+
+// One workgroup per tensor: stats[ti] = {mean, stddev}.
+template <typename T>
+__global__ void __launch_bounds__(OPT_THREADS) clip_finalize_kernel(const TensorTable<T> tab, const Moments* __restrict__ partial,
+                                                                    double* __restrict__ stats) {
+    const int ti = blockIdx.x;
+    double mean, stddev;
+    merge_tensor_chunks(partial, tab.t[ti].first_chunk, tab.t[ti].nchunks, mean, stddev);
+    if (threadIdx.x == 0) {
+        stats[2 * ti] = mean;
+        stats[2 * ti + 1] = stddev;
+    }
+}
+
+// Statistics of tensor ti for a workgroup of the clamping pass: read from stats when the finalize
+// launch ran, otherwise (tensors of few chunks) merged here by every workgroup for itself, in the
+// same order, which saves a launch where launches are what a step costs.
+constexpr int64_t INLINE_FINALIZE_CHUNKS = 256;
+template <typename T>
+__device__ __forceinline__ void tensor_stats(const DevTensor<T>& t, int ti, const double* __restrict__ stats,
+                                             const Moments* __restrict__ partial, T& mean, T& stddev) {
+    if (stats != nullptr) {
+        // PRADLite keeps mean and standard deviation in float.
+        mean = (T)stats[2 * ti];
+        stddev = (T)stats[2 * ti + 1];
+        return;
+    }
+    __shared__ double sh[2];
+    double m, sd;
+    merge_tensor_chunks(partial, t.first_chunk, t.nchunks, m, sd);
+    if (threadIdx.x == 0) { sh[0] = m; sh[1] = sd; }
+    __syncthreads();
+    mean = (T)sh[0];
+    stddev = (T)sh[1];
 }
 
 // .NET Math.Min: NaN when either argument is NaN.
@@ -193,18 +227,9 @@ __device__ __forceinline__ T dotnet_min(T a, T b) {
 }
 
 template <typename T>
-__global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTable<T> tab, const double* __restrict__ stats,
-                                                                 T clip_value, T min_value) {
-    const int64_t chunk = blockIdx.x;
-    const int ti = find_tensor(tab.t, tab.nt, chunk);
-    const DevTensor<T> t = tab.t[ti];
-    // PRADLite keeps mean and standard deviation in float.
-    const T mean = (T)stats[2 * ti];
-    const T stddev = (T)stats[2 * ti + 1];
-    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
-    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
-    constexpr int PER = OPT_CHUNK / OPT_THREADS;
-    auto clamp = [&](T g) -> T {
+struct Clamp {
+    T mean, stddev, clip_value, min_value;
+    __device__ __forceinline__ T operator()(T g) const {
         const T z = (g - mean) / stddev;
         const T value = dotnet_min<T>(clip_value, (T)1 + (z < (T)0 ? -z : z));
         if (g > value) g = value;
@@ -212,7 +237,36 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTab
         if (g > (T)0 && g < min_value) g = min_value;
         else if (g < (T)0 && g > -min_value) g = -min_value;
         return g;
-    };
+    }
+};
+
+template <typename T>
+struct AdamUpdate {
+    T lr, beta1, beta2, omb1, omb2, c1, c2, eps;
+    __device__ __forceinline__ void operator()(T& w, T& m, T& v, T g) const {
+        const T first = (beta1 * m) + (omb1 * g);
+        const T second = (beta2 * v) + (omb2 * (g * g));
+        const T mhat = c1 * first;
+        const T vhat = c2 * second;
+        const T red = lr * mhat / (sqrt(vhat) + eps);
+        w = w - red;
+        m = first;
+        v = second;
+    }
+};
+
+template <typename T>
+__global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTable<T> tab, const double* __restrict__ stats,
+                                                                 const Moments* __restrict__ partial, T clip_value, T min_value) {
+    const int64_t chunk = blockIdx.x;
+    const int ti = find_tensor(tab.t, tab.nt, chunk);
+    const DevTensor<T> t = tab.t[ti];
+    Clamp<T> clamp;
+    tensor_stats<T>(t, ti, stats, partial, clamp.mean, clamp.stddev);
+    clamp.clip_value = clip_value; clamp.min_value = min_value;
+    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
+    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
+    constexpr int PER = OPT_CHUNK / OPT_THREADS;
     if (vector_chunk<T>(t.g, nullptr, nullptr, nullptr, begin, end)) {
         typedef typename OptVec<T>::type V;
         constexpr int VN = OptVec<T>::N;
@@ -235,26 +289,24 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTab
     }
 }
 
-// Adam: one pass over w, m, v, g (7 element sizes of HBM traffic per element).
-template <typename T>
-__global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> tab, T lr, T beta1, T beta2, T omb1, T omb2,
-                                                           T c1, T c2, T eps) {
+// Adam: one pass over w, m, v, g (7 element sizes of HBM traffic per element).  With CLIP the clamping
+// pass of the clipper runs in the same pass (the clamped gradient is stored, as the clipper does in
+// place): 8 element sizes instead of 2 + 7 for the two passes.
+template <typename T, bool CLIP>
+__global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> tab, const AdamUpdate<T> update,
+                                                           const double* __restrict__ stats, const Moments* __restrict__ partial,
+                                                           T clip_value, T min_value) {
     const int64_t chunk = blockIdx.x;
     const int ti = find_tensor(tab.t, tab.nt, chunk);
     const DevTensor<T> t = tab.t[ti];
+    Clamp<T> clamp{};
+    if (CLIP) {
+        tensor_stats<T>(t, ti, stats, partial, clamp.mean, clamp.stddev);
+        clamp.clip_value = clip_value; clamp.min_value = min_value;
+    }
     const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
     const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
     constexpr int PER = OPT_CHUNK / OPT_THREADS;
-    auto update = [&](T& w, T& m, T& v, T g) {
-        const T first = (beta1 * m) + (omb1 * g);
-        const T second = (beta2 * v) + (omb2 * (g * g));
-        const T mhat = c1 * first;
-        const T vhat = c2 * second;
-        const T red = lr * mhat / (sqrt(vhat) + eps);
-        w = w - red;
-        m = first;
-        v = second;
-    };
     if (vector_chunk<T>(t.w, t.m, t.v, t.g, begin, end)) {
         typedef typename OptVec<T>::type V;
         constexpr int VN = OptVec<T>::N;
@@ -262,7 +314,7 @@ __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> 
         V* __restrict__ wv = reinterpret_cast<V*>(t.w + begin);
         V* __restrict__ mv = reinterpret_cast<V*>(t.m + begin);
         V* __restrict__ vv = reinterpret_cast<V*>(t.v + begin);
-        const V* __restrict__ gv = reinterpret_cast<const V*>(t.g + begin);
+        V* __restrict__ gv = reinterpret_cast<V*>(t.g + begin);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             V w[HALF], m[HALF], v[HALF], g[HALF];
@@ -280,9 +332,11 @@ __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> 
 #pragma unroll
                 for (int c = 0; c < VN; ++c) {
                     T wi = w[e][c], mi = m[e][c], vi = v[e][c];
+                    if (CLIP) g[e][c] = clamp(g[e][c]);
                     update(wi, mi, vi, g[e][c]);
                     w[e][c] = wi; m[e][c] = mi; v[e][c] = vi;
                 }
+                if (CLIP) __builtin_nontemporal_store(g[e], gv + iv);
                 __builtin_nontemporal_store(w[e], wv + iv);
                 __builtin_nontemporal_store(m[e], mv + iv);
                 __builtin_nontemporal_store(v[e], vv + iv);
@@ -294,8 +348,9 @@ __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> 
     for (int e = 0; e < PER; ++e) {
         const int64_t i = begin + (int64_t)e * OPT_THREADS + threadIdx.x;
         if (i < end) {
-            T wi = t.w[i], mi = t.m[i], vi = t.v[i];
-            update(wi, mi, vi, t.g[i]);
+            T wi = t.w[i], mi = t.m[i], vi = t.v[i], gi = t.g[i];
+            if (CLIP) { gi = clamp(gi); t.g[i] = gi; }
+            update(wi, mi, vi, gi);
             t.w[i] = wi; t.m[i] = mi; t.v[i] = vi;
         }
     }
@@ -327,6 +382,25 @@ size_t clip_workspace_bytes(const int64_t* n, int nt) {
     return worst + 64;
 }
 
+// Statistics passes of the clipper for one group of tensors; returns in *stats_out the finalized
+// statistics, or NULL when every tensor is small enough for the clamping pass to merge its chunks itself.
+template <typename T>
+static void enqueue_clip_stats(const TensorTable<T>& tab, int gn, int64_t chunks, void* workspace, const double** stats_out,
+                               const Moments** partial_out, hipStream_t s) {
+    double* dstats = reinterpret_cast<double*>(workspace);
+    Moments* dpartial = reinterpret_cast<Moments*>(static_cast<char*>(workspace) + (size_t)MAX_TABLE * 16);
+    hipLaunchKernelGGL((clip_stats_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, dpartial);
+    int64_t most = 0;
+    for (int i = 0; i < gn; ++i) most = tab.t[i].nchunks > most ? tab.t[i].nchunks : most;
+    if (most > INLINE_FINALIZE_CHUNKS) {
+        hipLaunchKernelGGL((clip_finalize_kernel<T>), dim3((unsigned)gn), dim3(OPT_THREADS), 0, s, tab, dpartial, dstats);
+        *stats_out = dstats;
+    } else {
+        *stats_out = nullptr;
+    }
+    *partial_out = dpartial;
+}
+
 template <typename T>
 hipError_t launch_clip(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value, hipStream_t s) {
     for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
@@ -334,11 +408,9 @@ hipError_t launch_clip(const TensorDesc<T>* host, int nt, void* workspace, T cli
         TensorTable<T> tab;
         const int64_t chunks = build_table(host + g0, gn, tab);
         if (chunks == 0) continue;
-        double* dstats = reinterpret_cast<double*>(workspace);
-        Moments* dpartial = reinterpret_cast<Moments*>(static_cast<char*>(workspace) + (size_t)MAX_TABLE * 16);
-        hipLaunchKernelGGL((clip_stats_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, dpartial);
-        hipLaunchKernelGGL((clip_finalize_kernel<T>), dim3((unsigned)gn), dim3(OPT_THREADS), 0, s, tab, dpartial, dstats);
-        hipLaunchKernelGGL((clip_apply_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, dstats, clip_value,
+        const double* stats; const Moments* partial;
+        enqueue_clip_stats<T>(tab, gn, chunks, workspace, &stats, &partial, s);
+        hipLaunchKernelGGL((clip_apply_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, stats, partial, clip_value,
                            min_value);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -348,14 +420,35 @@ hipError_t launch_clip(const TensorDesc<T>* host, int nt, void* workspace, T cli
 
 template <typename T>
 hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s) {
-    const T omb1 = (T)1 - beta1, omb2 = (T)1 - beta2;
+    const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps};
     for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
         const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
         TensorTable<T> tab;
         const int64_t chunks = build_table(host + g0, gn, tab);
         if (chunks == 0) continue;
-        hipLaunchKernelGGL((adam_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, lr, beta1, beta2, omb1, omb2,
-                           c1, c2, eps);
+        hipLaunchKernelGGL((adam_kernel<T, false>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, update,
+                           (const double*)nullptr, (const Moments*)nullptr, (T)0, (T)0);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+// GradientClipper.Clip followed by AdamOptimizer.Optimize over the same tensors: statistics pass, then
+// one pass that clamps the gradient and updates w, m, v.
+template <typename T>
+hipError_t launch_clip_adam(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value, T lr, T beta1, T beta2,
+                            T eps, T c1, T c2, hipStream_t s) {
+    const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps};
+    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
+        const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
+        TensorTable<T> tab;
+        const int64_t chunks = build_table(host + g0, gn, tab);
+        if (chunks == 0) continue;
+        const double* stats; const Moments* partial;
+        enqueue_clip_stats<T>(tab, gn, chunks, workspace, &stats, &partial, s);
+        hipLaunchKernelGGL((adam_kernel<T, true>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, update, stats, partial,
+                           clip_value, min_value);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -367,5 +460,9 @@ template hipError_t launch_clip<float>(const TensorDesc<float>*, int, void*, flo
 template hipError_t launch_adam<double>(const TensorDesc<double>*, int, double, double, double, double, double, double,
                                         hipStream_t);
 template hipError_t launch_adam<float>(const TensorDesc<float>*, int, float, float, float, float, float, float, hipStream_t);
+template hipError_t launch_clip_adam<double>(const TensorDesc<double>*, int, void*, double, double, double, double, double, double,
+                                             double, double, hipStream_t);
+template hipError_t launch_clip_adam<float>(const TensorDesc<float>*, int, void*, float, float, float, float, float, float, float,
+                                            float, hipStream_t);
 
 }  // namespace prad

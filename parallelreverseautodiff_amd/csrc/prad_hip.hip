@@ -33,17 +33,35 @@ namespace {
 constexpr uint32_t BUF_MAGIC = 0x50524144u;  // "PRAD"
 constexpr size_t STAGING_CHUNK = (size_t)256 << 20;
 
+constexpr int MAX_BRANCHES = PRAD_MAX_BRANCHES;
+
+// Branch 0 is the library stream; branches 1.. exist so that independent operations can overlap
+// (prad_fork / prad_branch / prad_join).  Each branch has its own kernel workspace, because two
+// kernels that run side by side cannot share partial-result storage.
+struct Branch {
+    hipStream_t stream = nullptr;
+    hipEvent_t done = nullptr;
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
+    unsigned* counter = nullptr;  // arrival counter for kernels whose last workgroup finishes the job; zero between launches
+    bool open = false;
+};
+
 struct Context {
     std::mutex mu;
     std::atomic<bool> initialized{false};
     int device = -1;
-    hipStream_t stream = nullptr;
+    hipStream_t stream = nullptr;  // == branch[0].stream
+    Branch branch[MAX_BRANCHES];
+    int cur = 0;
+    hipEvent_t fork_event = nullptr;
     void* pinned = nullptr;
     size_t pinned_bytes = 0;
-    void* workspace = nullptr;
-    size_t workspace_bytes = 0;
 };
 Context g_ctx;
+inline Branch& cur_branch() { return g_ctx.branch[g_ctx.cur]; }
+#define CUR_STREAM (g_ctx.branch[g_ctx.cur].stream)
+#define CUR_WORKSPACE (g_ctx.branch[g_ctx.cur].workspace)
 thread_local std::string tl_error;
 
 int32_t fail(int32_t code, const char* fmt, ...) {
@@ -79,9 +97,21 @@ inline int64_t count(prad_buf_t b) { return b->depth * b->rows * b->cols; }
     } while (0)
 
 // Lock must be held.
+// Waits for everything enqueued on the library stream and on every branch.
+int32_t sync_all() {
+    for (int i = 0; i < MAX_BRANCHES; ++i)
+        if (g_ctx.branch[i].stream) HIP_TRY(hipStreamSynchronize(g_ctx.branch[i].stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+// Copies run on the library stream; results that open branches still produce are waited for first.
+int32_t drain_open_branches() {
+    for (int i = 1; i < MAX_BRANCHES; ++i)
+        if (g_ctx.branch[i].open) HIP_TRY(hipStreamSynchronize(g_ctx.branch[i].stream), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
 int32_t ensure_pinned(size_t bytes) {
     if (bytes <= g_ctx.pinned_bytes) return PRAD_OK;
-    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    if (int32_t st = sync_all()) return st;
     if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
     g_ctx.pinned = nullptr;
     g_ctx.pinned_bytes = 0;
@@ -89,15 +119,18 @@ int32_t ensure_pinned(size_t bytes) {
     g_ctx.pinned_bytes = bytes;
     return PRAD_OK;
 }
+// Grows the workspace of the branch that is selected (its stream is drained first; while a launch
+// sequence is being recorded that fails, which is why a recording follows an eager warm-up).
 int32_t ensure_workspace(size_t bytes) {
-    if (bytes <= g_ctx.workspace_bytes) return PRAD_OK;
-    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
-    if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
-    g_ctx.workspace = nullptr;
-    g_ctx.workspace_bytes = 0;
+    Branch& b = cur_branch();
+    if (bytes <= b.workspace_bytes) return PRAD_OK;
+    HIP_TRY(hipStreamSynchronize(b.stream), PRAD_ERR_LAUNCH);
+    if (b.workspace) (void)hipFree(b.workspace);
+    b.workspace = nullptr;
+    b.workspace_bytes = 0;
     bytes = (bytes + 4095) & ~(size_t)4095;
-    HIP_TRY(hipMalloc(&g_ctx.workspace, bytes), PRAD_ERR_ALLOC);
-    g_ctx.workspace_bytes = bytes;
+    HIP_TRY(hipMalloc(&b.workspace, bytes), PRAD_ERR_ALLOC);
+    b.workspace_bytes = bytes;
     return PRAD_OK;
 }
 
@@ -131,7 +164,7 @@ int32_t attach_split_workspace(GemmArgs<T>& a) {
     const int splits = gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T));
     if (splits <= 1) return PRAD_OK;
     if (int32_t st = ensure_workspace((size_t)splits * a.batch * a.M * a.N * sizeof(T))) return st;
-    a.split_ws = static_cast<T*>(g_ctx.workspace);
+    a.split_ws = static_cast<T*>(CUR_WORKSPACE);
     return PRAD_OK;
 }
 
@@ -146,6 +179,9 @@ struct Epilogue {
     int act_bwd = PRAD_ACT_NONE;
     prad_buf_t act_src = nullptr;
     double alpha = 0.0;
+    // column sum riding along with the launch: colsum_dst (1 x cols) = column sums of colsum_src
+    prad_buf_t colsum_src = nullptr;
+    prad_buf_t colsum_dst = nullptr;
 };
 
 template <typename T>
@@ -159,6 +195,12 @@ int32_t enqueue_gemm_t(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_
     a.act_bwd = ep.act_bwd;
     if (ep.act_src) { a.act_src = static_cast<const T*>(ep.act_src->ptr); a.ld_act = ep.act_src->cols; }
     a.alpha = (T)ep.alpha;
+    if (ep.colsum_dst) {
+        a.colsum_src = static_cast<const T*>(ep.colsum_src->ptr);
+        a.colsum_dst = static_cast<T*>(ep.colsum_dst->ptr);
+        a.colsum_rows = ep.colsum_src->rows;
+        a.colsum_cols = ep.colsum_src->cols;
+    }
     if (batched) {
         a.batch = (int)C->depth;
         a.strideA = A->depth == 1 ? 0 : A->rows * A->cols;
@@ -166,7 +208,7 @@ int32_t enqueue_gemm_t(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_
         a.strideC = C->rows * C->cols;
     }
     if (int32_t st = attach_split_workspace(a)) return st;
-    HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);
+    HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
 
@@ -176,7 +218,7 @@ int32_t enqueue_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_bu
     REQUIRE_BUF(A); REQUIRE_BUF(B); REQUIRE_BUF(C);
     if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1) || (transA && transB))
         return fail(PRAD_ERR_ARG, "unsupported transpose combination (%d, %d)", transA, transB);
-    if (int32_t st = same_dtype({A, B, C, ep.bias, ep.Z, ep.act_src})) return st;
+    if (int32_t st = same_dtype({A, B, C, ep.bias, ep.Z, ep.act_src, ep.colsum_src, ep.colsum_dst})) return st;
     if (op_cols(A, transA) != op_rows(B, transB))
         return fail(PRAD_ERR_SHAPE, "Input 1 columns do not match Input 2 rows");
     if (C->rows != op_rows(A, transA) || C->cols != op_cols(B, transB))
@@ -230,7 +272,16 @@ int32_t prad_init(int32_t device_id) {
     HIP_TRY(hipGetDeviceProperties(&prop, device_id), PRAD_ERR_NOT_INITIALIZED);
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(PRAD_ERR_NOT_INITIALIZED, "device %d is %s; this library is built for gfx950 only", device_id, prop.gcnArchName);
-    HIP_TRY(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking), PRAD_ERR_NOT_INITIALIZED);
+    for (int i = 0; i < MAX_BRANCHES; ++i) {
+        HIP_TRY(hipStreamCreateWithFlags(&g_ctx.branch[i].stream, hipStreamNonBlocking), PRAD_ERR_NOT_INITIALIZED);
+        HIP_TRY(hipEventCreateWithFlags(&g_ctx.branch[i].done, hipEventDisableTiming), PRAD_ERR_NOT_INITIALIZED);
+        g_ctx.branch[i].open = false;
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.branch[i].counter), 256), PRAD_ERR_ALLOC);
+        HIP_TRY(hipMemset(g_ctx.branch[i].counter, 0, 256), PRAD_ERR_ALLOC);
+    }
+    HIP_TRY(hipEventCreateWithFlags(&g_ctx.fork_event, hipEventDisableTiming), PRAD_ERR_NOT_INITIALIZED);
+    g_ctx.stream = g_ctx.branch[0].stream;
+    g_ctx.cur = 0;
     g_ctx.device = device_id;
     g_ctx.initialized.store(true);
     return PRAD_OK;
@@ -240,13 +291,20 @@ int32_t prad_shutdown(void) {
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     if (!g_ctx.initialized.load()) return PRAD_OK;
     (void)hipSetDevice(g_ctx.device);
-    (void)hipStreamSynchronize(g_ctx.stream);
+    (void)sync_all();
     if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
-    if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
-    (void)hipStreamDestroy(g_ctx.stream);
+    for (Branch& b : g_ctx.branch) {
+        if (b.workspace) (void)hipFree(b.workspace);
+        if (b.counter) (void)hipFree(b.counter);
+        if (b.done) (void)hipEventDestroy(b.done);
+        if (b.stream) (void)hipStreamDestroy(b.stream);
+        b = Branch{};
+    }
+    if (g_ctx.fork_event) (void)hipEventDestroy(g_ctx.fork_event);
+    g_ctx.fork_event = nullptr;
     g_ctx.pinned = nullptr; g_ctx.pinned_bytes = 0;
-    g_ctx.workspace = nullptr; g_ctx.workspace_bytes = 0;
     g_ctx.stream = nullptr;
+    g_ctx.cur = 0;
     g_ctx.device = -1;
     g_ctx.initialized.store(false);
     return PRAD_OK;
@@ -259,8 +317,7 @@ void* prad_stream(void) { return g_ctx.stream; }
 
 int32_t prad_stream_sync(void) {
     REQUIRE_INIT();
-    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
-    return PRAD_OK;
+    return sync_all();
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -275,8 +332,8 @@ int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t 
     HIP_TRY(hipMalloc(&p, bytes), PRAD_ERR_ALLOC);
     {
         std::lock_guard<std::mutex> lock(g_ctx.mu);
-        hipError_t e = dtype == PRAD_F64 ? launch_fill_zero<double>(static_cast<double*>(p), depth * rows * cols, g_ctx.stream)
-                                         : launch_fill_zero<float>(static_cast<float*>(p), depth * rows * cols, g_ctx.stream);
+        hipError_t e = dtype == PRAD_F64 ? launch_fill_zero<double>(static_cast<double*>(p), depth * rows * cols, CUR_STREAM)
+                                         : launch_fill_zero<float>(static_cast<float*>(p), depth * rows * cols, CUR_STREAM);
         if (e != hipSuccess) { (void)hipFree(p); return fail(PRAD_ERR_LAUNCH, "zero fill failed: %s", hipGetErrorString(e)); }
     }
     prad_buf* b = new prad_buf{BUF_MAGIC, dtype, depth, rows, cols, p, true};
@@ -304,7 +361,7 @@ int32_t prad_buf_free(prad_buf_t b) {
         REQUIRE_INIT();
         std::lock_guard<std::mutex> lock(g_ctx.mu);
         // Work that still uses the buffer may be queued.
-        HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+        if (int32_t st = sync_all()) return st;
         HIP_TRY(hipFree(b->ptr), PRAD_ERR_ALLOC);
     }
     b->magic = 0;
@@ -327,8 +384,8 @@ int32_t prad_buf_zero(prad_buf_t b) {
     REQUIRE_INIT();
     REQUIRE_BUF(b);
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (b->dtype == PRAD_F64) HIP_TRY(launch_fill_zero<double>(static_cast<double*>(b->ptr), count(b), g_ctx.stream), PRAD_ERR_LAUNCH);
-    else HIP_TRY(launch_fill_zero<float>(static_cast<float*>(b->ptr), count(b), g_ctx.stream), PRAD_ERR_LAUNCH);
+    if (b->dtype == PRAD_F64) HIP_TRY(launch_fill_zero<double>(static_cast<double*>(b->ptr), count(b), CUR_STREAM), PRAD_ERR_LAUNCH);
+    else HIP_TRY(launch_fill_zero<float>(static_cast<float*>(b->ptr), count(b), CUR_STREAM), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
 
@@ -344,6 +401,7 @@ int32_t prad_buf_upload_rows(prad_buf_t b, const void* const* row_ptrs, const in
         if (row_ptrs[i] == nullptr) return fail(PRAD_ERR_NOT_RECTANGULAR, "The given jagged array is not rectangular.");
     const size_t row_bytes = (size_t)b->cols * elem_size(b->dtype);
     std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (int32_t st = drain_open_branches()) return st;
     int64_t rows_per_chunk = (int64_t)(STAGING_CHUNK / row_bytes);
     if (rows_per_chunk < 1) rows_per_chunk = 1;
     if (rows_per_chunk > nrows) rows_per_chunk = nrows;
@@ -368,6 +426,7 @@ int32_t prad_buf_download_rows(prad_buf_t b, void* const* row_ptrs) {
         if (row_ptrs[i] == nullptr) return fail(PRAD_ERR_NOT_RECTANGULAR, "The given jagged array is not rectangular.");
     const size_t row_bytes = (size_t)b->cols * elem_size(b->dtype);
     std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (int32_t st = drain_open_branches()) return st;
     int64_t rows_per_chunk = (int64_t)(STAGING_CHUNK / row_bytes);
     if (rows_per_chunk < 1) rows_per_chunk = 1;
     if (rows_per_chunk > nrows) rows_per_chunk = nrows;
@@ -389,6 +448,7 @@ int32_t prad_buf_upload(prad_buf_t b, const void* src, int64_t ld) {
     if (src == nullptr || ld < b->cols) return fail(PRAD_ERR_ARG, "bad source pointer or leading dimension");
     const size_t es = elem_size(b->dtype);
     std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (int32_t st = drain_open_branches()) return st;
     HIP_TRY(hipMemcpy2DAsync(b->ptr, (size_t)b->cols * es, src, (size_t)ld * es, (size_t)b->cols * es,
                              (size_t)(b->depth * b->rows), hipMemcpyHostToDevice, g_ctx.stream), PRAD_ERR_LAUNCH);
     HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
@@ -401,6 +461,7 @@ int32_t prad_buf_download(prad_buf_t b, void* dst, int64_t ld) {
     if (dst == nullptr || ld < b->cols) return fail(PRAD_ERR_ARG, "bad destination pointer or leading dimension");
     const size_t es = elem_size(b->dtype);
     std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (int32_t st = drain_open_branches()) return st;
     HIP_TRY(hipMemcpy2DAsync(dst, (size_t)ld * es, b->ptr, (size_t)b->cols * es, (size_t)b->cols * es,
                              (size_t)(b->depth * b->rows), hipMemcpyDeviceToHost, g_ctx.stream), PRAD_ERR_LAUNCH);
     HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
@@ -416,10 +477,10 @@ int32_t prad_buf_copy(prad_buf_t dst, prad_buf_t src) {
     // A kernel rather than hipMemcpyAsync: it can be recorded into a captured graph and shows up in
     // kernel traces as a plain copy of known size.
     if (src->dtype == PRAD_F64)
-        HIP_TRY(launch_copy<double>(static_cast<double*>(dst->ptr), static_cast<const double*>(src->ptr), count(src), g_ctx.stream),
+        HIP_TRY(launch_copy<double>(static_cast<double*>(dst->ptr), static_cast<const double*>(src->ptr), count(src), CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     else
-        HIP_TRY(launch_copy<float>(static_cast<float*>(dst->ptr), static_cast<const float*>(src->ptr), count(src), g_ctx.stream),
+        HIP_TRY(launch_copy<float>(static_cast<float*>(dst->ptr), static_cast<const float*>(src->ptr), count(src), CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -454,8 +515,14 @@ int32_t prad_matmul_fwd_fused(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_
 }
 
 static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, int32_t acc_dA,
-                                 int32_t acc_dB, const Epilogue& ep) {
+                                 int32_t acc_dB, const Epilogue& ep, prad_buf_t dbias = nullptr) {
     REQUIRE_BUF(dC); REQUIRE_BUF(A); REQUIRE_BUF(B);
+    if (dbias != nullptr) {
+        REQUIRE_BUF(dbias);
+        if (dbias->dtype != dC->dtype) return fail(PRAD_ERR_DTYPE, "buffers of different element types in one call");
+        if (dbias->cols != dC->cols || dbias->rows != 1 || dbias->depth != 1 || dC->depth != 1)
+            return fail(PRAD_ERR_ARG, "bias gradient must be 1 x cols");
+    }
     if (A->cols != B->rows) return fail(PRAD_ERR_SHAPE, "Input 1 columns do not match Input 2 rows");
     if (dC->rows != A->rows || dC->cols != B->cols)
         return fail(PRAD_ERR_ARG, "upstream gradient is %lldx%lld, the product is %lldx%lld", (long long)dC->rows,
@@ -464,7 +531,23 @@ static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad
         if (int32_t st = enqueue_gemm(0, 1, dC, B, dA, acc_dA, ep, false)) return st;  // dA = dC . B^T
     }
     if (dB != nullptr) {
-        if (int32_t st = enqueue_gemm(1, 0, A, dC, dB, acc_dB, Epilogue{}, false)) return st;  // dB = A^T . dC
+        Epilogue rider;
+        if (dbias != nullptr && dC->rows < COLSUM_CHUNK_ROWS) { rider.colsum_src = dC; rider.colsum_dst = dbias; }
+        if (int32_t st = enqueue_gemm(1, 0, A, dC, dB, acc_dB, rider, false)) return st;  // dB = A^T . dC
+        if (rider.colsum_dst != nullptr) dbias = nullptr;
+    }
+    if (dbias != nullptr) {  // no weight-gradient launch to ride along with, or a tall matrix: own launch(es)
+        double* ws = nullptr;
+        if (colsum_chunks(dC->rows) > 1) {
+            if (int32_t st = ensure_workspace((size_t)colsum_chunks(dC->rows) * dC->cols * sizeof(double))) return st;
+            ws = static_cast<double*>(CUR_WORKSPACE);
+        }
+        if (dC->dtype == PRAD_F64)
+            HIP_TRY(launch_colsum<double>(static_cast<const double*>(dC->ptr), static_cast<double*>(dbias->ptr), dC->rows, dC->cols, ws,
+                                          CUR_STREAM), PRAD_ERR_LAUNCH);
+        else
+            HIP_TRY(launch_colsum<float>(static_cast<const float*>(dC->ptr), static_cast<float*>(dbias->ptr), dC->rows, dC->cols, ws,
+                                         CUR_STREAM), PRAD_ERR_LAUNCH);
     }
     return PRAD_OK;
 }
@@ -485,6 +568,15 @@ int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_bu
     return matmul_bwd_locked(dC, A, B, dA, dB, 0, accumulate_dB, ep);
 }
 
+int32_t prad_matmul_bias_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, prad_buf_t dbias,
+                             int32_t accumulate_dB, int32_t act, prad_buf_t act_src, double alpha) {
+    REQUIRE_INIT();
+    Epilogue ep;
+    ep.act_bwd = act; ep.act_src = act_src; ep.alpha = alpha;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return matmul_bwd_locked(dC, A, B, dA, dB, 0, accumulate_dB, ep, dbias);
+}
+
 #define RAW_GEMM(SFX, T)                                                                                              \
     int32_t prad_gemm_##SFX(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const T* A, int64_t lda, \
                             const T* B, int64_t ldb, T* C, int64_t ldc, int32_t accumulate) {                         \
@@ -497,7 +589,7 @@ int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_bu
         GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                   \
         std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                   \
         if (int32_t st = attach_split_workspace(a)) return st;                                                        \
-        HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);                                                    \
+        HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);                                                    \
         return PRAD_OK;                                                                                               \
     }
 RAW_GEMM(f64, double)
@@ -519,7 +611,7 @@ RAW_GEMM(f32, float)
         GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                    \
         a.batch = batch; a.strideA = strideA; a.strideB = strideB; a.strideC = strideC;                                \
         std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                    \
-        HIP_TRY(launch_gemm<T>(a, g_ctx.stream), PRAD_ERR_LAUNCH);                                                     \
+        HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);                                                     \
         return PRAD_OK;                                                                                                \
     }
 RAW_BATCHED_GEMM(f64, double)
@@ -577,14 +669,14 @@ int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out) {
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     const size_t ws = (size_t)P * gemm_tiles_per_product(A->rows, B->cols) * sizeof(double);
     if (int32_t st = ensure_workspace(ws)) return st;
-    double* w = static_cast<double*>(g_ctx.workspace);
+    double* w = static_cast<double*>(CUR_WORKSPACE);
     if (A->dtype == PRAD_F64)
         HIP_TRY(launch_matmul_sum_fwd<double>(static_cast<const double*>(A->ptr), static_cast<const double*>(B->ptr),
-                                              static_cast<double*>(out->ptr), w, A->rows, A->cols, B->cols, P, g_ctx.stream),
+                                              static_cast<double*>(out->ptr), w, A->rows, A->cols, B->cols, P, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     else
         HIP_TRY(launch_matmul_sum_fwd<float>(static_cast<const float*>(A->ptr), static_cast<const float*>(B->ptr),
-                                             static_cast<float*>(out->ptr), w, A->rows, A->cols, B->cols, P, g_ctx.stream),
+                                             static_cast<float*>(out->ptr), w, A->rows, A->cols, B->cols, P, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -608,12 +700,12 @@ int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_bu
     if (A->dtype == PRAD_F64)
         HIP_TRY(launch_matmul_sum_bwd<double>(static_cast<const double*>(A->ptr), static_cast<const double*>(B->ptr),
                                               static_cast<const double*>(dOut->ptr), dA ? static_cast<double*>(dA->ptr) : nullptr,
-                                              dB ? static_cast<double*>(dB->ptr) : nullptr, M, K, N, P, g_ctx.stream),
+                                              dB ? static_cast<double*>(dB->ptr) : nullptr, M, K, N, P, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     else
         HIP_TRY(launch_matmul_sum_bwd<float>(static_cast<const float*>(A->ptr), static_cast<const float*>(B->ptr),
                                              static_cast<const float*>(dOut->ptr), dA ? static_cast<float*>(dA->ptr) : nullptr,
-                                             dB ? static_cast<float*>(dB->ptr) : nullptr, M, K, N, P, g_ctx.stream),
+                                             dB ? static_cast<float*>(dB->ptr) : nullptr, M, K, N, P, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -634,8 +726,8 @@ int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha) {
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "activation")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(x, launch_act_fwd<double>(act, D(x), D(y), count(x), alpha, g_ctx.stream),
-             launch_act_fwd<float>(act, F(x), F(y), count(x), (float)alpha, g_ctx.stream));
+    DISPATCH(x, launch_act_fwd<double>(act, D(x), D(y), count(x), alpha, CUR_STREAM),
+             launch_act_fwd<float>(act, F(x), F(y), count(x), (float)alpha, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -647,8 +739,8 @@ int32_t prad_act_bwd(int32_t act, prad_buf_t src, prad_buf_t dy, prad_buf_t dx, 
     if (int32_t st = same_shape(src, dy, "activation backward")) return st;
     if (int32_t st = same_shape(src, dx, "activation backward")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(src, launch_act_bwd<double>(act, D(src), D(dy), D(dx), count(src), alpha, g_ctx.stream),
-             launch_act_bwd<float>(act, F(src), F(dy), F(dx), count(src), (float)alpha, g_ctx.stream));
+    DISPATCH(src, launch_act_bwd<double>(act, D(src), D(dy), D(dx), count(src), alpha, CUR_STREAM),
+             launch_act_bwd<float>(act, F(src), F(dy), F(dx), count(src), (float)alpha, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -659,8 +751,8 @@ int32_t prad_hadamard_fwd(prad_buf_t a, prad_buf_t b, prad_buf_t y) {
     if (int32_t st = same_shape(a, b, "Hadamard product")) return st;
     if (int32_t st = same_shape(a, y, "Hadamard product")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(a, launch_hadamard_fwd<double>(D(a), D(b), D(y), count(a), g_ctx.stream),
-             launch_hadamard_fwd<float>(F(a), F(b), F(y), count(a), g_ctx.stream));
+    DISPATCH(a, launch_hadamard_fwd<double>(D(a), D(b), D(y), count(a), CUR_STREAM),
+             launch_hadamard_fwd<float>(F(a), F(b), F(y), count(a), CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -671,8 +763,8 @@ int32_t prad_hadamard_bwd(prad_buf_t a, prad_buf_t b, prad_buf_t dy, prad_buf_t 
     for (prad_buf_t o : {b, dy, da, db})
         if (int32_t st = same_shape(a, o, "Hadamard product")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(a, launch_hadamard_bwd<double>(D(a), D(b), D(dy), D(da), D(db), count(a), g_ctx.stream),
-             launch_hadamard_bwd<float>(F(a), F(b), F(dy), F(da), F(db), count(a), g_ctx.stream));
+    DISPATCH(a, launch_hadamard_bwd<double>(D(a), D(b), D(dy), D(da), D(db), count(a), CUR_STREAM),
+             launch_hadamard_bwd<float>(F(a), F(b), F(dy), F(da), F(db), count(a), CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -682,8 +774,8 @@ int32_t prad_scale(prad_buf_t x, prad_buf_t y, double scalar) {
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "multiply by scalar")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(x, launch_scale<double>(D(y), D(x), count(x), scalar, g_ctx.stream),
-             launch_scale<float>(F(y), F(x), count(x), (float)scalar, g_ctx.stream));
+    DISPATCH(x, launch_scale<double>(D(y), D(x), count(x), scalar, CUR_STREAM),
+             launch_scale<float>(F(y), F(x), count(x), (float)scalar, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -693,8 +785,8 @@ int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad) {
     if (int32_t st = same_dtype({dest, grad})) return st;
     if (int32_t st = same_shape(dest, grad, "accumulate")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(dest, launch_accumulate<double>(D(dest), D(grad), count(dest), g_ctx.stream),
-             launch_accumulate<float>(F(dest), F(grad), count(dest), g_ctx.stream));
+    DISPATCH(dest, launch_accumulate<double>(D(dest), D(grad), count(dest), CUR_STREAM),
+             launch_accumulate<float>(F(dest), F(grad), count(dest), CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -706,8 +798,8 @@ int32_t prad_add_broadcast_fwd(prad_buf_t x, prad_buf_t bias, prad_buf_t y) {
         return fail(PRAD_ERR_ARG, "The length of the bias vector must be the same as the number of columns in the input matrix.");
     if (int32_t st = same_shape(x, y, "add broadcasting")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(x, launch_add_broadcast_fwd<double>(D(x), D(bias), D(y), x->depth * x->rows, x->cols, g_ctx.stream),
-             launch_add_broadcast_fwd<float>(F(x), F(bias), F(y), x->depth * x->rows, x->cols, g_ctx.stream));
+    DISPATCH(x, launch_add_broadcast_fwd<double>(D(x), D(bias), D(y), x->depth * x->rows, x->cols, CUR_STREAM),
+             launch_add_broadcast_fwd<float>(F(x), F(bias), F(y), x->depth * x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -721,10 +813,10 @@ int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias) {
     double* ws = nullptr;
     if (colsum_chunks(dy->rows) > 1) {
         if (int32_t st = ensure_workspace((size_t)colsum_chunks(dy->rows) * dy->cols * sizeof(double))) return st;
-        ws = static_cast<double*>(g_ctx.workspace);
+        ws = static_cast<double*>(CUR_WORKSPACE);
     }
-    DISPATCH(dy, launch_colsum<double>(D(dy), D(dbias), dy->rows, dy->cols, ws, g_ctx.stream),
-             launch_colsum<float>(F(dy), F(dbias), dy->rows, dy->cols, ws, g_ctx.stream));
+    DISPATCH(dy, launch_colsum<double>(D(dy), D(dbias), dy->rows, dy->cols, ws, CUR_STREAM),
+             launch_colsum<float>(F(dy), F(dbias), dy->rows, dy->cols, ws, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -735,8 +827,8 @@ int32_t prad_softmax_fwd(prad_buf_t x, prad_buf_t y) {
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "softmax")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(x, launch_softmax_fwd<double>(D(x), D(y), x->depth * x->rows, x->cols, g_ctx.stream),
-             launch_softmax_fwd<float>(F(x), F(y), x->depth * x->rows, x->cols, g_ctx.stream));
+    DISPATCH(x, launch_softmax_fwd<double>(D(x), D(y), x->depth * x->rows, x->cols, CUR_STREAM),
+             launch_softmax_fwd<float>(F(x), F(y), x->depth * x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -747,8 +839,8 @@ int32_t prad_softmax_bwd(prad_buf_t y, prad_buf_t dy, prad_buf_t dx) {
     if (int32_t st = same_shape(y, dy, "softmax backward")) return st;
     if (int32_t st = same_shape(y, dx, "softmax backward")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(y, launch_softmax_bwd<double>(D(y), D(dy), D(dx), y->depth * y->rows, y->cols, g_ctx.stream),
-             launch_softmax_bwd<float>(F(y), F(dy), F(dx), y->depth * y->rows, y->cols, g_ctx.stream));
+    DISPATCH(y, launch_softmax_bwd<double>(D(y), D(dy), D(dx), y->depth * y->rows, y->cols, CUR_STREAM),
+             launch_softmax_bwd<float>(F(y), F(dy), F(dx), y->depth * y->rows, y->cols, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -760,8 +852,8 @@ int32_t prad_cce_fwd(prad_buf_t p, prad_buf_t target, prad_buf_t loss) {
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(p, launch_cce_fwd<double>(D(p), D(target), D(loss), p->rows, p->cols, g_ctx.stream),
-             launch_cce_fwd<float>(F(p), F(target), F(loss), p->rows, p->cols, g_ctx.stream));
+    DISPATCH(p, launch_cce_fwd<double>(D(p), D(target), D(loss), p->rows, p->cols, CUR_STREAM),
+             launch_cce_fwd<float>(F(p), F(target), F(loss), p->rows, p->cols, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -773,8 +865,8 @@ int32_t prad_cce_bwd(prad_buf_t p, prad_buf_t target, prad_buf_t dp) {
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (int32_t st = same_shape(p, dp, "cross-entropy backward")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(p, launch_cce_bwd<double>(D(p), D(target), D(dp), p->rows, p->cols, g_ctx.stream),
-             launch_cce_bwd<float>(F(p), F(target), F(dp), p->rows, p->cols, g_ctx.stream));
+    DISPATCH(p, launch_cce_bwd<double>(D(p), D(target), D(dp), p->rows, p->cols, CUR_STREAM),
+             launch_cce_bwd<float>(F(p), F(target), F(dp), p->rows, p->cols, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -787,9 +879,9 @@ int32_t prad_mse_fwd(prad_buf_t y, prad_buf_t target, prad_buf_t loss) {
     if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     if (int32_t st = ensure_workspace(mse_workspace_bytes())) return st;
-    double* w = static_cast<double*>(g_ctx.workspace);
-    DISPATCH(y, launch_mse_fwd<double>(D(y), D(target), D(loss), w, count(y), g_ctx.stream),
-             launch_mse_fwd<float>(F(y), F(target), F(loss), w, count(y), g_ctx.stream));
+    double* w = static_cast<double*>(CUR_WORKSPACE);
+    DISPATCH(y, launch_mse_fwd<double>(D(y), D(target), D(loss), w, count(y), CUR_STREAM),
+             launch_mse_fwd<float>(F(y), F(target), F(loss), w, count(y), CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -801,8 +893,8 @@ int32_t prad_mse_bwd(prad_buf_t y, prad_buf_t target, prad_buf_t dy) {
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (int32_t st = same_shape(y, dy, "mean squared error backward")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(y, launch_mse_bwd<double>(D(y), D(target), D(dy), count(y), g_ctx.stream),
-             launch_mse_bwd<float>(F(y), F(target), F(dy), count(y), g_ctx.stream));
+    DISPATCH(y, launch_mse_bwd<double>(D(y), D(target), D(dy), count(y), CUR_STREAM),
+             launch_mse_bwd<float>(F(y), F(target), F(dy), count(y), CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -816,8 +908,8 @@ int32_t prad_lstm_cell_fwd(prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_b
     for (prad_buf_t o : {c_prev, tanh_c, h})
         if (int32_t st = same_shape(c, o, "LSTM cell")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(c, launch_lstm_cell_fwd<double>(D(G), D(c_prev), D(c), D(tanh_c), D(h), rows, hidden, g_ctx.stream),
-             launch_lstm_cell_fwd<float>(F(G), F(c_prev), F(c), F(tanh_c), F(h), rows, hidden, g_ctx.stream));
+    DISPATCH(c, launch_lstm_cell_fwd<double>(D(G), D(c_prev), D(c), D(tanh_c), D(h), rows, hidden, CUR_STREAM),
+             launch_lstm_cell_fwd<float>(F(G), F(c_prev), F(c), F(tanh_c), F(h), rows, hidden, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -838,9 +930,9 @@ int32_t prad_lstm_cell_bwd(prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     DISPATCH(c_prev,
              launch_lstm_cell_bwd<double>(D(gates), D(c_prev), D(tanh_c), D(dh_a), dh_b ? D(dh_b) : nullptr, dc_in ? D(dc_in) : nullptr,
-                                          D(dG), D(dc_prev), rows, hidden, g_ctx.stream),
+                                          D(dG), D(dc_prev), rows, hidden, CUR_STREAM),
              launch_lstm_cell_bwd<float>(F(gates), F(c_prev), F(tanh_c), F(dh_a), dh_b ? F(dh_b) : nullptr, dc_in ? F(dc_in) : nullptr,
-                                         F(dG), F(dc_prev), rows, hidden, g_ctx.stream));
+                                         F(dG), F(dc_prev), rows, hidden, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -868,6 +960,8 @@ int32_t prad_graph_end(void** graph) {
     REQUIRE_INIT();
     if (graph == nullptr) return fail(PRAD_ERR_ARG, "graph is NULL");
     std::lock_guard<std::mutex> lock(g_ctx.mu);
+    for (int i = 1; i < MAX_BRANCHES; ++i)
+        if (g_ctx.branch[i].open) return fail(PRAD_ERR_ARG, "prad_join must close the open branches before prad_graph_end");
     hipGraph_t g = nullptr;
     HIP_TRY(hipStreamEndCapture(g_ctx.stream, &g), PRAD_ERR_LAUNCH);
     hipGraphExec_t exec = nullptr;
@@ -890,8 +984,64 @@ int32_t prad_graph_destroy(void* graph) {
     REQUIRE_INIT();
     if (graph == nullptr) return PRAD_OK;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    if (int32_t st = sync_all()) return st;
     HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)), PRAD_ERR_ARG);
+    return PRAD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Branches: operations that do not depend on each other (the reference's visitor runs their
+// Backward on pool threads, src/RMAD/OperationNeuralNetworkVisitor.cs:303-306) are enqueued on
+// different branches and may run side by side; recorded, they become parallel paths of the graph.
+int32_t prad_fork(int32_t branches) {
+    REQUIRE_INIT();
+    if (branches < 2 || branches > MAX_BRANCHES) return fail(PRAD_ERR_ARG, "branches must be 2..%d", MAX_BRANCHES);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    HIP_TRY(hipEventRecord(g_ctx.fork_event, g_ctx.stream), PRAD_ERR_LAUNCH);
+    for (int i = 1; i < branches; ++i) {
+        HIP_TRY(hipStreamWaitEvent(g_ctx.branch[i].stream, g_ctx.fork_event, 0), PRAD_ERR_LAUNCH);
+        g_ctx.branch[i].open = true;
+    }
+    return PRAD_OK;
+}
+
+int32_t prad_branch(int32_t index) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (index < 0 || index >= MAX_BRANCHES) return fail(PRAD_ERR_ARG, "branch %d out of range", index);
+    if (index > 0 && !g_ctx.branch[index].open) return fail(PRAD_ERR_ARG, "branch %d was not opened by prad_fork", index);
+    g_ctx.cur = index;
+    return PRAD_OK;
+}
+
+int32_t prad_join(void) {
+    REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    g_ctx.cur = 0;
+    for (int i = 1; i < MAX_BRANCHES; ++i) {
+        Branch& b = g_ctx.branch[i];
+        if (!b.open) continue;
+        b.open = false;
+        HIP_TRY(hipEventRecord(b.done, b.stream), PRAD_ERR_LAUNCH);
+        HIP_TRY(hipStreamWaitEvent(g_ctx.stream, b.done, 0), PRAD_ERR_LAUNCH);
+    }
+    return PRAD_OK;
+}
+
+int32_t prad_softmax_cce(prad_buf_t x, prad_buf_t target, prad_buf_t p, prad_buf_t loss, prad_buf_t dp, prad_buf_t dx) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(target); REQUIRE_BUF(p); REQUIRE_BUF(dp); REQUIRE_BUF(dx);
+    if (loss != nullptr) REQUIRE_BUF(loss);
+    if (int32_t st = same_dtype({x, target, p, loss, dp, dx})) return st;
+    if (x->depth != 1) return fail(PRAD_ERR_SHAPE, "deep buffer passed to softmax + cross-entropy");
+    if (x->rows != target->rows || x->cols != target->cols || target->depth != 1)
+        return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
+    if (loss != nullptr && (loss->depth != 1 || loss->rows != 1 || loss->cols != 1)) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
+    for (prad_buf_t o : {p, dp, dx})
+        if (int32_t st = same_shape(x, o, "softmax + cross-entropy")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_softmax_cce<double>(D(x), D(target), D(p), D(dp), D(dx), loss ? D(loss) : nullptr, cur_branch().counter, x->rows, x->cols, CUR_STREAM),
+             launch_softmax_cce<float>(F(x), F(target), F(p), F(dp), F(dx), loss ? F(loss) : nullptr, cur_branch().counter, x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -911,19 +1061,20 @@ int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, doubl
     if (g[0]->dtype == PRAD_F64) {
         std::vector<TensorDesc<double>> d((size_t)n);
         for (int i = 0; i < n; ++i) d[i] = TensorDesc<double>{D(g[i]), nullptr, nullptr, nullptr, sizes[i]};
-        HIP_TRY(launch_clip<double>(d.data(), n, g_ctx.workspace, clip_value, min_value, g_ctx.stream), PRAD_ERR_LAUNCH);
+        HIP_TRY(launch_clip<double>(d.data(), n, CUR_WORKSPACE, clip_value, min_value, CUR_STREAM), PRAD_ERR_LAUNCH);
     } else {
         std::vector<TensorDesc<float>> d((size_t)n);
         for (int i = 0; i < n; ++i) d[i] = TensorDesc<float>{F(g[i]), nullptr, nullptr, nullptr, sizes[i]};
-        HIP_TRY(launch_clip<float>(d.data(), n, g_ctx.workspace, (float)clip_value, (float)min_value, g_ctx.stream), PRAD_ERR_LAUNCH);
+        HIP_TRY(launch_clip<float>(d.data(), n, CUR_WORKSPACE, (float)clip_value, (float)min_value, CUR_STREAM), PRAD_ERR_LAUNCH);
     }
     return PRAD_OK;
 }
 
 int32_t prad_clip(prad_buf_t g, double clip_value, double min_value) { return prad_clip_multi(&g, 1, clip_value, min_value); }
 
-int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n, double lr,
-                        double beta1, double beta2, double eps, double t) {
+// Shared by prad_adam_multi (clip == false) and prad_clip_adam_multi.
+static int32_t adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n, bool clip,
+                          double clip_value, double min_value, double lr, double beta1, double beta2, double eps, double t) {
     REQUIRE_INIT();
     if (n < 0 || (n > 0 && (w == nullptr || m == nullptr || v == nullptr || g == nullptr))) return fail(PRAD_ERR_ARG, "bad tensor list");
     if (n == 0) return PRAD_OK;
@@ -934,23 +1085,46 @@ int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf
         for (prad_buf_t o : {m[i], v[i], g[i]})
             if (int32_t st = same_shape(w[i], o, "Adam")) return st;
     }
+    std::vector<int64_t> sizes((size_t)n);
+    for (int i = 0; i < n; ++i) sizes[i] = count(w[i]);
     std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (clip)
+        if (int32_t st = ensure_workspace(clip_workspace_bytes(sizes.data(), n))) return st;
     if (w[0]->dtype == PRAD_F64) {
         // 1 / (1 - Math.Pow(beta, AdamIteration)), src/RMAD/AdamOptimizer.cs:204-207
         const double c1 = 1 / (1 - std::pow(beta1, t)), c2 = 1 / (1 - std::pow(beta2, t));
         std::vector<TensorDesc<double>> d((size_t)n);
-        for (int i = 0; i < n; ++i) d[i] = TensorDesc<double>{D(g[i]), D(w[i]), D(m[i]), D(v[i]), count(w[i])};
-        HIP_TRY(launch_adam<double>(d.data(), n, lr, beta1, beta2, eps, c1, c2, g_ctx.stream), PRAD_ERR_LAUNCH);
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<double>{D(g[i]), D(w[i]), D(m[i]), D(v[i]), sizes[i]};
+        if (clip)
+            HIP_TRY(launch_clip_adam<double>(d.data(), n, CUR_WORKSPACE, clip_value, min_value, lr, beta1, beta2, eps, c1, c2, CUR_STREAM),
+                    PRAD_ERR_LAUNCH);
+        else
+            HIP_TRY(launch_adam<double>(d.data(), n, lr, beta1, beta2, eps, c1, c2, CUR_STREAM), PRAD_ERR_LAUNCH);
     } else {
         // PRADLite: every parameter is a float and PradMath.Pow(float, float) is (float)Math.Pow.
         const float b1 = (float)beta1, b2 = (float)beta2, tf = (float)t;
         const float c1 = 1 / (1 - (float)std::pow((double)b1, (double)tf));
         const float c2 = 1 / (1 - (float)std::pow((double)b2, (double)tf));
         std::vector<TensorDesc<float>> d((size_t)n);
-        for (int i = 0; i < n; ++i) d[i] = TensorDesc<float>{F(g[i]), F(w[i]), F(m[i]), F(v[i]), count(w[i])};
-        HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, g_ctx.stream), PRAD_ERR_LAUNCH);
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<float>{F(g[i]), F(w[i]), F(m[i]), F(v[i]), sizes[i]};
+        if (clip)
+            HIP_TRY(launch_clip_adam<float>(d.data(), n, CUR_WORKSPACE, (float)clip_value, (float)min_value, (float)lr, b1, b2,
+                                            (float)eps, c1, c2, CUR_STREAM),
+                    PRAD_ERR_LAUNCH);
+        else
+            HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, CUR_STREAM), PRAD_ERR_LAUNCH);
     }
     return PRAD_OK;
+}
+
+int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n, double lr,
+                        double beta1, double beta2, double eps, double t) {
+    return adam_multi(w, m, v, g, n, false, 0.0, 0.0, lr, beta1, beta2, eps, t);
+}
+
+int32_t prad_clip_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
+                             double clip_value, double min_value, double lr, double beta1, double beta2, double eps, double t) {
+    return adam_multi(w, m, v, g, n, true, clip_value, min_value, lr, beta1, beta2, eps, t);
 }
 
 int32_t prad_adam(prad_buf_t w, prad_buf_t m, prad_buf_t v, prad_buf_t g, double lr, double beta1, double beta2, double eps,

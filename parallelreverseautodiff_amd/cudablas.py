@@ -2,7 +2,7 @@
 
 Every example and test of the reference brackets GPU work with
 ``CudaBlas.Instance.DeviceId = 0; CudaBlas.Instance.Initialize(); ...; CudaBlas.Instance.Dispose()``
-(examples/feedforward/FeedForwardNeuralNetworkExample/Program.cs:17-25).  The name is kept so that
+(examples/feedforward/ParallelReverseAutoDiff.FeedForwardExample/Program.cs:17-25).  The name is kept so that
 code reads the same; what it starts is the HIP library, not cuBLAS.
 """
 from . import _lib

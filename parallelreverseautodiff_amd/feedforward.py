@@ -1,12 +1,18 @@
 """Device-resident training step of the feed-forward configuration: the call sequence the reference's
 training loop makes (forward walk over the operation list, loss, backward visitor with gradient
-accumulation, clip, Adam: examples/feedforward/FeedForwardNeuralNetworkExample/FeedForwardNeuralNetwork.cs:212-358)
+accumulation, clip, Adam: examples/feedforward/ParallelReverseAutoDiff.FeedForwardExample/FeedForwardNeuralNetwork.cs:212-358)
 replayed on pre-allocated device buffers, either launch by launch or as one recorded submission.
 
 Network: X (batch x n0) -> [MatrixMultiply(W_l) -> MatrixAddBroadcasting(b_l) -> LeakyReLU] x (L-1)
          -> MatrixMultiply(W_L) -> MatrixAddBroadcasting(b_L) -> Softmax -> CategoricalCrossEntropy.
 Per layer the product, the bias add and the activation are one launch (fused epilogue), and the
-activation's Backward is the epilogue of the next layer's dA product.
+activation's Backward is the epilogue of the next layer's dA product.  A step of this size costs what
+its chain of dependent launches costs, so fused=True (the default) uses the entry points that cover
+several reference operations per launch (softmax + cross-entropy forward and backward; the bias gradient
+next to the weight gradient; clip + Adam);
+overlap=True puts gradients that do not depend on each other on separate branches, as the reference's
+visitor hands independent Backward calls to pool threads.  The arithmetic of every operation is the
+same in all variants and the results are bit for bit equal.
 """
 import ctypes
 
@@ -20,7 +26,7 @@ from .optim import NeuralNetworkParameters
 
 
 class FeedForwardNetwork:
-    def __init__(self, sizes=(784, 256, 128, 10), batch=64, dtype=np.float64, seed=seeded.DEFAULT_SEED, parameters=None):
+    def __init__(self, sizes=(784, 256, 128, 10), batch=64, dtype=np.float64, seed=seeded.DEFAULT_SEED, parameters=None, fused=True, overlap=False):
         _ensure_initialized()
         self.lib = _lib.load()
         self.dtype = np.dtype(dtype)
@@ -50,6 +56,8 @@ class FeedForwardNetwork:
         self.dZ = [alloc(batch, sizes[l + 1]) for l in range(L)]
         self.dX = alloc(batch, sizes[0])
         self.iteration = 0
+        self.overlap = overlap
+        self.fused = fused
         self._graph = None
         self._weights = self.W + self.b
         self._grads = self.dW + self.db
@@ -61,7 +69,7 @@ class FeedForwardNetwork:
         self.T.upload(T)
 
     # ---- one step, launch by launch ------------------------------------------------------------
-    def _enqueue_forward_backward(self):
+    def _enqueue_forward(self):
         lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
         a = self.X
         for l in range(L):
@@ -71,23 +79,72 @@ class FeedForwardNetwork:
             check(lib.prad_matmul_fwd_fused(a.handle, self.W[l].handle, self.b[l].handle, z, out.handle,
                                             _lib.ACT_NONE if last else _lib.ACT_LEAKYRELU, alpha))
             a = out
-        check(lib.prad_softmax_fwd(self.Z[-1].handle, self.P.handle))
-        check(lib.prad_cce_fwd(self.P.handle, self.T.handle, self.loss.handle))
-        check(lib.prad_cce_bwd(self.P.handle, self.T.handle, self.dP.handle))
-        check(lib.prad_softmax_bwd(self.P.handle, self.dP.handle, self.dZ[-1].handle))
+
+    def _enqueue_forward_backward(self):
+        if self.overlap:
+            return self._enqueue_forward_backward_overlapped()
+        lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
+        self._enqueue_forward()
+        if self.fused:
+            check(lib.prad_softmax_cce(self.Z[-1].handle, self.T.handle, self.P.handle, self.loss.handle, self.dP.handle,
+                                       self.dZ[-1].handle))
+        else:
+            check(lib.prad_softmax_fwd(self.Z[-1].handle, self.P.handle))
+            check(lib.prad_cce_fwd(self.P.handle, self.T.handle, self.loss.handle))
+            check(lib.prad_cce_bwd(self.P.handle, self.T.handle, self.dP.handle))
+            check(lib.prad_softmax_bwd(self.P.handle, self.dP.handle, self.dZ[-1].handle))
         for l in range(L - 1, -1, -1):
             inp = self.X if l == 0 else self.H[l - 1]
+            # MatrixMultiplyOperation.Backward always forms both gradients, also for the network input (l == 0)
+            dA = self.dX if l == 0 else self.dZ[l - 1]
+            act, src = (_lib.ACT_NONE, None) if l == 0 else (_lib.ACT_LEAKYRELU, self.Z[l - 1].handle)
+            if self.fused:
+                check(lib.prad_matmul_bias_bwd(self.dZ[l].handle, inp.handle, self.W[l].handle, dA.handle, self.dW[l].handle,
+                                               self.db[l].handle, 0, act, src, alpha))
+                continue
             check(lib.prad_add_broadcast_bwd_bias(self.dZ[l].handle, self.db[l].handle))
             if l == 0:
-                # MatrixMultiplyOperation.Backward always forms both gradients, also for the input
                 check(lib.prad_matmul_bwd(self.dZ[0].handle, inp.handle, self.W[0].handle, self.dX.handle, self.dW[0].handle, 0, 0))
             else:
-                check(lib.prad_matmul_bwd_fused(self.dZ[l].handle, inp.handle, self.W[l].handle, self.dZ[l - 1].handle,
-                                                self.dW[l].handle, 0, _lib.ACT_LEAKYRELU, self.Z[l - 1].handle, alpha))
+                check(lib.prad_matmul_bwd_fused(self.dZ[l].handle, inp.handle, self.W[l].handle, dA.handle,
+                                                self.dW[l].handle, 0, act, src, alpha))
+
+    def _enqueue_forward_backward_overlapped(self):
+        """Branch 0 carries the chain forward -> loss gradient -> dA of every layer; branch 1 the weight
+        gradients, branch 2 the bias gradients and the loss value, branch 3 the input gradient."""
+        lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
+        self._enqueue_forward()
+        check(lib.prad_softmax_cce(self.Z[-1].handle, self.T.handle, self.P.handle, None, self.dP.handle, self.dZ[-1].handle))
+        try:
+            for l in range(L - 1, -1, -1):
+                inp = self.X if l == 0 else self.H[l - 1]
+                check(lib.prad_fork(4))                      # dZ[l] (and P) are ready for the side branches
+                check(lib.prad_branch(2))
+                if l == L - 1:
+                    check(lib.prad_cce_fwd(self.P.handle, self.T.handle, self.loss.handle))
+                check(lib.prad_add_broadcast_bwd_bias(self.dZ[l].handle, self.db[l].handle))
+                check(lib.prad_branch(1))
+                check(lib.prad_matmul_bwd(self.dZ[l].handle, inp.handle, self.W[l].handle, None, self.dW[l].handle, 0, 0))
+                if l == 0:
+                    check(lib.prad_branch(3))
+                    check(lib.prad_matmul_bwd(self.dZ[0].handle, inp.handle, self.W[0].handle, self.dX.handle, None, 0, 0))
+                    check(lib.prad_branch(0))
+                else:
+                    check(lib.prad_branch(0))
+                    check(lib.prad_matmul_bwd_fused(self.dZ[l].handle, inp.handle, self.W[l].handle, self.dZ[l - 1].handle,
+                                                    None, 0, _lib.ACT_LEAKYRELU, self.Z[l - 1].handle, alpha))
+        finally:
+            check(lib.prad_join())
 
     def _enqueue_update(self, t):
         p = self.params
         n = len(self._grads)
+        if self.fused:
+            check(self.lib.prad_clip_adam_multi(handle_array(self._weights), handle_array(self._m), handle_array(self._v),
+                                                handle_array(self._grads), n, float(p.ClipValue), float(p.MinimumClipValue),
+                                                float(p.LearningRate), float(p.AdamBeta1), float(p.AdamBeta2),
+                                                float(p.AdamEpsilon), float(t)))
+            return
         check(self.lib.prad_clip_multi(handle_array(self._grads), n, float(p.ClipValue), float(p.MinimumClipValue)))
         check(self.lib.prad_adam_multi(handle_array(self._weights), handle_array(self._m), handle_array(self._v),
                                        handle_array(self._grads), n, float(p.LearningRate), float(p.AdamBeta1),

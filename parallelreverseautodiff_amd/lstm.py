@@ -92,10 +92,10 @@ class LSTMLayer:
 
     def _enqueue_update(self, t):
         p = self.params
-        check(self.lib.prad_clip_multi(handle_array([self.dW, self.db]), 2, float(p.ClipValue), float(p.MinimumClipValue)))
-        check(self.lib.prad_adam_multi(handle_array([self.W, self.b]), handle_array([self.mW, self.mb]),
-                                       handle_array([self.vW, self.vb]), handle_array([self.dW, self.db]), 2,
-                                       float(p.LearningRate), float(p.AdamBeta1), float(p.AdamBeta2), float(p.AdamEpsilon), float(t)))
+        check(self.lib.prad_clip_adam_multi(handle_array([self.W, self.b]), handle_array([self.mW, self.mb]),
+                                            handle_array([self.vW, self.vb]), handle_array([self.dW, self.db]), 2,
+                                            float(p.ClipValue), float(p.MinimumClipValue), float(p.LearningRate),
+                                            float(p.AdamBeta1), float(p.AdamBeta2), float(p.AdamEpsilon), float(t)))
 
     def step(self, update=True):
         self.iteration += 1

@@ -120,9 +120,9 @@ class SwinBlock:
     def _enqueue_update(self, t):
         p, n = self.params, len(self.names)
         arr = lambda d: handle_array([d[k] for k in self.names])
-        check(self.lib.prad_clip_multi(arr(self.g), n, float(p.ClipValue), float(p.MinimumClipValue)))
-        check(self.lib.prad_adam_multi(arr(self.w), arr(self.m), arr(self.v), arr(self.g), n, float(p.LearningRate),
-                                       float(p.AdamBeta1), float(p.AdamBeta2), float(p.AdamEpsilon), float(t)))
+        check(self.lib.prad_clip_adam_multi(arr(self.w), arr(self.m), arr(self.v), arr(self.g), n, float(p.ClipValue),
+                                            float(p.MinimumClipValue), float(p.LearningRate), float(p.AdamBeta1),
+                                            float(p.AdamBeta2), float(p.AdamEpsilon), float(t)))
 
     def step(self, update=True):
         self.iteration += 1

@@ -111,3 +111,79 @@ def test_softmax_and_cross_entropy_operations(gpu, oracle, dtype):
     assert_parity(dx, oracle.softmax_bwd(rp, oracle.cce_bwd(rp, t)), dtype, "softmax backward")
     wide = seeded.normal(5, 3, (3, 1000), 3.0, dtype)  # more columns than a wavefront
     assert_parity(SoftmaxOperation().Forward(Matrix.from_numpy(wide)).to_numpy(), oracle.softmax_fwd(wide), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_overlapped_step_equals_sequential_step(gpu, dtype):
+    """Independent gradients on separate branches (and the fused softmax + cross-entropy launch) must give
+    bit for bit what the one-branch, operation-by-operation step gives; also when recorded and replayed."""
+    X = seeded.uniform(7, 1, (64, 784), 0.0, 1.0, dtype)
+    T = seeded.one_hot_labels(7, 2, 64, 10, dtype)
+    seq = FeedForwardNetwork(dtype=dtype, fused=False, overlap=False)   # one reference operation per launch
+    fus = FeedForwardNetwork(dtype=dtype, fused=True, overlap=False)
+    par, rec = (FeedForwardNetwork(dtype=dtype, overlap=True) for _ in range(2))
+    for net in (seq, fus, par, rec):
+        net.set_batch(X, T)
+        net.step()
+    rec.record(adam_iteration=2.0)
+    for replay in range(3):
+        for net in (seq, fus, par):
+            net.iteration = 1
+            net.step()
+        rec.replay()
+        gpu.Synchronize()
+        for name in ("_weights", "_grads", "_m", "_v"):
+            for a, f, b2, c in zip(getattr(seq, name), getattr(fus, name), getattr(par, name), getattr(rec, name)):
+                ref = a.download()
+                assert np.array_equal(ref, f.download()), "%s differs (fused launches, pass %d)" % (name, replay)
+                assert np.array_equal(ref, b2.download()), "%s differs (eager branches, pass %d)" % (name, replay)
+                assert np.array_equal(ref, c.download()), "%s differs (recorded branches, pass %d)" % (name, replay)
+        for other in (fus, par, rec):
+            assert np.array_equal(seq.loss.download(), other.loss.download())
+        assert np.array_equal(seq.dX.download(), par.dX.download())
+    rec.release()
+
+
+def test_branch_protocol_errors(gpu):
+    from parallelreverseautodiff_amd import _lib
+    from parallelreverseautodiff_amd.exceptions import ArgumentException, check
+    lib = _lib.load()
+    with pytest.raises(ArgumentException):
+        check(lib.prad_fork(1))
+    with pytest.raises(ArgumentException):
+        check(lib.prad_fork(5))
+    with pytest.raises(ArgumentException):
+        check(lib.prad_branch(2))          # not opened
+    check(lib.prad_fork(2))
+    check(lib.prad_branch(1))
+    with pytest.raises(ArgumentException):
+        check(lib.prad_branch(2))          # only branch 1 is open
+    check(lib.prad_join())
+    with pytest.raises(ArgumentException):
+        check(lib.prad_branch(1))          # closed again
+    check(lib.prad_join())                 # joining with nothing open is a no-op
+    check(lib.prad_branch(0))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(64, 10), (5, 200), (1, 1), (700, 12)])
+def test_fused_softmax_cross_entropy_equals_separate_launches(gpu, dtype, shape):
+    from parallelreverseautodiff_amd import _lib
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    x = seeded.normal(9, 1, shape, 2.0, dtype)
+    t = seeded.one_hot_labels(9, 2, shape[0], shape[1], dtype)
+    bx, bt = DeviceBuffer.alloc(dtype, *shape), DeviceBuffer.alloc(dtype, *shape)
+    bx.upload(x); bt.upload(t)
+    p1, dp1, dx1, p2, dp2, dx2 = (DeviceBuffer.alloc(dtype, *shape) for _ in range(6))
+    l1, l2 = DeviceBuffer.alloc(dtype, 1, 1), DeviceBuffer.alloc(dtype, 1, 1)
+    check(lib.prad_softmax_fwd(bx.handle, p1.handle))
+    check(lib.prad_cce_fwd(p1.handle, bt.handle, l1.handle))
+    check(lib.prad_cce_bwd(p1.handle, bt.handle, dp1.handle))
+    check(lib.prad_softmax_bwd(p1.handle, dp1.handle, dx1.handle))
+    check(lib.prad_softmax_cce(bx.handle, bt.handle, p2.handle, l2.handle, dp2.handle, dx2.handle))
+    for a, b2 in ((p1, p2), (dp1, dp2), (dx1, dx2), (l1, l2)):
+        assert np.array_equal(a.download(), b2.download())
+    check(lib.prad_softmax_cce(bx.handle, bt.handle, p2.handle, None, dp2.handle, dx2.handle))   # loss is optional
+    assert np.array_equal(dx1.download(), dx2.download())

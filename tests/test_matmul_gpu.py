@@ -364,3 +364,31 @@ def test_raw_pointer_entry_point_with_leading_dimensions(gpu, oracle):
     assert_parity(got[:, :N], oracle.matmul_fwd(np.ascontiguousarray(A[:, :K]), np.ascontiguousarray(B[:, :N])), np.float64)
     assert not got[:, N:].any()  # padding columns untouched
     assert lib.prad_gemm_f64(0, 0, M, N, K, dA_.ptr, K - 1, dB_.ptr, ldb, dC_.ptr, ldc, 0) == _lib.PRAD_ERR_ARG
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("shape", [(64, 784, 256), (64, 128, 10), (1024, 64, 64), (2500, 40, 70), (33, 17, 129)])
+def test_bias_gradient_riding_with_the_weight_gradient(gpu, dtype, shape):
+    """prad_matmul_bias_bwd = prad_add_broadcast_bwd_bias + prad_matmul_bwd_fused, bit for bit: the column sum
+    shares the launch of the dB product (also when that product is split along K: 1024 x 64 x 64) or gets its
+    own launches (no dB requested; 2500 rows, which are summed in row chunks)."""
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    M, K, N = shape
+    A, B, dC, Z = (seeded.normal(71, i, s, 1.0, dtype) for i, s in enumerate([(M, K), (K, N), (M, N), (M, K)]))
+    up = lambda a: (lambda b: (b.upload(a), b)[1])(DeviceBuffer.alloc(dtype, *a.shape))
+    bA, bB, bdC, bZ = up(A), up(B), up(dC), up(Z)
+    dA1, dA2 = DeviceBuffer.alloc(dtype, M, K), DeviceBuffer.alloc(dtype, M, K)
+    dB1, dB2 = DeviceBuffer.alloc(dtype, K, N), DeviceBuffer.alloc(dtype, K, N)
+    db1, db2, db3 = (DeviceBuffer.alloc(dtype, 1, N) for _ in range(3))
+    check(lib.prad_add_broadcast_bwd_bias(bdC.handle, db1.handle))
+    check(lib.prad_matmul_bwd_fused(bdC.handle, bA.handle, bB.handle, dA1.handle, dB1.handle, 0, _lib.ACT_LEAKYRELU, bZ.handle, 0.01))
+    check(lib.prad_matmul_bias_bwd(bdC.handle, bA.handle, bB.handle, dA2.handle, dB2.handle, db2.handle, 0, _lib.ACT_LEAKYRELU,
+                                   bZ.handle, 0.01))
+    check(lib.prad_matmul_bias_bwd(bdC.handle, bA.handle, bB.handle, None, None, db3.handle, 0, _lib.ACT_NONE, None, 0.0))
+    assert np.array_equal(dA1.download(), dA2.download())
+    assert np.array_equal(dB1.download(), dB2.download())
+    assert np.array_equal(db1.download(), db2.download())
+    assert np.array_equal(db1.download(), db3.download())
+    assert_parity(db2.download(), dC.astype(np.float64).sum(axis=0, keepdims=True).astype(dtype), dtype, "bias gradient")

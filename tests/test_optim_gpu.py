@@ -123,3 +123,49 @@ def test_many_tensors_cross_the_table_limit(gpu, oracle):
         assert_parity(gm[i].to_numpy(), cg, np.float64)
         w, _, _ = oracle.adam(ws[i], np.zeros_like(ws[i]), np.zeros_like(ws[i]), gm[i].to_numpy(), 1e-3, 0.9, 0.999, 1e-8, 1.0)
         assert_parity(wm[i].to_numpy(), w, np.float64)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fused_clip_adam_equals_clip_then_adam(gpu, oracle, dtype):
+    """prad_clip_adam_multi must leave exactly what prad_clip_multi followed by prad_adam_multi leaves, for
+    tensors whose chunk statistics are merged inside the clamping pass (few chunks) and for a tensor large
+    enough to take the separate finalize launch; the small ones are also checked against the oracle."""
+    from parallelreverseautodiff_amd import _lib
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    from parallelreverseautodiff_amd.operations import handle_array
+    lib = _lib.load()
+    for shapes in ([(784, 256), (1, 256), (1, 1), (3, 5000), (128, 10)], [(1100, 1024), (7, 3)]):   # 1100*1024 -> 275 chunks
+        host = {k: [] for k in "wmvg"}
+        dev = {tag: {k: [] for k in "wmvg"} for tag in ("two", "one")}
+        for i, s in enumerate(shapes):
+            host["w"].append(seeded.normal(61, 4 * i, s, 1.0, dtype))
+            host["m"].append(seeded.normal(61, 4 * i + 1, s, 0.1, dtype))
+            host["v"].append(np.abs(seeded.normal(61, 4 * i + 2, s, 0.1, dtype)))
+            g = seeded.normal(61, 4 * i + 3, s, 0.5, dtype)
+            if g.size > 100:
+                g.reshape(-1)[5] = 90.0
+                g.reshape(-1)[9] = 1e-20
+            host["g"].append(g)
+            for tag in dev:
+                for k in "wmvg":
+                    b = DeviceBuffer.alloc(dtype, *s)
+                    b.upload(host[k][i])
+                    dev[tag][k].append(b)
+        n = len(shapes)
+        arr = lambda tag, k: handle_array(dev[tag][k])
+        args = (4.0, 1e-16 if dtype == np.float64 else 1e-8, 1e-3, 0.9, 0.999, 1e-8, 3.0)
+        check(lib.prad_clip_multi(arr("two", "g"), n, args[0], args[1]))
+        check(lib.prad_adam_multi(arr("two", "w"), arr("two", "m"), arr("two", "v"), arr("two", "g"), n, *args[2:]))
+        check(lib.prad_clip_adam_multi(arr("one", "w"), arr("one", "m"), arr("one", "v"), arr("one", "g"), n, *args))
+        for k in "wmvg":
+            for i in range(n):
+                assert np.array_equal(dev["two"][k][i].download(), dev["one"][k][i].download()), (k, shapes[i])
+        if shapes[0] == (784, 256):
+            for i in range(n):
+                g = oracle.clip(host["g"][i], args[0], args[1])
+                assert_parity(dev["one"]["g"][i].download(), g, dtype, "clamped gradient")
+                w, m, v = oracle.adam(host["w"][i], host["m"][i], host["v"][i], dev["one"]["g"][i].download(), *args[2:])
+                assert_parity(dev["one"]["w"][i].download(), w, dtype, "weight")
+                assert_parity(dev["one"]["m"][i].download(), m, dtype, "first moment")
+                assert_parity(dev["one"]["v"][i].download(), v, dtype, "second moment")
