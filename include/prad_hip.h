@@ -146,6 +146,14 @@ int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out);
 /* As written in the reference: dB[q] = A^T * dOut[0][q] (deep (P, K, M)); dA = sum_q B[q]^T * dOut[0][q]
  * (needs N == M). */
 int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_buf_t dA, prad_buf_t dB);
+/* Independent products summed into one output plus a broadcast bias: C = sum_q A[q].B[q] + bias, A deep
+ * (P, M, K), B deep (P, K, N), bias 1 x N or NULL, C M x N.  The reference has no single operation of this
+ * form (it composes MatrixMultiplyOperation.Forward, src/RMAD/MatrixMultiplyOperation.cs:50-80, a sum of
+ * matrices and MatrixAddBroadcastingOperation.cs:32-54); results are those of that composition with the
+ * products added in slice order.  Backward for the upstream gradient dC: dA[q] = dC . B[q]^T,
+ * dB[q] = A[q]^T . dC, dbias = column sums of dC; each may be NULL. */
+int32_t prad_matmul_batch_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_buf_t C);
+int32_t prad_matmul_batch_sum_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, prad_buf_t dbias);
 
 /* ---- elementwise forward / backward (bandwidth kernels) ------------------------------------- */
 int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha);

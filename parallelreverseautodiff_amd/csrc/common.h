@@ -131,8 +131,15 @@ struct GemmArgs {
     // Scratch for products that are split along K (see gemm_split_factor): split_ws holds
     // split_factor * batch * M * N elements.  Filled in by the caller; nullptr disables splitting.
     T* split_ws;
-    // Set by launch_gemm for the kernels: K range per split (0 = not split).
+    // Set by launch_gemm for the kernels: K range per split (0 = not split) and the element offsets
+    // of split z's operand blocks from those of split 0.
     int64_t ksplit;
+    int64_t zstrideA, zstrideB;
+    // A sum of products C = sum_q op(A_q).op(B_q): nseg > 1 operand pairs, segstrideA / segstrideB
+    // elements apart, M x K and K x N each.  Runs as a product split along the joint reduction
+    // (one pair per split), so split_ws must hold nseg * M * N elements.  batch must be 1.
+    int nseg;
+    int64_t segstrideA, segstrideB;
     // A column sum that rides along with the product's launch (the bias gradient of
     // MatrixAddBroadcasting next to the weight gradient, both functions of the same upstream
     // gradient): colsum_dst[j] = sum_i colsum_src[i][j] over colsum_rows x colsum_cols, taken by extra

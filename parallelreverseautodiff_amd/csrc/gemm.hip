@@ -207,8 +207,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     if (p.ksplit > 0) {
         const int64_t kb = (int64_t)blockIdx.z * p.ksplit;
         K = min(p.ksplit, p.K - kb);
-        A += A_KC ? kb : kb * p.lda;
-        B += B_KC ? kb : kb * p.ldb;
+        A += (int64_t)blockIdx.z * p.zstrideA;
+        B += (int64_t)blockIdx.z * p.zstrideB;
     }
 
     const int tid = threadIdx.x;
@@ -432,6 +432,7 @@ static hipError_t launch_tile(const GemmArgs<T>& a, int epi, hipStream_t stream)
     const bool aligned = (a.M % BM == 0) && (a.N % BM == 0) && a.K > 0 && (a.lda % VEC == 0) &&
                          (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
+                         (a.zstrideA % VEC == 0) && (a.zstrideB % VEC == 0) &&
                          // per-thread element offsets inside one tile's slab are kept in 32 bits
                          (a.lda < (1 << 23)) && (a.ldb < (1 << 23));
     // Grid y carries the batch; the tile count must fit the 1-D grid.
@@ -526,11 +527,36 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
     const int epi = a.tile_sums != nullptr ? EPI_TILE_SUM
                     : (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) ? EPI_ELEMENTWISE
                                                                                                              : EPI_PLAIN;
+    if (a.nseg > 1) {
+        // Sum of nseg products: one operand pair per split, partial results added in pair order.
+        if (a.split_ws == nullptr || a.batch != 1 || epi == EPI_TILE_SUM) return hipErrorInvalidValue;
+        GemmArgs<T> part = a;
+        part.K = a.K * a.nseg;
+        part.ksplit = a.K;
+        part.zstrideA = a.segstrideA; part.zstrideB = a.segstrideB;
+        part.C = a.split_ws; part.ldc = a.N; part.strideC = a.M * a.N;
+        part.accumulate = 0;
+        part.bias = nullptr; part.Z = nullptr; part.act_fwd = ACT_NONE; part.act_bwd = ACT_NONE; part.act_src = nullptr;
+        hipError_t e;
+        switch (choose_tile(a.M, a.N, a.nseg, false)) {
+            case TILE_128x128: e = launch_tile<T, 4>(part, EPI_PLAIN, stream); break;
+            case TILE_64x64: e = launch_tile<T, 2>(part, EPI_PLAIN, stream); break;
+            default: e = launch_tile<T, 1>(part, EPI_PLAIN, stream); break;
+        }
+        if (e != hipSuccess) return e;
+        const int64_t total = a.M * a.N;
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL((split_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, a, a.split_ws, a.nseg);
+        return hipGetLastError();
+    }
     const int splits = (a.split_ws != nullptr && epi != EPI_TILE_SUM) ? gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T)) : 1;
     if (splits > 1) {
         constexpr int64_t bk = Slab<T, 1>::BK;
         GemmArgs<T> part = a;
         part.ksplit = ((a.K + splits - 1) / splits + bk - 1) / bk * bk;
+        part.zstrideA = a.transA ? part.ksplit * a.lda : part.ksplit;  // A stored [k][m] when transposed, else [m][k]
+        part.zstrideB = a.transB ? part.ksplit : part.ksplit * a.ldb;  // B stored [n][k] when transposed, else [k][n]
         part.C = a.split_ws; part.ldc = a.N; part.strideC = a.M * a.N;  // split z, batch b at ((z * batch) + b) * M * N
         part.accumulate = 0;
         part.bias = nullptr; part.Z = nullptr; part.act_fwd = ACT_NONE; part.act_bwd = ACT_NONE; part.act_src = nullptr;

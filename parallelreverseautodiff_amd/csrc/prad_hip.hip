@@ -246,6 +246,24 @@ int32_t enqueue_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_bu
     return enqueue_gemm_t<float>(transA, transB, A, B, C, accumulate, ep, batched);
 }
 
+// C = sum_q A[q].B[q] + bias: the pairs are the splits of one product along the joint reduction.
+template <typename T>
+int32_t batch_sum_fwd_t(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_buf_t C) {
+    GemmArgs<T> a = plain_gemm<T>(0, 0, A->rows, B->cols, A->cols, A->ptr, A->cols, B->ptr, B->cols, C->ptr, C->cols, 0);
+    if (bias) a.bias = static_cast<const T*>(bias->ptr);
+    if (A->depth > 1) {
+        a.nseg = (int)A->depth;
+        a.segstrideA = A->rows * A->cols;
+        a.segstrideB = B->rows * B->cols;
+        if (int32_t st = ensure_workspace((size_t)a.nseg * a.M * a.N * sizeof(T))) return st;
+        a.split_ws = static_cast<T*>(CUR_WORKSPACE);
+    } else if (int32_t st = attach_split_workspace(a)) {
+        return st;
+    }
+    HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
 int32_t same_shape(prad_buf_t a, prad_buf_t b, const char* what) {
     if (a->depth != b->depth || a->rows != b->rows || a->cols != b->cols)
         return fail(PRAD_ERR_ARG, "%s: Matrices must have the same dimensions.", what);
@@ -514,6 +532,26 @@ int32_t prad_matmul_fwd_fused(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_
     return enqueue_gemm(0, 0, A, B, H, 0, ep, false);
 }
 
+// Bias gradient by its own launch(es); lock held, handles validated by the caller.
+static int32_t matmul_bwd_bias_only_locked(prad_buf_t dC, prad_buf_t dbias) {
+    REQUIRE_BUF(dbias);
+    if (dbias->dtype != dC->dtype) return fail(PRAD_ERR_DTYPE, "buffers of different element types in one call");
+    if (dbias->cols != dC->cols || dbias->rows != 1 || dbias->depth != 1 || dC->depth != 1)
+        return fail(PRAD_ERR_ARG, "bias gradient must be 1 x cols");
+    double* ws = nullptr;
+    if (colsum_chunks(dC->rows) > 1) {
+        if (int32_t st = ensure_workspace((size_t)colsum_chunks(dC->rows) * dC->cols * sizeof(double))) return st;
+        ws = static_cast<double*>(CUR_WORKSPACE);
+    }
+    if (dC->dtype == PRAD_F64)
+        HIP_TRY(launch_colsum<double>(static_cast<const double*>(dC->ptr), static_cast<double*>(dbias->ptr), dC->rows, dC->cols, ws,
+                                      CUR_STREAM), PRAD_ERR_LAUNCH);
+    else
+        HIP_TRY(launch_colsum<float>(static_cast<const float*>(dC->ptr), static_cast<float*>(dbias->ptr), dC->rows, dC->cols, ws,
+                                     CUR_STREAM), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
 static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, int32_t acc_dA,
                                  int32_t acc_dB, const Epilogue& ep, prad_buf_t dbias = nullptr) {
     REQUIRE_BUF(dC); REQUIRE_BUF(A); REQUIRE_BUF(B);
@@ -536,19 +574,7 @@ static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad
         if (int32_t st = enqueue_gemm(1, 0, A, dC, dB, acc_dB, rider, false)) return st;  // dB = A^T . dC
         if (rider.colsum_dst != nullptr) dbias = nullptr;
     }
-    if (dbias != nullptr) {  // no weight-gradient launch to ride along with, or a tall matrix: own launch(es)
-        double* ws = nullptr;
-        if (colsum_chunks(dC->rows) > 1) {
-            if (int32_t st = ensure_workspace((size_t)colsum_chunks(dC->rows) * dC->cols * sizeof(double))) return st;
-            ws = static_cast<double*>(CUR_WORKSPACE);
-        }
-        if (dC->dtype == PRAD_F64)
-            HIP_TRY(launch_colsum<double>(static_cast<const double*>(dC->ptr), static_cast<double*>(dbias->ptr), dC->rows, dC->cols, ws,
-                                          CUR_STREAM), PRAD_ERR_LAUNCH);
-        else
-            HIP_TRY(launch_colsum<float>(static_cast<const float*>(dC->ptr), static_cast<float*>(dbias->ptr), dC->rows, dC->cols, ws,
-                                         CUR_STREAM), PRAD_ERR_LAUNCH);
-    }
+    if (dbias != nullptr) return matmul_bwd_bias_only_locked(dC, dbias);  // nothing to ride along with, or a tall matrix
     return PRAD_OK;
 }
 
@@ -566,6 +592,44 @@ int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_bu
     ep.act_bwd = act; ep.act_src = act_src; ep.alpha = alpha;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     return matmul_bwd_locked(dC, A, B, dA, dB, 0, accumulate_dB, ep);
+}
+
+int32_t prad_matmul_batch_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_buf_t C) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(A); REQUIRE_BUF(B); REQUIRE_BUF(C);
+    if (bias != nullptr) REQUIRE_BUF(bias);
+    if (int32_t st = same_dtype({A, B, bias, C})) return st;
+    if (A->depth != B->depth || A->depth > 65535) return fail(PRAD_ERR_SHAPE, "both operands must hold the same number of slices");
+    if (A->cols != B->rows) return fail(PRAD_ERR_SHAPE, "Input 1 columns do not match Input 2 rows");
+    if (C->depth != 1 || C->rows != A->rows || C->cols != B->cols)
+        return fail(PRAD_ERR_ARG, "output must be %lldx%lld", (long long)A->rows, (long long)B->cols);
+    if (bias && (bias->rows != 1 || bias->cols != C->cols || bias->depth != 1))
+        return fail(PRAD_ERR_ARG, "The length of the bias vector must be the same as the number of columns in the input matrix.");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return A->dtype == PRAD_F64 ? batch_sum_fwd_t<double>(A, B, bias, C) : batch_sum_fwd_t<float>(A, B, bias, C);
+}
+
+int32_t prad_matmul_batch_sum_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, prad_buf_t dbias) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(dC); REQUIRE_BUF(A); REQUIRE_BUF(B);
+    if (A->depth != B->depth) return fail(PRAD_ERR_SHAPE, "both operands must hold the same number of slices");
+    if (A->cols != B->rows) return fail(PRAD_ERR_SHAPE, "Input 1 columns do not match Input 2 rows");
+    if (dC->depth != 1 || dC->rows != A->rows || dC->cols != B->cols)
+        return fail(PRAD_ERR_ARG, "upstream gradient is %lldx%lld, the product is %lldx%lld", (long long)dC->rows,
+                    (long long)dC->cols, (long long)A->rows, (long long)B->cols);
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (dA != nullptr) {
+        REQUIRE_BUF(dA);
+        if (int32_t st = same_shape(A, dA, "gradient of the first operand")) return st;
+        if (int32_t st = enqueue_gemm(0, 1, dC, B, dA, 0, Epilogue{}, true)) return st;  // dA[q] = dC . B[q]^T
+    }
+    if (dB != nullptr) {
+        REQUIRE_BUF(dB);
+        if (int32_t st = same_shape(B, dB, "gradient of the second operand")) return st;
+        if (int32_t st = enqueue_gemm(1, 0, A, dC, dB, 0, Epilogue{}, true)) return st;  // dB[q] = A[q]^T . dC
+    }
+    if (dbias != nullptr) return matmul_bwd_bias_only_locked(dC, dbias);
+    return PRAD_OK;
 }
 
 int32_t prad_matmul_bias_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, prad_buf_t dbias,

@@ -306,6 +306,51 @@ class GpuMatrixMultiplyAndSumOperation(MatrixMultiplyAndSumOperation):
         return GpuMatrixMultiplyAndSumOperation()
 
 
+class BatchMatrixMultiplySumOperation(Operation):
+    """Independent products summed into one output plus a broadcast bias: C = sum_q A[q].B[q] + bias.
+    No operation of the reference has this form; it is the composition of MatrixMultiplyOperation.Forward
+    per slice (src/RMAD/MatrixMultiplyOperation.cs:50-80), a sum of the products in slice order and
+    MatrixAddBroadcastingOperation (src/RMAD/MatrixAddBroadcastingOperation.cs:32-70), run as one split
+    product.  Backward returns [dA (deep), dB (deep), dBias]."""
+
+    def __init__(self):
+        super().__init__()
+        self.a = self.b = self.bias = None
+
+    @staticmethod
+    def Instantiate(net):
+        return BatchMatrixMultiplySumOperation()
+
+    def _intermediates(self):
+        return [self.a, self.b, self.bias]
+
+    def _restore_from(self, items):
+        self.a, self.b, self.bias = items
+
+    def Forward(self, a, b, bias=None):
+        _ensure_initialized()
+        self.a, self.b, self.bias = a, b, bias
+        if a.Cols != b.Rows:
+            raise InvalidOperationException("Input 1 columns do not match Input 2 rows")
+        out = DeviceBuffer.alloc(a.dtype, a.Rows, b.Cols)
+        check(_lib.load().prad_matmul_batch_sum_fwd(a.device().handle, b.device().handle,
+                                                   None if bias is None else bias.device().handle, out.handle))
+        self.Output = Matrix._from_device(out)
+        return self.Output
+
+    def Backward(self, dOutput):
+        a, b = self.a, self.b
+        d_a = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols, depth=a.Depth)
+        d_b = DeviceBuffer.alloc(a.dtype, b.Rows, b.Cols, depth=b.Depth)
+        d_bias = None if self.bias is None else DeviceBuffer.alloc(a.dtype, 1, b.Cols)
+        check(_lib.load().prad_matmul_batch_sum_bwd(dOutput.device().handle, a.device().handle, b.device().handle, d_a.handle,
+                                                   d_b.handle, None if d_bias is None else d_bias.handle))
+        builder = BackwardResultBuilder().AddInputGradient(DeepMatrix._from_device(d_a)).AddInputGradient(DeepMatrix._from_device(d_b))
+        if d_bias is not None:
+            builder.AddBiasGradient(Matrix._from_device(d_bias))
+        return builder.Build()
+
+
 class _ActivationOperation(Operation):
     """Elementwise activation; ``_caches`` says whether Backward needs the input or the output."""
 

@@ -68,3 +68,35 @@ def test_shape_errors(gpu):
     op = GpuMatrixMultiplyAndSumOperation.Instantiate(None)
     with pytest.raises(InvalidOperationException, match="compatible for multiplication"):
         op.Forward(Matrix(4, 5), DeepMatrix(2, 6, 4))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 64, 96, 64), (3, 33, 50, 17), (32, 128, 192, 128), (1, 40, 24, 56)])
+def test_batch_of_products_summed_with_bias(gpu, oracle, dtype, shape):
+    """C = sum_q A[q].B[q] + bias against the oracle's composition: MatrixMultiplyOperation.Forward per slice,
+    the products added in slice order, MatrixAddBroadcasting; and its backward against matmul_bwd per slice.
+    (The reference has no single operation of this form, so the composition is the bar.)"""
+    from conftest import dot_bound
+    from parallelreverseautodiff_amd.operations import BatchMatrixMultiplySumOperation
+    P, M, K, N = shape
+    A = seeded.normal(83, 1, (P, M, K), 1.0, dtype)
+    B = seeded.normal(83, 2, (P, K, N), 1.0, dtype)
+    bias = seeded.normal(83, 3, (1, N), 1.0, dtype)
+    dC = seeded.normal(83, 4, (M, N), 1.0, dtype)
+    ref = np.zeros((M, N), dtype)
+    for q in range(P):
+        ref = ref + oracle.matmul_fwd(A[q], B[q], threads=4)
+    ref = oracle.add_broadcast_fwd(ref, bias)
+    op = BatchMatrixMultiplySumOperation.Instantiate(None)
+    C = op.Forward(DeepMatrix.from_numpy(A), DeepMatrix.from_numpy(B), Matrix.from_numpy(bias))
+    bound = sum(dot_bound(A[q], B[q], dtype) for q in range(P)) + P * np.finfo(dtype).eps * np.abs(ref)
+    assert_parity(C.to_numpy(), ref, dtype, "sum of products + bias", bound=bound)
+    res = op.Backward(Matrix.from_numpy(dC))
+    dA, dB, db = res.Results
+    for q in range(P):
+        rA, rB = oracle.matmul_bwd(dC, A[q], B[q], threads=4)
+        assert_parity(dA.to_numpy()[q], rA, dtype, "dA[%d]" % q)
+        assert_parity(dB.to_numpy()[q], rB, dtype, "dB[%d]" % q)
+    assert_parity(db.to_numpy(), oracle.add_broadcast_bwd_bias(dC), dtype, "bias gradient")
+    with pytest.raises(InvalidOperationException):
+        BatchMatrixMultiplySumOperation().Forward(DeepMatrix.from_numpy(A), DeepMatrix.from_numpy(A))
