@@ -75,7 +75,17 @@ struct Slab {
     static constexpr int MN = 32 * WT;
     static constexpr int BK = Mfma<T>::SLAB_ELEMS / MN;
     static constexpr int LDK = BK + Mfma<T>::KPAD;  // pitch of a KC row: 16 bytes past a multiple of 128/256/512 bytes
-    static constexpr int LDM = MN + 16;             // pitch of an MC row
+    // MC rows (one k each, MN elements): the 128 tile pads the pitch by 16 elements; the smaller tiles, whose
+    // padded slabs would let only one workgroup live on a compute unit, keep the pitch at MN and rotate row k
+    // by mc_shift(k) elements instead, which gives the MFMA lane read (16 columns x 4 consecutive k) the same
+    // conflict-free bank pattern.
+    static constexpr bool ROTATE_MC = WT < 4;
+    static constexpr int LDM = ROTATE_MC ? MN : MN + 16;
+    static __device__ __forceinline__ int mc_shift(int k) {
+        if (!ROTATE_MC) return 0;
+        if (sizeof(T) == 8) return 16 * (k & 1);           // a row spans all banks (MN = 32) or twice (64)
+        return MN == 32 ? 16 * ((k >> 1) & 1) : 16 * (k & 3);  // floats: rows start 32 banks apart, or at the same bank
+    }
     static constexpr int TPR_KC = BK / Mfma<T>::VEC;        // threads covering one KC row
     static constexpr int ROWS_KC = GEMM_THREADS / TPR_KC;   // KC rows per pass
     static constexpr int TPR_MC = MN / Mfma<T>::VEC;        // threads covering one MC row
@@ -139,14 +149,19 @@ __device__ __forceinline__ void store_slab(T* __restrict__ s, const typename Mfm
 #pragma unroll
     for (int p = 0; p < NV; ++p) {
         if (KC) *reinterpret_cast<Vec*>(s + (tid / S::TPR_KC + S::ROWS_KC * p) * S::LDK + (tid % S::TPR_KC) * VEC) = r[p];
-        else *reinterpret_cast<Vec*>(s + (tid / S::TPR_MC + S::ROWS_MC * p) * S::LDM + (tid % S::TPR_MC) * VEC) = r[p];
+        else {
+            const int k = tid / S::TPR_MC + S::ROWS_MC * p;
+            const int col = ((tid % S::TPR_MC) * VEC + S::mc_shift(k)) & (S::ROTATE_MC ? S::MN - 1 : ~0);
+            *reinterpret_cast<Vec*>(s + k * S::LDM + col) = r[p];
+        }
     }
 }
 
 // Element (mn, k) of a slab in LDS.
 template <typename T, int WT, bool KC>
 __device__ __forceinline__ T slab_at(const T* __restrict__ s, int mn, int k) {
-    return KC ? s[mn * Slab<T, WT>::LDK + k] : s[k * Slab<T, WT>::LDM + mn];
+    typedef Slab<T, WT> S;
+    return KC ? s[mn * S::LDK + k] : s[k * S::LDM + ((mn + S::mc_shift(k)) & (S::ROTATE_MC ? S::MN - 1 : ~0))];
 }
 
 // Maps the linear workgroup id to an output tile.  Hardware deals consecutive workgroup ids
@@ -349,7 +364,54 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         return;
     }
 
-    T* __restrict__ C = p.C + batch * p.strideC + (p.ksplit > 0 ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
+    if (EPI != EPI_TILE_SUM && p.pair_counters != nullptr) {
+        // Two workgroups share this tile, half of K each.  Both park their partial tile in the workspace and
+        // count their arrival; the one that arrives second adds the other's tile to its own accumulators and
+        // goes on to the epilogue.  No workgroup waits for another, and a + b = b + a makes the result
+        // independent of which one that is.
+        const int64_t mn = p.M * p.N;
+        T* __restrict__ mine = p.split_ws + ((int64_t)blockIdx.z * gridDim.y + batch) * mn;
+#pragma unroll
+        for (int x = 0; x < WTM; ++x)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t i = row0 + wm * WS + x * 16 + MF::row(r, g);
+#pragma unroll
+                for (int y = 0; y < WTN; ++y) {
+                    const int64_t j = col0 + wn * WS + y * 16 + li;
+                    if (EDGE && (i >= p.M || j >= p.N)) continue;
+                    __hip_atomic_store(&mine[i * p.N + j], acc[x][y][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        // The partial tile travels as device-coherent stores and loads (written through, read past the
+        // caches) and the barriers wait for their completion: a cache-wide write-back and invalidate
+        // (what a device-scope fence costs) would evict the operand panels of every workgroup nearby.
+        __syncthreads();
+        __shared__ unsigned arrived;
+        if (tid == 0) {
+            unsigned* c = p.pair_counters + (int64_t)batch * tilesM * tilesN + (int64_t)tm * tilesN + tn;
+            arrived = atomicAdd(c, 1u);
+            if (arrived == 1u) *c = 0u;  // left zeroed for the next launch
+        }
+        __syncthreads();
+        if (arrived == 0u) return;
+        const T* other = p.split_ws + ((int64_t)(blockIdx.z ^ 1u) * gridDim.y + batch) * mn;
+#pragma unroll
+        for (int x = 0; x < WTM; ++x)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t i = row0 + wm * WS + x * 16 + MF::row(r, g);
+#pragma unroll
+                for (int y = 0; y < WTN; ++y) {
+                    const int64_t j = col0 + wn * WS + y * 16 + li;
+                    if (EDGE && (i >= p.M || j >= p.N)) continue;
+                    acc[x][y][r] = acc[x][y][r] + __hip_atomic_load(&other[i * p.N + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+    }
+
+    T* __restrict__ C = p.C + batch * p.strideC +
+                        ((p.ksplit > 0 && p.pair_counters == nullptr) ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
         // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
         // row-major: the elementwise arithmetic (which includes exp/tanh code) then sits in one runtime loop
@@ -500,6 +562,23 @@ int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size)
     return (int)((K + ksplit - 1) / ksplit);
 }
 
+static int64_t slab_depth(TileShape t, int elem_size) {
+    if (elem_size == 8) return t == TILE_128x128 ? Slab<double, 4>::BK : t == TILE_64x64 ? Slab<double, 2>::BK : Slab<double, 1>::BK;
+    return t == TILE_128x128 ? Slab<float, 4>::BK : t == TILE_64x64 ? Slab<float, 2>::BK : Slab<float, 1>::BK;
+}
+
+// A product whose chosen tile yields between half and one and a half workgroups per compute unit leaves
+// workgroup slots empty (two fit per compute unit) and has nothing to hide a workgroup's barriers behind:
+// when K is long enough it runs as pairs of workgroups per tile.  PRAD_GEMM_PAIRS=0 switches this off.
+bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_PAIRS"); return !(e && e[0] == '0'); }();
+    if (!enabled || gemm_split_factor(M, N, K, batch, elem_size) > 1) return false;
+    const TileShape t = choose_tile(M, N, batch, false);
+    const int64_t e = t == TILE_128x128 ? 128 : t == TILE_64x64 ? 64 : 32;
+    const int64_t wgs = ((M + e - 1) / e) * ((N + e - 1) / e) * batch;
+    return wgs >= 128 && wgs <= GEMM_PAIR_MAX_TILES && K >= 16 * slab_depth(t, elem_size);
+}
+
 // Adds the partial results of a split product in split order and applies the epilogue.
 template <typename T>
 __global__ void __launch_bounds__(256) split_reduce_kernel(const GemmArgs<T> p, const T* __restrict__ ws, int splits) {
@@ -523,7 +602,7 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
     if (a_in.M <= 0 || a_in.N <= 0 || a_in.batch <= 0) return hipSuccess;
     if (a_in.transA && a_in.transB) return hipErrorInvalidValue;
     GemmArgs<T> a = a_in;
-    a.ksplit = 0;
+    a.ksplit = 0; a.zstrideA = 0; a.zstrideB = 0;
     const int epi = a.tile_sums != nullptr ? EPI_TILE_SUM
                     : (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) ? EPI_ELEMENTWISE
                                                                                                              : EPI_PLAIN;
@@ -531,6 +610,7 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         // Sum of nseg products: one operand pair per split, partial results added in pair order.
         if (a.split_ws == nullptr || a.batch != 1 || epi == EPI_TILE_SUM) return hipErrorInvalidValue;
         GemmArgs<T> part = a;
+        part.pair_counters = nullptr;
         part.K = a.K * a.nseg;
         part.ksplit = a.K;
         part.zstrideA = a.segstrideA; part.zstrideB = a.segstrideB;
@@ -554,6 +634,7 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
     if (splits > 1) {
         constexpr int64_t bk = Slab<T, 1>::BK;
         GemmArgs<T> part = a;
+        part.pair_counters = nullptr;
         part.ksplit = ((a.K + splits - 1) / splits + bk - 1) / bk * bk;
         part.zstrideA = a.transA ? part.ksplit * a.lda : part.ksplit;  // A stored [k][m] when transposed, else [m][k]
         part.zstrideB = a.transB ? part.ksplit : part.ksplit * a.ldb;  // B stored [n][k] when transposed, else [k][n]
@@ -568,7 +649,17 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         hipLaunchKernelGGL((split_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, a, a.split_ws, splits);
         return hipGetLastError();
     }
-    switch (choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr)) {
+    const TileShape tile = choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr);
+    if (a.pair_counters != nullptr && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
+        gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T))) {
+        const int64_t bk = slab_depth(tile, (int)sizeof(T));
+        a.ksplit = ((a.K + 1) / 2 + bk - 1) / bk * bk;
+        a.zstrideA = a.transA ? a.ksplit * a.lda : a.ksplit;
+        a.zstrideB = a.transB ? a.ksplit : a.ksplit * a.ldb;
+    } else {
+        a.pair_counters = nullptr;
+    }
+    switch (tile) {
         case TILE_128x128: return launch_tile<T, 4>(a, epi, stream);
         case TILE_64x64: return launch_tile<T, 2>(a, epi, stream);
         default: return launch_tile<T, 1>(a, epi, stream);

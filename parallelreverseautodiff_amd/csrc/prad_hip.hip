@@ -34,6 +34,8 @@ constexpr uint32_t BUF_MAGIC = 0x50524144u;  // "PRAD"
 constexpr size_t STAGING_CHUNK = (size_t)256 << 20;
 
 constexpr int MAX_BRANCHES = PRAD_MAX_BRANCHES;
+constexpr size_t COUNTER_BYTES = 4096;  // arrival counters of a branch: one per tile of a paired product, and a few
+static_assert(COUNTER_BYTES >= GEMM_PAIR_MAX_TILES * sizeof(unsigned), "a paired product needs a counter per tile");
 
 // Branch 0 is the library stream; branches 1.. exist so that independent operations can overlap
 // (prad_fork / prad_branch / prad_join).  Each branch has its own kernel workspace, because two
@@ -158,13 +160,16 @@ GemmArgs<T> plain_gemm(int transA, int transB, int64_t M, int64_t N, int64_t K, 
     return a;
 }
 
-// Products split along K need room for their partial results; the shared workspace is grown here (lock held).
+// Products split along K (in several passes, or as pairs of workgroups per tile) need room for their
+// partial results; the selected branch's workspace is grown here (lock held).
 template <typename T>
 int32_t attach_split_workspace(GemmArgs<T>& a) {
     const int splits = gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T));
-    if (splits <= 1) return PRAD_OK;
-    if (int32_t st = ensure_workspace((size_t)splits * a.batch * a.M * a.N * sizeof(T))) return st;
+    const bool pairs = splits <= 1 && gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T));
+    if (splits <= 1 && !pairs) return PRAD_OK;
+    if (int32_t st = ensure_workspace((size_t)(pairs ? 2 : splits) * a.batch * a.M * a.N * sizeof(T))) return st;
     a.split_ws = static_cast<T*>(CUR_WORKSPACE);
+    if (pairs) a.pair_counters = cur_branch().counter;
     return PRAD_OK;
 }
 
@@ -294,8 +299,8 @@ int32_t prad_init(int32_t device_id) {
         HIP_TRY(hipStreamCreateWithFlags(&g_ctx.branch[i].stream, hipStreamNonBlocking), PRAD_ERR_NOT_INITIALIZED);
         HIP_TRY(hipEventCreateWithFlags(&g_ctx.branch[i].done, hipEventDisableTiming), PRAD_ERR_NOT_INITIALIZED);
         g_ctx.branch[i].open = false;
-        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.branch[i].counter), 256), PRAD_ERR_ALLOC);
-        HIP_TRY(hipMemset(g_ctx.branch[i].counter, 0, 256), PRAD_ERR_ALLOC);
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.branch[i].counter), COUNTER_BYTES), PRAD_ERR_ALLOC);
+        HIP_TRY(hipMemset(g_ctx.branch[i].counter, 0, COUNTER_BYTES), PRAD_ERR_ALLOC);
     }
     HIP_TRY(hipEventCreateWithFlags(&g_ctx.fork_event, hipEventDisableTiming), PRAD_ERR_NOT_INITIALIZED);
     g_ctx.stream = g_ctx.branch[0].stream;

@@ -392,3 +392,43 @@ def test_bias_gradient_riding_with_the_weight_gradient(gpu, dtype, shape):
     assert np.array_equal(db1.download(), db2.download())
     assert np.array_equal(db1.download(), db3.download())
     assert_parity(db2.download(), dC.astype(np.float64).sum(axis=0, keepdims=True).astype(dtype), dtype, "bias gradient")
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("shape", [(512, 2048, 512), (1024, 1024, 1024), (384, 2100, 500)])
+def test_products_run_as_workgroup_pairs(gpu, oracle, dtype, shape):
+    """Shapes whose tiles fill between half and one and a half of the chip's workgroup slots and whose K is
+    long run with two workgroups per tile (half of K each; the later one adds the other's partial tile):
+    parity with the oracle for the forward and both backward layouts, fused epilogue included, and the same
+    bits on every run, whichever workgroup of a pair arrives last."""
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    M, K, N = shape
+    A = seeded.uniform(91, 1, (M, K), -1.0, 1.0, dtype)
+    B = seeded.uniform(91, 2, (K, N), -1.0, 1.0, dtype)
+    dC = seeded.normal(91, 3, (M, N), 1.0, dtype)
+    bias = seeded.normal(91, 4, (1, N), 1.0, dtype)
+    up = lambda a: (lambda b: (b.upload(a), b)[1])(DeviceBuffer.alloc(dtype, *a.shape))
+    bA, bB, bdC, bbias = up(A), up(B), up(dC), up(bias)
+    C, Z, H = (DeviceBuffer.alloc(dtype, M, N) for _ in range(3))
+    dA, dB = DeviceBuffer.alloc(dtype, M, K), DeviceBuffer.alloc(dtype, K, N)
+    first = None
+    for run in range(4):
+        check(lib.prad_matmul_fwd(bA.handle, bB.handle, C.handle))
+        check(lib.prad_matmul_fwd_fused(bA.handle, bB.handle, bbias.handle, Z.handle, H.handle, _lib.ACT_LEAKYRELU, 0.01))
+        check(lib.prad_matmul_bwd(bdC.handle, bA.handle, bB.handle, dA.handle, dB.handle, 0, 0))
+        got = [x.download() for x in (C, Z, H, dA, dB)]
+        if first is None:
+            first = got
+        else:
+            for a, b2 in zip(first, got):
+                assert np.array_equal(a, b2), "run %d differs from run 0" % run
+    rC = oracle.matmul_fwd(A, B, threads=8)
+    rdA, rdB = oracle.matmul_bwd(dC, A, B, threads=8)
+    rZ = oracle.add_broadcast_fwd(rC, bias)
+    assert_parity(first[0], rC, dtype, "C", bound=dot_bound(A, B, dtype))
+    assert_parity(first[1], rZ, dtype, "Z")
+    assert_parity(first[2], oracle.leakyrelu_fwd(rZ, dtype(0.01)), dtype, "H")
+    assert_parity(first[3], rdA, dtype, "dA", bound=dot_bound(dC, B.T, dtype))
+    assert_parity(first[4], rdB, dtype, "dB", bound=dot_bound(A.T, dC, dtype))
