@@ -50,17 +50,17 @@ constexpr int Q_PER_WG = 2;  // slices written per workgroup of the dB kernel
 // dB[q][k][m] = A[m][k] * dOut[q]: the A tile is transposed through LDS once and scaled into
 // Q_PER_WG slices; reads walk k, writes walk m, both contiguous.
 template <typename T>
-__global__ void __launch_bounds__(256) sum_bwd_db_kernel(const T* __restrict__ A, const T* __restrict__ dOut, T* __restrict__ dB,
-                                                         int64_t M, int64_t K, int64_t P) {
-    __shared__ T tile[TS][TS + 1];
-    const int64_t m0 = (int64_t)blockIdx.x * TS, k0 = (int64_t)blockIdx.y * TS;
+__device__ __forceinline__ void sum_bwd_db_block(T (*tile)[TS + 1], const T* __restrict__ A, const T* __restrict__ dOut,
+                                                 T* __restrict__ dB, int64_t M, int64_t K, int64_t P, int64_t bx, int64_t by,
+                                                 int64_t bz) {
+    const int64_t m0 = bx * TS, k0 = by * TS;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int r = ty; r < TS; r += 4) {
         const int64_t m = m0 + r, k = k0 + tx;
         tile[r][tx] = (m < M && k < K) ? A[m * K + k] : (T)0;
     }
     __syncthreads();
-    const int64_t q0 = (int64_t)blockIdx.z * Q_PER_WG;
+    const int64_t q0 = bz * Q_PER_WG;
     for (int64_t q = q0; q < q0 + Q_PER_WG && q < P; ++q) {
         const T sc = dOut[q];
         T* __restrict__ out = dB + q * K * M;
@@ -75,12 +75,12 @@ __global__ void __launch_bounds__(256) sum_bwd_db_kernel(const T* __restrict__ A
 // dA = dA + t).  A thread owns dA elements in the orientation B is stored in (i contiguous), keeps
 // their running sums in registers over all q, and the finished tile is transposed through LDS so
 // that the single write of dA walks j.
+constexpr int TJ = 16;  // rows of B (j) per workgroup of the dA part; 64 columns (i)
 template <typename T>
-__global__ void __launch_bounds__(256) sum_bwd_da_kernel(const T* __restrict__ B, const T* __restrict__ dOut, T* __restrict__ dA,
-                                                         int64_t M, int64_t K, int64_t N, int64_t P) {
-    constexpr int TJ = 16;  // rows of B (j) per workgroup; 64 columns (i)
-    __shared__ T tile[TJ][TS + 1];
-    const int64_t i0 = (int64_t)blockIdx.x * TS, j0 = (int64_t)blockIdx.y * TJ;
+__device__ __forceinline__ void sum_bwd_da_block(T (*tile)[TS + 1], const T* __restrict__ B, const T* __restrict__ dOut,
+                                                 T* __restrict__ dA, int64_t M, int64_t K, int64_t N, int64_t P, int64_t bx,
+                                                 int64_t by) {
+    const int64_t i0 = bx * TS, j0 = by * TJ;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // ty in 0..3, rows ty, ty+4, ty+8, ty+12
     T acc[4] = {(T)0, (T)0, (T)0, (T)0};
     const int64_t i = i0 + tx;
@@ -125,18 +125,33 @@ __global__ void __launch_bounds__(256) sum_bwd_da_kernel(const T* __restrict__ B
     }
 }
 
+// Both gradients in one launch: the workgroups of the dA part (each walks all P slices) come first in the
+// grid, those of the dB part fill in behind them.
+template <typename T>
+__global__ void __launch_bounds__(256) sum_bwd_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ dOut,
+                                                      T* __restrict__ dA, T* __restrict__ dB, int64_t M, int64_t K, int64_t N,
+                                                      int64_t P, int64_t da_blocks, int64_t bm, int64_t db_by) {
+    __shared__ T tile[TS][TS + 1];
+    int64_t id = blockIdx.x;
+    if (id < da_blocks) {
+        sum_bwd_da_block<T>(tile, B, dOut, dA, M, K, N, P, id % bm, id / bm);
+        return;
+    }
+    id -= da_blocks;
+    sum_bwd_db_block<T>(tile, A, dOut, dB, M, K, P, id % bm, (id / bm) % db_by, id / (bm * db_by));
+}
+
 template <typename T>
 hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T* dB, int64_t M, int64_t K, int64_t N, int64_t P,
                                  hipStream_t s) {
     if (M <= 0 || K <= 0) return hipSuccess;
-    if (dB != nullptr && P > 0) {
-        dim3 grid((unsigned)((M + TS - 1) / TS), (unsigned)((K + TS - 1) / TS), (unsigned)((P + Q_PER_WG - 1) / Q_PER_WG));
-        hipLaunchKernelGGL((sum_bwd_db_kernel<T>), grid, dim3(256), 0, s, A, dOut, dB, M, K, P);
-    }
-    if (dA != nullptr) {
-        dim3 grid((unsigned)((M + TS - 1) / TS), (unsigned)((K + 15) / 16), 1);
-        hipLaunchKernelGGL((sum_bwd_da_kernel<T>), grid, dim3(256), 0, s, B, dOut, dA, M, K, N, P);
-    }
+    const int64_t bm = (M + TS - 1) / TS, db_by = (K + TS - 1) / TS;
+    const int64_t da_blocks = dA != nullptr ? bm * ((K + TJ - 1) / TJ) : 0;
+    const int64_t db_blocks = (dB != nullptr && P > 0) ? bm * db_by * ((P + Q_PER_WG - 1) / Q_PER_WG) : 0;
+    if (da_blocks + db_blocks == 0) return hipSuccess;
+    if (da_blocks + db_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((sum_bwd_kernel<T>), dim3((unsigned)(da_blocks + db_blocks)), dim3(256), 0, s, A, B, dOut, dA, dB, M, K, N, P,
+                       da_blocks, bm, db_by);
     return hipGetLastError();
 }
 

@@ -4,7 +4,7 @@
 // group of a model, replacing the Parallel.For over layers of GradientClipper.Clip (:31-71)
 // and AdamOptimizer.Optimize (:32-91) and the five temporaries per weight of the reference.
 //
-// Work is cut into chunks of CHUNK elements; chunk c of the launch belongs to the tensor whose
+// Work is cut into chunks of OPT_CHUNK elements; chunk c of the launch belongs to the tensor whose
 // [first_chunk, first_chunk + nchunks) range contains it (binary search in the descriptor table).
 //
 // Clip statistics: the reference makes two passes (mean, then sum of squared deviations).  Here
@@ -17,7 +17,12 @@
 namespace prad {
 
 constexpr int OPT_THREADS = 256;
-constexpr int OPT_CHUNK = 4096;  // elements per workgroup
+// Elements per workgroup (template argument CHUNK of the kernels): 4096, or for large float tensors 8192, so
+// that a float workgroup keeps as many bytes in flight as a double one (float clip was 4 points of HBM peak
+// behind with 4096-element chunks); a small model keeps the small chunk, which spreads it over more workgroups.
+constexpr int OPT_CHUNK_SMALL = 4096;
+template <typename T> constexpr int OPT_CHUNK_LARGE = 32768 / (int)sizeof(T);
+constexpr int64_t LARGE_CHUNK_FROM = (int64_t)4 << 20;  // total elements of a launch
 
 template <typename T>
 struct DevTensor {
@@ -77,34 +82,34 @@ __device__ __forceinline__ Moments shfl_down(const Moments& a, int off) {
 }
 
 // A chunk is processed with 16-byte vector accesses when it is full and its tensor's pointers are
-// 16-byte aligned (chunks start at multiples of 4096 elements); partial last chunks and borrowed,
+// 16-byte aligned (chunks start at multiples of 32 KiB); partial last chunks and borrowed,
 // unaligned buffers take the scalar path.
 template <typename T> struct OptVec;
 template <> struct OptVec<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
 template <> struct OptVec<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
 
-template <typename T>
+template <typename T, int CHUNK>
 __device__ __forceinline__ bool vector_chunk(const void* a, const void* b, const void* c, const void* d, int64_t begin, int64_t end) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c) |
                            reinterpret_cast<uintptr_t>(d);
-    return (end - begin == OPT_CHUNK) && (bits % 16 == 0);
+    return (end - begin == CHUNK) && (bits % 16 == 0);
 }
 
 // Per-chunk moments -> partial[chunk].
-template <typename T>
+template <typename T, int CHUNK>
 __global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTable<T> tab, Moments* __restrict__ partial) {
     typedef typename OptVec<T>::type V;
     constexpr int VN = OptVec<T>::N;
     const int64_t chunk = blockIdx.x;
     const int ti = find_tensor(tab.t, tab.nt, chunk);
     const DevTensor<T> t = tab.t[ti];
-    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
-    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
-    constexpr int PER = OPT_CHUNK / OPT_THREADS;  // 16 elements per thread
+    const int64_t begin = (chunk - t.first_chunk) * CHUNK;
+    const int64_t end = min(begin + (int64_t)CHUNK, t.n);
+    constexpr int PER = CHUNK / OPT_THREADS;  // 16 (double) or 32 (float) elements per thread
     double x[PER];
     int cnt = 0;
     double sum = 0.0;
-    if (vector_chunk<T>(t.g, nullptr, nullptr, nullptr, begin, end)) {
+    if (vector_chunk<T, CHUNK>(t.g, nullptr, nullptr, nullptr, begin, end)) {
         const V* __restrict__ gv = reinterpret_cast<const V*>(t.g + begin);
         V v[PER / VN];
 #pragma unroll
@@ -135,7 +140,7 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTab
             if (i < end) { const double d = x[e] - mo.mean; mo.m2 += d * d; }
         }
     }
-    const bool full = end - begin == OPT_CHUNK;  // uniform over the workgroup
+    const bool full = end - begin == CHUNK;  // uniform over the workgroup
     if (full) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) mo = merge_equal(mo, shfl_down(mo, off));
@@ -255,7 +260,7 @@ struct AdamUpdate {
     }
 };
 
-template <typename T>
+template <typename T, int CHUNK>
 __global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTable<T> tab, const double* __restrict__ stats,
                                                                  const Moments* __restrict__ partial, T clip_value, T min_value) {
     const int64_t chunk = blockIdx.x;
@@ -264,10 +269,10 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTab
     Clamp<T> clamp;
     tensor_stats<T>(t, ti, stats, partial, clamp.mean, clamp.stddev);
     clamp.clip_value = clip_value; clamp.min_value = min_value;
-    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
-    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
-    constexpr int PER = OPT_CHUNK / OPT_THREADS;
-    if (vector_chunk<T>(t.g, nullptr, nullptr, nullptr, begin, end)) {
+    const int64_t begin = (chunk - t.first_chunk) * CHUNK;
+    const int64_t end = min(begin + (int64_t)CHUNK, t.n);
+    constexpr int PER = CHUNK / OPT_THREADS;
+    if (vector_chunk<T, CHUNK>(t.g, nullptr, nullptr, nullptr, begin, end)) {
         typedef typename OptVec<T>::type V;
         constexpr int VN = OptVec<T>::N;
         V* __restrict__ gv = reinterpret_cast<V*>(t.g + begin);
@@ -292,7 +297,7 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_apply_kernel(const TensorTab
 // Adam: one pass over w, m, v, g (7 element sizes of HBM traffic per element).  With CLIP the clamping
 // pass of the clipper runs in the same pass (the clamped gradient is stored, as the clipper does in
 // place): 8 element sizes instead of 2 + 7 for the two passes.
-template <typename T, bool CLIP>
+template <typename T, int CHUNK, bool CLIP>
 __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> tab, const AdamUpdate<T> update,
                                                            const double* __restrict__ stats, const Moments* __restrict__ partial,
                                                            T clip_value, T min_value) {
@@ -304,10 +309,10 @@ __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> 
         tensor_stats<T>(t, ti, stats, partial, clamp.mean, clamp.stddev);
         clamp.clip_value = clip_value; clamp.min_value = min_value;
     }
-    const int64_t begin = (chunk - t.first_chunk) * OPT_CHUNK;
-    const int64_t end = min(begin + (int64_t)OPT_CHUNK, t.n);
-    constexpr int PER = OPT_CHUNK / OPT_THREADS;
-    if (vector_chunk<T>(t.w, t.m, t.v, t.g, begin, end)) {
+    const int64_t begin = (chunk - t.first_chunk) * CHUNK;
+    const int64_t end = min(begin + (int64_t)CHUNK, t.n);
+    constexpr int PER = CHUNK / OPT_THREADS;
+    if (vector_chunk<T, CHUNK>(t.w, t.m, t.v, t.g, begin, end)) {
         typedef typename OptVec<T>::type V;
         constexpr int VN = OptVec<T>::N;
         constexpr int HALF = PER / VN / 2;  // two passes keep the register footprint moderate
@@ -357,14 +362,14 @@ __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> 
 }
 
 template <typename T>
-static int64_t build_table(const TensorDesc<T>* host, int nt, TensorTable<T>& tab) {
+static int64_t build_table(const TensorDesc<T>* host, int nt, TensorTable<T>& tab, int CHUNK) {
     int64_t chunks = 0;
     tab.nt = nt;
     for (int i = 0; i < nt; ++i) {
         tab.t[i].g = host[i].g; tab.t[i].w = host[i].w; tab.t[i].m = host[i].m; tab.t[i].v = host[i].v;
         tab.t[i].n = host[i].n;
         tab.t[i].first_chunk = chunks;
-        tab.t[i].nchunks = (host[i].n + OPT_CHUNK - 1) / OPT_CHUNK;
+        tab.t[i].nchunks = (host[i].n + CHUNK - 1) / CHUNK;
         chunks += tab.t[i].nchunks;
     }
     return chunks;
@@ -375,63 +380,69 @@ size_t clip_workspace_bytes(const int64_t* n, int nt) {
     size_t worst = 0;
     for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
         int64_t chunks = 0;
-        for (int i = g0; i < nt && i < g0 + MAX_TABLE; ++i) chunks += (n[i] + OPT_CHUNK - 1) / OPT_CHUNK;
+        for (int i = g0; i < nt && i < g0 + MAX_TABLE; ++i) chunks += (n[i] + OPT_CHUNK_SMALL - 1) / OPT_CHUNK_SMALL;  // the smaller chunk: an upper bound
         const size_t need = (size_t)chunks * sizeof(Moments) + (size_t)MAX_TABLE * 16;
         if (need > worst) worst = need;
     }
     return worst + 64;
 }
 
-// Statistics passes of the clipper for one group of tensors; returns in *stats_out the finalized
-// statistics, or NULL when every tensor is small enough for the clamping pass to merge its chunks itself.
-template <typename T>
-static void enqueue_clip_stats(const TensorTable<T>& tab, int gn, int64_t chunks, void* workspace, const double** stats_out,
-                               const Moments** partial_out, hipStream_t s) {
-    double* dstats = reinterpret_cast<double*>(workspace);
-    Moments* dpartial = reinterpret_cast<Moments*>(static_cast<char*>(workspace) + (size_t)MAX_TABLE * 16);
-    hipLaunchKernelGGL((clip_stats_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, dpartial);
-    int64_t most = 0;
-    for (int i = 0; i < gn; ++i) most = tab.t[i].nchunks > most ? tab.t[i].nchunks : most;
-    if (most > INLINE_FINALIZE_CHUNKS) {
-        hipLaunchKernelGGL((clip_finalize_kernel<T>), dim3((unsigned)gn), dim3(OPT_THREADS), 0, s, tab, dpartial, dstats);
-        *stats_out = dstats;
-    } else {
-        *stats_out = nullptr;
+// One group of at most MAX_TABLE tensors: clip only (ADAM false), Adam only (CLIP false) or both in one pass.
+template <typename T, int CHUNK, bool CLIP, bool ADAM>
+static hipError_t launch_group(const TensorDesc<T>* host, int gn, void* workspace, T clip_value, T min_value,
+                               const AdamUpdate<T>& update, hipStream_t s) {
+    TensorTable<T> tab;
+    const int64_t chunks = build_table(host, gn, tab, CHUNK);
+    if (chunks == 0) return hipSuccess;
+    if (chunks > 0x7fffffffLL) return hipErrorInvalidValue;
+    const double* stats = nullptr;
+    const Moments* partial = nullptr;
+    if (CLIP) {
+        double* dstats = reinterpret_cast<double*>(workspace);
+        Moments* dpartial = reinterpret_cast<Moments*>(static_cast<char*>(workspace) + (size_t)MAX_TABLE * 16);
+        hipLaunchKernelGGL((clip_stats_kernel<T, CHUNK>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, dpartial);
+        int64_t most = 0;
+        for (int i = 0; i < gn; ++i) most = tab.t[i].nchunks > most ? tab.t[i].nchunks : most;
+        // Tensors of few chunks: the clamping pass merges the chunk moments itself and the finalize launch is skipped.
+        if (most > INLINE_FINALIZE_CHUNKS) {
+            hipLaunchKernelGGL((clip_finalize_kernel<T>), dim3((unsigned)gn), dim3(OPT_THREADS), 0, s, tab, dpartial, dstats);
+            stats = dstats;
+        }
+        partial = dpartial;
     }
-    *partial_out = dpartial;
+    if (ADAM)
+        hipLaunchKernelGGL((adam_kernel<T, CHUNK, CLIP>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, update, stats, partial,
+                           clip_value, min_value);
+    else
+        hipLaunchKernelGGL((clip_apply_kernel<T, CHUNK>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, stats, partial,
+                           clip_value, min_value);
+    return hipGetLastError();
+}
+
+template <typename T, bool CLIP, bool ADAM>
+static hipError_t launch_groups(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value,
+                                const AdamUpdate<T>& update, hipStream_t s) {
+    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
+        const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
+        int64_t total = 0;
+        for (int i = 0; i < gn; ++i) total += host[g0 + i].n;
+        const hipError_t e = (OPT_CHUNK_LARGE<T> != OPT_CHUNK_SMALL && total >= LARGE_CHUNK_FROM)
+                                 ? launch_group<T, OPT_CHUNK_LARGE<T>, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s)
+                                 : launch_group<T, OPT_CHUNK_SMALL, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 template <typename T>
 hipError_t launch_clip(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value, hipStream_t s) {
-    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
-        const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
-        TensorTable<T> tab;
-        const int64_t chunks = build_table(host + g0, gn, tab);
-        if (chunks == 0) continue;
-        const double* stats; const Moments* partial;
-        enqueue_clip_stats<T>(tab, gn, chunks, workspace, &stats, &partial, s);
-        hipLaunchKernelGGL((clip_apply_kernel<T>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, stats, partial, clip_value,
-                           min_value);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    return hipSuccess;
+    return launch_groups<T, true, false>(host, nt, workspace, clip_value, min_value, AdamUpdate<T>{}, s);
 }
 
 template <typename T>
 hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s) {
     const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps};
-    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
-        const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
-        TensorTable<T> tab;
-        const int64_t chunks = build_table(host + g0, gn, tab);
-        if (chunks == 0) continue;
-        hipLaunchKernelGGL((adam_kernel<T, false>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, update,
-                           (const double*)nullptr, (const Moments*)nullptr, (T)0, (T)0);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    return hipSuccess;
+    return launch_groups<T, false, true>(host, nt, nullptr, (T)0, (T)0, update, s);
 }
 
 // GradientClipper.Clip followed by AdamOptimizer.Optimize over the same tensors: statistics pass, then
@@ -440,19 +451,7 @@ template <typename T>
 hipError_t launch_clip_adam(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value, T lr, T beta1, T beta2,
                             T eps, T c1, T c2, hipStream_t s) {
     const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps};
-    for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
-        const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
-        TensorTable<T> tab;
-        const int64_t chunks = build_table(host + g0, gn, tab);
-        if (chunks == 0) continue;
-        const double* stats; const Moments* partial;
-        enqueue_clip_stats<T>(tab, gn, chunks, workspace, &stats, &partial, s);
-        hipLaunchKernelGGL((adam_kernel<T, true>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, update, stats, partial,
-                           clip_value, min_value);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    return hipSuccess;
+    return launch_groups<T, true, true>(host, nt, workspace, clip_value, min_value, update, s);
 }
 
 template hipError_t launch_clip<double>(const TensorDesc<double>*, int, void*, double, double, hipStream_t);
