@@ -77,7 +77,8 @@ def gpu_leg(n, dtype_name, steps, warmup):
 def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
     """Times each bandwidth kernel on n_elems elements (default 64 Mi: beyond the 256 MB last-level cache).
     Algorithmic bytes per element, s = element size: activation backward 3s (read src, dy; write dx),
-    Hadamard backward 5s, accumulate 3s, copy 2s, clip 3s (read for statistics; read + write), Adam 7s."""
+    Hadamard backward 5s, accumulate 3s, copy 2s, clip 3s (read for statistics; read + write), Adam 7s,
+    add 3s, add three 4s, transpose 2s, layer normalization 2s forward / 3s backward (rows of 4096)."""
     from parallelreverseautodiff_amd import _lib, seeded
     from parallelreverseautodiff_amd.cudablas import CudaBlas
     from parallelreverseautodiff_amd.exceptions import check
@@ -96,6 +97,8 @@ def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
     for i in range(3):
         b[i].upload(host[i])
     h = [x.handle for x in b]
+    tr = DeviceBuffer.alloc(dtype, cols, rows)                      # transpose target
+    mean, std = DeviceBuffer.alloc(dtype, 1, rows), DeviceBuffer.alloc(dtype, 1, rows)
     cases = {
         "copy": (2, lambda: lib.prad_buf_copy(h[3], h[0])),
         "leakyrelu_bwd": (3, lambda: lib.prad_act_bwd(_lib.ACT_LEAKYRELU, h[0], h[1], h[3], 0.01)),
@@ -106,6 +109,12 @@ def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
         "accumulate": (3, lambda: lib.prad_accumulate(h[3], h[1])),
         "clip": (3, lambda: lib.prad_clip(h[1], 4.0, 1e-16 if dtype_name == "f64" else 1e-8)),
         "adam": (7, lambda: lib.prad_adam(h[0], h[3], h[2], h[1], 1e-3, 0.9, 0.999, 1e-8, 1.0)),
+        "amplified_sigmoid_bwd": (3, lambda: lib.prad_act_bwd(_lib.ACT_AMPLIFIED_SIGMOID, h[0], h[1], h[3], 0.0)),
+        "add": (3, lambda: lib.prad_add(h[0], h[1], h[3])),
+        "add_three": (4, lambda: lib.prad_add_three(h[0], h[1], h[2], h[3])),
+        "transpose": (2, lambda: lib.prad_transpose(h[0], tr.handle)),
+        "layernorm_fwd": (2, lambda: lib.prad_layernorm_fwd(h[0], h[3], mean.handle, std.handle)),
+        "layernorm_bwd": (3, lambda: lib.prad_layernorm_bwd(h[0], mean.handle, std.handle, h[1], h[3])),
     }
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     check(lib.prad_event_create(ctypes.byref(e0)))

@@ -47,7 +47,8 @@ enum {
     PRAD_ACT_LEAKYRELU = 1, /* src = x; src/RMAD/LeakyReLUOperation.cs:54-93 */
     PRAD_ACT_SIGMOID = 2,   /* src = y; src/RMAD/SigmoidOperation.cs:46-84 */
     PRAD_ACT_TANH = 3,      /* src = y; src/RMAD/TanhOperation.cs:42-79 */
-    PRAD_ACT_GELU = 4       /* src = x; src/RMAD/GELUOperation.cs:44-101 (the reference's own derivative formula) */
+    PRAD_ACT_GELU = 4,      /* src = x; src/RMAD/GELUOperation.cs:44-101 (the reference's own derivative formula) */
+    PRAD_ACT_AMPLIFIED_SIGMOID = 5 /* src = x; src/RMAD/AmplifiedSigmoidOperation.cs:44-84 (derivative as written there) */
 };
 
 typedef struct prad_buf* prad_buf_t;
@@ -157,7 +158,7 @@ int32_t prad_matmul_batch_sum_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, pra
 
 /* ---- elementwise forward / backward (bandwidth kernels) ------------------------------------- */
 int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha);
-/* dx = dy (.) act'(src); src is x for LeakyReLU/GELU and y for Sigmoid/Tanh. */
+/* dx = dy (.) act'(src); src is x for LeakyReLU/GELU/AmplifiedSigmoid and y for Sigmoid/Tanh. */
 int32_t prad_act_bwd(int32_t act, prad_buf_t src, prad_buf_t dy, prad_buf_t dx, double alpha);
 /* HadamardProductOperation, src/RMAD/HadamardProductOperation.cs:50-118 */
 int32_t prad_hadamard_fwd(prad_buf_t a, prad_buf_t b, prad_buf_t y);
@@ -169,6 +170,18 @@ int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad);
 /* y = x + bias broadcast over rows; db[0][j] = sum_i dy[i][j]; src/RMAD/MatrixAddBroadcastingOperation.cs:32-70 */
 int32_t prad_add_broadcast_fwd(prad_buf_t x, prad_buf_t bias, prad_buf_t y);
 int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias);
+/* MatrixAddOperation.Forward, src/RMAD/MatrixAddOperation.cs:30-45 (Backward returns dy for both inputs), and
+ * MatrixAddThreeOperation.Forward, src/RMAD/MatrixAddThreeOperation.cs:35-50: y = (a + b) + c. */
+int32_t prad_add(prad_buf_t a, prad_buf_t b, prad_buf_t y);
+int32_t prad_add_three(prad_buf_t a, prad_buf_t b, prad_buf_t c, prad_buf_t y);
+/* MatrixTransposeOperation, src/RMAD/MatrixTransposeOperation.cs:30-64: y (cols x rows) = x^T; Backward is the
+ * same call on dy. */
+int32_t prad_transpose(prad_buf_t x, prad_buf_t y);
+/* LayerNormalizationOperation, src/RMAD/LayerNormalizationOperation.cs:56-110: per row, y = (x - mean) /
+ * (stddev + 1e-9) with the population deviation; mean and stddev (1 x rows) are what the operation caches.
+ * Backward as written there: dx = dy * ((1 - 1/cols) / (stddev + eps) - (x - mean)^2 / (cols * (stddev + eps)^3)). */
+int32_t prad_layernorm_fwd(prad_buf_t x, prad_buf_t y, prad_buf_t mean, prad_buf_t stddev);
+int32_t prad_layernorm_bwd(prad_buf_t x, prad_buf_t mean, prad_buf_t stddev, prad_buf_t dy, prad_buf_t dx);
 
 /* ---- operations that close a training step on the device ------------------------------------ */
 /* Row-wise softmax, src/RMAD/SoftmaxOperation.cs:45-110 (backward: dx = J^T . dy per row). */

@@ -256,6 +256,52 @@ def mse_bwd(y, t):
     return dy
 
 
+def matrix_add(a, b):
+    return _binary("matrix_add", a, b)
+
+
+def matrix_add_three(a, b, c):
+    dt = a.dtype
+    a, b, c = _c(a, dt), _c(b, dt), _c(c, dt)
+    y = np.empty_like(a)
+    _fn("matrix_add_three", dt)(_p(a), _p(b), _p(c), _p(y), ctypes.c_int64(a.size))
+    return y
+
+
+def matrix_transpose(x):
+    dt = x.dtype
+    x = _c(x, dt)
+    y = np.empty((x.shape[1], x.shape[0]), dt)
+    _fn("matrix_transpose", dt)(_p(x), _p(y), x.shape[0], x.shape[1])
+    return y
+
+
+def layernorm_fwd(x):
+    """Returns (y, mean, stddev); mean and stddev have one entry per row."""
+    dt = x.dtype
+    x = _c(x, dt)
+    y = np.empty_like(x)
+    mean, std = np.empty(x.shape[0], dt), np.empty(x.shape[0], dt)
+    _fn("layernorm_fwd", dt)(_p(x), _p(y), _p(mean), _p(std), x.shape[0], x.shape[1])
+    return y, mean, std
+
+
+def layernorm_bwd(x, mean, stddev, dy):
+    dt = x.dtype
+    x, mean, stddev, dy = _c(x, dt), _c(mean, dt), _c(stddev, dt), _c(dy, dt)
+    dx = np.empty_like(x)
+    _fn("layernorm_bwd", dt)(_p(x), _p(mean), _p(stddev), _p(dy), _p(dx), x.shape[0], x.shape[1])
+    return dx
+
+
+def amplified_sigmoid_fwd(x):
+    return _unary("amplified_sigmoid_fwd", x)
+
+
+def amplified_sigmoid_bwd(x, dy):
+    return _binary("amplified_sigmoid_bwd", x, dy)
+
+
 def time_matmul_fwdbwd(n, dtype=np.float64, threads=1, iters=1):
     """Seconds for `iters` forward+backward passes of an n x n x n product on jagged rows."""
     chk = ctypes.c_double()

@@ -385,6 +385,72 @@ template <class T> void mse_bwd(const T* y, const T* t, T* dy, int rows, int col
 }
 
 // ---------------------------------------------------------------------------------------
+// Operations adjacent to the products in the reference's example graphs.
+// ---------------------------------------------------------------------------------------
+
+// MatrixAddOperation (src/RMAD/MatrixAddOperation.cs:30-68): y = a + b; both input gradients are copies of dy.
+template <class T> void matrix_add(const T* a, const T* b, T* y, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) y[i] = a[i] + b[i];
+}
+// MatrixAddThreeOperation (src/RMAD/MatrixAddThreeOperation.cs:35-70): y = a + b + bias, left to right.
+template <class T> void matrix_add_three(const T* a, const T* b, const T* c, T* y, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) y[i] = a[i] + b[i] + c[i];
+}
+// MatrixTransposeOperation (src/RMAD/MatrixTransposeOperation.cs:30-64): y[i][j] = x[j][i]; backward transposes dy.
+template <class T> void matrix_transpose(const T* x, T* y, int rows, int cols) {
+    for (int i = 0; i < cols; ++i) for (int j = 0; j < rows; ++j) y[(size_t)i * rows + j] = x[(size_t)j * cols + i];
+}
+
+// LINQ Average: double[] sums in double and divides by the count; float[] sums in double and
+// returns (float)(sum / count).
+inline double linq_average(const double* x, int n) { double s = 0; for (int i = 0; i < n; ++i) s += x[i]; return s / n; }
+inline float linq_average(const float* x, int n) { double s = 0; for (int i = 0; i < n; ++i) s += (double)x[i]; return (float)(s / n); }
+
+// LayerNormalizationOperation (src/RMAD/LayerNormalizationOperation.cs:56-110, EPSILON = 1e-9 :17):
+// per row mean = Average(), stdDev = sqrt(Sum(pow(x - mean, 2)) / cols), y = (x - mean) / (stdDev + eps).
+// Backward AS WRITTEN (:87-110): dx = dy * ((1 - 1/cols) / (stdDev + eps) - (x - mean)^2 / (cols * (stdDev + eps)^3)),
+// the diagonal of the Jacobian only (not the full layer-norm gradient).
+template <class T> void layernorm_fwd(const T* x, T* y, T* mean, T* stddev, int rows, int cols) {
+    const T eps = (T)1e-9;
+    std::vector<T> sq((size_t)cols);
+    for (int i = 0; i < rows; ++i) {
+        const T* xr = x + (size_t)i * cols;
+        mean[i] = linq_average(xr, cols);
+        for (int j = 0; j < cols; ++j) sq[j] = p_pow(xr[j] - mean[i], (T)2);
+        stddev[i] = (T)std::sqrt((double)(linq_sum(sq.data(), cols) / cols));
+        for (int j = 0; j < cols; ++j) y[(size_t)i * cols + j] = (xr[j] - mean[i]) / (stddev[i] + eps);
+    }
+}
+template <class T> void layernorm_bwd(const T* x, const T* mean, const T* stddev, const T* dy, T* dx, int rows, int cols) {
+    const T eps = (T)1e-9;
+    for (int i = 0; i < rows; ++i) {
+        const T inv = 1 / (stddev[i] + eps);
+        const T exp1 = (1 - ((T)1.0 / cols)) * inv;
+        for (int j = 0; j < cols; ++j) {
+            const size_t e = (size_t)i * cols + j;
+            const T exp2 = p_pow(x[e] - mean[i], (T)2) / (cols * p_pow(stddev[i] + eps, (T)3));
+            dx[e] = dy[e] * (exp1 - exp2);
+        }
+    }
+}
+
+// AmplifiedSigmoidOperation (src/RMAD/AmplifiedSigmoidOperation.cs:44-84): y = 1 / (1 + pow(PI - 2, -x)) where
+// PradMath.PI is a float ((float)Math.PI, src/PRAD/PradMath.cs:20) and PI - 2 a float subtraction, widened to
+// double for Math.Pow in the double build.  Backward AS WRITTEN: dx = dy * pow(b, -x) / pow(1 + pow(b, -x), 2)
+// (without the ln(b) factor of the derivative).  PRADLite has no such operation; the float instantiation
+// follows the same text with PradMath.Pow(float, float) = (float)Math.Pow.
+template <class T> inline T amp_base() { return (T)((float)3.14159265358979323846 - 2.0f); }
+template <class T> void amplified_sigmoid_fwd(const T* x, T* y, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) y[i] = (T)1 / ((T)1 + p_pow(amp_base<T>(), -x[i]));
+}
+template <class T> void amplified_sigmoid_bwd(const T* x, const T* dy, T* dx, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) {
+        const T d = p_pow(amp_base<T>(), -x[i]) / p_pow((T)1 + p_pow(amp_base<T>(), -x[i]), (T)2);
+        dx[i] = dy[i] * d;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Seeded fill used only by the timing entry point: SplitMix64 of (seed, tensor, index).
 // ---------------------------------------------------------------------------------------
 inline uint64_t splitmix64(uint64_t z) {
@@ -504,6 +570,22 @@ double time_matmul_fwdbwd(int N, int threads, int iters, double* checksum) {
     EXPORT void oracle_cce_bwd_##SFX(const T* p, const T* t, T* dp, int rows, int cols) { cce_bwd<T>(p, t, dp, rows, cols); } \
     EXPORT T oracle_mse_fwd_##SFX(const T* y, const T* t, int rows, int cols) { return mse_fwd<T>(y, t, rows, cols); } \
     EXPORT void oracle_mse_bwd_##SFX(const T* y, const T* t, T* dy, int rows, int cols) { mse_bwd<T>(y, t, dy, rows, cols); } \
+    EXPORT void oracle_matrix_add_##SFX(const T* a, const T* b, T* y, int64_t n) { matrix_add<T>(a, b, y, n); } \
+    EXPORT void oracle_matrix_add_three_##SFX(const T* a, const T* b, const T* c, T* y, int64_t n) {           \
+        matrix_add_three<T>(a, b, c, y, n);                                                                    \
+    }                                                                                                          \
+    EXPORT void oracle_matrix_transpose_##SFX(const T* x, T* y, int rows, int cols) { matrix_transpose<T>(x, y, rows, cols); } \
+    EXPORT void oracle_layernorm_fwd_##SFX(const T* x, T* y, T* mean, T* stddev, int rows, int cols) {         \
+        layernorm_fwd<T>(x, y, mean, stddev, rows, cols);                                                      \
+    }                                                                                                          \
+    EXPORT void oracle_layernorm_bwd_##SFX(const T* x, const T* mean, const T* stddev, const T* dy, T* dx, int rows, \
+                                           int cols) {                                                         \
+        layernorm_bwd<T>(x, mean, stddev, dy, dx, rows, cols);                                                 \
+    }                                                                                                          \
+    EXPORT void oracle_amplified_sigmoid_fwd_##SFX(const T* x, T* y, int64_t n) { amplified_sigmoid_fwd<T>(x, y, n); } \
+    EXPORT void oracle_amplified_sigmoid_bwd_##SFX(const T* x, const T* dy, T* dx, int64_t n) {                \
+        amplified_sigmoid_bwd<T>(x, dy, dx, n);                                                                \
+    }                                                                                                          \
     EXPORT double oracle_time_matmul_fwdbwd_##SFX(int N, int threads, int iters, double* checksum) {           \
         return time_matmul_fwdbwd<T>(N, threads, iters, checksum);                                             \
     }

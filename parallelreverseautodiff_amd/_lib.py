@@ -23,7 +23,7 @@ PRAD_ERR_DTYPE = -8
 PRAD_F64 = 0
 PRAD_F32 = 1
 
-ACT_NONE, ACT_LEAKYRELU, ACT_SIGMOID, ACT_TANH, ACT_GELU = 0, 1, 2, 3, 4
+ACT_NONE, ACT_LEAKYRELU, ACT_SIGMOID, ACT_TANH, ACT_GELU, ACT_AMPLIFIED_SIGMOID = 0, 1, 2, 3, 4, 5
 
 _c = ctypes
 _i32, _i64, _f64, _vp = _c.c_int32, _c.c_int64, _c.c_double, _c.c_void_p
@@ -77,6 +77,11 @@ SIGNATURES = {
     "prad_accumulate": (_i32, [_vp, _vp]),
     "prad_add_broadcast_fwd": (_i32, [_vp, _vp, _vp]),
     "prad_add_broadcast_bwd_bias": (_i32, [_vp, _vp]),
+    "prad_add": (_i32, [_vp, _vp, _vp]),
+    "prad_add_three": (_i32, [_vp, _vp, _vp, _vp]),
+    "prad_transpose": (_i32, [_vp, _vp]),
+    "prad_layernorm_fwd": (_i32, [_vp, _vp, _vp, _vp]),
+    "prad_layernorm_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp]),
     "prad_softmax_fwd": (_i32, [_vp, _vp]),
     "prad_softmax_bwd": (_i32, [_vp, _vp, _vp]),
     "prad_cce_fwd": (_i32, [_vp, _vp, _vp]),

@@ -10,12 +10,14 @@
 namespace prad {
 
 // Activation selectors: same values as PRAD_ACT_* in include/prad_hip.h.
-enum Act : int { ACT_NONE = 0, ACT_LEAKYRELU = 1, ACT_SIGMOID = 2, ACT_TANH = 3, ACT_GELU = 4 };
+enum Act : int { ACT_NONE = 0, ACT_LEAKYRELU = 1, ACT_SIGMOID = 2, ACT_TANH = 3, ACT_GELU = 4, ACT_AMPLIFIED_SIGMOID = 5 };
+constexpr int ACT_LAST = ACT_AMPLIFIED_SIGMOID;
 
 // ---- activation arithmetic, shared by the bandwidth kernels and the GEMM epilogues ----------
 // Formulas follow the reference operation by operation (association order included):
 //   LeakyReLU src/RMAD/LeakyReLUOperation.cs:54-93, Sigmoid src/RMAD/SigmoidOperation.cs:46-84,
-//   Tanh src/RMAD/TanhOperation.cs:42-79, GELU src/RMAD/GELUOperation.cs:86-101.
+//   Tanh src/RMAD/TanhOperation.cs:42-79, GELU src/RMAD/GELUOperation.cs:86-101,
+//   AmplifiedSigmoid src/RMAD/AmplifiedSigmoidOperation.cs:44-84.
 template <typename T> struct GeluConst;
 template <> struct GeluConst<double> {
     // sqrt(2 / pi) in double
@@ -66,6 +68,14 @@ __device__ __forceinline__ float gelu_tanh(float u) {
 __device__ __forceinline__ float gelu_cube(float x) { return x * x * x; }
 __device__ __forceinline__ double gelu_cube(double x) { return x * x * x; }
 
+// AmplifiedSigmoid: pow(b, -x) with b = (float)pi - 2 (PradMath.PI is a float, src/PRAD/PradMath.cs:20, and the
+// subtraction a float one), evaluated as exp(-x * ln b).
+template <typename T>
+__device__ __forceinline__ T amp_pow_neg(T x) {
+    const double ln_b = 0.13242442855180583;  // log(1.1415927410125732421875)
+    return (T)exp(-(double)x * ln_b);
+}
+
 template <typename T>
 __device__ __forceinline__ T act_forward(int act, T x, T alpha) {
     switch (act) {
@@ -76,11 +86,12 @@ __device__ __forceinline__ T act_forward(int act, T x, T alpha) {
             T a = (T)0.5 * ((T)1 + gelu_tanh(GeluConst<T>::s() * (x + (GeluConst<T>::c0() * gelu_cube(x)))));
             return a * x;
         }
+        case ACT_AMPLIFIED_SIGMOID: return (T)1 / ((T)1 + amp_pow_neg<T>(x));
         default: return x;
     }
 }
 
-// Derivative factor act'(src): src is the cached input x (LeakyReLU, GELU) or output y (Sigmoid, Tanh).
+// Derivative factor act'(src): src is the cached input x (LeakyReLU, GELU, AmplifiedSigmoid) or output y (Sigmoid, Tanh).
 template <typename T>
 __device__ __forceinline__ T act_derivative(int act, T s, T alpha) {
     switch (act) {
@@ -93,6 +104,11 @@ __device__ __forceinline__ T act_derivative(int act, T s, T alpha) {
             T c = omb * omb;
             T d = GeluConst<T>::s() * ((GeluConst<T>::c0() * (T)3 * (s * s)) + (T)1);
             return ((T)0.5 * s * ((c * d) + b)) + ((T)0.5 * ((T)1 + b));
+        }
+        case ACT_AMPLIFIED_SIGMOID: {  // as written: pow(b, -x) / pow(1 + pow(b, -x), 2), no ln(b) factor
+            const T e = amp_pow_neg<T>(s);
+            const T q = (T)1 + e;
+            return e / (q * q);
         }
         default: return (T)1;
     }
@@ -191,6 +207,12 @@ inline int64_t gemm_tiles_per_product(int64_t M, int64_t N) { return ((M + 127) 
 template <typename T> hipError_t launch_gemm(const GemmArgs<T>& args, hipStream_t stream);
 
 // ---- bandwidth kernels ----------------------------------------------------------------------
+template <typename T> hipError_t launch_add(const T* a, const T* b, T* y, int64_t n, hipStream_t s);
+template <typename T> hipError_t launch_add_three(const T* a, const T* b, const T* c, T* y, int64_t n, hipStream_t s);
+template <typename T> hipError_t launch_transpose(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_layernorm_fwd(const T* x, T* y, T* mean, T* stddev, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_layernorm_bwd(const T* x, const T* mean, const T* stddev, const T* dy, T* dx, int64_t rows,
+                                                      int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_act_fwd(int act, const T* x, T* y, int64_t n, T alpha, hipStream_t s);
 template <typename T> hipError_t launch_act_bwd(int act, const T* src, const T* dy, T* dx, int64_t n, T alpha, hipStream_t s);
 template <typename T> hipError_t launch_hadamard_fwd(const T* a, const T* b, T* y, int64_t n, hipStream_t s);

@@ -138,6 +138,12 @@ template <typename T> struct Scale {
 template <typename T> struct Copy {
     __device__ __forceinline__ void apply(const T (&in)[1], T (&out)[1]) const { out[0] = in[0]; }
 };
+template <typename T> struct Add2 {  // MatrixAddOperation, src/RMAD/MatrixAddOperation.cs:30-45
+    __device__ __forceinline__ void apply(const T (&in)[2], T (&out)[1]) const { out[0] = in[0] + in[1]; }
+};
+template <typename T> struct Add3 {  // MatrixAddThreeOperation, src/RMAD/MatrixAddThreeOperation.cs:35-50: (a + b) + c
+    __device__ __forceinline__ void apply(const T (&in)[3], T (&out)[1]) const { out[0] = (in[0] + in[1]) + in[2]; }
+};
 template <typename T> struct Accum {  // in: dest, grad ; out: dest
     __device__ __forceinline__ void apply(const T (&in)[2], T (&out)[1]) const { out[0] = in[0] + in[1]; }
 };
@@ -150,6 +156,7 @@ hipError_t launch_act_fwd(int act, const T* x, T* y, int64_t n, T alpha, hipStre
         case ACT_SIGMOID: return launch_stream(p, n, ActFwd<T, ACT_SIGMOID>{alpha}, s);
         case ACT_TANH: return launch_stream(p, n, ActFwd<T, ACT_TANH>{alpha}, s);
         case ACT_GELU: return launch_stream(p, n, ActFwd<T, ACT_GELU>{alpha}, s);
+        case ACT_AMPLIFIED_SIGMOID: return launch_stream(p, n, ActFwd<T, ACT_AMPLIFIED_SIGMOID>{alpha}, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -161,6 +168,7 @@ hipError_t launch_act_bwd(int act, const T* src, const T* dy, T* dx, int64_t n, 
         case ACT_SIGMOID: return launch_stream(p, n, ActBwd<T, ACT_SIGMOID>{alpha}, s);
         case ACT_TANH: return launch_stream(p, n, ActBwd<T, ACT_TANH>{alpha}, s);
         case ACT_GELU: return launch_stream(p, n, ActBwd<T, ACT_GELU>{alpha}, s);
+        case ACT_AMPLIFIED_SIGMOID: return launch_stream(p, n, ActBwd<T, ACT_AMPLIFIED_SIGMOID>{alpha}, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -173,6 +181,16 @@ template <typename T>
 hipError_t launch_hadamard_bwd(const T* a, const T* b, const T* dy, T* da, T* db, int64_t n, hipStream_t s) {
     StreamPtrs<T, 3, 2> p{{a, b, dy}, {da, db}};
     return launch_stream(p, n, HadBwd<T>{}, s);
+}
+template <typename T>
+hipError_t launch_add(const T* a, const T* b, T* y, int64_t n, hipStream_t s) {
+    StreamPtrs<T, 2, 1> p{{a, b}, {y}};
+    return launch_stream(p, n, Add2<T>{}, s);
+}
+template <typename T>
+hipError_t launch_add_three(const T* a, const T* b, const T* c, T* y, int64_t n, hipStream_t s) {
+    StreamPtrs<T, 3, 1> p{{a, b, c}, {y}};
+    return launch_stream(p, n, Add3<T>{}, s);
 }
 template <typename T>
 hipError_t launch_accumulate(T* dest, const T* grad, int64_t n, hipStream_t s) {
@@ -270,6 +288,8 @@ hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double*
     template hipError_t launch_act_bwd<T>(int, const T*, const T*, T*, int64_t, T, hipStream_t);                   \
     template hipError_t launch_hadamard_fwd<T>(const T*, const T*, T*, int64_t, hipStream_t);                      \
     template hipError_t launch_hadamard_bwd<T>(const T*, const T*, const T*, T*, T*, int64_t, hipStream_t);        \
+    template hipError_t launch_add<T>(const T*, const T*, T*, int64_t, hipStream_t);                               \
+    template hipError_t launch_add_three<T>(const T*, const T*, const T*, T*, int64_t, hipStream_t);               \
     template hipError_t launch_accumulate<T>(T*, const T*, int64_t, hipStream_t);                                  \
     template hipError_t launch_copy<T>(T*, const T*, int64_t, hipStream_t);                                        \
     template hipError_t launch_scale<T>(T*, const T*, int64_t, T, hipStream_t);                                    \

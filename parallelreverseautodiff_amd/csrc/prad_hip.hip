@@ -245,7 +245,7 @@ int32_t enqueue_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_bu
         if (ep.act_src->rows != C->rows || ep.act_src->cols != C->cols || ep.act_src->depth != C->depth)
             return fail(PRAD_ERR_ARG, "act_src must have the shape of the gradient it scales");
     }
-    if (ep.act_fwd < 0 || ep.act_fwd > PRAD_ACT_GELU || ep.act_bwd < 0 || ep.act_bwd > PRAD_ACT_GELU)
+    if (ep.act_fwd < 0 || ep.act_fwd > PRAD_ACT_AMPLIFIED_SIGMOID || ep.act_bwd < 0 || ep.act_bwd > PRAD_ACT_AMPLIFIED_SIGMOID)
         return fail(PRAD_ERR_ARG, "unknown activation selector");
     if (A->dtype == PRAD_F64) return enqueue_gemm_t<double>(transA, transB, A, B, C, accumulate, ep, batched);
     return enqueue_gemm_t<float>(transA, transB, A, B, C, accumulate, ep, batched);
@@ -791,7 +791,7 @@ int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_bu
 int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha) {
     REQUIRE_INIT();
     REQUIRE_BUF(x); REQUIRE_BUF(y);
-    if (act < PRAD_ACT_LEAKYRELU || act > PRAD_ACT_GELU) return fail(PRAD_ERR_ARG, "unknown activation selector");
+    if (act < PRAD_ACT_LEAKYRELU || act > PRAD_ACT_AMPLIFIED_SIGMOID) return fail(PRAD_ERR_ARG, "unknown activation selector");
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "activation")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
@@ -803,7 +803,7 @@ int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha) {
 int32_t prad_act_bwd(int32_t act, prad_buf_t src, prad_buf_t dy, prad_buf_t dx, double alpha) {
     REQUIRE_INIT();
     REQUIRE_BUF(src); REQUIRE_BUF(dy); REQUIRE_BUF(dx);
-    if (act < PRAD_ACT_LEAKYRELU || act > PRAD_ACT_GELU) return fail(PRAD_ERR_ARG, "unknown activation selector");
+    if (act < PRAD_ACT_LEAKYRELU || act > PRAD_ACT_AMPLIFIED_SIGMOID) return fail(PRAD_ERR_ARG, "unknown activation selector");
     if (int32_t st = same_dtype({src, dy, dx})) return st;
     if (int32_t st = same_shape(src, dy, "activation backward")) return st;
     if (int32_t st = same_shape(src, dx, "activation backward")) return st;
@@ -856,6 +856,75 @@ int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad) {
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     DISPATCH(dest, launch_accumulate<double>(D(dest), D(grad), count(dest), CUR_STREAM),
              launch_accumulate<float>(F(dest), F(grad), count(dest), CUR_STREAM));
+    return PRAD_OK;
+}
+
+int32_t prad_add(prad_buf_t a, prad_buf_t b, prad_buf_t y) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(a); REQUIRE_BUF(b); REQUIRE_BUF(y);
+    if (int32_t st = same_dtype({a, b, y})) return st;
+    if (int32_t st = same_shape(a, b, "add")) return st;
+    if (int32_t st = same_shape(a, y, "add")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(a, launch_add<double>(D(a), D(b), D(y), count(a), CUR_STREAM), launch_add<float>(F(a), F(b), F(y), count(a), CUR_STREAM));
+    return PRAD_OK;
+}
+
+int32_t prad_add_three(prad_buf_t a, prad_buf_t b, prad_buf_t c, prad_buf_t y) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(a); REQUIRE_BUF(b); REQUIRE_BUF(c); REQUIRE_BUF(y);
+    if (int32_t st = same_dtype({a, b, c, y})) return st;
+    for (prad_buf_t o : {b, c, y})
+        if (int32_t st = same_shape(a, o, "add three")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(a, launch_add_three<double>(D(a), D(b), D(c), D(y), count(a), CUR_STREAM),
+             launch_add_three<float>(F(a), F(b), F(c), F(y), count(a), CUR_STREAM));
+    return PRAD_OK;
+}
+
+int32_t prad_transpose(prad_buf_t x, prad_buf_t y) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(y);
+    if (int32_t st = same_dtype({x, y})) return st;
+    if (x->depth != 1 || y->depth != 1 || y->rows != x->cols || y->cols != x->rows)
+        return fail(PRAD_ERR_ARG, "the transpose of a %lldx%lld matrix is %lldx%lld", (long long)x->rows, (long long)x->cols,
+                    (long long)x->cols, (long long)x->rows);
+    if (x->ptr == y->ptr) return fail(PRAD_ERR_ARG, "transpose in place is not supported");
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_transpose<double>(D(x), D(y), x->rows, x->cols, CUR_STREAM),
+             launch_transpose<float>(F(x), F(y), x->rows, x->cols, CUR_STREAM));
+    return PRAD_OK;
+}
+
+static int32_t layernorm_shapes(prad_buf_t x, prad_buf_t mean, prad_buf_t stddev) {
+    if (x->depth != 1) return fail(PRAD_ERR_SHAPE, "deep buffer passed to layer normalization");
+    for (prad_buf_t o : {mean, stddev})
+        if (o->depth != 1 || o->rows != 1 || o->cols != x->rows) return fail(PRAD_ERR_ARG, "mean and stddev must be 1 x rows");
+    return PRAD_OK;
+}
+
+int32_t prad_layernorm_fwd(prad_buf_t x, prad_buf_t y, prad_buf_t mean, prad_buf_t stddev) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(y); REQUIRE_BUF(mean); REQUIRE_BUF(stddev);
+    if (int32_t st = same_dtype({x, y, mean, stddev})) return st;
+    if (int32_t st = same_shape(x, y, "layer normalization")) return st;
+    if (int32_t st = layernorm_shapes(x, mean, stddev)) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_layernorm_fwd<double>(D(x), D(y), D(mean), D(stddev), x->rows, x->cols, CUR_STREAM),
+             launch_layernorm_fwd<float>(F(x), F(y), F(mean), F(stddev), x->rows, x->cols, CUR_STREAM));
+    return PRAD_OK;
+}
+
+int32_t prad_layernorm_bwd(prad_buf_t x, prad_buf_t mean, prad_buf_t stddev, prad_buf_t dy, prad_buf_t dx) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(x); REQUIRE_BUF(mean); REQUIRE_BUF(stddev); REQUIRE_BUF(dy); REQUIRE_BUF(dx);
+    if (int32_t st = same_dtype({x, mean, stddev, dy, dx})) return st;
+    if (int32_t st = same_shape(x, dy, "layer normalization backward")) return st;
+    if (int32_t st = same_shape(x, dx, "layer normalization backward")) return st;
+    if (int32_t st = layernorm_shapes(x, mean, stddev)) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    DISPATCH(x, launch_layernorm_bwd<double>(D(x), D(mean), D(stddev), D(dy), D(dx), x->rows, x->cols, CUR_STREAM),
+             launch_layernorm_bwd<float>(F(x), F(mean), F(stddev), F(dy), F(dx), x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
 }
 

@@ -470,6 +470,112 @@ class HadamardProductOperation(Operation):
                 .Build())
 
 
+class AmplifiedSigmoidOperation(_ActivationOperation):
+    """src/RMAD/AmplifiedSigmoidOperation.cs:44-84: 1 / (1 + pow(PI - 2, -x)); Backward as written there."""
+
+    _act = _lib.ACT_AMPLIFIED_SIGMOID
+
+    @staticmethod
+    def Instantiate(net):
+        return AmplifiedSigmoidOperation()
+
+
+class MatrixAddOperation(Operation):
+    """y = a + b; Backward returns two copies of dOutput (src/RMAD/MatrixAddOperation.cs:30-68).  The copies are
+    the upstream gradient itself here: nothing writes into a gradient it received."""
+
+    @staticmethod
+    def Instantiate(net):
+        return MatrixAddOperation()
+
+    def Forward(self, inputA, inputB):
+        _ensure_initialized()
+        out = DeviceBuffer.alloc(inputA.dtype, inputA.Rows, inputA.Cols)
+        check(_lib.load().prad_add(inputA.device().handle, inputB.device().handle, out.handle))
+        self.Output = Matrix._from_device(out)
+        return self.Output
+
+    def Backward(self, dOutput):
+        return BackwardResultBuilder().AddInputGradient(dOutput).AddInputGradient(dOutput).Build()
+
+
+class MatrixAddThreeOperation(Operation):
+    """y = a + b + bias; Backward returns dOutput for a, b and as the bias gradient
+    (src/RMAD/MatrixAddThreeOperation.cs:35-70)."""
+
+    @staticmethod
+    def Instantiate(net):
+        return MatrixAddThreeOperation()
+
+    def Forward(self, inputA, inputB, bias):
+        _ensure_initialized()
+        out = DeviceBuffer.alloc(inputA.dtype, inputA.Rows, inputA.Cols)
+        check(_lib.load().prad_add_three(inputA.device().handle, inputB.device().handle, bias.device().handle, out.handle))
+        self.Output = Matrix._from_device(out)
+        return self.Output
+
+    def Backward(self, dOutput):
+        return BackwardResultBuilder().AddInputGradient(dOutput).AddInputGradient(dOutput).AddBiasGradient(dOutput).Build()
+
+
+class MatrixTransposeOperation(Operation):
+    """src/RMAD/MatrixTransposeOperation.cs:30-64"""
+
+    @staticmethod
+    def Instantiate(net):
+        return MatrixTransposeOperation()
+
+    @staticmethod
+    def _transpose(m):
+        _ensure_initialized()
+        out = DeviceBuffer.alloc(m.dtype, m.Cols, m.Rows)
+        check(_lib.load().prad_transpose(m.device().handle, out.handle))
+        return Matrix._from_device(out)
+
+    def Forward(self, input):
+        self.Output = self._transpose(input)
+        return self.Output
+
+    def Backward(self, dOutput):
+        return BackwardResultBuilder().AddInputGradient(self._transpose(dOutput)).Build()
+
+
+class LayerNormalizationOperation(Operation):
+    """src/RMAD/LayerNormalizationOperation.cs:56-110: row-wise (x - mean) / (stddev + 1e-9); caches the input and
+    the per-row mean and deviation (device buffers here); Backward as written in the reference."""
+
+    def __init__(self):
+        super().__init__()
+        self.input = self.mean = self.stdDev = None
+
+    @staticmethod
+    def Instantiate(net):
+        return LayerNormalizationOperation()
+
+    def _intermediates(self):
+        return [self.input, self.mean, self.stdDev]
+
+    def _restore_from(self, items):
+        self.input, self.mean, self.stdDev = items
+
+    def Forward(self, input):
+        _ensure_initialized()
+        self.input = input
+        out = DeviceBuffer.alloc(input.dtype, input.Rows, input.Cols)
+        self.mean = DeviceBuffer.alloc(input.dtype, 1, input.Rows)
+        self.stdDev = DeviceBuffer.alloc(input.dtype, 1, input.Rows)
+        check(_lib.load().prad_layernorm_fwd(input.device().handle, out.handle, self.mean.handle, self.stdDev.handle))
+        self.Output = Matrix._from_device(out)
+        return self.Output
+
+    def Backward(self, gradOutput):
+        _ensure_initialized()
+        dx = DeviceBuffer.alloc(self.input.dtype, self.input.Rows, self.input.Cols)
+        check(_lib.load().prad_layernorm_bwd(self.input.device().handle, self.mean.handle, self.stdDev.handle,
+                                             gradOutput.device().handle, dx.handle))
+        return BackwardResultBuilder().AddInputGradient(Matrix._from_device(dx)).Build()
+
+
 class MatrixAddBroadcastingOperation(Operation):
     """y = x + bias (1 x N); Backward returns [dOutput itself, dBias] with HasMultipleInputs false
     (src/RMAD/MatrixAddBroadcastingOperation.cs:32-70)."""

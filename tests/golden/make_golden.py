@@ -61,6 +61,13 @@ def optim_inputs(dtype, rows=24, cols=17):
     return g, w, m, v
 
 
+def adjacent_inputs(dtype, rows=7, cols=13):
+    a = seeded.normal(SEED, 31, (rows, cols), 2.0, dtype)
+    b = seeded.normal(SEED, 32, (rows, cols), 1.0, dtype)
+    c = seeded.uniform(SEED, 33, (rows, cols), -3.0, 3.0, dtype)
+    return a, b, c
+
+
 def encode(a):
     a = np.ascontiguousarray(a)
     entry = {"shape": list(a.shape), "sha256": hashlib.sha256(a.tobytes()).hexdigest()}
@@ -74,7 +81,7 @@ def encode(a):
 
 
 def main():
-    out = {"seed": SEED, "matmul": {}, "elementwise": {}, "optim": {}}
+    out = {"seed": SEED, "matmul": {}, "elementwise": {}, "optim": {}, "adjacent": {}}
     for name, dt, M, K, N in MATMUL_CASES:
         dtype = np.dtype(dt)
         A, B, dC = matmul_inputs(dtype, M, K, N)
@@ -104,6 +111,19 @@ def main():
         w1, m1, v1 = oracle.adam(w, m, v, g, 1e-3, 0.9, 0.999, 1e-8, 3.0)
         out["optim"][dt] = {"clip": encode(oracle.clip(g, 4.0, minv)), "adam_w": encode(w1), "adam_m": encode(m1),
                             "adam_v": encode(v1)}
+    for dt in ("float64", "float32"):
+        dtype = np.dtype(dt)
+        a, b, c = adjacent_inputs(dtype)
+        y, mean, std = oracle.layernorm_fwd(a)
+        # sums, square roots and divisions only: exact fixtures; pow(b, -x) depends on libm: values within a few ulp
+        out["adjacent"][dt] = {
+            "add": encode(oracle.matrix_add(a, b)), "add_three": encode(oracle.matrix_add_three(a, b, c)),
+            "transpose": encode(oracle.matrix_transpose(a)),
+            "layernorm_y": encode(y), "layernorm_mean": encode(mean), "layernorm_std": encode(std),
+            "layernorm_bwd": encode(oracle.layernorm_bwd(a, mean, std, b)),
+            "values": {"amplified_sigmoid_fwd": [float(v).hex() for v in oracle.amplified_sigmoid_fwd(a).reshape(-1)[:32]],
+                       "amplified_sigmoid_bwd": [float(v).hex() for v in oracle.amplified_sigmoid_bwd(a, b).reshape(-1)[:32]]},
+        }
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden.json")
     with open(path, "w") as f:
         json.dump(out, f, indent=1, sort_keys=True)

@@ -65,3 +65,21 @@ def test_elementwise_and_optim_golden(oracle, dt):
     matches(w1, op["adam_w"])
     matches(m1, op["adam_m"])
     matches(v1, op["adam_v"])
+
+
+@pytest.mark.parametrize("dt", ["float64", "float32"])
+def test_adjacent_operations_golden(oracle, dt):
+    dtype = np.dtype(dt)
+    gold = GOLDEN["adjacent"][dt]
+    a, b, c = make_golden.adjacent_inputs(dtype)
+    matches(oracle.matrix_add(a, b), gold["add"])
+    matches(oracle.matrix_add_three(a, b, c), gold["add_three"])
+    matches(oracle.matrix_transpose(a), gold["transpose"])
+    y, mean, std = oracle.layernorm_fwd(a)
+    matches(y, gold["layernorm_y"])
+    matches(mean, gold["layernorm_mean"])
+    matches(std, gold["layernorm_std"])
+    matches(oracle.layernorm_bwd(a, mean, std, b), gold["layernorm_bwd"])
+    ulp = np.finfo(dtype).eps
+    for key, got in (("amplified_sigmoid_fwd", oracle.amplified_sigmoid_fwd(a)), ("amplified_sigmoid_bwd", oracle.amplified_sigmoid_bwd(a, b))):
+        assert np.allclose(got.reshape(-1)[:32], decode_values(gold["values"][key], dtype), rtol=64 * ulp, atol=4 * ulp)

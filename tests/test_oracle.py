@@ -18,6 +18,13 @@ term, a wrong sign or index, or a transposed operand fails at least one of them:
   clip                      constant / one-element matrices unchanged (NaN path of Math.Min),
                             tiny magnitudes floored, outlier clamped to min(clip, 1 + |z|)
   adam                      closed form at t = 1 with zero moments; ReverseAdamUpdate round trip
+  add / add_three           bit-for-bit vs numpy; (a + b) + c on an input where a + (b + c) differs
+  transpose                 numpy .T bit-for-bit, involution, non-square shape
+  layernorm fwd / bwd       closed form on [1, 2, 3, 4]; zero-variance row gives zeros (0 / 1e-9); numpy statement
+                            of the written formulas; dy = ones gives a non-zero gradient (the reference keeps
+                            only the Jacobian's diagonal; the full layer-norm gradient would be zero)
+  amplified sigmoid         f(0) = 0.5, f(1) = b / (1 + b) with b = float32(pi) - 2; f'(0) as written = 0.25
+                            (the analytic derivative would be ln(b) / 4 = 0.0331)
 """
 from fractions import Fraction
 
@@ -281,3 +288,59 @@ def test_generator_matches_c_copy(oracle):
         assert u[i] == oracle.u01(seeded.DEFAULT_SEED, 3, i)
     assert np.array_equal(seeded.uniform(5, 1, (4, 4)), seeded.uniform(5, 1, (16,)).reshape(4, 4))
     assert 0.0 <= u.min() and u.max() < 1.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_and_transpose(oracle, dtype):
+    a = seeded.normal(41, 1, (9, 14), 3.0, dtype)
+    b = seeded.normal(41, 2, (9, 14), 1.0, dtype)
+    c = seeded.normal(41, 3, (9, 14), 1e-3, dtype)
+    assert np.array_equal(oracle.matrix_add(a, b), a + b)
+    assert np.array_equal(oracle.matrix_add_three(a, b, c), (a + b) + c)
+    big, small = dtype(1.0), dtype(np.finfo(dtype).eps / 2)   # (1 + e/2) + e/2 = 1 but 1 + (e/2 + e/2) = 1 + e
+    got = oracle.matrix_add_three(np.full((1, 1), big), np.full((1, 1), small), np.full((1, 1), small))
+    assert got[0, 0] == big and big + (small + small) != big
+    t = oracle.matrix_transpose(a)
+    assert t.shape == (14, 9) and np.array_equal(t, a.T)
+    assert np.array_equal(oracle.matrix_transpose(t), a)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layernorm_as_written(oracle, dtype):
+    x = np.array([[1, 2, 3, 4], [5, 5, 5, 5], [0, 0, 0, 8]], dtype=dtype)
+    y, mean, std = oracle.layernorm_fwd(x)
+    rt = 8 * np.finfo(dtype).eps
+    assert np.allclose(mean, [2.5, 5.0, 2.0], rtol=rt)
+    assert np.allclose(std, [np.sqrt(1.25), 0.0, np.sqrt(12.0)], rtol=rt)
+    assert np.allclose(y[0], np.array([-1.5, -0.5, 0.5, 1.5]) / np.sqrt(1.25), rtol=1e-6)
+    assert np.array_equal(y[1], np.zeros(4, dtype))                 # 0 / (0 + 1e-9)
+    assert np.allclose(y[2], np.array([-2, -2, -2, 6]) / np.sqrt(12.0), rtol=1e-6)
+    # independent statement of the written formulas in float64
+    xr = seeded.normal(43, 1, (6, 33), 2.0, dtype)
+    dy = seeded.normal(43, 2, (6, 33), 1.0, dtype)
+    y, mean, std = oracle.layernorm_fwd(xr)
+    x64 = xr.astype(np.float64)
+    mu = x64.mean(axis=1, keepdims=True)
+    sd = np.sqrt(((x64 - mu) ** 2).sum(axis=1, keepdims=True) / 33)
+    tol = 1e-12 if dtype == np.float64 else 2e-6
+    assert np.allclose(y, (x64 - mu) / (sd + 1e-9), rtol=tol, atol=tol)
+    dx = oracle.layernorm_bwd(xr, mean, std, dy)
+    want = dy.astype(np.float64) * ((1 - 1 / 33) / (sd + 1e-9) - (x64 - mu) ** 2 / (33 * (sd + 1e-9) ** 3))
+    assert np.allclose(dx, want, rtol=tol * 10, atol=tol * 10)
+    # diagonal of the Jacobian only: a constant upstream gradient does not cancel
+    ones = oracle.layernorm_bwd(xr, mean, std, np.ones_like(xr))
+    assert np.abs(ones.sum(axis=1)).min() > 1.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_amplified_sigmoid_as_written(oracle, dtype):
+    b = np.float64(np.float32(np.pi) - np.float32(2))
+    x = np.array([[0.0, 1.0, -1.0, 20.0]], dtype=dtype)
+    y = oracle.amplified_sigmoid_fwd(x)
+    rt = 1e-14 if dtype == np.float64 else 1e-6
+    assert y[0, 0] == dtype(0.5)
+    assert np.allclose(y[0, 1:], [b / (1 + b), 1 / (1 + b), 1 / (1 + b ** -20.0)], rtol=rt)
+    d = oracle.amplified_sigmoid_bwd(x, np.ones_like(x))
+    assert d[0, 0] == dtype(0.25)                                    # the true derivative is ln(b) / 4 = 0.0331
+    assert np.allclose(d[0, 1], (1 / b) / (1 + 1 / b) ** 2, rtol=rt)
+    assert abs(np.log(b) / 4 - 0.25) > 0.2
