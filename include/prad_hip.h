@@ -140,6 +140,18 @@ int32_t prad_matmul_bwd_host(int32_t dtype, const void* const* dc_rows, const vo
                              const void* const* b_rows, void* const* da_rows, void* const* db_rows, int64_t M,
                              int64_t K, int64_t N);
 
+/* ---- the tape engine's products on flat row-major arrays (no jagged marshalling):
+ *      Tensor.MatrixMultiply, src/PRAD/Tensor.cs:572-608: c (m x n) = alpha * a (m x k) . b (k2 x n); the reference's
+ *      beta multiplies a freshly zeroed result and has no effect, so it is not a parameter; k != k2 is the
+ *      reference's ArgumentException("Incompatible shapes for matrix multiplication.") (status PRAD_ERR_SHAPE).
+ *      TensorReverse.MatrixMultiplyReverse, src/PRAD/TensorReverse.cs:94-157: da = dc . b^T, db = a^T . dc.
+ *      Device-resident tensors use prad_buf_upload / prad_matmul_fwd / prad_matmul_bwd or prad_gemm_f64/f32
+ *      on their own device pointers. */
+int32_t prad_tensor_matmul_host(int32_t dtype, const void* a, const void* b, void* c, int64_t m, int64_t k, int64_t k2,
+                                int64_t n, double alpha);
+int32_t prad_tensor_matmul_reverse_host(int32_t dtype, const void* dc, const void* a, const void* b, void* da, void* db,
+                                        int64_t m, int64_t k, int64_t n);
+
 /* ---- MatrixMultiplyAndSumOperation / GpuMatrixMultiplyAndSumOperation,
  *      src/RMAD/MatrixMultiplyAndSumOperation.cs:50-89, GpuMatrixMultiplyAndSumOperation.cs:114-154 */
 /* out[0][q] = sum_ij (A . B[q])_ij ; A is M x K, B is deep (P, K, N), out is 1 x P. */

@@ -58,6 +58,8 @@ SIGNATURES = {
     "prad_matmul_bwd_fused": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp, _f64]),
     "prad_matmul_batch_sum_fwd": (_i32, [_vp, _vp, _vp, _vp]),
     "prad_matmul_batch_sum_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp]),
+    "prad_tensor_matmul_host": (_i32, [_i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64]),
+    "prad_tensor_matmul_reverse_host": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64]),
     "prad_matmul_bias_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp, _f64]),
     "prad_gemm": (_i32, [_i32, _i32, _vp, _vp, _vp, _i32]),
     "prad_gemm_batched": (_i32, [_i32, _i32, _vp, _vp, _vp, _i32]),

@@ -726,6 +726,51 @@ int32_t prad_matmul_bwd_host(int32_t dtype, const void* const* dc_rows, const vo
     return st;
 }
 
+// The tape engine's products on flat row-major host arrays: Tensor.MatrixMultiply (src/PRAD/Tensor.cs:572-608,
+// which hands the arrays to a BLAS gemm) and TensorReverse.MatrixMultiplyReverse (src/PRAD/TensorReverse.cs:94-157).
+int32_t prad_tensor_matmul_host(int32_t dtype, const void* a, const void* b, void* c, int64_t m, int64_t k, int64_t k2, int64_t n,
+                                double alpha) {
+    REQUIRE_INIT();
+    if (k != k2) return fail(PRAD_ERR_SHAPE, "Incompatible shapes for matrix multiplication.");
+    if (m < 0 || k < 0 || n < 0 || a == nullptr || b == nullptr || c == nullptr) return fail(PRAD_ERR_ARG, "bad tensor arguments");
+    prad_buf_t A = nullptr, B = nullptr, C = nullptr;
+    int32_t st = prad_buf_alloc(dtype, m, k, &A);
+    if (!st) st = prad_buf_alloc(dtype, k, n, &B);
+    if (!st) st = prad_buf_alloc(dtype, m, n, &C);
+    if (!st) st = prad_buf_upload(A, a, k);
+    if (!st) st = prad_buf_upload(B, b, n);
+    if (!st) st = prad_matmul_fwd(A, B, C);
+    if (!st && alpha != 1.0) st = prad_scale(C, C, alpha);
+    if (!st) st = prad_buf_download(C, c, n);
+    std::string keep = tl_error;
+    prad_buf_free(A); prad_buf_free(B); prad_buf_free(C);
+    if (st) tl_error = keep;
+    return st;
+}
+
+int32_t prad_tensor_matmul_reverse_host(int32_t dtype, const void* dc, const void* a, const void* b, void* da, void* db, int64_t m,
+                                        int64_t k, int64_t n) {
+    REQUIRE_INIT();
+    if (m < 0 || k < 0 || n < 0 || dc == nullptr || a == nullptr || b == nullptr || da == nullptr || db == nullptr)
+        return fail(PRAD_ERR_ARG, "bad tensor arguments");
+    prad_buf_t dC = nullptr, A = nullptr, B = nullptr, dA = nullptr, dB = nullptr;
+    int32_t st = prad_buf_alloc(dtype, m, n, &dC);
+    if (!st) st = prad_buf_alloc(dtype, m, k, &A);
+    if (!st) st = prad_buf_alloc(dtype, k, n, &B);
+    if (!st) st = prad_buf_alloc(dtype, m, k, &dA);
+    if (!st) st = prad_buf_alloc(dtype, k, n, &dB);
+    if (!st) st = prad_buf_upload(dC, dc, n);
+    if (!st) st = prad_buf_upload(A, a, k);
+    if (!st) st = prad_buf_upload(B, b, n);
+    if (!st) st = prad_matmul_bwd(dC, A, B, dA, dB, 0, 0);
+    if (!st) st = prad_buf_download(dA, da, k);
+    if (!st) st = prad_buf_download(dB, db, n);
+    std::string keep = tl_error;
+    prad_buf_free(dC); prad_buf_free(A); prad_buf_free(B); prad_buf_free(dA); prad_buf_free(dB);
+    if (st) tl_error = keep;
+    return st;
+}
+
 // ---------------------------------------------------------------------------------------------
 int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out) {
     REQUIRE_INIT();
