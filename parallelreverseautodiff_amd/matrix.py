@@ -16,6 +16,7 @@ when needed:
 """
 import ctypes
 import itertools
+import struct
 import threading
 
 import numpy as np
@@ -233,6 +234,42 @@ class Matrix:
             return np.stack(self._rows)
         return self._dev.download()
 
+    # ---- wire and file formats ------------------------------------------------------------------
+    def Serialize(self, transpose=False):
+        """The byte layout of Matrix.Serialize (src/RMAD/Matrix.cs:856-877; float elements in PRADLite): one byte
+        transpose flag, int32 UniqueId, int32 Rows, int32 Cols (little endian, as BitConverter writes on x64), then
+        the values row-major.  The flag is carried, not applied."""
+        head = struct.pack("<Biii", 1 if transpose else 0, int(self.UniqueId), self._nrows, self._ncols)
+        return head + np.ascontiguousarray(self.to_numpy(), dtype=self.dtype.newbyteorder("<")).tobytes()
+
+    @staticmethod
+    def DeserializeToFlatArray(buffer, dtype=np.float64):
+        """Matrix.DeserializeToFlatArray (src/RMAD/Matrix.cs:357-374): the values of a serialized matrix as one flat array."""
+        _, _, rows, cols = struct.unpack_from("<Biii", buffer, 0)
+        return np.frombuffer(buffer, dtype=np.dtype(dtype).newbyteorder("<"), count=rows * cols, offset=13).astype(dtype)
+
+    @classmethod
+    def Deserialize(cls, buffer, dtype=np.float64):
+        """(transpose flag, Matrix) from the byte layout of Serialize; the UniqueId travels with the matrix."""
+        flag, uid, rows, cols = struct.unpack_from("<Biii", buffer, 0)
+        m = cls.from_numpy(cls.DeserializeToFlatArray(buffer, dtype).reshape(rows, cols))
+        m.UniqueId = uid
+        return bool(flag), m
+
+    def to_json_object(self):
+        """What MatrixJsonConverter.WriteJson emits (src/RMAD/MatrixJsonConverter.cs:34-47)."""
+        return {"UniqueId": int(self.UniqueId), "MatrixValues": [[float(v) for v in row] for row in self.to_numpy()],
+                "Shape": [self._nrows, self._ncols], "NumDimensions": 2}
+
+    @classmethod
+    def from_json_object(cls, obj, dtype=np.float64):
+        """MatrixJsonConverter.ReadJson (src/RMAD/MatrixJsonConverter.cs:57-72); Shape and NumDimensions are optional,
+        as in files written by older versions."""
+        values = obj["MatrixValues"]
+        m = cls([np.array(row, dtype=dtype) for row in values])
+        m.UniqueId = int(obj["UniqueId"])
+        return m
+
 
 class DeepMatrix:
     """Array of Matrix (src/RMAD/DeepMatrix.cs:22) whose device twin is one contiguous deep buffer."""
@@ -305,3 +342,13 @@ class DeepMatrix:
 
     def to_numpy(self):
         return np.stack([m.to_numpy() for m in self._mats])
+
+    def to_json_object(self):
+        """DeepMatrixJsonConverter.WriteJson (src/RMAD/DeepMatrixJsonConverter.cs:33-42)."""
+        return {"UniqueId": int(self.UniqueId), "MatrixArrayValues": [m.to_json_object() for m in self._mats]}
+
+    @classmethod
+    def from_json_object(cls, obj, dtype=np.float64):
+        d = cls([Matrix.from_json_object(o, dtype) for o in obj["MatrixArrayValues"]])
+        d.UniqueId = int(obj["UniqueId"])
+        return d

@@ -6,6 +6,8 @@ src/RMAD/AdamOptimizer.cs:32-91 (Optimize over layers), :195-239 (UpdateWeightWi
 parameters and defaults from src/RMAD/NeuralNetworkParameters.cs:18-88 (PRADLite:
 lite/src/ParallelReverseAutoDiffLite/Lite/NeuralNetworkParameters.cs).
 """
+import json
+
 from . import _lib
 from .exceptions import InvalidOperationException, check
 from .matrix import DeepMatrix, Matrix
@@ -62,6 +64,43 @@ class ModelLayer:
 
     def WeightMatrix(self, identifier):
         return self[identifier, "Weight"]
+
+    # ---- files (src/RMAD/ModelLayer.cs:219-320): Newtonsoft JSON of the Matrix / DeepMatrix converters; the
+    # (weights, firstMoments, secondMoments) tuple serializes as {"Item1": .., "Item2": .., "Item3": ..}.  Values
+    # that live on the device are downloaded for saving; loaded values replace the element objects and reach
+    # the device on their next use.
+    def _dump(self, element):
+        return {i: self._elements[i][element].to_json_object() for i in self.Identifiers}
+
+    def _load(self, objects, element):
+        for identifier, obj in objects.items():
+            if identifier in self._elements:       # unknown identifiers in the file are ignored, as in the reference
+                current = self._elements[identifier][element]
+                kind = DeepMatrix if isinstance(current, DeepMatrix) else Matrix
+                self._elements[identifier][element] = kind.from_json_object(obj, current.dtype)
+
+    def SaveWeights(self, path):
+        with open(path, "w") as f:
+            json.dump(self._dump("Weight"), f, indent=2)
+
+    def LoadWeights(self, path):
+        with open(path) as f:
+            weights = json.load(f)
+        if weights is None:
+            raise InvalidOperationException("Weights must not be null.")
+        self._load(weights, "Weight")
+
+    def SaveWeightsAndMoments(self, path):
+        with open(path, "w") as f:
+            json.dump({"Item1": self._dump("Weight"), "Item2": self._dump("FirstMoment"), "Item3": self._dump("SecondMoment")},
+                      f, indent=2)
+
+    def LoadWeightsAndMoments(self, path):
+        with open(path) as f:
+            items = json.load(f)
+        self._load(items["Item1"], "Weight")
+        self._load(items["Item2"], "FirstMoment")
+        self._load(items["Item3"], "SecondMoment")
 
     def GradientMatrix(self, identifier):
         return self[identifier, "Gradient"]

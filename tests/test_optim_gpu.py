@@ -169,3 +169,27 @@ def test_fused_clip_adam_equals_clip_then_adam(gpu, oracle, dtype):
                 assert_parity(dev["one"]["w"][i].download(), w, dtype, "weight")
                 assert_parity(dev["one"]["m"][i].download(), m, dtype, "first moment")
                 assert_parity(dev["one"]["v"][i].download(), v, dtype, "second moment")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_device_resident_state_survives_a_checkpoint(gpu, tmp_path, dtype):
+    """Weights and moments that live on the device are written in the reference's JSON layout
+    (ModelLayer.SaveWeightsAndMoments), loaded into a fresh layer and trained on: both layers stay bit-identical."""
+    params = NeuralNetworkParameters(lite=dtype == np.float32)
+    shapes = [(33, 17), (1, 17), (5, 4099)]
+    grads = [seeded.normal(72, i, s, 1.0, dtype) for i, s in enumerate(shapes)]
+    a = layer_of([Matrix.from_numpy(seeded.xavier(71, i, *s).astype(dtype)) for i, s in enumerate(shapes)],
+                 [Matrix.from_numpy(g) for g in grads])
+    for step in (1, 2):
+        params.AdamIteration = float(step)
+        AdamOptimizer(params).Optimize([a])                  # state now device-resident
+    path = str(tmp_path / "state.json")
+    a.SaveWeightsAndMoments(path)
+    b = layer_of([Matrix(*s, dtype) for s in shapes], [Matrix.from_numpy(g) for g in grads])
+    b.LoadWeightsAndMoments(path)
+    params.AdamIteration = 3.0
+    AdamOptimizer(params).Optimize([a])
+    AdamOptimizer(params).Optimize([b])
+    for i in range(len(shapes)):
+        for element in ("Weight", "FirstMoment", "SecondMoment"):
+            assert np.array_equal(a["W%d" % i, element].to_numpy(), b["W%d" % i, element].to_numpy()), (i, element)
