@@ -151,10 +151,11 @@ struct GemmArgs {
     // of split z's operand blocks from those of split 0.
     int64_t ksplit;
     int64_t zstrideA, zstrideB;
-    // Products whose tiles would leave half of the chip's workgroup slots empty run as pairs of
-    // workgroups per tile, each reducing half of K (see gemm_pairs): pair_counters points at one zeroed
-    // unsigned per tile and batch (left zeroed), split_ws holds 2 * batch * M * N elements.  nullptr = off.
-    unsigned* pair_counters;
+    // One zeroed unsigned per tile and batch (left zeroed): with it, a product split along K (several ways, see
+    // gemm_split_factor, or two ways, see gemm_pairs) runs as one launch in which the workgroup that arrives
+    // last at a tile's counter adds the partial tiles; without it, a several-way split takes a second launch
+    // and a product that would run as pairs runs unsplit.
+    unsigned* split_counters;
     // A sum of products C = sum_q op(A_q).op(B_q): nseg > 1 operand pairs, segstrideA / segstrideB
     // elements apart, M x K and K x N each.  Runs as a product split along the joint reduction
     // (one pair per split), so split_ws must hold nseg * M * N elements.  batch must be 1.
@@ -196,10 +197,10 @@ constexpr int64_t COLSUM_CHUNK_ROWS = 2048;  // taller matrices are summed in ro
 // the chip (1 = not split).  A split product writes its partial results to GemmArgs::split_ws and a
 // second kernel adds them in split order and applies the epilogue.
 int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size);
-// Whether launch_gemm would run the product as pairs of workgroups per tile (needs GemmArgs::pair_counters and
-// split_ws); at most GEMM_PAIR_MAX_TILES counters are used.
+// Whether launch_gemm would run the product as pairs of workgroups per tile (needs GemmArgs::split_counters and
+// split_ws: 2 * batch * M * N elements).  In-kernel reduction uses at most GEMM_SPLIT_MAX_TILES counters.
 bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size);
-constexpr int GEMM_PAIR_MAX_TILES = 384;
+constexpr int GEMM_SPLIT_MAX_TILES = 384;
 
 // Number of 128 x 128 output tiles of one product (the tile_sums layout).
 inline int64_t gemm_tiles_per_product(int64_t M, int64_t N) { return ((M + 127) / 128) * ((N + 127) / 128); }

@@ -124,14 +124,19 @@ __device__ __forceinline__ void load_slab_guarded(typename Mfma<T>::Vec (&r)[NV]
 // Unguarded loads of one slab, addressed as a wavefront-uniform base (scalar registers, advanced slab
 // by slab) plus a per-thread 32-bit element offset that never changes: the loads take the
 // scalar-base form and the two prefetch register sets share one set of offsets.
+// A tile that hangs over the edge of the matrix (`valid` < MN rows or columns of it exist) clamps its offsets to
+// the last valid row / vector: the threads concerned load duplicates of valid data, which only reach output
+// rows or columns that are never stored (row i of the product depends on row i of A alone, column j on column j
+// of B alone).  A vector that starts below the edge may run past it, inside the padding of the leading dimension.
 template <typename T, int WT, bool KC>
-__device__ __forceinline__ void slab_offsets(unsigned (&off)[NV], int64_t ld, int tid) {
+__device__ __forceinline__ void slab_offsets(unsigned (&off)[NV], int64_t ld, int tid, int valid) {
     typedef Slab<T, WT> S;
     constexpr int VEC = Mfma<T>::VEC;
+    const int last_vec = ((valid - 1) / VEC) * VEC;
 #pragma unroll
     for (int p = 0; p < NV; ++p)
-        off[p] = KC ? (unsigned)((tid / S::TPR_KC + S::ROWS_KC * p) * ld + (tid % S::TPR_KC) * VEC)
-                    : (unsigned)((tid / S::TPR_MC + S::ROWS_MC * p) * ld + (tid % S::TPR_MC) * VEC);
+        off[p] = KC ? (unsigned)(min(tid / S::TPR_KC + S::ROWS_KC * p, valid - 1) * ld + (tid % S::TPR_KC) * VEC)
+                    : (unsigned)((tid / S::TPR_MC + S::ROWS_MC * p) * ld + min((tid % S::TPR_MC) * VEC, last_vec));
 }
 template <typename T>
 __device__ __forceinline__ void load_slab_fast(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ ubase,
@@ -269,8 +274,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         // that the sets are named statically.
         Vec ra0[NV], rb0[NV], ra1[NV], rb1[NV];
         unsigned offa[NV], offb[NV];
-        slab_offsets<T, WT, A_KC>(offa, p.lda, tid);
-        slab_offsets<T, WT, B_KC>(offb, p.ldb, tid);
+        slab_offsets<T, WT, A_KC>(offa, p.lda, tid, (int)min((int64_t)BM, p.M - row0));
+        slab_offsets<T, WT, B_KC>(offb, p.ldb, tid, (int)min((int64_t)BN, p.N - col0));
         // uniform bases of slab 0 and their per-slab strides
         const T* __restrict__ ua = A + (A_KC ? row0 * p.lda : row0);
         const T* __restrict__ ub = B + (B_KC ? col0 * p.ldb : col0);
@@ -364,12 +369,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         return;
     }
 
-    if (EPI != EPI_TILE_SUM && p.pair_counters != nullptr) {
-        // Two workgroups share this tile, half of K each.  Both park their partial tile in the workspace and
-        // count their arrival; the one that arrives second adds the other's tile to its own accumulators and
-        // goes on to the epilogue.  No workgroup waits for another, and a + b = b + a makes the result
-        // independent of which one that is.
+    if (EPI != EPI_TILE_SUM && p.split_counters != nullptr) {
+        // Several workgroups share this tile, a K range each.  Every one parks its partial tile in the workspace
+        // and counts its arrival; the one that arrives last adds the partial tiles in split order (its own
+        // included, read back like the others, so that the sum does not depend on who arrives last) and goes on
+        // to the epilogue.  No workgroup waits for another.  The partial tiles travel as device-coherent stores and
+        // loads (written through, read past the caches) whose completion the barriers wait for: a device-scope
+        // fence would write back and invalidate the whole L2 and evict the operand panels of every workgroup nearby.
         const int64_t mn = p.M * p.N;
+        const int splits = (int)gridDim.z;
         T* __restrict__ mine = p.split_ws + ((int64_t)blockIdx.z * gridDim.y + batch) * mn;
 #pragma unroll
         for (int x = 0; x < WTM; ++x)
@@ -379,39 +387,56 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
 #pragma unroll
                 for (int y = 0; y < WTN; ++y) {
                     const int64_t j = col0 + wn * WS + y * 16 + li;
-                    if (EDGE && (i >= p.M || j >= p.N)) continue;
+                    if (i >= p.M || j >= p.N) continue;
                     __hip_atomic_store(&mine[i * p.N + j], acc[x][y][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-        // The partial tile travels as device-coherent stores and loads (written through, read past the
-        // caches) and the barriers wait for their completion: a cache-wide write-back and invalidate
-        // (what a device-scope fence costs) would evict the operand panels of every workgroup nearby.
         __syncthreads();
         __shared__ unsigned arrived;
         if (tid == 0) {
-            unsigned* c = p.pair_counters + (int64_t)batch * tilesM * tilesN + (int64_t)tm * tilesN + tn;
+            unsigned* c = p.split_counters + (int64_t)batch * tilesM * tilesN + (int64_t)tm * tilesN + tn;
             arrived = atomicAdd(c, 1u);
-            if (arrived == 1u) *c = 0u;  // left zeroed for the next launch
+            if (arrived == (unsigned)splits - 1u) *c = 0u;  // left zeroed for the next launch
         }
         __syncthreads();
-        if (arrived == 0u) return;
-        const T* other = p.split_ws + ((int64_t)(blockIdx.z ^ 1u) * gridDim.y + batch) * mn;
+        if (arrived != (unsigned)splits - 1u) return;
+        // Partial tiles of ZU splits are fetched together, 16 rows of the wavefront's share at a time, so that
+        // enough loads are in flight without holding a second copy of the whole tile in registers.
+        constexpr int ZU = WT == 4 ? 1 : (WT == 2 ? 4 : 8);
+        for (int z0 = 0; z0 < splits; z0 += ZU) {
 #pragma unroll
-        for (int x = 0; x < WTM; ++x)
+            for (int x = 0; x < WTM; ++x) {
+                T part[ZU][WTN][4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int64_t i = row0 + wm * WS + x * 16 + MF::row(r, g);
+                for (int u = 0; u < ZU; ++u) {
+                    if (z0 + u >= splits) break;
+                    const T* other = p.split_ws + ((int64_t)(z0 + u) * gridDim.y + batch) * mn;
 #pragma unroll
-                for (int y = 0; y < WTN; ++y) {
-                    const int64_t j = col0 + wn * WS + y * 16 + li;
-                    if (EDGE && (i >= p.M || j >= p.N)) continue;
-                    acc[x][y][r] = acc[x][y][r] + __hip_atomic_load(&other[i * p.N + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int r = 0; r < 4; ++r) {
+                        const int64_t i = row0 + wm * WS + x * 16 + MF::row(r, g);
+#pragma unroll
+                        for (int y = 0; y < WTN; ++y) {
+                            const int64_t j = col0 + wn * WS + y * 16 + li;
+                            part[u][y][r] = (i >= p.M || j >= p.N)
+                                                ? (T)0
+                                                : __hip_atomic_load(&other[i * p.N + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < ZU; ++u) {
+                    if (z0 + u >= splits) break;
+#pragma unroll
+                    for (int y = 0; y < WTN; ++y)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[x][y][r] = (z0 + u == 0) ? part[u][y][r] : acc[x][y][r] + part[u][y][r];
                 }
             }
+        }
     }
 
     T* __restrict__ C = p.C + batch * p.strideC +
-                        ((p.ksplit > 0 && p.pair_counters == nullptr) ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
+                        ((p.ksplit > 0 && p.split_counters == nullptr) ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
         // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
         // row-major: the elementwise arithmetic (which includes exp/tanh code) then sits in one runtime loop
@@ -431,7 +456,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
                 const int rr = idx / WS, c = idx % WS;
                 const int64_t i = row0 + wm * WS + x * 16 + rr;
                 const int64_t j = col0 + wn * WS + c;
-                if (EDGE && (i >= p.M || j >= p.N)) continue;
+                if (i >= p.M || j >= p.N) continue;
                 T v = stage[rr * LDW + c];
                 if (p.bias != nullptr) v = v + p.bias[j];
                 if (p.Z != nullptr) p.Z[i * p.ldz + j] = v;
@@ -454,7 +479,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
 #pragma unroll
             for (int y = 0; y < WTN; ++y) {
                 const int64_t j = col0 + wn * WS + y * 16 + li;
-                if (EDGE && (i >= p.M || j >= p.N)) continue;
+                if (i >= p.M || j >= p.N) continue;
                 T v = acc[x][y][r];
                 T* c = C + i * p.ldc + j;
                 if (p.accumulate) v = *c + v;
@@ -490,8 +515,11 @@ template <typename T, int WT>
 static hipError_t launch_tile(const GemmArgs<T>& a, int epi, hipStream_t stream) {
     constexpr int VEC = Mfma<T>::VEC;
     constexpr int BM = 32 * WT;
-    // The unguarded kernels use 16-byte loads on whole tiles (any K: a ragged end is handled inside).
-    const bool aligned = (a.M % BM == 0) && (a.N % BM == 0) && a.K > 0 && (a.lda % VEC == 0) &&
+    // The unguarded kernels use 16-byte loads (any M, N, K: tiles over the edge clamp their loads, a ragged end of K
+    // is handled inside); they need operands whose rows start 16-byte aligned.  The tile-sum epilogue adds up whole
+    // tiles and therefore needs the zero fill of the guarded kernels when the output does not fill its tiles.
+    const bool whole = (a.M % BM == 0) && (a.N % BM == 0);
+    const bool aligned = (whole || epi != EPI_TILE_SUM) && a.K > 0 && (a.lda % VEC == 0) &&
                          (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
                          (a.zstrideA % VEC == 0) && (a.zstrideB % VEC == 0) &&
@@ -576,7 +604,7 @@ bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
     const TileShape t = choose_tile(M, N, batch, false);
     const int64_t e = t == TILE_128x128 ? 128 : t == TILE_64x64 ? 64 : 32;
     const int64_t wgs = ((M + e - 1) / e) * ((N + e - 1) / e) * batch;
-    return wgs >= 128 && wgs <= GEMM_PAIR_MAX_TILES && K >= 16 * slab_depth(t, elem_size);
+    return wgs >= 128 && wgs <= GEMM_SPLIT_MAX_TILES && K >= 16 * slab_depth(t, elem_size);
 }
 
 // Adds the partial results of a split product in split order and applies the epilogue.
@@ -610,7 +638,7 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         // Sum of nseg products: one operand pair per split, partial results added in pair order.
         if (a.split_ws == nullptr || a.batch != 1 || epi == EPI_TILE_SUM) return hipErrorInvalidValue;
         GemmArgs<T> part = a;
-        part.pair_counters = nullptr;
+        part.split_counters = nullptr;
         part.K = a.K * a.nseg;
         part.ksplit = a.K;
         part.zstrideA = a.segstrideA; part.zstrideB = a.segstrideB;
@@ -633,11 +661,15 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
     const int splits = (a.split_ws != nullptr && epi != EPI_TILE_SUM) ? gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T)) : 1;
     if (splits > 1) {
         constexpr int64_t bk = Slab<T, 1>::BK;
+        const int64_t tiles = ((a.M + 31) / 32) * ((a.N + 31) / 32) * a.batch;
         GemmArgs<T> part = a;
-        part.pair_counters = nullptr;
         part.ksplit = ((a.K + splits - 1) / splits + bk - 1) / bk * bk;
         part.zstrideA = a.transA ? part.ksplit * a.lda : part.ksplit;  // A stored [k][m] when transposed, else [m][k]
         part.zstrideB = a.transB ? part.ksplit : part.ksplit * a.ldb;  // B stored [n][k] when transposed, else [k][n]
+        if (a.split_counters != nullptr && tiles <= GEMM_SPLIT_MAX_TILES)
+            return launch_tile<T, 1>(part, epi, stream);  // one launch: the last workgroup of a tile reduces
+        // two passes: partial products, then a kernel that adds them in split order and applies the epilogue
+        part.split_counters = nullptr;
         part.C = a.split_ws; part.ldc = a.N; part.strideC = a.M * a.N;  // split z, batch b at ((z * batch) + b) * M * N
         part.accumulate = 0;
         part.bias = nullptr; part.Z = nullptr; part.act_fwd = ACT_NONE; part.act_bwd = ACT_NONE; part.act_src = nullptr;
@@ -650,14 +682,14 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         return hipGetLastError();
     }
     const TileShape tile = choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr);
-    if (a.pair_counters != nullptr && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
+    if (a.split_counters != nullptr && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
         gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T))) {
         const int64_t bk = slab_depth(tile, (int)sizeof(T));
         a.ksplit = ((a.K + 1) / 2 + bk - 1) / bk * bk;
         a.zstrideA = a.transA ? a.ksplit * a.lda : a.ksplit;
         a.zstrideB = a.transB ? a.ksplit : a.ksplit * a.ldb;
     } else {
-        a.pair_counters = nullptr;
+        a.split_counters = nullptr;
     }
     switch (tile) {
         case TILE_128x128: return launch_tile<T, 4>(a, epi, stream);

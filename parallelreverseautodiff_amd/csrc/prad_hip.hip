@@ -35,7 +35,7 @@ constexpr size_t STAGING_CHUNK = (size_t)256 << 20;
 
 constexpr int MAX_BRANCHES = PRAD_MAX_BRANCHES;
 constexpr size_t COUNTER_BYTES = 4096;  // arrival counters of a branch: one per tile of a paired product, and a few
-static_assert(COUNTER_BYTES >= GEMM_PAIR_MAX_TILES * sizeof(unsigned), "a paired product needs a counter per tile");
+static_assert(COUNTER_BYTES >= GEMM_SPLIT_MAX_TILES * sizeof(unsigned), "a split product needs a counter per tile");
 
 // Branch 0 is the library stream; branches 1.. exist so that independent operations can overlap
 // (prad_fork / prad_branch / prad_join).  Each branch has its own kernel workspace, because two
@@ -169,7 +169,7 @@ int32_t attach_split_workspace(GemmArgs<T>& a) {
     if (splits <= 1 && !pairs) return PRAD_OK;
     if (int32_t st = ensure_workspace((size_t)(pairs ? 2 : splits) * a.batch * a.M * a.N * sizeof(T))) return st;
     a.split_ws = static_cast<T*>(CUR_WORKSPACE);
-    if (pairs) a.pair_counters = cur_branch().counter;
+    a.split_counters = cur_branch().counter;
     return PRAD_OK;
 }
 
