@@ -219,6 +219,16 @@ int32_t prad_lstm_cell_fwd(prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_b
  * gradient of the pre-activations) and dc_prev. */
 int32_t prad_lstm_cell_bwd(prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_c, prad_buf_t dh_a, prad_buf_t dh_b,
                            prad_buf_t dc_in, prad_buf_t dG, prad_buf_t dc_prev);
+/* One time step in one launch each way (the recurrent product with the cell arithmetic as its epilogue; same
+ * results as the product followed by prad_lstm_cell_fwd / preceded by prad_lstm_cell_bwd):
+ * forward: G (rows x 4*hidden, holding x_t . W_x + b) becomes the activated gates of G + h_prev . Wh, and c, tanh_c, h
+ * are written; backward for step t: dh = dh_loss + dG_next . Wh^T (dG_next = gate gradients of step t + 1), then the
+ * cell's backward writes dG and dc_prev.  dc_in may be NULL.  dh_scratch (rows x hidden) is only written when the
+ * shape needs the two-launch path (hidden not a multiple of the kernels' K slab, unaligned buffers). */
+int32_t prad_lstm_step_fwd(prad_buf_t h_prev, prad_buf_t Wh, prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_buf_t tanh_c,
+                           prad_buf_t h);
+int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_c,
+                           prad_buf_t dh_loss, prad_buf_t dc_in, prad_buf_t dG, prad_buf_t dc_prev, prad_buf_t dh_scratch);
 /* Borrowed view of rows [row0, row0 + rows) of a 2-D buffer (a block of a fused weight, a time step of a
  * stacked sequence).  The view must be freed before its parent. */
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out);

@@ -92,6 +92,8 @@ SIGNATURES = {
     "prad_mse_bwd": (_i32, [_vp, _vp, _vp]),
     "prad_lstm_cell_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp]),
     "prad_lstm_cell_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "prad_lstm_step_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "prad_lstm_step_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_buf_view_rows": (_i32, [_vp, _i64, _i64, _vpp]),
     "prad_fork": (_i32, [_i32]),
     "prad_branch": (_i32, [_i32]),

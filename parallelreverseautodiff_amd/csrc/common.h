@@ -156,6 +156,11 @@ struct GemmArgs {
     // last at a tile's counter adds the partial tiles; without it, a several-way split takes a second launch
     // and a product that would run as pairs runs unsplit.
     unsigned* split_counters;
+    // LSTM step epilogues (launch_lstm_step_fwd / _bwd; see there).  All matrices are rows x lstm_hidden with
+    // leading dimension lstm_hidden, except gates / dG (rows x 4 * lstm_hidden, blocks [i | f | g | o]).
+    int64_t lstm_hidden;
+    const T* lstm_c_prev; const T* lstm_tanh_c_in; const T* lstm_gates; const T* lstm_dh_loss; const T* lstm_dc_in;
+    T* lstm_c; T* lstm_tanh_c; T* lstm_h; T* lstm_dG; T* lstm_dc_prev;
     // A sum of products C = sum_q op(A_q).op(B_q): nseg > 1 operand pairs, segstrideA / segstrideB
     // elements apart, M x K and K x N each.  Runs as a product split along the joint reduction
     // (one pair per split), so split_ws must hold nseg * M * N elements.  batch must be 1.
@@ -206,6 +211,18 @@ constexpr int GEMM_SPLIT_MAX_TILES = 384;
 inline int64_t gemm_tiles_per_product(int64_t M, int64_t N) { return ((M + 127) / 128) * ((N + 127) / 128); }
 
 template <typename T> hipError_t launch_gemm(const GemmArgs<T>& args, hipStream_t stream);
+
+// One LSTM time step forward in one launch: gates = act(C + A . B) with C (rows x 4H) holding the input
+// projection plus bias, A = h_{t-1} (rows x H), B = W_h (H x 4H); then c = f.c_prev + i.g, tanh_c, h = o.tanh_c.
+// The activated gates replace C.  A workgroup's tile gathers the four gate columns of 8 hidden units, so the
+// cell arithmetic has all it needs.  Same arithmetic as the product followed by launch_lstm_cell_fwd.
+// Returns hipErrorNotSupported for shapes it does not take (H not a multiple of the slab depth, unaligned
+// operands): the caller then runs the two launches.
+template <typename T> hipError_t launch_lstm_step_fwd(const GemmArgs<T>& args, hipStream_t stream);
+// One LSTM time step backward in one launch: dh = dh_loss + A . B^T with A = dG_{t+1} (rows x 4H), B = W_h,
+// then the cell's backward (as launch_lstm_cell_bwd) writes dG_t and dc_prev.  split_ws / split_counters as for
+// launch_gemm.
+template <typename T> hipError_t launch_lstm_step_bwd(const GemmArgs<T>& args, hipStream_t stream);
 
 // ---- bandwidth kernels ----------------------------------------------------------------------
 template <typename T> hipError_t launch_add(const T* a, const T* b, T* y, int64_t n, hipStream_t s);

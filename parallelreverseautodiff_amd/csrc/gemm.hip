@@ -128,15 +128,20 @@ __device__ __forceinline__ void load_slab_guarded(typename Mfma<T>::Vec (&r)[NV]
 // the last valid row / vector: the threads concerned load duplicates of valid data, which only reach output
 // rows or columns that are never stored (row i of the product depends on row i of A alone, column j on column j
 // of B alone).  A vector that starts below the edge may run past it, inside the padding of the leading dimension.
+// gather_stride > 0 (MC operands only): the MN columns of the tile are four segments of MN / 4 columns that lie
+// gather_stride elements apart in memory (the four gate blocks of a fused LSTM weight).
 template <typename T, int WT, bool KC>
-__device__ __forceinline__ void slab_offsets(unsigned (&off)[NV], int64_t ld, int tid, int valid) {
+__device__ __forceinline__ void slab_offsets(unsigned (&off)[NV], int64_t ld, int tid, int valid, int64_t gather_stride = 0) {
     typedef Slab<T, WT> S;
     constexpr int VEC = Mfma<T>::VEC;
     const int last_vec = ((valid - 1) / VEC) * VEC;
+    int col = min((tid % S::TPR_MC) * VEC, last_vec);
+    int64_t col_off = col;
+    if (!KC && gather_stride > 0) col_off = (col / (S::MN / 4)) * gather_stride + col % (S::MN / 4);
 #pragma unroll
     for (int p = 0; p < NV; ++p)
         off[p] = KC ? (unsigned)(min(tid / S::TPR_KC + S::ROWS_KC * p, valid - 1) * ld + (tid % S::TPR_KC) * VEC)
-                    : (unsigned)((tid / S::TPR_MC + S::ROWS_MC * p) * ld + min((tid % S::TPR_MC) * VEC, last_vec));
+                    : (unsigned)((tid / S::TPR_MC + S::ROWS_MC * p) * ld + col_off);
 }
 template <typename T>
 __device__ __forceinline__ void load_slab_fast(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ ubase,
@@ -193,6 +198,8 @@ constexpr int min_blocks(int) { return 2; }
 constexpr int EPI_PLAIN = 0;      // store (or accumulate into) C
 constexpr int EPI_ELEMENTWISE = 1;  // bias / pre-activation copy / activation forward / upstream activation backward
 constexpr int EPI_TILE_SUM = 2;   // reduce the tile to one double (MatrixMultiplyAndSum forward)
+constexpr int EPI_LSTM_FWD = 3;   // gates, cell state and hidden state of one LSTM step (32 x 32 tile gathering 4 gates x 8 units)
+constexpr int EPI_LSTM_BWD = 4;   // cell backward of one LSTM step on the recurrent gradient tile
 
 template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI>
 __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
@@ -275,10 +282,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         Vec ra0[NV], rb0[NV], ra1[NV], rb1[NV];
         unsigned offa[NV], offb[NV];
         slab_offsets<T, WT, A_KC>(offa, p.lda, tid, (int)min((int64_t)BM, p.M - row0));
-        slab_offsets<T, WT, B_KC>(offb, p.ldb, tid, (int)min((int64_t)BN, p.N - col0));
+        constexpr bool GATHER = EPI == EPI_LSTM_FWD;  // B columns: 4 gate segments of BN / 4 hidden units each
+        if (GATHER) slab_offsets<T, WT, B_KC>(offb, p.ldb, tid, BN, p.lstm_hidden);
+        else slab_offsets<T, WT, B_KC>(offb, p.ldb, tid, (int)min((int64_t)BN, p.N - col0));
         // uniform bases of slab 0 and their per-slab strides
         const T* __restrict__ ua = A + (A_KC ? row0 * p.lda : row0);
-        const T* __restrict__ ub = B + (B_KC ? col0 * p.ldb : col0);
+        const T* __restrict__ ub = B + (GATHER ? (int64_t)tn * (BN / 4) : (B_KC ? col0 * p.ldb : col0));
         const int64_t stepa = A_KC ? (int64_t)BK : (int64_t)BK * p.lda;
         const int64_t stepb = B_KC ? (int64_t)BK : (int64_t)BK * p.ldb;
         if (ntiles > 0) {
@@ -435,6 +444,86 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         }
     }
 
+    if (EPI == EPI_LSTM_FWD) {
+        // The tile holds h_{t-1} . W_h for 32 rows and, column block q of 8, gate q of hidden units [8 tn, 8 tn + 8).
+        // It goes through LDS so that one thread gets the four gates of one (row, unit); then the arithmetic of
+        // lstm_cell_fwd_kernel, statement for statement.
+        static_assert(EPI != EPI_LSTM_FWD || WT == 1, "the gate gather is laid out for the 32 x 32 tile");
+        constexpr int LDT = BN + 1;
+        __syncthreads();  // every wavefront is done with the slab stages
+        T* __restrict__ stage = &smem[0][0];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) stage[(wm * WS + MF::row(r, g)) * LDT + wn * WS + li] = acc[0][0][r];
+        __syncthreads();
+        const int row = tid / 8, jj = tid % 8;
+        const int64_t i = row0 + row, H = p.lstm_hidden, j = (int64_t)tn * 8 + jj;
+        if (i < p.M) {
+            T* __restrict__ gr = p.C + i * p.ldc;  // pre-activations (input projection + bias) in, activated gates out
+            const T* __restrict__ st = stage + row * LDT + jj;
+            const T i_ = act_forward<T>(ACT_SIGMOID, gr[j] + st[0], (T)0);
+            const T f_ = act_forward<T>(ACT_SIGMOID, gr[H + j] + st[8], (T)0);
+            const T g_ = act_forward<T>(ACT_TANH, gr[2 * H + j] + st[16], (T)0);
+            const T o_ = act_forward<T>(ACT_SIGMOID, gr[3 * H + j] + st[24], (T)0);
+            gr[j] = i_; gr[H + j] = f_; gr[2 * H + j] = g_; gr[3 * H + j] = o_;
+            const int64_t idx = i * H + j;
+            const T cn = (f_ * p.lstm_c_prev[idx]) + (i_ * g_);
+            const T tc = act_forward<T>(ACT_TANH, cn, (T)0);
+            p.lstm_c[idx] = cn;
+            p.lstm_tanh_c[idx] = tc;
+            p.lstm_h[idx] = o_ * tc;
+        }
+        return;
+    }
+
+    if (EPI == EPI_LSTM_BWD) {
+        // The tile is (dG_{t+1} . W_h^T), the recurrent part of dh, for 32 rows x 32 hidden units.  It goes through
+        // LDS so that a thread takes four elements of consecutive rows with all their loads in flight at once; then
+        // the arithmetic of lstm_cell_bwd_kernel, statement for statement.
+        static_assert(EPI != EPI_LSTM_BWD || WT == 1, "laid out for the 32 x 32 tile");
+        constexpr int LDT = BN + 1;
+        __syncthreads();  // every wavefront is done with the slab stages
+        T* __restrict__ stage = &smem[0][0];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) stage[(wm * WS + MF::row(r, g)) * LDT + wn * WS + li] = acc[0][0][r];
+        __syncthreads();
+        const int64_t H = p.lstm_hidden;
+        const int cc = tid & 31, rbase = tid >> 5;  // rows rbase, rbase + 8, rbase + 16, rbase + 24
+        const int64_t j = col0 + cc;
+        T i_[4], f_[4], g_[4], o_[4], tc[4], dhl[4], dci[4], cp[4];
+        bool ok[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t i = row0 + rbase + 8 * u;
+            ok[u] = i < p.M && j < H;
+            if (ok[u]) {
+                const T* __restrict__ gt = p.lstm_gates + i * 4 * H;
+                const int64_t idx = i * H + j;
+                i_[u] = gt[j]; f_[u] = gt[H + j]; g_[u] = gt[2 * H + j]; o_[u] = gt[3 * H + j];
+                tc[u] = p.lstm_tanh_c_in[idx];
+                dhl[u] = p.lstm_dh_loss[idx];
+                dci[u] = p.lstm_dc_in != nullptr ? p.lstm_dc_in[idx] : (T)0;
+                cp[u] = p.lstm_c_prev[idx];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (!ok[u]) continue;
+            const int64_t i = row0 + rbase + 8 * u, idx = i * H + j;
+            T* __restrict__ dg = p.lstm_dG + i * 4 * H;
+            const T dh = dhl[u] + stage[(rbase + 8 * u) * LDT + cc];
+            const T d_o = dh * tc[u];
+            T dc = (dh * o_[u]) * act_derivative<T>(ACT_TANH, tc[u], (T)0);
+            if (p.lstm_dc_in != nullptr) dc = dc + dci[u];
+            const T d_i = dc * g_[u], d_g = dc * i_[u], d_f = dc * cp[u];
+            p.lstm_dc_prev[idx] = dc * f_[u];
+            dg[j] = d_i * act_derivative<T>(ACT_SIGMOID, i_[u], (T)0);
+            dg[H + j] = d_f * act_derivative<T>(ACT_SIGMOID, f_[u], (T)0);
+            dg[2 * H + j] = d_g * act_derivative<T>(ACT_TANH, g_[u], (T)0);
+            dg[3 * H + j] = d_o * act_derivative<T>(ACT_SIGMOID, o_[u], (T)0);
+        }
+        return;
+    }
+
     T* __restrict__ C = p.C + batch * p.strideC +
                         ((p.ksplit > 0 && p.split_counters == nullptr) ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
@@ -582,8 +671,9 @@ int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size)
     if (tiles >= 192) return 1;
     const int64_t bk = (elem_size == 8 ? Slab<double, 1>::BK : Slab<float, 1>::BK);
     if ((K + bk - 1) / bk < split_min_slabs()) return 1;
+    static const int max_splits = [] { const char* e = getenv("PRAD_GEMM_SPLIT_MAX"); const int x = e ? atoi(e) : 0; return x > 0 ? x : 32; }();
     int64_t s = 512 / tiles;
-    if (s > 32) s = 32;
+    if (s > max_splits) s = max_splits;
     if (s > K / (2 * bk)) s = K / (2 * bk);  // at least two slabs per split
     if (s < 2) return 1;
     const int64_t ksplit = ((K + s - 1) / s + bk - 1) / bk * bk;
@@ -698,6 +788,58 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
     }
 }
 
+template <typename T>
+static bool lstm_operands_aligned(const GemmArgs<T>& a) {
+    constexpr int VEC = Mfma<T>::VEC;
+    return a.lda % VEC == 0 && a.ldb % VEC == 0 && reinterpret_cast<uintptr_t>(a.A) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(a.B) % 16 == 0 && a.lda < (1 << 23) && a.ldb < (1 << 23) && a.batch == 1;
+}
+
+template <typename T>
+hipError_t launch_lstm_step_fwd(const GemmArgs<T>& a_in, hipStream_t stream) {
+    GemmArgs<T> a = a_in;
+    const int64_t H = a.lstm_hidden;
+    constexpr int64_t bk = Slab<T, 1>::BK;
+    // M x 4H = (M x H) . (H x 4H); whole slabs of K (the gather has no guarded tail) and whole groups of 8 units
+    if (a.M <= 0 || H <= 0) return hipSuccess;
+    if (a.transA || a.transB || a.K != H || a.N != 4 * H || H % bk != 0 || H % 8 != 0 || !lstm_operands_aligned(a) ||
+        (a.M + 31) / 32 * (H / 8) > 0x7fffffffLL)
+        return hipErrorNotSupported;
+    a.ksplit = 0; a.zstrideA = 0; a.zstrideB = 0; a.split_counters = nullptr; a.colsum_dst = nullptr; a.nseg = 0;
+    const int tilesM = (int)((a.M + 31) / 32), tilesN = (int)(H / 8);
+    hipLaunchKernelGGL((gemm_kernel<T, 1, true, false, false, EPI_LSTM_FWD>), dim3((unsigned)(tilesM * tilesN)), dim3(GEMM_THREADS), 0,
+                       stream, a, tilesM, tilesN);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_lstm_step_bwd(const GemmArgs<T>& a_in, hipStream_t stream) {
+    GemmArgs<T> a = a_in;
+    const int64_t H = a.lstm_hidden;
+    if (a.M <= 0 || H <= 0) return hipSuccess;
+    if (a.transA || !a.transB || a.N != H || a.K != 4 * H || !lstm_operands_aligned(a)) return hipErrorNotSupported;
+    a.ksplit = 0; a.zstrideA = 0; a.zstrideB = 0; a.colsum_dst = nullptr; a.nseg = 0;
+    const int tilesM = (int)((a.M + 31) / 32), tilesN = (int)((H + 31) / 32);
+    const int splits = (a.split_ws != nullptr && a.split_counters != nullptr && (int64_t)tilesM * tilesN <= GEMM_SPLIT_MAX_TILES)
+                           ? gemm_split_factor(a.M, a.N, a.K, 1, (int)sizeof(T)) : 1;
+    if (splits > 1) {
+        constexpr int64_t bk = Slab<T, 1>::BK;
+        a.ksplit = ((a.K + splits - 1) / splits + bk - 1) / bk * bk;
+        a.zstrideA = a.ksplit;   // A stored [m][k]
+        a.zstrideB = a.ksplit;   // B stored [n][k]
+    } else {
+        a.split_counters = nullptr;
+    }
+    const unsigned gz = a.ksplit > 0 ? (unsigned)((a.K + a.ksplit - 1) / a.ksplit) : 1u;
+    hipLaunchKernelGGL((gemm_kernel<T, 1, true, true, false, EPI_LSTM_BWD>), dim3((unsigned)(tilesM * tilesN), 1, gz),
+                       dim3(GEMM_THREADS), 0, stream, a, tilesM, tilesN);
+    return hipGetLastError();
+}
+
+template hipError_t launch_lstm_step_fwd<double>(const GemmArgs<double>&, hipStream_t);
+template hipError_t launch_lstm_step_fwd<float>(const GemmArgs<float>&, hipStream_t);
+template hipError_t launch_lstm_step_bwd<double>(const GemmArgs<double>&, hipStream_t);
+template hipError_t launch_lstm_step_bwd<float>(const GemmArgs<float>&, hipStream_t);
 template hipError_t launch_gemm<double>(const GemmArgs<double>&, hipStream_t);
 template hipError_t launch_gemm<float>(const GemmArgs<float>&, hipStream_t);
 

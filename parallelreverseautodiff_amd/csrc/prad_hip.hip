@@ -269,6 +269,46 @@ int32_t batch_sum_fwd_t(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_buf_t 
     return PRAD_OK;
 }
 
+// One LSTM time step in one launch each way; shapes the fused kernels do not take run as product + cell kernel.
+template <typename T>
+int32_t lstm_step_fwd_t(prad_buf_t h_prev, prad_buf_t Wh, prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_buf_t tanh_c,
+                        prad_buf_t h) {
+    const int64_t rows = c->rows, H = c->cols;
+    GemmArgs<T> a = plain_gemm<T>(0, 0, rows, 4 * H, H, h_prev->ptr, H, Wh->ptr, 4 * H, G->ptr, 4 * H, 1);
+    a.lstm_hidden = H;
+    a.lstm_c_prev = static_cast<const T*>(c_prev->ptr);
+    a.lstm_c = static_cast<T*>(c->ptr); a.lstm_tanh_c = static_cast<T*>(tanh_c->ptr); a.lstm_h = static_cast<T*>(h->ptr);
+    hipError_t e = launch_lstm_step_fwd<T>(a, CUR_STREAM);
+    if (e == hipErrorNotSupported) {
+        if (int32_t st = attach_split_workspace(a)) return st;
+        HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);
+        e = launch_lstm_cell_fwd<T>(static_cast<T*>(G->ptr), a.lstm_c_prev, a.lstm_c, a.lstm_tanh_c, a.lstm_h, rows, H, CUR_STREAM);
+    }
+    HIP_TRY(e, PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+template <typename T>
+int32_t lstm_step_bwd_t(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_c,
+                        prad_buf_t dh_loss, prad_buf_t dc_in, prad_buf_t dG, prad_buf_t dc_prev, prad_buf_t dh_scratch) {
+    const int64_t rows = c_prev->rows, H = c_prev->cols;
+    GemmArgs<T> a = plain_gemm<T>(0, 1, rows, H, 4 * H, dG_next->ptr, 4 * H, Wh->ptr, 4 * H, dh_scratch->ptr, H, 0);
+    if (int32_t st = attach_split_workspace(a)) return st;
+    a.lstm_hidden = H;
+    a.lstm_gates = static_cast<const T*>(gates->ptr); a.lstm_c_prev = static_cast<const T*>(c_prev->ptr);
+    a.lstm_tanh_c_in = static_cast<const T*>(tanh_c->ptr); a.lstm_dh_loss = static_cast<const T*>(dh_loss->ptr);
+    a.lstm_dc_in = dc_in ? static_cast<const T*>(dc_in->ptr) : nullptr;
+    a.lstm_dG = static_cast<T*>(dG->ptr); a.lstm_dc_prev = static_cast<T*>(dc_prev->ptr);
+    hipError_t e = launch_lstm_step_bwd<T>(a, CUR_STREAM);
+    if (e == hipErrorNotSupported) {
+        HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);  // dh_scratch = dG_next . Wh^T
+        e = launch_lstm_cell_bwd<T>(a.lstm_gates, a.lstm_c_prev, a.lstm_tanh_c_in, a.lstm_dh_loss, static_cast<const T*>(dh_scratch->ptr),
+                                    a.lstm_dc_in, a.lstm_dG, a.lstm_dc_prev, rows, H, CUR_STREAM);
+    }
+    HIP_TRY(e, PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
 int32_t same_shape(prad_buf_t a, prad_buf_t b, const char* what) {
     if (a->depth != b->depth || a->rows != b->rows || a->cols != b->cols)
         return fail(PRAD_ERR_ARG, "%s: Matrices must have the same dimensions.", what);
@@ -1117,6 +1157,44 @@ int32_t prad_lstm_cell_bwd(prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_
              launch_lstm_cell_bwd<float>(F(gates), F(c_prev), F(tanh_c), F(dh_a), dh_b ? F(dh_b) : nullptr, dc_in ? F(dc_in) : nullptr,
                                          F(dG), F(dc_prev), rows, hidden, CUR_STREAM));
     return PRAD_OK;
+}
+
+int32_t prad_lstm_step_fwd(prad_buf_t h_prev, prad_buf_t Wh, prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_buf_t tanh_c,
+                           prad_buf_t h) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(h_prev); REQUIRE_BUF(Wh); REQUIRE_BUF(G); REQUIRE_BUF(c_prev); REQUIRE_BUF(c); REQUIRE_BUF(tanh_c); REQUIRE_BUF(h);
+    if (int32_t st = same_dtype({h_prev, Wh, G, c_prev, c, tanh_c, h})) return st;
+    const int64_t rows = c->rows, hidden = c->cols;
+    if (G->depth != 1 || c->depth != 1 || G->rows != rows || G->cols != 4 * hidden)
+        return fail(PRAD_ERR_ARG, "gate pre-activations must be rows x 4*hidden");
+    if (Wh->depth != 1 || Wh->rows != hidden || Wh->cols != 4 * hidden) return fail(PRAD_ERR_SHAPE, "recurrent weight must be hidden x 4*hidden");
+    for (prad_buf_t o : {h_prev, c_prev, tanh_c, h})
+        if (int32_t st = same_shape(c, o, "LSTM step")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return G->dtype == PRAD_F64 ? lstm_step_fwd_t<double>(h_prev, Wh, G, c_prev, c, tanh_c, h)
+                                : lstm_step_fwd_t<float>(h_prev, Wh, G, c_prev, c, tanh_c, h);
+}
+
+int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_c,
+                           prad_buf_t dh_loss, prad_buf_t dc_in, prad_buf_t dG, prad_buf_t dc_prev, prad_buf_t dh_scratch) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(dG_next); REQUIRE_BUF(Wh); REQUIRE_BUF(gates); REQUIRE_BUF(c_prev); REQUIRE_BUF(tanh_c); REQUIRE_BUF(dh_loss);
+    REQUIRE_BUF(dG); REQUIRE_BUF(dc_prev); REQUIRE_BUF(dh_scratch);
+    if (dc_in != nullptr) REQUIRE_BUF(dc_in);
+    if (int32_t st = same_dtype({dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch})) return st;
+    const int64_t rows = c_prev->rows, hidden = c_prev->cols;
+    if (gates->rows != rows || gates->cols != 4 * hidden || c_prev->depth != 1 || gates->depth != 1)
+        return fail(PRAD_ERR_ARG, "gates must be rows x 4*hidden");
+    if (Wh->depth != 1 || Wh->rows != hidden || Wh->cols != 4 * hidden) return fail(PRAD_ERR_SHAPE, "recurrent weight must be hidden x 4*hidden");
+    for (prad_buf_t o : {dG_next, dG})
+        if (int32_t st = same_shape(gates, o, "LSTM step backward")) return st;
+    for (prad_buf_t o : {tanh_c, dh_loss, dc_in, dc_prev, dh_scratch})
+        if (o != nullptr)
+            if (int32_t st = same_shape(c_prev, o, "LSTM step backward")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return gates->dtype == PRAD_F64
+               ? lstm_step_bwd_t<double>(dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch)
+               : lstm_step_bwd_t<float>(dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch);
 }
 
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out) {

@@ -27,7 +27,7 @@ from .optim import NeuralNetworkParameters
 
 class LSTMLayer:
     def __init__(self, input_dim=256, hidden=512, batch=128, steps=64, dtype=np.float32, seed=seeded.DEFAULT_SEED,
-                 parameters=None):
+                 parameters=None, fused=True):
         _ensure_initialized()
         self.lib = _lib.load()
         self.dtype = np.dtype(dtype)
@@ -67,11 +67,16 @@ class LSTMLayer:
         self.H_out = self.Hs.view_rows(B, T * B)
         self.iteration = 0
         self._graph = None
+        self.fused = fused   # one launch per time step each way (cell arithmetic as the recurrent product's epilogue)
 
     def _enqueue_forward_backward(self):
         lib, T = self.lib, self.steps
         check(lib.prad_matmul_fwd_fused(self.X.handle, self.Wx.handle, self.b.handle, None, self.G.handle, _lib.ACT_NONE, 0.0))
         for t in range(T):
+            if self.fused:
+                check(lib.prad_lstm_step_fwd(self.H_t[t].handle, self.Wh.handle, self.G_t[t].handle, self.C_t[t].handle,
+                                             self.C_t[t + 1].handle, self.TC_t[t].handle, self.H_t[t + 1].handle))
+                continue
             check(lib.prad_gemm(0, 0, self.H_t[t].handle, self.Wh.handle, self.G_t[t].handle, 1))  # G_t += h_{t-1} . W_h
             check(lib.prad_lstm_cell_fwd(self.G_t[t].handle, self.C_t[t].handle, self.C_t[t + 1].handle, self.TC_t[t].handle,
                                          self.H_t[t + 1].handle))
@@ -80,11 +85,20 @@ class LSTMLayer:
         for t in range(T - 1, -1, -1):
             last = t == T - 1
             rec, dc_in, dc_out = self.dh[t % 2], self.dc[t % 2], self.dc[(t + 1) % 2]
+            if self.fused and not last:
+                # dh_t = dHl_t + dG_{t+1} . W_h^T and the cell's backward in one launch
+                check(lib.prad_lstm_step_bwd(self.dG_t[t + 1].handle, self.Wh.handle, self.G_t[t].handle, self.C_t[t].handle,
+                                             self.TC_t[t].handle, self.dHl_t[t].handle, dc_in.handle, self.dG_t[t].handle,
+                                             dc_out.handle, rec.handle))
+                continue
             check(lib.prad_lstm_cell_bwd(self.G_t[t].handle, self.C_t[t].handle, self.TC_t[t].handle, self.dHl_t[t].handle,
                                          None if last else rec.handle, None if last else dc_in.handle,
                                          self.dG_t[t].handle, dc_out.handle))
-            # dh_{t-1} = dG_t . W_h^T (formed for t = 0 too: MatrixMultiplyOperation.Backward always returns both gradients)
-            check(lib.prad_gemm(0, 1, self.dG_t[t].handle, self.Wh.handle, self.dh[(t + 1) % 2].handle, 0))
+            if not self.fused:
+                # dh_{t-1} = dG_t . W_h^T (formed for t = 0 too: MatrixMultiplyOperation.Backward always returns both gradients)
+                check(lib.prad_gemm(0, 1, self.dG_t[t].handle, self.Wh.handle, self.dh[(t + 1) % 2].handle, 0))
+        if self.fused:
+            check(lib.prad_gemm(0, 1, self.dG_t[0].handle, self.Wh.handle, self.dh[1].handle, 0))   # dh_{-1}, as above
         check(lib.prad_gemm(1, 0, self.X.handle, self.dG.handle, self.dWx.handle, 0))
         check(lib.prad_gemm(1, 0, self.H_prev_all.handle, self.dG.handle, self.dWh.handle, 0))
         check(lib.prad_add_broadcast_bwd_bias(self.dG.handle, self.db.handle))

@@ -38,3 +38,18 @@ def test_lstm_recorded_step_equals_eager(gpu):
         for x, y in ((a.W, b.W), (a.b, b.b), (a.dW, b.dW), (a.mW, b.mW), (a.vW, b.vW), (a.loss, b.loss)):
             assert np.array_equal(x.download(), y.download())
     b.release()
+
+
+@pytest.mark.parametrize("dtype,cfg", [(np.float64, (24, 64, 40, 5)), (np.float64, (16, 128, 32, 4)), (np.float32, (32, 128, 40, 5)),
+                                       (np.float32, (256, 512, 128, 3)), (np.float32, (16, 32, 8, 4))])
+def test_one_launch_per_time_step_equals_product_plus_cell_kernels(gpu, dtype, cfg):
+    """The recurrent product with the cell arithmetic as its epilogue (forward: gate columns gathered per tile;
+    backward: on the product split along K) gives the bits of the product followed by the cell kernel; row counts
+    that do not fill the tiles and a hidden size that takes the two-launch path (32) included."""
+    I, H, B, T = cfg
+    a, b = LSTMLayer(I, H, B, T, dtype=dtype, fused=True), LSTMLayer(I, H, B, T, dtype=dtype, fused=False)
+    for step in range(2):
+        a.step(); b.step()
+        for name in ("G", "C", "Hs", "TC", "dG", "dX", "dW", "db", "W", "b", "loss"):
+            assert np.array_equal(getattr(a, name).download(), getattr(b, name).download()), (name, step)
+        assert np.array_equal(a.dh[1].download(), b.dh[1].download())
