@@ -259,6 +259,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     auto compute = [&](const T* __restrict__ st) {
         const T* __restrict__ sA = st;
         const T* __restrict__ sB = st + SA;
+        // While a wavefront multiplies it outranks its SIMD's other wavefront (which is then loading or waiting at a
+        // barrier) at instruction issue: measured +2.3 % at N = 4096 in double.
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int s = 0; s < BK / 4; ++s) {
             const int k = 4 * s + g;
@@ -272,6 +275,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
 #pragma unroll
                 for (int y = 0; y < WTN; ++y) acc[x][y] = MF::run(a[x], b[y], acc[x][y]);
         }
+        __builtin_amdgcn_s_setprio(0);
     };
 
     if (!EDGE) {
