@@ -248,7 +248,7 @@ hipError_t launch_add_broadcast_fwd(const T* x, const T* bias, T* y, int64_t row
 // wavefronts take rows i = w, w+4, w+8, ... with four independent loads in flight each, and the four
 // partial sums are added in wavefront order, so the result does not depend on timing.  Neighbouring
 // lanes read neighbouring columns: every row is one coalesced read.  Tall matrices (a whole sequence of
-// gate gradients) are cut into up to 64 row chunks whose partial sums a second kernel adds in chunk order.
+// gate gradients) are cut into row chunks whose partial sums a second pass adds (see colsum_chunks).
 // Rows [blockIdx.y * rows_per_chunk, ...) of 64 columns; out is db itself (one chunk) or a row of partial sums.
 template <typename T, typename OUT>
 __global__ void __launch_bounds__(256) colsum_kernel(const T* __restrict__ dy, OUT* __restrict__ out, int64_t rows, int64_t cols,
@@ -258,15 +258,13 @@ __global__ void __launch_bounds__(256) colsum_kernel(const T* __restrict__ dy, O
     __shared__ double part[4 * 64];
     colsum_block<T, OUT>(dy, out + (int64_t)blockIdx.y * cols, cols, r0, r1, blockIdx.x, part);
 }
-template <typename T>
-__global__ void __launch_bounds__(64) colsum_final_kernel(const double* __restrict__ partial, T* __restrict__ db, int chunks, int64_t cols) {
-    const int64_t j = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (j >= cols) return;
-    double s = 0.0;
-    for (int c = 0; c < chunks; ++c) s += partial[(int64_t)c * cols + j];
-    db[j] = (T)s;
+// Tall matrices are summed in row chunks of at least 64 rows (up to 256 chunks, so that the first stage fills the
+// chip); the chunk sums, a chunks x cols matrix of doubles, are then summed by the same kernel.
+int colsum_chunks(int64_t rows) {
+    if (rows < COLSUM_CHUNK_ROWS) return 1;
+    const int64_t c = rows / 64;
+    return (int)(c > 256 ? 256 : c);
 }
-int colsum_chunks(int64_t rows) { return rows >= COLSUM_CHUNK_ROWS ? (int)((rows + 255) / 256 > 64 ? 64 : (rows + 255) / 256) : 1; }
 // workspace: colsum_chunks(rows) * cols doubles when colsum_chunks(rows) > 1.
 template <typename T>
 hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double* workspace, hipStream_t s) {
@@ -278,7 +276,8 @@ hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double*
     } else {
         const int64_t per = (rows + chunks - 1) / chunks;
         hipLaunchKernelGGL((colsum_kernel<T, double>), dim3(gx, (unsigned)chunks), dim3(256), 0, s, dy, workspace, rows, cols, per);
-        hipLaunchKernelGGL((colsum_final_kernel<T>), dim3(gx), dim3(64), 0, s, workspace, db, chunks, cols);
+        hipLaunchKernelGGL((colsum_kernel<double, T>), dim3(gx, 1), dim3(256), 0, s, workspace, db, (int64_t)chunks, cols,
+                           (int64_t)chunks);
     }
     return hipGetLastError();
 }

@@ -537,12 +537,30 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         constexpr int LDW = WS + 4;
         __syncthreads();  // every wavefront is done with the slab stages
         T* __restrict__ stage = &smem[0][0] + wave * (16 * LDW);
+        T* __restrict__ side = &smem[0][0] + (4 + wave) * (16 * LDW);  // the values act' is taken of, fetched ahead
+        static_assert(8 * 16 * LDW <= 2 * (SA + SB), "both staging areas fit into the slab stages");
 #pragma unroll
         for (int x = 0; x < WTM; ++x) {
 #pragma unroll
             for (int y = 0; y < WTN; ++y)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) stage[MF::row(r, g) * LDW + y * 16 + li] = acc[x][y][r];
+            if (p.act_bwd != ACT_NONE) {
+                // All loads of this pass are issued together (one memory latency instead of one per iteration of
+                // the loop below); each lane parks what it will need in LDS at the position it reads back itself.
+                T src[16 * WS / 64];
+#pragma unroll
+                for (int it = 0; it < 16 * WS / 64; ++it) {
+                    const int idx = lane + 64 * it, rr = idx / WS, c = idx % WS;
+                    const int64_t i = row0 + wm * WS + x * 16 + rr, j = col0 + wn * WS + c;
+                    src[it] = (i < p.M && j < p.N) ? p.act_src[i * p.ld_act + j] : (T)0;
+                }
+#pragma unroll
+                for (int it = 0; it < 16 * WS / 64; ++it) {
+                    const int idx = lane + 64 * it;
+                    side[(idx / WS) * LDW + idx % WS] = src[it];
+                }
+            }
             __syncthreads();
 #pragma unroll 1
             for (int idx = lane; idx < 16 * WS; idx += 64) {
@@ -554,7 +572,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
                 if (p.bias != nullptr) v = v + p.bias[j];
                 if (p.Z != nullptr) p.Z[i * p.ldz + j] = v;
                 if (p.act_fwd != ACT_NONE) v = act_forward<T>(p.act_fwd, v, p.alpha);
-                if (p.act_bwd != ACT_NONE) v = v * act_derivative<T>(p.act_bwd, p.act_src[i * p.ld_act + j], p.alpha);
+                if (p.act_bwd != ACT_NONE) v = v * act_derivative<T>(p.act_bwd, side[rr * LDW + c], p.alpha);
                 T* c_out = C + i * p.ldc + j;
                 if (p.accumulate) v = *c_out + v;
                 *c_out = v;

@@ -37,6 +37,32 @@ __global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x
     for (int64_t j = threadIdx.x; j < cols; j += 64) yr[j] = yr[j] / s;
 }
 
+// Rows of at most 64 columns (attention windows: 49): a lane holds one element, the row is read once and written
+// once, four rows per workgroup.  Same arithmetic as softmax_fwd_kernel (which re-reads y for the division).
+template <typename T>
+__global__ void __launch_bounds__(256) softmax_fwd_short_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols) {
+    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const bool on = lane < cols;
+    const T xv = on ? x[i * cols + lane] : (T)0;
+    const T m = (T)wave_max(on ? (double)xv : -INFINITY);
+    const T e = on ? dev_exp(xv - m) : (T)0;
+    const T s = (T)wave_sum(on ? (double)e : 0.0);
+    if (on) y[i * cols + lane] = e / s;
+}
+template <typename T>
+__global__ void __launch_bounds__(256) softmax_bwd_short_kernel(const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx,
+                                                                int64_t rows, int64_t cols) {
+    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const bool on = lane < cols;
+    const T yv = on ? y[i * cols + lane] : (T)0, gv = on ? dy[i * cols + lane] : (T)0;
+    const double dot = wave_sum(on ? (double)gv * (double)yv : 0.0);
+    if (on) dx[i * cols + lane] = (T)((double)yv * ((double)gv - dot));
+}
+
 // The reference multiplies dy with the explicit Jacobian row by row (O(cols^2)):
 //   dx[j] = dy[j]*y[j]*(1-y[j]) - sum_{k != j} dy[k]*y[j]*y[k]  =  y[j] * (dy[j] - sum_k dy[k]*y[k]).
 template <typename T>
@@ -195,12 +221,20 @@ hipError_t launch_mse_bwd(const T* y, const T* t, T* dy, int64_t n, hipStream_t 
 template <typename T>
 hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
+    if (cols <= 64) {
+        hipLaunchKernelGGL((softmax_fwd_short_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, x, y, rows, cols);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL((softmax_fwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, x, y, rows, cols);
     return hipGetLastError();
 }
 template <typename T>
 hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
+    if (cols <= 64) {
+        hipLaunchKernelGGL((softmax_bwd_short_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, y, dy, dx, rows, cols);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, y, dy, dx, rows, cols);
     return hipGetLastError();
 }
