@@ -539,6 +539,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         T* __restrict__ stage = &smem[0][0] + wave * (16 * LDW);
         T* __restrict__ side = &smem[0][0] + (4 + wave) * (16 * LDW);  // the values act' is taken of, fetched ahead
         static_assert(8 * 16 * LDW <= 2 * (SA + SB), "both staging areas fit into the slab stages");
+        constexpr int VEC = MF::VEC;
+        auto vec_aligned = [](const void* q, int64_t ld) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) % 16 == 0 && ld % VEC == 0); };
+        const bool vec_ok = p.N % VEC == 0 && vec_aligned(C, p.ldc) && vec_aligned(p.Z, p.ldz) && vec_aligned(p.act_src, p.ld_act) &&
+                            vec_aligned(p.bias, VEC);
 #pragma unroll
         for (int x = 0; x < WTM; ++x) {
 #pragma unroll
@@ -562,6 +566,41 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
                 }
             }
             __syncthreads();
+            if (vec_ok) {
+                // 16 bytes per lane and access: whole rows of the tile leave in 1 KiB pieces.
+#pragma unroll 1
+                for (int idx = lane; idx < 16 * WS / VEC; idx += 64) {
+                    const int rr = idx / (WS / VEC), c = (idx % (WS / VEC)) * VEC;
+                    const int64_t i = row0 + wm * WS + x * 16 + rr;
+                    const int64_t j = col0 + wn * WS + c;
+                    if (i >= p.M || j >= p.N) continue;  // N is a multiple of VEC here: a vector is inside or outside
+                    Vec v = *reinterpret_cast<const Vec*>(stage + rr * LDW + c);
+                    if (p.bias != nullptr) {
+                        const Vec b = *reinterpret_cast<const Vec*>(p.bias + j);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) v[e] = v[e] + b[e];
+                    }
+                    if (p.Z != nullptr) *reinterpret_cast<Vec*>(p.Z + i * p.ldz + j) = v;
+                    if (p.act_fwd != ACT_NONE) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) v[e] = act_forward<T>(p.act_fwd, v[e], p.alpha);
+                    }
+                    if (p.act_bwd != ACT_NONE) {
+                        const Vec sv = *reinterpret_cast<const Vec*>(side + rr * LDW + c);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) v[e] = v[e] * act_derivative<T>(p.act_bwd, sv[e], p.alpha);
+                    }
+                    Vec* c_out = reinterpret_cast<Vec*>(C + i * p.ldc + j);
+                    if (p.accumulate) {
+                        const Vec old = *c_out;
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) v[e] = old[e] + v[e];
+                    }
+                    *c_out = v;
+                }
+                __syncthreads();
+                continue;
+            }
 #pragma unroll 1
             for (int idx = lane; idx < 16 * WS; idx += 64) {
                 const int rr = idx / WS, c = idx % WS;
