@@ -130,6 +130,16 @@ int32_t prad_gemm_strided_batched_f64(int32_t transA, int32_t transB, int64_t M,
 int32_t prad_gemm_strided_batched_f32(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const float* A,
                                       int64_t lda, int64_t strideA, const float* B, int64_t ldb, int64_t strideB, float* C,
                                       int64_t ldc, int64_t strideC, int32_t batch, int32_t accumulate);
+/* Two-level batches (attention: windows x heads) in one launch: product (o, i), o < batch_outer, i < batch_inner,
+ * takes its operand blocks at o * stride + i * istride elements from the base pointers. */
+int32_t prad_gemm_strided_batched_2d_f64(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const double* A,
+                                         int64_t lda, int64_t strideA, int64_t istrideA, const double* B, int64_t ldb,
+                                         int64_t strideB, int64_t istrideB, double* C, int64_t ldc, int64_t strideC,
+                                         int64_t istrideC, int32_t batch_outer, int32_t batch_inner, int32_t accumulate);
+int32_t prad_gemm_strided_batched_2d_f32(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const float* A,
+                                         int64_t lda, int64_t strideA, int64_t istrideA, const float* B, int64_t ldb,
+                                         int64_t strideB, int64_t istrideB, float* C, int64_t ldc, int64_t strideC,
+                                         int64_t istrideC, int32_t batch_outer, int32_t batch_inner, int32_t accumulate);
 
 /* One-shot host-pointer forms with today's call-per-operation behaviour of
  * GpuMatrixMultiplyOperation.Forward/Backward (src/RMAD/GpuMatrixMultiplyOperation.cs:113-161):

@@ -67,6 +67,8 @@ SIGNATURES = {
     "prad_gemm_f32": (_i32, [_i32, _i32, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i32]),
     "prad_gemm_strided_batched_f64": (_i32, [_i32, _i32, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32]),
     "prad_gemm_strided_batched_f32": (_i32, [_i32, _i32, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32]),
+    "prad_gemm_strided_batched_2d_f64": (_i32, [_i32, _i32, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i32, _i32, _i32]),
+    "prad_gemm_strided_batched_2d_f32": (_i32, [_i32, _i32, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i32, _i32, _i32]),
     "prad_scale": (_i32, [_vp, _vp, _f64]),
     "prad_matmul_fwd_host": (_i32, [_i32, _vpp, _vpp, _vpp, _i64, _i64, _i64, _i64]),
     "prad_matmul_bwd_host": (_i32, [_i32, _vpp, _vpp, _vpp, _vpp, _vpp, _i64, _i64, _i64]),

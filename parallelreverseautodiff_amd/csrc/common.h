@@ -141,6 +141,10 @@ struct GemmArgs {
     T alpha;
     int batch;
     int64_t strideA, strideB, strideC;
+    // Two-level batches (windows x heads): with batch_inner > 1, product b takes operand blocks at
+    // (b / batch_inner) * stride + (b % batch_inner) * istride.
+    int batch_inner;
+    int64_t istrideA, istrideB, istrideC;
     // When set, C is not written: each workgroup stores the sum of its finished tile to
     // tile_sums[batch_index * tiles_per_product + tile_index] (MatrixMultiplyAndSum forward).
     double* tile_sums;

@@ -227,8 +227,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     tile_of_workgroup(blockIdx.x, tilesM, tilesN, tm, tn);
     const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
     const int batch = blockIdx.y;
-    const T* __restrict__ A = p.A + batch * p.strideA;
-    const T* __restrict__ B = p.B + batch * p.strideB;
+    const int b_outer = p.batch_inner > 1 ? batch / p.batch_inner : batch;
+    const int b_inner = p.batch_inner > 1 ? batch - b_outer * p.batch_inner : 0;
+    const T* __restrict__ A = p.A + b_outer * p.strideA + b_inner * p.istrideA;
+    const T* __restrict__ B = p.B + b_outer * p.strideB + b_inner * p.istrideB;
     // A product split along K: this workgroup reduces [kb, kb + K) and writes its own M x N partial result.
     int64_t K = p.K;
     if (p.ksplit > 0) {
@@ -528,7 +530,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         return;
     }
 
-    T* __restrict__ C = p.C + batch * p.strideC +
+    T* __restrict__ C = p.C + b_outer * p.strideC + b_inner * p.istrideC +
                         ((p.ksplit > 0 && p.split_counters == nullptr) ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
         // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
@@ -672,7 +674,7 @@ static hipError_t launch_tile(const GemmArgs<T>& a, int epi, hipStream_t stream)
     const bool aligned = (whole || epi != EPI_TILE_SUM) && a.K > 0 && (a.lda % VEC == 0) &&
                          (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
-                         (a.zstrideA % VEC == 0) && (a.zstrideB % VEC == 0) &&
+                         (a.zstrideA % VEC == 0) && (a.zstrideB % VEC == 0) && (a.istrideA % VEC == 0) && (a.istrideB % VEC == 0) &&
                          // per-thread element offsets inside one tile's slab are kept in 32 bits
                          (a.lda < (1 << 23)) && (a.ldb < (1 << 23));
     // Grid y carries the batch; the tile count must fit the 1-D grid.
@@ -809,7 +811,12 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         hipLaunchKernelGGL((split_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, a, a.split_ws, a.nseg);
         return hipGetLastError();
     }
-    const int splits = (a.split_ws != nullptr && epi != EPI_TILE_SUM) ? gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T)) : 1;
+    int splits = (a.split_ws != nullptr && epi != EPI_TILE_SUM) ? gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T)) : 1;
+    {
+        // the two-pass reduction addresses C with one batch stride
+        const int64_t tiles = ((a.M + 31) / 32) * ((a.N + 31) / 32) * a.batch;
+        if (a.batch_inner > 1 && !(a.split_counters != nullptr && tiles <= GEMM_SPLIT_MAX_TILES)) splits = 1;
+    }
     if (splits > 1) {
         constexpr int64_t bk = Slab<T, 1>::BK;
         const int64_t tiles = ((a.M + 31) / 32) * ((a.N + 31) / 32) * a.batch;

@@ -37,30 +37,46 @@ __global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x
     for (int64_t j = threadIdx.x; j < cols; j += 64) yr[j] = yr[j] / s;
 }
 
-// Rows of at most 64 columns (attention windows: 49): a lane holds one element, the row is read once and written
-// once, four rows per workgroup.  Same arithmetic as softmax_fwd_kernel (which re-reads y for the division).
+// Rows of at most 64 columns (attention windows: 49): a lane holds one element of each of SHORT_ROWS consecutive
+// rows, whose loads are all issued before the first reduction (a row is under 256 bytes: one row per wavefront
+// leaves the memory system idle).  Each row is read once and written once.  Same arithmetic as softmax_fwd_kernel.
+constexpr int SHORT_ROWS = 8;
 template <typename T>
 __global__ void __launch_bounds__(256) softmax_fwd_short_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols) {
-    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (i >= rows) return;
+    const int64_t i0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * SHORT_ROWS;
     const int lane = threadIdx.x & 63;
     const bool on = lane < cols;
-    const T xv = on ? x[i * cols + lane] : (T)0;
-    const T m = (T)wave_max(on ? (double)xv : -INFINITY);
-    const T e = on ? dev_exp(xv - m) : (T)0;
-    const T s = (T)wave_sum(on ? (double)e : 0.0);
-    if (on) y[i * cols + lane] = e / s;
+    T xv[SHORT_ROWS];
+#pragma unroll
+    for (int r = 0; r < SHORT_ROWS; ++r) xv[r] = (on && i0 + r < rows) ? x[(i0 + r) * cols + lane] : (T)0;
+#pragma unroll
+    for (int r = 0; r < SHORT_ROWS; ++r) {
+        if (i0 + r >= rows) break;
+        const T m = (T)wave_max(on ? (double)xv[r] : -INFINITY);
+        const T e = on ? dev_exp(xv[r] - m) : (T)0;
+        const T s = (T)wave_sum(on ? (double)e : 0.0);
+        if (on) y[(i0 + r) * cols + lane] = e / s;
+    }
 }
 template <typename T>
 __global__ void __launch_bounds__(256) softmax_bwd_short_kernel(const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx,
                                                                 int64_t rows, int64_t cols) {
-    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (i >= rows) return;
+    const int64_t i0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * SHORT_ROWS;
     const int lane = threadIdx.x & 63;
     const bool on = lane < cols;
-    const T yv = on ? y[i * cols + lane] : (T)0, gv = on ? dy[i * cols + lane] : (T)0;
-    const double dot = wave_sum(on ? (double)gv * (double)yv : 0.0);
-    if (on) dx[i * cols + lane] = (T)((double)yv * ((double)gv - dot));
+    T yv[SHORT_ROWS], gv[SHORT_ROWS];
+#pragma unroll
+    for (int r = 0; r < SHORT_ROWS; ++r) {
+        const bool ok = on && i0 + r < rows;
+        yv[r] = ok ? y[(i0 + r) * cols + lane] : (T)0;
+        gv[r] = ok ? dy[(i0 + r) * cols + lane] : (T)0;
+    }
+#pragma unroll
+    for (int r = 0; r < SHORT_ROWS; ++r) {
+        if (i0 + r >= rows) break;
+        const double dot = wave_sum(on ? (double)gv[r] * (double)yv[r] : 0.0);
+        if (on) dx[(i0 + r) * cols + lane] = (T)((double)yv[r] * ((double)gv[r] - dot));
+    }
 }
 
 // The reference multiplies dy with the explicit Jacobian row by row (O(cols^2)):
@@ -222,7 +238,8 @@ template <typename T>
 hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
     if (cols <= 64) {
-        hipLaunchKernelGGL((softmax_fwd_short_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, x, y, rows, cols);
+        hipLaunchKernelGGL((softmax_fwd_short_kernel<T>), dim3((unsigned)((rows + 4 * SHORT_ROWS - 1) / (4 * SHORT_ROWS))), dim3(256), 0, s, x, y,
+                           rows, cols);
         return hipGetLastError();
     }
     hipLaunchKernelGGL((softmax_fwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, x, y, rows, cols);
@@ -232,7 +249,8 @@ template <typename T>
 hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
     if (cols <= 64) {
-        hipLaunchKernelGGL((softmax_bwd_short_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, y, dy, dx, rows, cols);
+        hipLaunchKernelGGL((softmax_bwd_short_kernel<T>), dim3((unsigned)((rows + 4 * SHORT_ROWS - 1) / (4 * SHORT_ROWS))), dim3(256), 0, s, y, dy,
+                           dx, rows, cols);
         return hipGetLastError();
     }
     hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, y, dy, dx, rows, cols);

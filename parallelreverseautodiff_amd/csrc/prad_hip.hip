@@ -726,6 +726,30 @@ RAW_GEMM(f32, float)
 RAW_BATCHED_GEMM(f64, double)
 RAW_BATCHED_GEMM(f32, float)
 
+#define RAW_BATCHED_GEMM_2D(SFX, T)                                                                                    \
+    int32_t prad_gemm_strided_batched_2d_##SFX(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K, const T* A, \
+                                               int64_t lda, int64_t strideA, int64_t istrideA, const T* B, int64_t ldb,  \
+                                               int64_t strideB, int64_t istrideB, T* C, int64_t ldc, int64_t strideC,    \
+                                               int64_t istrideC, int32_t batch_outer, int32_t batch_inner, int32_t accumulate) { \
+        REQUIRE_INIT();                                                                                                \
+        if (A == nullptr || B == nullptr || C == nullptr) return fail(PRAD_ERR_ARG, "NULL matrix pointer");            \
+        if (M < 0 || N < 0 || K < 0 || batch_outer < 0 || batch_inner < 1 || strideA < 0 || strideB < 0 || strideC < 0 || \
+            istrideA < 0 || istrideB < 0 || istrideC < 0)                                                              \
+            return fail(PRAD_ERR_ARG, "negative dimension");                                                           \
+        if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1) || (transA && transB))                        \
+            return fail(PRAD_ERR_ARG, "unsupported transpose combination (%d, %d)", transA, transB);                   \
+        if (lda < (transA ? M : K) || ldb < (transB ? K : N) || ldc < N) return fail(PRAD_ERR_ARG, "leading dimension too small"); \
+        if ((int64_t)batch_outer * batch_inner > 65535) return fail(PRAD_ERR_ARG, "at most 65535 products per call");  \
+        GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                    \
+        a.batch = batch_outer * batch_inner; a.strideA = strideA; a.strideB = strideB; a.strideC = strideC;            \
+        a.batch_inner = batch_inner; a.istrideA = istrideA; a.istrideB = istrideB; a.istrideC = istrideC;              \
+        std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                    \
+        HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);                                                     \
+        return PRAD_OK;                                                                                                \
+    }
+RAW_BATCHED_GEMM_2D(f64, double)
+RAW_BATCHED_GEMM_2D(f32, float)
+
 // ---------------------------------------------------------------------------------------------
 int32_t prad_matmul_fwd_host(int32_t dtype, const void* const* a_rows, const void* const* b_rows, void* const* c_rows, int64_t M,
                              int64_t K, int64_t K2, int64_t N) {

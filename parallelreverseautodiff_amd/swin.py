@@ -9,7 +9,8 @@ Tokens arrive window-major: rows [w*49, (w+1)*49) of X are the 7 x 7 tokens of w
   Y1 = O . Wo + bo ;  Y2 = GELU(Y1 . W1 + b1) . W2 + b2   (GELUOperation, with the reference's own derivative)
   loss = MSE(Y2, target)
 and the backward of every node in reverse order, then clip and Adam.  The 3 x windows small products of a kind
-are one strided-batched launch per head over the columns of the shared QKV / gradient matrices (no gather).
+are one launch over windows x heads (two-level strided batch over the columns of the shared QKV / gradient
+matrices, no gather).
 """
 import ctypes
 
@@ -64,14 +65,16 @@ class SwinBlock:
         self.scale = 1.0 / float(np.sqrt(self.hd))
         self.iteration = 0
         self._graph = None
-        self._batched = self.lib.prad_gemm_strided_batched_f64 if self.dtype == np.float64 else self.lib.prad_gemm_strided_batched_f32
+        self._batched = (self.lib.prad_gemm_strided_batched_2d_f64 if self.dtype == np.float64
+                         else self.lib.prad_gemm_strided_batched_2d_f32)
 
     def _ptr(self, buf, elem_offset):
         return ctypes.c_void_p(buf.ptr + elem_offset * self.dtype.itemsize)
 
-    def _per_head(self, tA, tB, M, N, K, A, a_off, lda, sA, B, b_off, ldb, sB, Cb, c_off, ldc, sC):
-        check(self._batched(tA, tB, M, N, K, self._ptr(A, a_off), lda, sA, self._ptr(B, b_off), ldb, sB,
-                            self._ptr(Cb, c_off), ldc, sC, self.nw, 0))
+    def _all_heads(self, tA, tB, M, N, K, A, a_off, lda, sA, hA, B, b_off, ldb, sB, hB, Cb, c_off, ldc, sC, hC):
+        """One launch over windows x heads: s* are the element strides between windows, h* between heads."""
+        check(self._batched(tA, tB, M, N, K, self._ptr(A, a_off), lda, sA, hA, self._ptr(B, b_off), ldb, sB, hB,
+                            self._ptr(Cb, c_off), ldc, sC, hC, self.nw, self.heads, 0))
 
     def _enqueue_forward_backward(self):
         lib, C, wt, hd, nw = self.lib, self.C, self.wt, self.hd, self.nw
@@ -79,16 +82,13 @@ class SwinBlock:
         q3 = 3 * C
         fused = lib.prad_matmul_fwd_fused
         check(fused(self.X.handle, w["Wqkv"].handle, w["bqkv"].handle, None, self.QKV.handle, _lib.ACT_NONE, 0.0))
-        for h in range(self.heads):
-            s_off = h * nw * wt * wt
-            # S = Q . K^T per window
-            self._per_head(0, 1, wt, wt, hd, self.QKV, h * hd, q3, wt * q3, self.QKV, C + h * hd, q3, wt * q3, self.S, s_off, wt, wt * wt)
+        hs = nw * wt * wt                 # scores are stored head-major: [head][window][wt][wt]
+        # S = Q . K^T per window and head
+        self._all_heads(0, 1, wt, wt, hd, self.QKV, 0, q3, wt * q3, hd, self.QKV, C, q3, wt * q3, hd, self.S, 0, wt, wt * wt, hs)
         check(lib.prad_scale(self.S.handle, self.S.handle, self.scale))
         check(lib.prad_softmax_fwd(self.S.handle, self.P.handle))
-        for h in range(self.heads):
-            s_off = h * nw * wt * wt
-            # O = P . V per window, written into head h's columns of O
-            self._per_head(0, 0, wt, hd, wt, self.P, s_off, wt, wt * wt, self.QKV, 2 * C + h * hd, q3, wt * q3, self.O, h * hd, C, wt * C)
+        # O = P . V per window, written into each head's columns of O
+        self._all_heads(0, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.QKV, 2 * C, q3, wt * q3, hd, self.O, 0, C, wt * C, hd)
         check(fused(self.O.handle, w["Wo"].handle, w["bo"].handle, None, self.Y1.handle, _lib.ACT_NONE, 0.0))
         check(fused(self.Y1.handle, w["W1"].handle, w["b1"].handle, self.Z1.handle, self.H1.handle, _lib.ACT_GELU, 0.0))
         check(fused(self.H1.handle, w["W2"].handle, w["b2"].handle, None, self.Y2.handle, _lib.ACT_NONE, 0.0))
@@ -102,18 +102,14 @@ class SwinBlock:
         check(lib.prad_matmul_bwd(self.dZ1.handle, self.Y1.handle, w["W1"].handle, self.dY1.handle, g["W1"].handle, 0, 0))
         check(lib.prad_add_broadcast_bwd_bias(self.dY1.handle, g["bo"].handle))
         check(lib.prad_matmul_bwd(self.dY1.handle, self.O.handle, w["Wo"].handle, self.dO.handle, g["Wo"].handle, 0, 0))
-        for h in range(self.heads):
-            s_off = h * nw * wt * wt
-            # dP = dO . V^T ; dV = P^T . dO
-            self._per_head(0, 1, wt, wt, hd, self.dO, h * hd, C, wt * C, self.QKV, 2 * C + h * hd, q3, wt * q3, self.dP, s_off, wt, wt * wt)
-            self._per_head(1, 0, wt, hd, wt, self.P, s_off, wt, wt * wt, self.dO, h * hd, C, wt * C, self.dQKV, 2 * C + h * hd, q3, wt * q3)
+        # dP = dO . V^T ; dV = P^T . dO
+        self._all_heads(0, 1, wt, wt, hd, self.dO, 0, C, wt * C, hd, self.QKV, 2 * C, q3, wt * q3, hd, self.dP, 0, wt, wt * wt, hs)
+        self._all_heads(1, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.dO, 0, C, wt * C, hd, self.dQKV, 2 * C, q3, wt * q3, hd)
         check(lib.prad_softmax_bwd(self.P.handle, self.dP.handle, self.dS.handle))
         check(lib.prad_scale(self.dS.handle, self.dS.handle, self.scale))
-        for h in range(self.heads):
-            s_off = h * nw * wt * wt
-            # dQ = dS . K ; dK = dS^T . Q
-            self._per_head(0, 0, wt, hd, wt, self.dS, s_off, wt, wt * wt, self.QKV, C + h * hd, q3, wt * q3, self.dQKV, h * hd, q3, wt * q3)
-            self._per_head(1, 0, wt, hd, wt, self.dS, s_off, wt, wt * wt, self.QKV, h * hd, q3, wt * q3, self.dQKV, C + h * hd, q3, wt * q3)
+        # dQ = dS . K ; dK = dS^T . Q
+        self._all_heads(0, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, C, q3, wt * q3, hd, self.dQKV, 0, q3, wt * q3, hd)
+        self._all_heads(1, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, 0, q3, wt * q3, hd, self.dQKV, C, q3, wt * q3, hd)
         check(lib.prad_add_broadcast_bwd_bias(self.dQKV.handle, g["bqkv"].handle))
         check(lib.prad_matmul_bwd(self.dQKV.handle, self.X.handle, w["Wqkv"].handle, self.dX.handle, g["Wqkv"].handle, 0, 0))
 
