@@ -18,6 +18,24 @@ __device__ __forceinline__ double wave_max(double v) {
     return v;
 }
 
+// Reductions and exponentials in the element type for the short-row kernels: in float they move one register per
+// shuffle step instead of two and use the hardware exponential (within 2e-7 of the double evaluation rounded to
+// float, far inside the 1e-5 parity bar), which is what those kernels' time goes into.
+__device__ __forceinline__ float wave_sum_t(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_sum_t(double v) { return wave_sum(v); }
+__device__ __forceinline__ float wave_max_t(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ double wave_max_t(double v) { return wave_max(v); }
+__device__ __forceinline__ float short_exp(float x) { return __expf(x); }
+__device__ __forceinline__ double short_exp(double x) { return exp(x); }
+
 // y[i][j] = exp(x[i][j] - max_i) / sum_j exp(x[i][j] - max_i)
 template <typename T>
 __global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols) {
@@ -39,7 +57,7 @@ __global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x
 
 // Rows of at most 64 columns (attention windows: 49): a lane holds one element of each of SHORT_ROWS consecutive
 // rows, whose loads are all issued before the first reduction (a row is under 256 bytes: one row per wavefront
-// leaves the memory system idle).  Each row is read once and written once.  Same arithmetic as softmax_fwd_kernel.
+// leaves the memory system idle).  Each row is read once and written once.
 constexpr int SHORT_ROWS = 8;
 template <typename T>
 __global__ void __launch_bounds__(256) softmax_fwd_short_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols) {
@@ -52,9 +70,9 @@ __global__ void __launch_bounds__(256) softmax_fwd_short_kernel(const T* __restr
 #pragma unroll
     for (int r = 0; r < SHORT_ROWS; ++r) {
         if (i0 + r >= rows) break;
-        const T m = (T)wave_max(on ? (double)xv[r] : -INFINITY);
-        const T e = on ? dev_exp(xv[r] - m) : (T)0;
-        const T s = (T)wave_sum(on ? (double)e : 0.0);
+        const T m = wave_max_t(on ? xv[r] : (T)-INFINITY);
+        const T e = on ? short_exp(xv[r] - m) : (T)0;
+        const T s = wave_sum_t(e);
         if (on) y[(i0 + r) * cols + lane] = e / s;
     }
 }
@@ -74,8 +92,8 @@ __global__ void __launch_bounds__(256) softmax_bwd_short_kernel(const T* __restr
 #pragma unroll
     for (int r = 0; r < SHORT_ROWS; ++r) {
         if (i0 + r >= rows) break;
-        const double dot = wave_sum(on ? (double)gv[r] * (double)yv[r] : 0.0);
-        if (on) dx[(i0 + r) * cols + lane] = (T)((double)yv[r] * ((double)gv[r] - dot));
+        const T dot = wave_sum_t(on ? gv[r] * yv[r] : (T)0);
+        if (on) dx[(i0 + r) * cols + lane] = yv[r] * (gv[r] - dot);
     }
 }
 
@@ -125,6 +143,19 @@ __global__ void __launch_bounds__(256) cce_bwd_kernel(const T* __restrict__ p, c
 template <typename T>
 __device__ __forceinline__ void softmax_cce_row(const T* __restrict__ xr, const T* __restrict__ tr, T* __restrict__ yr,
                                                 T* __restrict__ gr, T* __restrict__ dxr, int64_t rows, int64_t cols, int lane) {
+    if (cols <= 64) {  // the arithmetic of the short-row kernels, which the separate launches use for such rows
+        const bool on = lane < cols;
+        const T xv = on ? xr[lane] : (T)0;
+        const T m = wave_max_t(on ? xv : (T)-INFINITY);
+        const T e = on ? short_exp(xv - m) : (T)0;
+        const T s = wave_sum_t(e);
+        const T p = e / s;
+        const T scale = (T)1 / (T)rows;
+        const T g = on ? -scale * tr[lane] / (p + (T)1e-15) : (T)0;
+        const T dot = wave_sum_t(on ? g * p : (T)0);
+        if (on) { yr[lane] = p; gr[lane] = g; dxr[lane] = p * (g - dot); }
+        return;
+    }
     double mx = -INFINITY;
     for (int64_t j = lane; j < cols; j += 64) mx = fmax(mx, (double)xr[j]);
     const T m = (T)wave_max(mx);
