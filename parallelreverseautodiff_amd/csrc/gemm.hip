@@ -22,9 +22,17 @@
 //       layout was measured too: same speed in double, 6 % slower in float because the compiler
 //       can no longer merge neighbouring LDS reads);
 //   stored with mn contiguous ("MC": B of the forward, both operands of dB)
-//       S[k][mn], row pitch MN + 16 elements.
+//       S[k][mn], row pitch MN + 16 elements for the 128 tile; the smaller tiles keep the pitch at MN and
+//       rotate row k instead (Slab::mc_shift), so that two of their workgroups fit on a compute unit.
 // An MFMA lane (mn = lane % 16, k = lane / 16) reads one element from either placement without
 // bank conflicts, so no transposed copy is ever written.
+//
+// Around the main loop: tiles that hang over the edge of the output clamp their loads and guard their stores
+// (only operands whose rows are not 16-byte aligned take the guarded scalar kernels); products with few tiles
+// are split along K and reduced inside the kernel by the last workgroup to arrive at a tile (gemm_split_factor,
+// gemm_pairs); the epilogue is a plain store, an elementwise pass staged through LDS (bias, activation, upstream
+// activation's backward), a per-tile sum, or the cell arithmetic of an LSTM step; a column sum (bias gradient)
+// can ride along on extra workgroups of the grid.
 #include "common.h"
 
 #include <cstdlib>
