@@ -28,6 +28,9 @@ SHAPES = [  # M, K, N: tile-aligned, ragged in every dimension, degenerate vecto
     (64, 784, 256), (64, 256, 128), (64, 128, 10), (100, 100, 1), (1, 100, 100), (384, 512, 256), (130, 260, 390),
     # whole tiles with a ragged reduction: one slab plus a tail, a tail only, an odd number of slabs
     (128, 70, 64), (64, 40, 32), (256, 200, 256), (512, 1000, 512), (2048, 24, 2048),
+    # rows that start 16-byte aligned but tiles that hang over the edge (vector loads clamped at the edge), on the
+    # 64 and 128 tiles, with a tiny M and with a narrow N
+    (1000, 64, 1000), (2052, 36, 2060), (4, 8, 260), (3000, 100, 12),
 ]
 
 
