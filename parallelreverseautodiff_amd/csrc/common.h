@@ -215,6 +215,9 @@ constexpr int GEMM_SPLIT_MAX_TILES = 384;
 inline int64_t gemm_tiles_per_product(int64_t M, int64_t N) { return ((M + 127) / 128) * ((N + 127) / 128); }
 
 template <typename T> hipError_t launch_gemm(const GemmArgs<T>& args, hipStream_t stream);
+// first = dC . B^T (transB) and second = A^T . dC (transA, may carry the column-sum rider) in one launch;
+// hipErrorNotSupported (nothing launched) unless each alone would run unsplit on the smallest tile.
+template <typename T> hipError_t launch_gemm_pair(const GemmArgs<T>& first, const GemmArgs<T>& second, hipStream_t stream);
 
 // One LSTM time step forward in one launch: gates = act(C + A . B) with C (rows x 4H) holding the input
 // projection plus bias, A = h_{t-1} (rows x H), B = W_h (H x 4H); then c = f.c_prev + i.g, tanh_c, h = o.tanh_c.

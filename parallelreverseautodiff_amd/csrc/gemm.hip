@@ -209,9 +209,15 @@ constexpr int EPI_TILE_SUM = 2;   // reduce the tile to one double (MatrixMultip
 constexpr int EPI_LSTM_FWD = 3;   // gates, cell state and hidden state of one LSTM step (32 x 32 tile gathering 4 gates x 8 units)
 constexpr int EPI_LSTM_BWD = 4;   // cell backward of one LSTM step on the recurrent gradient tile
 
+// Workgroup coordinates of a product inside a launch: what blockIdx / gridDim are when the launch holds one product.
+struct GridPos {
+    unsigned bx, by, bz;  // tile (or rider) index, batch index, split index
+    unsigned gy, gz;      // batch count, split count
+};
+
+// One workgroup's share of one product (a tile, or the column-sum rider).
 template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI>
-__global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
-                                                                            const int tilesN) {
+__device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM, const int tilesN, const GridPos g_) {
     typedef Mfma<T> MF;
     typedef Slab<T, WT> S;
     typedef typename MF::Acc Acc;
@@ -225,16 +231,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     __shared__ __attribute__((aligned(16))) T smem[2][SA + SB];  // [stage][A slab | B slab]
 
     // Workgroups beyond the tiles carry a column sum that rides along with this launch.
-    if (blockIdx.x >= (unsigned)(tilesM * tilesN)) {
-        if (blockIdx.y == 0 && blockIdx.z == 0)
-            colsum_block<T, T>(p.colsum_src, p.colsum_dst, p.colsum_cols, 0, p.colsum_rows, blockIdx.x - tilesM * tilesN,
+    if (g_.bx >= (unsigned)(tilesM * tilesN)) {
+        if (g_.by == 0 && g_.bz == 0)
+            colsum_block<T, T>(p.colsum_src, p.colsum_dst, p.colsum_cols, 0, p.colsum_rows, g_.bx - tilesM * tilesN,
                                reinterpret_cast<double*>(&smem[0][0]));
         return;
     }
     int tm, tn;
-    tile_of_workgroup(blockIdx.x, tilesM, tilesN, tm, tn);
+    tile_of_workgroup(g_.bx, tilesM, tilesN, tm, tn);
     const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
-    const int batch = blockIdx.y;
+    const int batch = g_.by;
     const int b_outer = p.batch_inner > 1 ? batch / p.batch_inner : batch;
     const int b_inner = p.batch_inner > 1 ? batch - b_outer * p.batch_inner : 0;
     const T* __restrict__ A = p.A + b_outer * p.strideA + b_inner * p.istrideA;
@@ -242,10 +248,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     // A product split along K: this workgroup reduces [kb, kb + K) and writes its own M x N partial result.
     int64_t K = p.K;
     if (p.ksplit > 0) {
-        const int64_t kb = (int64_t)blockIdx.z * p.ksplit;
+        const int64_t kb = (int64_t)g_.bz * p.ksplit;
         K = min(p.ksplit, p.K - kb);
-        A += (int64_t)blockIdx.z * p.zstrideA;
-        B += (int64_t)blockIdx.z * p.zstrideB;
+        A += (int64_t)g_.bz * p.zstrideA;
+        B += (int64_t)g_.bz * p.zstrideB;
     }
 
     const int tid = threadIdx.x;
@@ -400,8 +406,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
         // loads (written through, read past the caches) whose completion the barriers wait for: a device-scope
         // fence would write back and invalidate the whole L2 and evict the operand panels of every workgroup nearby.
         const int64_t mn = p.M * p.N;
-        const int splits = (int)gridDim.z;
-        T* __restrict__ mine = p.split_ws + ((int64_t)blockIdx.z * gridDim.y + batch) * mn;
+        const int splits = (int)g_.gz;
+        T* __restrict__ mine = p.split_ws + ((int64_t)g_.bz * g_.gy + batch) * mn;
 #pragma unroll
         for (int x = 0; x < WTM; ++x)
 #pragma unroll
@@ -433,7 +439,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
 #pragma unroll
                 for (int u = 0; u < ZU; ++u) {
                     if (z0 + u >= splits) break;
-                    const T* other = p.split_ws + ((int64_t)(z0 + u) * gridDim.y + batch) * mn;
+                    const T* other = p.split_ws + ((int64_t)(z0 + u) * g_.gy + batch) * mn;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int64_t i = row0 + wm * WS + x * 16 + MF::row(r, g);
@@ -539,7 +545,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     }
 
     T* __restrict__ C = p.C + b_outer * p.strideC + b_inner * p.istrideC +
-                        ((p.ksplit > 0 && p.split_counters == nullptr) ? (int64_t)blockIdx.z * gridDim.y * p.strideC : 0);
+                        ((p.ksplit > 0 && p.split_counters == nullptr) ? (int64_t)g_.bz * g_.gy * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
         // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
         // row-major: the elementwise arithmetic (which includes exp/tanh code) then sits in one runtime loop
@@ -649,6 +655,26 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     }
 }
 
+template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI>
+__global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
+                                                                            const int tilesN) {
+    gemm_tile<T, WT, A_KC, B_KC, EDGE, EPI>(p, tilesM, tilesN, GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z});
+}
+
+// The two gradient products of a layer, dA = dC . B^T (both operands k-contiguous; the upstream activation's
+// backward may be its epilogue) and dB = A^T . dC (both operands mn-contiguous; the bias gradient may ride along),
+// in one launch on 32 x 32 tiles: small layers cost what their chain of dependent launches costs.  Workgroups
+// [0, first) belong to the first product, the rest to the second.  Neither product is split or batched.
+template <typename T, bool EDGE1, int EPI1, bool EDGE2>
+__global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_pair_kernel(const GemmArgs<T> p1, const int tilesM1, const int tilesN1,
+                                                                     const GemmArgs<T> p2, const int tilesM2, const int tilesN2,
+                                                                     const unsigned first) {
+    // (each product's slab stages are LDS of their own: 133 KB together, one workgroup per compute unit, which is
+    // all such small products put there anyway)
+    if (blockIdx.x < first) gemm_tile<T, 1, true, true, EDGE1, EPI1>(p1, tilesM1, tilesN1, GridPos{blockIdx.x, 0u, 0u, 1u, 1u});
+    else gemm_tile<T, 1, false, false, EDGE2, EPI_PLAIN>(p2, tilesM2, tilesN2, GridPos{blockIdx.x - first, 0u, 0u, 1u, 1u});
+}
+
 template <typename T, int WT, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStream_t stream) {
     constexpr int BM = 32 * WT;
@@ -671,20 +697,25 @@ static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStr
     return hipGetLastError();
 }
 
+// The unguarded kernels use 16-byte loads (any M, N, K: tiles over the edge clamp their loads, a ragged end of K
+// is handled inside); they need operands whose rows start 16-byte aligned.  The tile-sum epilogue adds up whole
+// tiles and therefore needs the zero fill of the guarded kernels when the output does not fill its tiles.
+template <typename T>
+static bool vector_loads_ok(const GemmArgs<T>& a, int epi, int BM) {
+    constexpr int VEC = Mfma<T>::VEC;
+    const bool whole = (a.M % BM == 0) && (a.N % BM == 0);
+    return (whole || epi != EPI_TILE_SUM) && a.K > 0 && (a.lda % VEC == 0) &&
+           (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
+           (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
+           (a.zstrideA % VEC == 0) && (a.zstrideB % VEC == 0) && (a.istrideA % VEC == 0) && (a.istrideB % VEC == 0) &&
+           // per-thread element offsets inside one tile's slab are kept in 32 bits
+           (a.lda < (1 << 23)) && (a.ldb < (1 << 23));
+}
+
 template <typename T, int WT>
 static hipError_t launch_tile(const GemmArgs<T>& a, int epi, hipStream_t stream) {
-    constexpr int VEC = Mfma<T>::VEC;
     constexpr int BM = 32 * WT;
-    // The unguarded kernels use 16-byte loads (any M, N, K: tiles over the edge clamp their loads, a ragged end of K
-    // is handled inside); they need operands whose rows start 16-byte aligned.  The tile-sum epilogue adds up whole
-    // tiles and therefore needs the zero fill of the guarded kernels when the output does not fill its tiles.
-    const bool whole = (a.M % BM == 0) && (a.N % BM == 0);
-    const bool aligned = (whole || epi != EPI_TILE_SUM) && a.K > 0 && (a.lda % VEC == 0) &&
-                         (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
-                         (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
-                         (a.zstrideA % VEC == 0) && (a.zstrideB % VEC == 0) && (a.istrideA % VEC == 0) && (a.istrideB % VEC == 0) &&
-                         // per-thread element offsets inside one tile's slab are kept in 32 bits
-                         (a.lda < (1 << 23)) && (a.ldb < (1 << 23));
+    const bool aligned = vector_loads_ok(a, epi, BM);
     // Grid y carries the batch; the tile count must fit the 1-D grid.
     if ((int64_t)((a.M + BM - 1) / BM) * ((a.N + BM - 1) / BM) > 0x7fffffffLL || a.batch > 65535) return hipErrorInvalidValue;
     if (!a.transA && !a.transB) return launch_layout<T, WT, true, false>(a, !aligned, epi, stream);
@@ -864,6 +895,49 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
     }
 }
 
+// Both gradient products of a layer in one launch (gemm_pair_kernel).  Taken only where each product alone would
+// run unsplit on 32 x 32 tiles, so that the results are those of the two separate launches bit for bit, and where
+// the two together still give every workgroup a compute unit of its own.  hipErrorNotSupported otherwise: the
+// caller then launches the products one after the other.
+template <typename T>
+hipError_t launch_gemm_pair(const GemmArgs<T>& first_in, const GemmArgs<T>& second_in, hipStream_t stream) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_DUAL"); return !(e && e[0] == '0'); }();  // tuning aid
+    if (!enabled) return hipErrorNotSupported;
+    GemmArgs<T> p1 = first_in, p2 = second_in;
+    auto epilogue = [](const GemmArgs<T>& a) {
+        return (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) ? EPI_ELEMENTWISE : EPI_PLAIN;
+    };
+    auto small = [](const GemmArgs<T>& a) {
+        return a.M > 0 && a.N > 0 && a.K > 0 && a.batch == 1 && a.batch_inner <= 1 && a.nseg <= 1 && a.tile_sums == nullptr &&
+               choose_tile(a.M, a.N, 1, false) == TILE_32x32 && gemm_split_factor(a.M, a.N, a.K, 1, (int)sizeof(T)) == 1 &&
+               !gemm_pairs(a.M, a.N, a.K, 1, (int)sizeof(T));
+    };
+    if (p1.transA || !p1.transB || !p2.transA || p2.transB || !small(p1) || !small(p2)) return hipErrorNotSupported;
+    if (epilogue(p2) != EPI_PLAIN || p1.colsum_dst != nullptr) return hipErrorNotSupported;
+    for (GemmArgs<T>* p : {&p1, &p2}) { p->ksplit = 0; p->zstrideA = 0; p->zstrideB = 0; p->split_counters = nullptr; }
+    const int tilesM1 = (int)((p1.M + 31) / 32), tilesN1 = (int)((p1.N + 31) / 32);
+    const int tilesM2 = (int)((p2.M + 31) / 32), tilesN2 = (int)((p2.N + 31) / 32);
+    const unsigned first = (unsigned)(tilesM1 * tilesN1);
+    const unsigned riders = p2.colsum_dst != nullptr ? (unsigned)((p2.colsum_cols + 63) / 64) : 0u;
+    const unsigned total = first + (unsigned)(tilesM2 * tilesN2) + riders;
+    if (total > 256u) return hipErrorNotSupported;
+    const int epi1 = epilogue(p1);
+    const bool edge1 = !vector_loads_ok(p1, epi1, 32), edge2 = !vector_loads_ok(p2, EPI_PLAIN, 32);
+    const dim3 grid(total), block(GEMM_THREADS);
+#define PRAD_LAUNCH(E1_, EPI_, E2_) \
+    hipLaunchKernelGGL((gemm_pair_kernel<T, E1_, EPI_, E2_>), grid, block, 0, stream, p1, tilesM1, tilesN1, p2, tilesM2, tilesN2, first)
+    if (edge1 || edge2) {
+        // misaligned operands: both products on the guarded loads
+        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(true, EPI_PLAIN, true);
+        else PRAD_LAUNCH(true, EPI_ELEMENTWISE, true);
+    } else {
+        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(false, EPI_PLAIN, false);
+        else PRAD_LAUNCH(false, EPI_ELEMENTWISE, false);
+    }
+#undef PRAD_LAUNCH
+    return hipGetLastError();
+}
+
 template <typename T>
 static bool lstm_operands_aligned(const GemmArgs<T>& a) {
     constexpr int VEC = Mfma<T>::VEC;
@@ -916,6 +990,8 @@ template hipError_t launch_lstm_step_fwd<double>(const GemmArgs<double>&, hipStr
 template hipError_t launch_lstm_step_fwd<float>(const GemmArgs<float>&, hipStream_t);
 template hipError_t launch_lstm_step_bwd<double>(const GemmArgs<double>&, hipStream_t);
 template hipError_t launch_lstm_step_bwd<float>(const GemmArgs<float>&, hipStream_t);
+template hipError_t launch_gemm_pair<double>(const GemmArgs<double>&, const GemmArgs<double>&, hipStream_t);
+template hipError_t launch_gemm_pair<float>(const GemmArgs<float>&, const GemmArgs<float>&, hipStream_t);
 template hipError_t launch_gemm<double>(const GemmArgs<double>&, hipStream_t);
 template hipError_t launch_gemm<float>(const GemmArgs<float>&, hipStream_t);
 

@@ -190,8 +190,8 @@ struct Epilogue {
 };
 
 template <typename T>
-int32_t enqueue_gemm_t(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int accumulate, const Epilogue& ep,
-                       bool batched) {
+GemmArgs<T> gemm_args_of(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int accumulate, const Epilogue& ep,
+                         bool batched) {
     const int64_t M = op_rows(A, transA), K = op_cols(A, transA), N = op_cols(B, transB);
     GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A->ptr, A->cols, B->ptr, B->cols, C->ptr, C->cols, accumulate);
     if (ep.bias) a.bias = static_cast<const T*>(ep.bias->ptr);
@@ -212,14 +212,20 @@ int32_t enqueue_gemm_t(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_
         a.strideB = B->depth == 1 ? 0 : B->rows * B->cols;
         a.strideC = C->rows * C->cols;
     }
+    return a;
+}
+
+template <typename T>
+int32_t enqueue_gemm_t(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int accumulate, const Epilogue& ep,
+                       bool batched) {
+    GemmArgs<T> a = gemm_args_of<T>(transA, transB, A, B, C, accumulate, ep, batched);
     if (int32_t st = attach_split_workspace(a)) return st;
     HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
 
-// Validates shapes with the reference's messages and enqueues C = op(A).op(B).
-int32_t enqueue_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int accumulate, const Epilogue& ep,
-                     bool batched) {
+// Checks the operands of C = op(A).op(B) and of its epilogue, with the reference's messages.
+int32_t validate_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, const Epilogue& ep, bool batched) {
     REQUIRE_BUF(A); REQUIRE_BUF(B); REQUIRE_BUF(C);
     if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1) || (transA && transB))
         return fail(PRAD_ERR_ARG, "unsupported transpose combination (%d, %d)", transA, transB);
@@ -247,8 +253,28 @@ int32_t enqueue_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_bu
     }
     if (ep.act_fwd < 0 || ep.act_fwd > PRAD_ACT_AMPLIFIED_SIGMOID || ep.act_bwd < 0 || ep.act_bwd > PRAD_ACT_AMPLIFIED_SIGMOID)
         return fail(PRAD_ERR_ARG, "unknown activation selector");
+    return PRAD_OK;
+}
+
+// Validates and enqueues C = op(A).op(B).
+int32_t enqueue_gemm(int transA, int transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int accumulate, const Epilogue& ep,
+                     bool batched) {
+    if (int32_t st = validate_gemm(transA, transB, A, B, C, ep, batched)) return st;
     if (A->dtype == PRAD_F64) return enqueue_gemm_t<double>(transA, transB, A, B, C, accumulate, ep, batched);
     return enqueue_gemm_t<float>(transA, transB, A, B, C, accumulate, ep, batched);
+}
+
+// dA = dC . B^T (epilogue ep) and dB = A^T . dC (epilogue rider) in one launch where launch_gemm_pair takes them;
+// *done says whether it did.  Operands already validated.
+template <typename T>
+int32_t enqueue_gradient_pair_t(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, int acc_dA, int acc_dB,
+                                const Epilogue& ep, const Epilogue& rider, bool* done) {
+    const GemmArgs<T> first = gemm_args_of<T>(0, 1, dC, B, dA, acc_dA, ep, false);
+    const GemmArgs<T> second = gemm_args_of<T>(1, 0, A, dC, dB, acc_dB, rider, false);
+    const hipError_t e = launch_gemm_pair<T>(first, second, CUR_STREAM);
+    *done = e == hipSuccess;
+    if (e != hipSuccess && e != hipErrorNotSupported) HIP_TRY(e, PRAD_ERR_LAUNCH);
+    return PRAD_OK;
 }
 
 // C = sum_q A[q].B[q] + bias: the pairs are the splits of one product along the joint reduction.
@@ -610,15 +636,33 @@ static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad
     if (dC->rows != A->rows || dC->cols != B->cols)
         return fail(PRAD_ERR_ARG, "upstream gradient is %lldx%lld, the product is %lldx%lld", (long long)dC->rows,
                     (long long)dC->cols, (long long)A->rows, (long long)B->cols);
-    if (dA != nullptr) {
+    Epilogue rider;
+    if (dB != nullptr && dbias != nullptr && dC->rows < COLSUM_CHUNK_ROWS) { rider.colsum_src = dC; rider.colsum_dst = dbias; }
+    bool paired = false;
+    // (one launch only if the first product's output is not an operand of the second: launched one after the other,
+    // the second would read what the first wrote)
+    auto overlap = [](prad_buf_t x, prad_buf_t y) {
+        const char* x0 = static_cast<const char*>(x->ptr);
+        const char* y0 = static_cast<const char*>(y->ptr);
+        const size_t xb = (size_t)count(x) * elem_size(x->dtype), yb = (size_t)count(y) * elem_size(y->dtype);
+        return x0 < y0 + yb && y0 < x0 + xb;
+    };
+    if (dA != nullptr && dB != nullptr && valid(dA) && valid(dB) && !overlap(dA, dC) && !overlap(dA, A) && !overlap(dA, dB) &&
+        !overlap(dB, dC) && !overlap(dB, B) && (dbias == nullptr || !overlap(dbias, dA))) {
+        if (int32_t st = validate_gemm(0, 1, dC, B, dA, ep, false)) return st;
+        if (int32_t st = validate_gemm(1, 0, A, dC, dB, rider, false)) return st;
+        if (int32_t st = dC->dtype == PRAD_F64
+                             ? enqueue_gradient_pair_t<double>(dC, A, B, dA, dB, acc_dA, acc_dB, ep, rider, &paired)
+                             : enqueue_gradient_pair_t<float>(dC, A, B, dA, dB, acc_dA, acc_dB, ep, rider, &paired))
+            return st;
+    }
+    if (dA != nullptr && !paired) {
         if (int32_t st = enqueue_gemm(0, 1, dC, B, dA, acc_dA, ep, false)) return st;  // dA = dC . B^T
     }
-    if (dB != nullptr) {
-        Epilogue rider;
-        if (dbias != nullptr && dC->rows < COLSUM_CHUNK_ROWS) { rider.colsum_src = dC; rider.colsum_dst = dbias; }
+    if (dB != nullptr && !paired) {
         if (int32_t st = enqueue_gemm(1, 0, A, dC, dB, acc_dB, rider, false)) return st;  // dB = A^T . dC
-        if (rider.colsum_dst != nullptr) dbias = nullptr;
     }
+    if (rider.colsum_dst != nullptr) dbias = nullptr;
     if (dbias != nullptr) return matmul_bwd_bias_only_locked(dC, dbias);  // nothing to ride along with, or a tall matrix
     return PRAD_OK;
 }

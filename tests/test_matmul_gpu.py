@@ -398,6 +398,40 @@ def test_bias_gradient_riding_with_the_weight_gradient(gpu, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("accumulate", [0, 1])
+@pytest.mark.parametrize("shape", [(64, 784, 256), (64, 256, 128), (64, 128, 10), (33, 17, 129), (50, 49, 49), (1, 1, 1),
+                                   (96, 200, 72), (300, 300, 300)])
+def test_both_gradients_in_one_launch(gpu, dtype, accumulate, shape):
+    """Small layers get dA = dC . B^T (with the activation's backward) and dB = A^T . dC (+ bias gradient) from one
+    launch; asking for one gradient at a time takes the single-product launches.  Same bits either way, for aligned
+    and misaligned operands, with and without accumulation into dB, and for a shape too large for the joint launch."""
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    M, K, N = shape
+    A, B, dC, Z, dB0 = (seeded.normal(73, i, s, 1.0, dtype) for i, s in enumerate([(M, K), (K, N), (M, N), (M, K), (K, N)]))
+    up = lambda a: (lambda b: (b.upload(a), b)[1])(DeviceBuffer.alloc(dtype, *a.shape))
+    bA, bB, bdC, bZ = up(A), up(B), up(dC), up(Z)
+    dA1, dA2, dB1, dB2 = DeviceBuffer.alloc(dtype, M, K), DeviceBuffer.alloc(dtype, M, K), up(dB0), up(dB0)
+    db1, db2 = DeviceBuffer.alloc(dtype, 1, N), DeviceBuffer.alloc(dtype, 1, N)
+    args = (accumulate, _lib.ACT_TANH, bZ.handle, 0.0)
+    check(lib.prad_matmul_bias_bwd(bdC.handle, bA.handle, bB.handle, dA1.handle, None, None, *args))
+    check(lib.prad_matmul_bias_bwd(bdC.handle, bA.handle, bB.handle, None, dB1.handle, db1.handle, *args))
+    check(lib.prad_matmul_bias_bwd(bdC.handle, bA.handle, bB.handle, dA2.handle, dB2.handle, db2.handle, *args))
+    assert np.array_equal(dA1.download(), dA2.download())
+    assert np.array_equal(dB1.download(), dB2.download())
+    assert np.array_equal(db1.download(), db2.download())
+    # plain upstream gradient (no activation): prad_matmul_bwd against the two single products
+    check(lib.prad_gemm(0, 1, bdC.handle, bB.handle, dA1.handle, 0))
+    check(lib.prad_gemm(1, 0, bA.handle, bdC.handle, dB1.handle, 0))
+    check(lib.prad_matmul_bwd(bdC.handle, bA.handle, bB.handle, dA2.handle, dB2.handle, 0, 0))
+    assert np.array_equal(dA1.download(), dA2.download())
+    assert np.array_equal(dB1.download(), dB2.download())
+    ref_dA = dC.astype(np.float64) @ B.astype(np.float64).T
+    assert_parity(dA2.download(), ref_dA.astype(dtype), dtype, "dA", bound=dot_bound(dC, B.T, dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("shape", [(512, 2048, 512), (1024, 1024, 1024), (384, 2100, 500)])
 def test_products_run_as_workgroup_pairs(gpu, oracle, dtype, shape):
     """Shapes whose tiles fill between half and one and a half of the chip's workgroup slots and whose K is
