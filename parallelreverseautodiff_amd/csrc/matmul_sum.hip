@@ -125,33 +125,124 @@ __device__ __forceinline__ void sum_bwd_da_block(T (*tile)[TS + 1], const T* __r
     }
 }
 
+// The same two blocks on 16-byte loads and stores, for operands whose rows are whole, aligned vectors.
+template <typename T> struct SumVec;
+template <> struct SumVec<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
+template <> struct SumVec<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
+constexpr int Q_PER_WG_VEC = 4;  // the transposed tile stays in registers while it is scaled into this many slices
+
+template <typename T>
+__device__ __forceinline__ void sum_bwd_db_block_vec(T (*tile)[TS + 1], const T* __restrict__ A, const T* __restrict__ dOut,
+                                                     T* __restrict__ dB, int64_t M, int64_t K, int64_t P, int64_t bx, int64_t by,
+                                                     int64_t bz) {
+    typedef typename SumVec<T>::type V;
+    constexpr int VEC = SumVec<T>::N, VPR = TS / VEC, ROWS = 256 / VPR, PASSES = TS / ROWS;
+    const int64_t m0 = bx * TS, k0 = by * TS;
+    const int t = threadIdx.x, row = t / VPR, col = (t % VPR) * VEC;
+    V v[PASSES];
+#pragma unroll
+    for (int e = 0; e < PASSES; ++e) {
+        const int64_t m = m0 + row + e * ROWS, k = k0 + col;
+        if (m < M && k < K) v[e] = *reinterpret_cast<const V*>(A + m * K + k);
+        else v[e] = (V)(T)0;
+    }
+#pragma unroll
+    for (int e = 0; e < PASSES; ++e)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) tile[row + e * ROWS][col + j] = v[e][j];
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < PASSES; ++e)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[e][j] = tile[col + j][row + e * ROWS];  // rows of the output walk k, vectors walk m
+    const int64_t q0 = bz * Q_PER_WG_VEC;
+    for (int64_t q = q0; q < q0 + Q_PER_WG_VEC && q < P; ++q) {
+        const T sc = dOut[q];
+        T* __restrict__ out = dB + q * K * M;
+#pragma unroll
+        for (int e = 0; e < PASSES; ++e) {
+            const int64_t k = k0 + row + e * ROWS, m = m0 + col;
+            if (k < K && m < M) __builtin_nontemporal_store(v[e] * sc, reinterpret_cast<V*>(out + k * M + m));
+        }
+    }
+}
+
+// 16 vectors (i) x 16 rows (j) of dA^T per workgroup; eight slices' loads are in flight before their ordered additions.
+template <typename T>
+__device__ __forceinline__ void sum_bwd_da_block_vec(T (*tile)[TS + 1], const T* __restrict__ B, const T* __restrict__ dOut,
+                                                     T* __restrict__ dA, int64_t M, int64_t K, int64_t N, int64_t P, int64_t bx,
+                                                     int64_t by) {
+    typedef typename SumVec<T>::type V;
+    constexpr int VEC = SumVec<T>::N, IW = 16 * VEC, DEPTH = 8;
+    const int64_t i0 = bx * IW, j0 = by * TJ;
+    const int t = threadIdx.x, jr = t >> 4, iv = (t & 15) * VEC;
+    const int64_t i = i0 + iv, j = j0 + jr;
+    const bool inside = i < N && j < K;
+    const T* __restrict__ src = B + j * N + i;
+    const int64_t slice = K * N;
+    V acc = (V)(T)0;
+    int64_t q = 0;
+    for (; q + DEPTH <= P; q += DEPTH) {
+        V b[DEPTH];
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            if (inside) b[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + (q + u) * slice));
+            else b[u] = (V)(T)0;
+        }
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) acc = acc + (b[u] * dOut[q + u]);
+    }
+    for (; q < P; ++q) {
+        V b = (V)(T)0;
+        if (inside) b = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + q * slice));
+        acc = acc + (b * dOut[q]);
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) tile[jr][iv + e] = acc[e];
+    __syncthreads();
+    const int jj = t & 15, ib = t >> 4;
+    for (int r = 0; r < IW; r += 16) {
+        const int64_t ii = i0 + ib + r, jo = j0 + jj;
+        if (ii < M && jo < K) dA[ii * K + jo] = tile[jj][ib + r];
+    }
+}
+
 // Both gradients in one launch: the workgroups of the dA part (each walks all P slices) come first in the
 // grid, those of the dB part fill in behind them.
-template <typename T>
+template <typename T, bool VECTOR>
 __global__ void __launch_bounds__(256) sum_bwd_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ dOut,
                                                       T* __restrict__ dA, T* __restrict__ dB, int64_t M, int64_t K, int64_t N,
-                                                      int64_t P, int64_t da_blocks, int64_t bm, int64_t db_by) {
+                                                      int64_t P, int64_t da_blocks, int64_t da_bm, int64_t bm, int64_t db_by) {
     __shared__ T tile[TS][TS + 1];
     int64_t id = blockIdx.x;
     if (id < da_blocks) {
-        sum_bwd_da_block<T>(tile, B, dOut, dA, M, K, N, P, id % bm, id / bm);
+        if (VECTOR) sum_bwd_da_block_vec<T>(tile, B, dOut, dA, M, K, N, P, id % da_bm, id / da_bm);
+        else sum_bwd_da_block<T>(tile, B, dOut, dA, M, K, N, P, id % da_bm, id / da_bm);
         return;
     }
     id -= da_blocks;
-    sum_bwd_db_block<T>(tile, A, dOut, dB, M, K, P, id % bm, (id / bm) % db_by, id / (bm * db_by));
+    if (VECTOR) sum_bwd_db_block_vec<T>(tile, A, dOut, dB, M, K, P, id % bm, (id / bm) % db_by, id / (bm * db_by));
+    else sum_bwd_db_block<T>(tile, A, dOut, dB, M, K, P, id % bm, (id / bm) % db_by, id / (bm * db_by));
 }
 
 template <typename T>
 hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T* dB, int64_t M, int64_t K, int64_t N, int64_t P,
                                  hipStream_t s) {
     if (M <= 0 || K <= 0) return hipSuccess;
-    const int64_t bm = (M + TS - 1) / TS, db_by = (K + TS - 1) / TS;
-    const int64_t da_blocks = dA != nullptr ? bm * ((K + TJ - 1) / TJ) : 0;
-    const int64_t db_blocks = (dB != nullptr && P > 0) ? bm * db_by * ((P + Q_PER_WG - 1) / Q_PER_WG) : 0;
+    constexpr int VEC = SumVec<T>::N;
+    auto aligned = [](const void* p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const bool vec = M % VEC == 0 && K % VEC == 0 && N % VEC == 0 && aligned(A) && aligned(B) && aligned(dA) && aligned(dB);
+    const int64_t iw = vec ? 16 * VEC : TS, qpw = vec ? Q_PER_WG_VEC : Q_PER_WG;
+    const int64_t bm = (M + TS - 1) / TS, db_by = (K + TS - 1) / TS, da_bm = (M + iw - 1) / iw;
+    const int64_t da_blocks = dA != nullptr ? da_bm * ((K + TJ - 1) / TJ) : 0;
+    const int64_t db_blocks = (dB != nullptr && P > 0) ? bm * db_by * ((P + qpw - 1) / qpw) : 0;
     if (da_blocks + db_blocks == 0) return hipSuccess;
     if (da_blocks + db_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((sum_bwd_kernel<T>), dim3((unsigned)(da_blocks + db_blocks)), dim3(256), 0, s, A, B, dOut, dA, dB, M, K, N, P,
-                       da_blocks, bm, db_by);
+    const dim3 grid((unsigned)(da_blocks + db_blocks)), block(256);
+    if (vec)
+        hipLaunchKernelGGL((sum_bwd_kernel<T, true>), grid, block, 0, s, A, B, dOut, dA, dB, M, K, N, P, da_blocks, da_bm, bm, db_by);
+    else
+        hipLaunchKernelGGL((sum_bwd_kernel<T, false>), grid, block, 0, s, A, B, dOut, dA, dB, M, K, N, P, da_blocks, da_bm, bm, db_by);
     return hipGetLastError();
 }
 

@@ -31,7 +31,7 @@ def test_add_and_add_three_are_exact(gpu, oracle, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", [(1, 1), (1, 100), (100, 1), (64, 64), (65, 127), (300, 1000)])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 100), (100, 1), (64, 64), (65, 127), (300, 1000), (128, 200), (1000, 36), (4, 4)])
 def test_transpose(gpu, oracle, dtype, shape):
     x = seeded.normal(102, 1, shape, 1.0, dtype)
     op = MatrixTransposeOperation.Instantiate(None)
