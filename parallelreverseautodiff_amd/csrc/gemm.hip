@@ -130,8 +130,10 @@ __device__ __forceinline__ void load_slab_guarded(typename Mfma<T>::Vec (&r)[NV]
 }
 
 // Unguarded loads of one slab, addressed as a wavefront-uniform base (scalar registers, advanced slab
-// by slab) plus a per-thread 32-bit element offset that never changes: the loads take the
-// scalar-base form and the two prefetch register sets share one set of offsets.
+// by slab) plus a per-thread 32-bit byte offset that never changes.  They are issued as buffer loads so
+// that no vector register is ever written to form an address: with per-lane 64-bit pointers the compiler
+// advances them with vector adds into registers that loads still in flight are about to fill, and waits
+// for those loads (the slab being prefetched) first, which undoes the prefetch.
 // A tile that hangs over the edge of the matrix (`valid` < MN rows or columns of it exist) clamps its offsets to
 // the last valid row / vector: the threads concerned load duplicates of valid data, which only reach output
 // rows or columns that are never stored (row i of the product depends on row i of A alone, column j on column j
@@ -148,15 +150,17 @@ __device__ __forceinline__ void slab_offsets(unsigned (&off)[NV], int64_t ld, in
     if (!KC && gather_stride > 0) col_off = (col / (S::MN / 4)) * gather_stride + col % (S::MN / 4);
 #pragma unroll
     for (int p = 0; p < NV; ++p)
-        off[p] = KC ? (unsigned)(min(tid / S::TPR_KC + S::ROWS_KC * p, valid - 1) * ld + (tid % S::TPR_KC) * VEC)
-                    : (unsigned)((tid / S::TPR_MC + S::ROWS_MC * p) * ld + col_off);
+        off[p] = (unsigned)sizeof(T) * (KC ? (unsigned)(min(tid / S::TPR_KC + S::ROWS_KC * p, valid - 1) * ld + (tid % S::TPR_KC) * VEC)
+                                           : (unsigned)((tid / S::TPR_MC + S::ROWS_MC * p) * ld + col_off));
 }
 template <typename T>
 __device__ __forceinline__ void load_slab_fast(typename Mfma<T>::Vec (&r)[NV], const T* __restrict__ ubase,
                                                const unsigned (&off)[NV]) {
     typedef typename Mfma<T>::Vec Vec;
+    // A buffer load: descriptor (the base, no bounds in use) in scalar registers, byte offset in one vector register.
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ubase), 0, -1, 0x00020000);
 #pragma unroll
-    for (int p = 0; p < NV; ++p) r[p] = *reinterpret_cast<const Vec*>(ubase + off[p]);
+    for (int p = 0; p < NV; ++p) r[p] = __builtin_bit_cast(Vec, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off[p], 0, 0));
 }
 
 template <typename T, int WT, bool KC>
@@ -296,9 +300,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
 
     if (!EDGE) {
         // Two register sets: while slab t is multiplied out of LDS, slab t+1 waits in one set and the loads
-        // of slab t+2 are issued into the other, so a global load has two slabs of MFMAs to arrive
-        // (measured +5 % at N = 4096 over a prefetch distance of one slab).  The loop is unrolled by two so
-        // that the sets are named statically.
+        // of slab t+2 are issued into the other, so a global load has two slabs of MFMAs to arrive.  The loop
+        // is unrolled by two so that the sets are named statically.
         Vec ra0[NV], rb0[NV], ra1[NV], rb1[NV];
         unsigned offa[NV], offb[NV];
         slab_offsets<T, WT, A_KC>(offa, p.lda, tid, (int)min((int64_t)BM, p.M - row0));
@@ -310,44 +313,56 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         const T* __restrict__ ub = B + (GATHER ? (int64_t)tn * (BN / 4) : (B_KC ? col0 * p.ldb : col0));
         const int64_t stepa = A_KC ? (int64_t)BK : (int64_t)BK * p.lda;
         const int64_t stepb = B_KC ? (int64_t)BK : (int64_t)BK * p.ldb;
+        // The loads inside the loop stand in straight-line code: at a branch around a load the compiler loses count
+        // of the loads in flight and from then on waits for all of them before every use, which undoes the prefetch.
+        // The loop therefore runs while both slabs it fetches exist, and the last one to three slabs drain after it.
         if (ntiles > 0) {
             load_slab_fast<T>(ra0, ua, offa);
             load_slab_fast<T>(rb0, ub, offb);
-        }
-        if (ntiles > 1) {
-            load_slab_fast<T>(ra1, ua + stepa, offa);
-            load_slab_fast<T>(rb1, ub + stepb, offb);
-        }
-        if (ntiles > 0) {
+            load_slab_fast<T>(ra1, ua + min(1, ntiles - 1) * stepa, offa);  // (the only slab twice if K holds just one)
+            load_slab_fast<T>(rb1, ub + min(1, ntiles - 1) * stepb, offb);
             store_slab<T, WT, A_KC>(smem[0], ra0, tid);
             store_slab<T, WT, B_KC>(smem[0] + SA, rb0, tid);
-        }
-        __syncthreads();
-        for (int kt = 0; kt + 1 < ntiles; kt += 2) {
-            // LDS stage 0 holds slab kt, set 1 holds slab kt+1 (in flight), set 0 is free.
+            __syncthreads();
+            int kt = 0;
+            for (; kt + 3 < ntiles; kt += 2) {
+                // LDS stage 0 holds slab kt, set 1 holds slab kt+1 (in flight), set 0 is free.
+                load_slab_fast<T>(ra0, ua + (kt + 2) * stepa, offa);
+                load_slab_fast<T>(rb0, ub + (kt + 2) * stepb, offb);
+                compute(smem[0]);
+                store_slab<T, WT, A_KC>(smem[1], ra1, tid);
+                store_slab<T, WT, B_KC>(smem[1] + SA, rb1, tid);
+                __syncthreads();
+                load_slab_fast<T>(ra1, ua + (kt + 3) * stepa, offa);
+                load_slab_fast<T>(rb1, ub + (kt + 3) * stepb, offb);
+                compute(smem[1]);
+                store_slab<T, WT, A_KC>(smem[0], ra0, tid);
+                store_slab<T, WT, B_KC>(smem[0] + SA, rb0, tid);
+                __syncthreads();
+            }
+            // left: slab kt in stage 0, slab kt+1 (if any) in set 1, slab kt+2 (if any) still to be fetched
             if (kt + 2 < ntiles) {
                 load_slab_fast<T>(ra0, ua + (kt + 2) * stepa, offa);
                 load_slab_fast<T>(rb0, ub + (kt + 2) * stepb, offb);
             }
             compute(smem[0]);
-            store_slab<T, WT, A_KC>(smem[1], ra1, tid);
-            store_slab<T, WT, B_KC>(smem[1] + SA, rb1, tid);
-            __syncthreads();
-            if (kt + 3 < ntiles) {
-                load_slab_fast<T>(ra1, ua + (kt + 3) * stepa, offa);
-                load_slab_fast<T>(rb1, ub + (kt + 3) * stepb, offb);
+            if (kt + 1 < ntiles) {
+                store_slab<T, WT, A_KC>(smem[1], ra1, tid);
+                store_slab<T, WT, B_KC>(smem[1] + SA, rb1, tid);
+                __syncthreads();
+                compute(smem[1]);
             }
-            compute(smem[1]);
             if (kt + 2 < ntiles) {
                 store_slab<T, WT, A_KC>(smem[0], ra0, tid);
                 store_slab<T, WT, B_KC>(smem[0] + SA, rb0, tid);
+                __syncthreads();
+                compute(smem[0]);
             }
-            __syncthreads();
         }
-        if (ntiles & 1) compute(smem[0]);  // an odd last slab was staged into stage 0
         if ((int64_t)ntiles * BK < K) {    // ragged end of K: one guarded slab through stage 1
             load_slab_guarded<T, WT, A_KC>(ra1, A, p.lda, row0, p.M, (int64_t)ntiles * BK, K, tid);
             load_slab_guarded<T, WT, B_KC>(rb1, B, p.ldb, col0, p.N, (int64_t)ntiles * BK, K, tid);
+            __syncthreads();  // every wavefront is done with the last whole slab, whichever stage held it
             store_slab<T, WT, A_KC>(smem[1], ra1, tid);
             store_slab<T, WT, B_KC>(smem[1] + SA, rb1, tid);
             __syncthreads();
@@ -708,8 +723,8 @@ static bool vector_loads_ok(const GemmArgs<T>& a, int epi, int BM) {
            (a.ldb % VEC == 0) && (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) && (a.strideA % VEC == 0) && (a.strideB % VEC == 0) &&
            (a.zstrideA % VEC == 0) && (a.zstrideB % VEC == 0) && (a.istrideA % VEC == 0) && (a.istrideB % VEC == 0) &&
-           // per-thread element offsets inside one tile's slab are kept in 32 bits
-           (a.lda < (1 << 23)) && (a.ldb < (1 << 23));
+           // per-thread byte offsets inside one tile's slab are kept in 32 bits
+           (a.lda < (1 << 21)) && (a.ldb < (1 << 21));
 }
 
 template <typename T, int WT>
@@ -942,7 +957,7 @@ template <typename T>
 static bool lstm_operands_aligned(const GemmArgs<T>& a) {
     constexpr int VEC = Mfma<T>::VEC;
     return a.lda % VEC == 0 && a.ldb % VEC == 0 && reinterpret_cast<uintptr_t>(a.A) % 16 == 0 &&
-           reinterpret_cast<uintptr_t>(a.B) % 16 == 0 && a.lda < (1 << 23) && a.ldb < (1 << 23) && a.batch == 1;
+           reinterpret_cast<uintptr_t>(a.B) % 16 == 0 && a.lda < (1 << 21) && a.ldb < (1 << 21) && a.batch == 1;
 }
 
 template <typename T>
