@@ -803,15 +803,19 @@ static int64_t slab_depth(TileShape t, int elem_size) {
 }
 
 // A product whose chosen tile yields between half and one and a half workgroups per compute unit leaves
-// workgroup slots empty (two fit per compute unit) and has nothing to hide a workgroup's barriers behind:
-// when K is long enough it runs as pairs of workgroups per tile.  PRAD_GEMM_PAIRS=0 switches this off.
+// workgroup slots empty (two fit per compute unit).  On the 64 x 64 and 32 x 32 tiles a lone workgroup has too
+// few MFMAs per fragment read to keep its compute unit busy, so with a K of 32 slabs or more such a product runs
+// as pairs of workgroups per tile (measured +4 to +20 %; at 16 slabs the exchange of the partial tiles costs
+// more than the pairing gains: -3 %).  The 128 x 128 tile keeps a compute unit busy on its own and only pays for
+// the exchange (-5 % at N = 2048 in double, -16 % on a 1024 x 4096 output): it never pairs.
+// PRAD_GEMM_PAIRS=0 switches pairing off.
 bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
     static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_PAIRS"); return !(e && e[0] == '0'); }();
     if (!enabled || gemm_split_factor(M, N, K, batch, elem_size) > 1) return false;
     const TileShape t = choose_tile(M, N, batch, false);
     const int64_t e = t == TILE_128x128 ? 128 : t == TILE_64x64 ? 64 : 32;
     const int64_t wgs = ((M + e - 1) / e) * ((N + e - 1) / e) * batch;
-    return wgs >= 128 && wgs <= GEMM_SPLIT_MAX_TILES && K >= 16 * slab_depth(t, elem_size);
+    return t != TILE_128x128 && wgs >= 128 && wgs <= GEMM_SPLIT_MAX_TILES && K >= 32 * slab_depth(t, elem_size);
 }
 
 // Adds the partial results of a split product in split order and applies the epilogue.

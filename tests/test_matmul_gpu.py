@@ -432,10 +432,11 @@ def test_both_gradients_in_one_launch(gpu, dtype, accumulate, shape):
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
-@pytest.mark.parametrize("shape", [(512, 2048, 512), (1024, 1024, 1024), (384, 2100, 500)])
+@pytest.mark.parametrize("shape", [(512, 2048, 512), (1024, 1024, 1024), (384, 2100, 500), (512, 4096, 512)])
 def test_products_run_as_workgroup_pairs(gpu, oracle, dtype, shape):
-    """Shapes whose tiles fill between half and one and a half of the chip's workgroup slots and whose K is
-    long run with two workgroups per tile (half of K each; the later one adds the other's partial tile):
+    """Shapes whose 64 x 64 or 32 x 32 tiles fill between half and one and a half of the chip's workgroup slots and
+    whose K holds at least 32 slabs (which of these shapes do depends on the element type) run with two workgroups
+    per tile (half of K each; the later one adds the other's partial tile):
     parity with the oracle for the forward and both backward layouts, fused epilogue included, and the same
     bits on every run, whichever workgroup of a pair arrives last."""
     from parallelreverseautodiff_amd.exceptions import check
