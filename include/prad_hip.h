@@ -87,7 +87,10 @@ int32_t prad_buf_copy(prad_buf_t dst, prad_buf_t src);
 int32_t prad_matmul_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t C);
 /* dA[M x K] = dC . B^T ; dB[K x N] = A^T . dC.  dA or dB may be NULL to skip that product.
  * accumulate_dA / accumulate_dB != 0 adds into the destination instead of overwriting it
- * (the dest += grad of OperationBase.AccumulateGradient, src/RMAD/OperationBase.cs:295-303). */
+ * (the dest += grad of OperationBase.AccumulateGradient, src/RMAD/OperationBase.cs:295-303).
+ * When both are requested for a small layer they may share one launch; the results are those of
+ * the two products computed one after the other, bit for bit (a dA that overlaps dC, A or dB in
+ * memory is always computed first, in a launch of its own). */
 int32_t prad_matmul_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB,
                         int32_t accumulate_dA, int32_t accumulate_dB);
 /* Forward with the next operations of the graph fused into the product's epilogue:
