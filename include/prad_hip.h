@@ -286,6 +286,12 @@ int32_t prad_adam(prad_buf_t w, prad_buf_t m, prad_buf_t v, prad_buf_t g, double
 int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, double min_value);
 int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
                         double lr, double beta1, double beta2, double eps, double t);
+/* AdamOptimizer.Revert -> ReverseAdamUpdate, src/RMAD/AdamOptimizer.cs:97-156 and :158-193: undoes the
+ * update that produced the given w, m, v from the given gradient, statement for statement
+ * (w += lr * mhat / (sqrt(vhat) + eps) from the current moments, then m = (m - (1 - beta1) g) / beta1,
+ * v = (v - (1 - beta2) g g) / beta2).  t is the AdamIteration of the update being undone. */
+int32_t prad_adam_revert_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
+                               double lr, double beta1, double beta2, double eps, double t);
 /* GradientClipper.Clip immediately followed by AdamOptimizer.Optimize over the same tensors, as every
  * training loop of the reference calls them
  * (examples/feedforward/ParallelReverseAutoDiff.FeedForwardExample/FeedForwardNeuralNetwork.cs:287-303): the clamping

@@ -262,8 +262,9 @@ struct TensorDesc {
 size_t clip_workspace_bytes(const int64_t* n, int ntensors);
 template <typename T> hipError_t launch_clip(const TensorDesc<T>* host_descs, int ntensors, void* workspace, T clip_value,
                                              T min_value, hipStream_t s);
+// reverse: AdamOptimizer.ReverseAdamUpdate instead of UpdateWeightWithAdam
 template <typename T> hipError_t launch_adam(const TensorDesc<T>* host_descs, int ntensors, T lr, T beta1, T beta2, T eps, T c1,
-                                             T c2, hipStream_t s);
+                                             T c2, bool reverse, hipStream_t s);
 template <typename T> hipError_t launch_clip_adam(const TensorDesc<T>* host_descs, int ntensors, void* workspace, T clip_value,
                                                   T min_value, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s);
 

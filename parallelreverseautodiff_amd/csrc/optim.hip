@@ -248,7 +248,17 @@ struct Clamp {
 template <typename T>
 struct AdamUpdate {
     T lr, beta1, beta2, omb1, omb2, c1, c2, eps;
+    int reverse;  // 0: UpdateWeightWithAdam; 1: ReverseAdamUpdate (src/RMAD/AdamOptimizer.cs:158-193), statement for statement
     __device__ __forceinline__ void operator()(T& w, T& m, T& v, T g) const {
+        if (reverse) {
+            const T mhat = c1 * m;
+            const T vhat = c2 * v;
+            const T red = lr * mhat / (sqrt(vhat) + eps);
+            w = w + red;
+            m = (m - (omb1 * g)) / beta1;
+            v = (v - ((omb2 * g) * g)) / beta2;
+            return;
+        }
         const T first = (beta1 * m) + (omb1 * g);
         const T second = (beta2 * v) + (omb2 * (g * g));
         const T mhat = c1 * first;
@@ -440,8 +450,8 @@ hipError_t launch_clip(const TensorDesc<T>* host, int nt, void* workspace, T cli
 }
 
 template <typename T>
-hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s) {
-    const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps};
+hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2, T eps, T c1, T c2, bool reverse, hipStream_t s) {
+    const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps, reverse ? 1 : 0};
     return launch_groups<T, false, true>(host, nt, nullptr, (T)0, (T)0, update, s);
 }
 
@@ -450,15 +460,15 @@ hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2
 template <typename T>
 hipError_t launch_clip_adam(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value, T lr, T beta1, T beta2,
                             T eps, T c1, T c2, hipStream_t s) {
-    const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps};
+    const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps, 0};
     return launch_groups<T, true, true>(host, nt, workspace, clip_value, min_value, update, s);
 }
 
 template hipError_t launch_clip<double>(const TensorDesc<double>*, int, void*, double, double, hipStream_t);
 template hipError_t launch_clip<float>(const TensorDesc<float>*, int, void*, float, float, hipStream_t);
-template hipError_t launch_adam<double>(const TensorDesc<double>*, int, double, double, double, double, double, double,
+template hipError_t launch_adam<double>(const TensorDesc<double>*, int, double, double, double, double, double, double, bool,
                                         hipStream_t);
-template hipError_t launch_adam<float>(const TensorDesc<float>*, int, float, float, float, float, float, float, hipStream_t);
+template hipError_t launch_adam<float>(const TensorDesc<float>*, int, float, float, float, float, float, float, bool, hipStream_t);
 template hipError_t launch_clip_adam<double>(const TensorDesc<double>*, int, void*, double, double, double, double, double, double,
                                              double, double, hipStream_t);
 template hipError_t launch_clip_adam<float>(const TensorDesc<float>*, int, void*, float, float, float, float, float, float, float,

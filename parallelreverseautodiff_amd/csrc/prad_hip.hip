@@ -1403,7 +1403,8 @@ int32_t prad_clip(prad_buf_t g, double clip_value, double min_value) { return pr
 
 // Shared by prad_adam_multi (clip == false) and prad_clip_adam_multi.
 static int32_t adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n, bool clip,
-                          double clip_value, double min_value, double lr, double beta1, double beta2, double eps, double t) {
+                          double clip_value, double min_value, double lr, double beta1, double beta2, double eps, double t,
+                          bool reverse = false) {
     REQUIRE_INIT();
     if (n < 0 || (n > 0 && (w == nullptr || m == nullptr || v == nullptr || g == nullptr))) return fail(PRAD_ERR_ARG, "bad tensor list");
     if (n == 0) return PRAD_OK;
@@ -1428,7 +1429,7 @@ static int32_t adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_b
             HIP_TRY(launch_clip_adam<double>(d.data(), n, CUR_WORKSPACE, clip_value, min_value, lr, beta1, beta2, eps, c1, c2, CUR_STREAM),
                     PRAD_ERR_LAUNCH);
         else
-            HIP_TRY(launch_adam<double>(d.data(), n, lr, beta1, beta2, eps, c1, c2, CUR_STREAM), PRAD_ERR_LAUNCH);
+            HIP_TRY(launch_adam<double>(d.data(), n, lr, beta1, beta2, eps, c1, c2, reverse, CUR_STREAM), PRAD_ERR_LAUNCH);
     } else {
         // PRADLite: every parameter is a float and PradMath.Pow(float, float) is (float)Math.Pow.
         const float b1 = (float)beta1, b2 = (float)beta2, tf = (float)t;
@@ -1441,7 +1442,7 @@ static int32_t adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_b
                                             (float)eps, c1, c2, CUR_STREAM),
                     PRAD_ERR_LAUNCH);
         else
-            HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, CUR_STREAM), PRAD_ERR_LAUNCH);
+            HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, reverse, CUR_STREAM), PRAD_ERR_LAUNCH);
     }
     return PRAD_OK;
 }
@@ -1449,6 +1450,11 @@ static int32_t adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_b
 int32_t prad_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n, double lr,
                         double beta1, double beta2, double eps, double t) {
     return adam_multi(w, m, v, g, n, false, 0.0, 0.0, lr, beta1, beta2, eps, t);
+}
+
+int32_t prad_adam_revert_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
+                               double lr, double beta1, double beta2, double eps, double t) {
+    return adam_multi(w, m, v, g, n, false, 0.0, 0.0, lr, beta1, beta2, eps, t, true);
 }
 
 int32_t prad_clip_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,

@@ -147,6 +147,14 @@ class AdamOptimizer:
 
     def Optimize(self, layers):
         """One Adam step on every (w, m, v, g) group of every layer, in place on the device."""
+        self._apply(layers, "prad_adam_multi")
+
+    def Revert(self, layers):
+        """Undoes the last update (src/RMAD/AdamOptimizer.cs:97-156): as in the reference, the gradients must still be
+        those of that update and Parameters.AdamIteration the iteration it was made with."""
+        self._apply(layers, "prad_adam_revert_multi")
+
+    def _apply(self, layers, entry_point):
         _ensure_initialized()
         w = _collect(layers, "Weight")
         if not w:
@@ -158,7 +166,7 @@ class AdamOptimizer:
         wb, mb, vb, gb = ([x.device() for x in xs] for xs in (w, m, v, g))
         for dtype in {b.dtype for b in wb}:
             idx = [i for i, b in enumerate(wb) if b.dtype == dtype]
-            check(_lib.load().prad_adam_multi(
+            check(getattr(_lib.load(), entry_point)(
                 handle_array([wb[i] for i in idx]), handle_array([mb[i] for i in idx]),
                 handle_array([vb[i] for i in idx]), handle_array([gb[i] for i in idx]), len(idx),
                 float(p.LearningRate), float(p.AdamBeta1), float(p.AdamBeta2), float(p.AdamEpsilon), float(p.AdamIteration)))

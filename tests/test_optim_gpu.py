@@ -107,6 +107,43 @@ def test_adam_matches_oracle_over_steps(gpu, oracle, dtype):
             assert_parity(layer[name, "SecondMoment"].to_numpy(), v, dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_adam_revert_matches_oracle_and_undoes_the_step(gpu, oracle, dtype):
+    """AdamOptimizer.Revert (src/RMAD/AdamOptimizer.cs:97-193) on the device: the same numbers as the oracle's
+    restatement of ReverseAdamUpdate, and, as its algebra promises, the weights and moments of the step before
+    (to rounding: the moments are divided by beta again, which amplifies their last bits by 1/beta)."""
+    params = NeuralNetworkParameters(lite=dtype == np.float32)
+    shapes = [(784, 256), (1, 256), (128, 10), (1, 1), (7, 4099)]
+    ws = [seeded.xavier(63, i, *s).astype(dtype) for i, s in enumerate(shapes)]
+    gs = [seeded.normal(64, i, s, 1.0, dtype) for i, s in enumerate(shapes)]
+    wm = [Matrix.from_numpy(w) for w in ws]
+    gm = [Matrix.from_numpy(g) for g in gs]
+    layer = layer_of(wm, gm)
+    opt = AdamOptimizer(params)
+    ref = [(w.copy(), np.zeros_like(w), np.zeros_like(w)) for w in ws]
+    before = None
+    for step in (1, 2, 3):
+        before = ref
+        params.AdamIteration = float(step)
+        opt.Optimize([layer])
+        ref = [oracle.adam(w, m, v, g, params.LearningRate, params.AdamBeta1, params.AdamBeta2, params.AdamEpsilon, float(step))
+               for (w, m, v), g in zip(ref, gs)]
+    opt.Revert([layer])  # AdamIteration is still 3: the iteration of the update being undone
+    undone = [oracle.adam(w, m, v, g, params.LearningRate, params.AdamBeta1, params.AdamBeta2, params.AdamEpsilon, 3.0, reverse=True)
+              for (w, m, v), g in zip(ref, gs)]
+    for i, ((w, m, v), (w2, m2, v2)) in enumerate(zip(undone, before)):
+        name = "W%d" % i
+        got = [layer[name, kind].to_numpy() for kind in ("Weight", "FirstMoment", "SecondMoment")]
+        for a, b in zip(got, (w, m, v)):
+            if dtype == np.float64:
+                assert np.array_equal(a, b)
+            else:
+                assert_parity(a, b, dtype)
+        tol = 1e-9 if dtype == np.float64 else 2e-3
+        for a, b in zip(got, (w2, m2, v2)):
+            assert rel_err(a, b) <= tol
+
+
 def test_many_tensors_cross_the_table_limit(gpu, oracle):
     """More tensors than one launch's descriptor table holds."""
     params = NeuralNetworkParameters()
