@@ -477,3 +477,37 @@ def test_products_run_as_workgroup_pairs(gpu, oracle, dtype, shape):
     assert_parity(first[2], oracle.leakyrelu_fwd(rZ, dtype(0.01)), dtype, "H")
     assert_parity(first[3], rdA, dtype, "dA", bound=dot_bound(dC, B.T, dtype))
     assert_parity(first[4], rdB, dtype, "dB", bound=dot_bound(A.T, dC, dtype))
+
+
+def test_operand_larger_than_four_gib(gpu):
+    """A 40000 x 30000 float operand (4.8 GB): tile bases lie beyond 2^32 bytes while the per-lane offsets inside a
+    slab stay 32-bit.  The operand is 40 copies of one 1000-row block, so every block of 1000 output rows of
+    A . B equals the first one, and that one the product taken in double; the same operand read mn-contiguously
+    (A^T . dC, dC with the same period) gives 40 times one block's contribution."""
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    block_rows, copies, K, N = 1000, 40, 30000, 64
+    M = block_rows * copies
+    block = seeded.uniform(97, 1, (block_rows, K), -1, 1, np.float32)
+    B = seeded.uniform(97, 2, (K, N), -1, 1, np.float32)
+    dblock = seeded.uniform(97, 3, (block_rows, N), -1, 1, np.float32)
+    A, dC = DeviceBuffer.alloc(np.float32, M, K), DeviceBuffer.alloc(np.float32, M, N)
+    for c in range(copies):
+        A.view_rows(c * block_rows, block_rows).upload(block)
+        dC.view_rows(c * block_rows, block_rows).upload(dblock)
+    bB = DeviceBuffer.alloc(np.float32, K, N)
+    bB.upload(B)
+    C, dB = DeviceBuffer.alloc(np.float32, M, N), DeviceBuffer.alloc(np.float32, K, N)
+    check(lib.prad_matmul_fwd(A.handle, bB.handle, C.handle))
+    check(lib.prad_gemm(1, 0, A.handle, dC.handle, dB.handle, 0))
+    got = C.download()
+    first = got[:block_rows]
+    ref = block.astype(np.float64) @ B.astype(np.float64)
+    assert np.max(np.abs(first - ref)) <= 1e-5 * np.max(np.abs(ref))
+    for c in (1, 17, 26, copies - 1):  # 1000 rows are not a multiple of the 128-row tile: compare within tolerance
+        assert np.max(np.abs(got[c * block_rows:(c + 1) * block_rows] - ref)) <= 1e-5 * np.max(np.abs(ref))
+    ref_dB = copies * (block.astype(np.float64).T @ dblock.astype(np.float64))
+    # (40000 float terms per entry that add up coherently, block after block: the rounding of the running sums
+    # is what the wider bar is for; a wrong tile base would be off by the size of the entries themselves)
+    assert np.max(np.abs(dB.download() - ref_dB)) <= 1e-4 * np.max(np.abs(ref_dB))
