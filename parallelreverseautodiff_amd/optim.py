@@ -102,6 +102,22 @@ class ModelLayer:
         self._load(items["Item2"], "FirstMoment")
         self._load(items["Item3"], "SecondMoment")
 
+    # ---- HDF5 files (src/RMAD/ModelLayer.cs:258-271): <path>.json names what is stored, <path>.hdf5 holds the rows
+    # of every weight, first moment and second moment.  Loading replaces the rows of the existing element objects.
+    _BINARY_GETS = (lambda e: e["Weight"], lambda e: e["FirstMoment"], lambda e: e["SecondMoment"])
+
+    def _ordered_elements(self):
+        return {i: self._elements[i] for i in self.Identifiers}
+
+    def SaveWeightsAndMomentsBinary(self, path):
+        from . import hdf5
+        if not hdf5.SerializeElements(path, self._ordered_elements(), self._BINARY_GETS):
+            self.SaveWeightsAndMoments(str(path) + ".json")
+
+    def LoadWeightsAndMomentsBinary(self, path):
+        from . import hdf5
+        hdf5.DeserializeElements(path, self._elements, self._BINARY_GETS)
+
     def GradientMatrix(self, identifier):
         return self[identifier, "Gradient"]
 

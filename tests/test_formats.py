@@ -1,7 +1,8 @@
 """Wire and file formats of Matrix / DeepMatrix / ModelLayer (host logic; no GPU):
 Matrix.Serialize byte layout (src/RMAD/Matrix.cs:856-877, read back by CudaBlas.cs:355-381 and
 Matrix.DeserializeToFlatArray :357-374), the Newtonsoft JSON of MatrixJsonConverter / DeepMatrixJsonConverter, and
-ModelLayer.SaveWeights / SaveWeightsAndMoments (src/RMAD/ModelLayer.cs:219-320).  The JSON reader is pinned by Matrix
+ModelLayer.SaveWeights / SaveWeightsAndMoments / SaveWeightsAndMomentsBinary (src/RMAD/ModelLayer.cs:219-320; the
+HDF5 files of src/Interprocess/HDF5Helper.cs).  The JSON reader is pinned by Matrix
 objects taken from the reference's own test data (tests/golden/reference_matrix_json.json)."""
 import json
 import os
@@ -10,6 +11,7 @@ import struct
 import numpy as np
 import pytest
 
+from parallelreverseautodiff_amd.exceptions import InvalidOperationException
 from parallelreverseautodiff_amd.matrix import DeepMatrix, Matrix
 from parallelreverseautodiff_amd.optim import ModelLayer
 
@@ -87,3 +89,75 @@ def test_model_layer_files_round_trip(tmp_path, dtype):
     only = ModelLayer().AddModelElementGroup("W", Matrix(5, 7, dtype))
     only.LoadWeights(wpath)
     assert np.array_equal(only["W", "Weight"].to_numpy(), src["W", "Weight"].to_numpy())
+
+
+# ---- HDF5 files (src/Interprocess/HDF5Helper.cs), through the HDF5 C library that the reference also calls ----
+def _hdf5():
+    from parallelreverseautodiff_amd import hdf5
+    from parallelreverseautodiff_amd.exceptions import InvalidOperationException
+    try:
+        hdf5.library()
+    except InvalidOperationException as e:
+        pytest.skip(str(e))
+    return hdf5
+
+
+def test_hdf5_rows_are_native_double_datasets(tmp_path):
+    hdf5 = _hdf5()
+    rng = np.random.default_rng(11)
+    a, b = rng.standard_normal((3, 5)), rng.standard_normal((2, 7))
+    path = str(tmp_path / "m.hdf5")
+    hdf5.Serialize(path, [Matrix.from_numpy(a), Matrix.from_numpy(b)])
+    raw = open(path, "rb").read()
+    assert raw[:8] == b"\x89HDF\r\n\x1a\n"
+    # Independent of the reader: every row lies in the file as contiguous little-endian doubles, and the
+    # datasets are named row0.. through both matrices.
+    for row in list(a) + list(b):
+        assert row.astype("<f8").tobytes() in raw
+    for n in range(5):
+        assert b"row%d\x00" % n in raw
+    assert b"row5\x00" not in raw
+    rows = hdf5.Deserialize(path)
+    assert [r.shape[0] for r in rows] == [5, 5, 5, 7, 7]
+    assert np.array_equal(np.stack(rows[:3]), a) and np.array_equal(np.stack(rows[3:]), b)
+    assert hdf5.Validate(path, [5, 5, 5, 7, 7]) and hdf5.Validate(path, [5, 5])     # fewer sizes than rows is valid
+    assert not hdf5.Validate(path, [5, 5, 5, 7, 8]) and not hdf5.Validate(path, [5, 5, 5, 7, 7, 7])
+    hdf5.Serialize(path, Matrix.from_numpy(a))                                        # truncates
+    assert len(hdf5.Deserialize(path)) == 3
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_model_layer_binary_files_round_trip(tmp_path, dtype):
+    hdf5 = _hdf5()
+    rng = np.random.default_rng(6)
+    mk = lambda *shape: rng.standard_normal(shape).astype(dtype)
+    src = ModelLayer()
+    src.AddModelElementGroup("W", Matrix.from_numpy(mk(5, 7)), None, Matrix.from_numpy(mk(5, 7)), Matrix.from_numpy(mk(5, 7)))
+    src.AddModelElementGroup("K", DeepMatrix.from_numpy(mk(3, 2, 4)), None, DeepMatrix.from_numpy(mk(3, 2, 4)), DeepMatrix.from_numpy(mk(3, 2, 4)))
+    path = str(tmp_path / "layer")
+    src.SaveWeightsAndMomentsBinary(path)
+    with open(path + ".json") as f:
+        meta = json.load(f)
+    # DataSet / DataSetItem as Newtonsoft writes them; rows are numbered through weight, first moment,
+    # second moment of each identifier in turn.
+    assert list(meta) == ["Items"] and len(meta["Items"]) == 6
+    assert [list(i) for i in meta["Items"]] == [["StartIndex", "Rows", "DeserializeKey", "TypeName"]] * 6
+    assert [(i["DeserializeKey"]["Item1"], i["DeserializeKey"]["Item2"]) for i in meta["Items"]] == \
+        [("W", 0), ("W", 1), ("W", 2), ("K", 0), ("K", 1), ("K", 2)]
+    assert [i["StartIndex"] for i in meta["Items"]] == [0, 5, 10, 15, 21, 27] and [i["Rows"] for i in meta["Items"]] == [5, 5, 5, 6, 6, 6]
+    assert [i["TypeName"] for i in meta["Items"]] == ["ParallelReverseAutoDiff.RMAD.Matrix"] * 3 + ["ParallelReverseAutoDiff.RMAD.DeepMatrix"] * 3
+    rows = hdf5.Deserialize(path + ".hdf5")
+    assert len(rows) == 33 and np.array_equal(np.stack(rows[5:10]), src["W", "FirstMoment"].to_numpy().astype(np.float64))
+    dst = ModelLayer()
+    dst.AddModelElementGroup("W", Matrix(5, 7, dtype))
+    dst.AddModelElementGroup("K", DeepMatrix(3, 2, 4, dtype))
+    kept = dst["K", "Weight"]
+    dst.LoadWeightsAndMomentsBinary(path)
+    assert dst["K", "Weight"] is kept                      # rows are replaced inside the existing objects
+    for ident in ("W", "K"):
+        for element in ("Weight", "FirstMoment", "SecondMoment"):
+            got, want = dst[ident, element], src[ident, element]
+            assert got.dtype == dtype and np.array_equal(got.to_numpy(), want.to_numpy())
+    wrong = ModelLayer().AddModelElementGroup("W", Matrix(5, 8, dtype)).AddModelElementGroup("K", DeepMatrix(3, 2, 4, dtype))
+    with pytest.raises(InvalidOperationException):
+        wrong.LoadWeightsAndMomentsBinary(path)
