@@ -129,6 +129,7 @@ __device__ __forceinline__ void sum_bwd_da_block(T (*tile)[TS + 1], const T* __r
 template <typename T> struct SumVec;
 template <> struct SumVec<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
 template <> struct SumVec<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
+constexpr int SUM_DA_DEPTH = 32;  // slices of the dA walk in flight per lane (32 x 16 bytes of registers)
 constexpr int Q_PER_WG_VEC = 4;  // the transposed tile stays in registers while it is scaled into this many slices
 
 template <typename T>
@@ -167,13 +168,30 @@ __device__ __forceinline__ void sum_bwd_db_block_vec(T (*tile)[TS + 1], const T*
     }
 }
 
-// 16 vectors (i) x 16 rows (j) of dA^T per workgroup; eight slices' loads are in flight before their ordered additions.
+// DEPTH slices of one (i, j) vector are loaded before their additions, which stay in ascending slice order.
+template <typename T, int DEPTH>
+__device__ __forceinline__ void sum_da_slices(typename SumVec<T>::type& acc, const T* __restrict__ src, int64_t slice,
+                                              const T* __restrict__ dOut, int64_t q, bool inside) {
+    typedef typename SumVec<T>::type V;
+    V b[DEPTH];
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+        if (inside) b[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + (q + u) * slice));
+        else b[u] = (V)(T)0;
+    }
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) acc = acc + (b[u] * dOut[q + u]);
+}
+
+// 16 vectors (i) x 16 rows (j) of dA^T per workgroup.  The walk over the slices is a chain of load latencies,
+// so up to SUM_DA_DEPTH slices are in flight at a time (all of them at the usual slice counts), and what is
+// left over goes in halving groups rather than one by one.
 template <typename T>
 __device__ __forceinline__ void sum_bwd_da_block_vec(T (*tile)[TS + 1], const T* __restrict__ B, const T* __restrict__ dOut,
                                                      T* __restrict__ dA, int64_t M, int64_t K, int64_t N, int64_t P, int64_t bx,
                                                      int64_t by) {
     typedef typename SumVec<T>::type V;
-    constexpr int VEC = SumVec<T>::N, IW = 16 * VEC, DEPTH = 8;
+    constexpr int VEC = SumVec<T>::N, IW = 16 * VEC;
     const int64_t i0 = bx * IW, j0 = by * TJ;
     const int t = threadIdx.x, jr = t >> 4, iv = (t & 15) * VEC;
     const int64_t i = i0 + iv, j = j0 + jr;
@@ -182,21 +200,12 @@ __device__ __forceinline__ void sum_bwd_da_block_vec(T (*tile)[TS + 1], const T*
     const int64_t slice = K * N;
     V acc = (V)(T)0;
     int64_t q = 0;
-    for (; q + DEPTH <= P; q += DEPTH) {
-        V b[DEPTH];
-#pragma unroll
-        for (int u = 0; u < DEPTH; ++u) {
-            if (inside) b[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + (q + u) * slice));
-            else b[u] = (V)(T)0;
-        }
-#pragma unroll
-        for (int u = 0; u < DEPTH; ++u) acc = acc + (b[u] * dOut[q + u]);
-    }
-    for (; q < P; ++q) {
-        V b = (V)(T)0;
-        if (inside) b = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + q * slice));
-        acc = acc + (b * dOut[q]);
-    }
+    for (; q + SUM_DA_DEPTH <= P; q += SUM_DA_DEPTH) sum_da_slices<T, SUM_DA_DEPTH>(acc, src, slice, dOut, q, inside);
+    if (SUM_DA_DEPTH > 16 && q + 16 <= P) { sum_da_slices<T, 16>(acc, src, slice, dOut, q, inside); q += 16; }
+    if (SUM_DA_DEPTH > 8 && q + 8 <= P) { sum_da_slices<T, 8>(acc, src, slice, dOut, q, inside); q += 8; }
+    if (q + 4 <= P) { sum_da_slices<T, 4>(acc, src, slice, dOut, q, inside); q += 4; }
+    if (q + 2 <= P) { sum_da_slices<T, 2>(acc, src, slice, dOut, q, inside); q += 2; }
+    if (q < P) sum_da_slices<T, 1>(acc, src, slice, dOut, q, inside);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) tile[jr][iv + e] = acc[e];
     __syncthreads();

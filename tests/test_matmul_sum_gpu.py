@@ -24,7 +24,8 @@ def check_forward(out, A, B, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", [(6, 9, 3), (64, 96, 5), (130, 70, 4), (128, 256, 8), (100, 36, 9), (68, 200, 13)])
+@pytest.mark.parametrize("shape", [(6, 9, 3), (64, 96, 5), (130, 70, 4), (128, 256, 8), (100, 36, 9), (68, 200, 13),
+                                   (64, 96, 31), (32, 48, 47), (16, 32, 63), (64, 64, 32), (8, 16, 1)])
 def test_forward_backward(gpu, oracle, dtype, shape):
     M, K, P = shape
     A = seeded.normal(81, 1, (M, K), 1.0, dtype)
