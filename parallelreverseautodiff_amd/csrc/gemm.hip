@@ -220,7 +220,11 @@ struct GridPos {
 };
 
 // One workgroup's share of one product (a tile, or the column-sum rider).
-template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI>
+// SHORT: thousands of small products whose K is a slab or less (the attention products of a windowed block,
+// K = 32 or 49).  Software pipelining has nothing to work with there, so the kernel keeps one LDS stage instead
+// of two and no prefetch registers: more workgroups share a compute unit and overlap one another's loads,
+// products and stores.  It multiplies only the k steps that the last slab has.
+template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI, bool SHORT = false>
 __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM, const int tilesN, const GridPos g_) {
     typedef Mfma<T> MF;
     typedef Slab<T, WT> S;
@@ -232,7 +236,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     constexpr int WTM = WT, WTN = WT;
     constexpr int SA = S::template elems<A_KC>(), SB = S::template elems<B_KC>();
 
-    __shared__ __attribute__((aligned(16))) T smem[2][SA + SB];  // [stage][A slab | B slab]
+    static_assert(!SHORT || (EDGE && EPI == EPI_PLAIN), "the single-stage kernel is guarded and stores plainly");
+    __shared__ __attribute__((aligned(16))) T smem[SHORT ? 1 : 2][SA + SB];  // [stage][A slab | B slab]
 
     // Workgroups beyond the tiles carry a column sum that rides along with this launch.
     if (g_.bx >= (unsigned)(tilesM * tilesN)) {
@@ -298,7 +303,36 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         __builtin_amdgcn_s_setprio(0);
     };
 
-    if (!EDGE) {
+    if (SHORT) {
+        // One LDS stage and no prefetch: the loads of a slab are hidden by the other workgroups of the compute unit.
+        Vec ra[NV], rb[NV];
+        const int nslabs = (int)((K + BK - 1) / BK);  // one where the launch rules send products here
+        for (int kt = 0; kt < nslabs; ++kt) {
+            const int64_t k0 = (int64_t)kt * BK;
+            load_slab_guarded<T, WT, A_KC>(ra, A, p.lda, row0, p.M, k0, K, tid);
+            load_slab_guarded<T, WT, B_KC>(rb, B, p.ldb, col0, p.N, k0, K, tid);
+            if (kt > 0) __syncthreads();  // every wavefront is done with the slab before
+            store_slab<T, WT, A_KC>(smem[0], ra, tid);
+            store_slab<T, WT, B_KC>(smem[0] + SA, rb, tid);
+            __syncthreads();
+            const T* __restrict__ sA = smem[0];
+            const T* __restrict__ sB = smem[0] + SA;
+            const int ksteps = (int)((min((int64_t)BK, K - k0) + 3) / 4);  // the slab is zero beyond K
+#pragma unroll 2
+            for (int s = 0; s < ksteps; ++s) {
+                const int k = 4 * s + g;
+                T a[WTM], b[WTN];
+#pragma unroll
+                for (int x = 0; x < WTM; ++x) a[x] = slab_at<T, WT, A_KC>(sA, wm * WS + x * 16 + li, k);
+#pragma unroll
+                for (int y = 0; y < WTN; ++y) b[y] = slab_at<T, WT, B_KC>(sB, wn * WS + y * 16 + li, k);
+#pragma unroll
+                for (int x = 0; x < WTM; ++x)
+#pragma unroll
+                    for (int y = 0; y < WTN; ++y) acc[x][y] = MF::run(a[x], b[y], acc[x][y]);
+            }
+        }
+    } else if (!EDGE) {
         // Two register sets: while slab t is multiplied out of LDS, slab t+1 waits in one set and the loads
         // of slab t+2 are issued into the other, so a global load has two slabs of MFMAs to arrive.  The loop
         // is unrolled by two so that the sets are named statically.
@@ -676,6 +710,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(cons
     gemm_tile<T, WT, A_KC, B_KC, EDGE, EPI>(p, tilesM, tilesN, GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z});
 }
 
+template <typename T, int WT, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(GEMM_THREADS, 4) gemm_short_kernel(const GemmArgs<T> p, const int tilesM, const int tilesN) {
+    gemm_tile<T, WT, A_KC, B_KC, true, EPI_PLAIN, true>(p, tilesM, tilesN,
+                                                        GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z});
+}
+
 // The two gradient products of a layer, dA = dC . B^T (both operands k-contiguous; the upstream activation's
 // backward may be its epilogue) and dB = A^T . dC (both operands mn-contiguous; the bias gradient may ride along),
 // in one launch on 32 x 32 tiles: small layers cost what their chain of dependent launches costs.  Workgroups
@@ -690,6 +730,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_pair_kernel(const GemmAr
     else gemm_tile<T, 1, false, false, EDGE2, EPI_PLAIN>(p2, tilesM2, tilesN2, GridPos{blockIdx.x - first, 0u, 0u, 1u, 1u});
 }
 
+// Which products go to the single-stage kernel (PRAD_GEMM_SHORT=0 switches it off: tuning aid): batches of small
+// products whose K fits one slab.  (128 x 128 tiles of three K slabs, a thousand of them, were measured on it too,
+// three workgroups to a compute unit: 10 to 25 % slower than the pipelined kernel at two.)
+template <typename T, int WT>
+static bool gemm_short_eligible(const GemmArgs<T>& a, int epi) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_SHORT"); return !(e && e[0] == '0'); }();
+    return enabled && WT != 4 && epi == EPI_PLAIN && a.ksplit == 0 && a.colsum_dst == nullptr && a.K <= Slab<T, WT>::BK &&
+           a.batch >= 64;
+}
+
 template <typename T, int WT, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStream_t stream) {
     constexpr int BM = 32 * WT;
@@ -697,6 +747,12 @@ static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStr
     const unsigned splits = a.ksplit > 0 ? (unsigned)((a.K + a.ksplit - 1) / a.ksplit) : 1u;
     const unsigned riders = a.colsum_dst != nullptr ? (unsigned)((a.colsum_cols + 63) / 64) : 0u;
     dim3 grid((unsigned)(tilesM * tilesN) + riders, (unsigned)a.batch, splits), block(GEMM_THREADS, 1, 1);
+    if constexpr (WT != 4) {
+        if (gemm_short_eligible<T, WT>(a, epi)) {
+            hipLaunchKernelGGL((gemm_short_kernel<T, WT, A_KC, B_KC>), grid, block, 0, stream, a, tilesM, tilesN);
+            return hipGetLastError();
+        }
+    }
 #define PRAD_LAUNCH(EDGE_, EPI_) \
     hipLaunchKernelGGL((gemm_kernel<T, WT, A_KC, B_KC, EDGE_, EPI_>), grid, block, 0, stream, a, tilesM, tilesN)
     if (edge) {
