@@ -608,6 +608,26 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         auto vec_aligned = [](const void* q, int64_t ld) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) % 16 == 0 && ld % VEC == 0); };
         const bool vec_ok = p.N % VEC == 0 && vec_aligned(C, p.ldc) && vec_aligned(p.Z, p.ldz) && vec_aligned(p.act_src, p.ld_act) &&
                             vec_aligned(p.bias, VEC);
+        // Each wavefront stages, reads back and stores its own share, so the passes are ordered inside the wavefront
+        // only: a workgroup barrier here would also make every pass wait for the global stores of the pass before.
+        auto wave_sync = [] {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        };
+        // The values act' is taken of, for one pass: all its loads are issued together, and a pass ahead, so that
+        // they are in flight during the arithmetic and the stores of the pass before.
+        constexpr int SRC_N = 16 * WS / 64;
+        T src[SRC_N];
+        auto fetch_src = [&](int x) {
+#pragma unroll
+            for (int it = 0; it < SRC_N; ++it) {
+                const int idx = lane + 64 * it, rr = idx / WS, c = idx % WS;
+                const int64_t i = row0 + wm * WS + x * 16 + rr, j = col0 + wn * WS + c;
+                src[it] = (i < p.M && j < p.N) ? p.act_src[i * p.ld_act + j] : (T)0;
+            }
+        };
+        if (p.act_bwd != ACT_NONE) fetch_src(0);
 #pragma unroll
         for (int x = 0; x < WTM; ++x) {
 #pragma unroll
@@ -615,22 +635,15 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
 #pragma unroll
                 for (int r = 0; r < 4; ++r) stage[MF::row(r, g) * LDW + y * 16 + li] = acc[x][y][r];
             if (p.act_bwd != ACT_NONE) {
-                // All loads of this pass are issued together (one memory latency instead of one per iteration of
-                // the loop below); each lane parks what it will need in LDS at the position it reads back itself.
-                T src[16 * WS / 64];
+                // each lane parks what it fetched in LDS at the position it was fetched for
 #pragma unroll
-                for (int it = 0; it < 16 * WS / 64; ++it) {
-                    const int idx = lane + 64 * it, rr = idx / WS, c = idx % WS;
-                    const int64_t i = row0 + wm * WS + x * 16 + rr, j = col0 + wn * WS + c;
-                    src[it] = (i < p.M && j < p.N) ? p.act_src[i * p.ld_act + j] : (T)0;
-                }
-#pragma unroll
-                for (int it = 0; it < 16 * WS / 64; ++it) {
+                for (int it = 0; it < SRC_N; ++it) {
                     const int idx = lane + 64 * it;
                     side[(idx / WS) * LDW + idx % WS] = src[it];
                 }
+                if (x + 1 < WTM) fetch_src(x + 1);
             }
-            __syncthreads();
+            wave_sync();
             if (vec_ok) {
                 // 16 bytes per lane and access: whole rows of the tile leave in 1 KiB pieces.
 #pragma unroll 1
@@ -663,7 +676,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                     }
                     *c_out = v;
                 }
-                __syncthreads();
+                wave_sync();
                 continue;
             }
 #pragma unroll 1
@@ -681,7 +694,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                 if (p.accumulate) v = *c_out + v;
                 *c_out = v;
             }
-            __syncthreads();
+            wave_sync();
         }
         return;
     }
