@@ -451,6 +451,7 @@ def main():
     ap.add_argument("--n", type=int, default=4096)
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-also", action="store_true", help="gemm mode: skip the other-precision and MLP legs")
     ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum", "lstm", "swin", "oneshot"], default="gemm",
                     help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
                          "mlp: the feed-forward training step of configs[0]")
@@ -531,9 +532,34 @@ def main():
                      ("double" if args.dtype == "f64" else "float"), "launch_ms": launch_ms},
         "wall_ms_per_step": wall_ms / args.steps, "spot_check_error": spot,
     }
+    if not args.no_also:
+        line["also"] = also_legs(args)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_leg()
     print(json.dumps(line))
+
+
+def also_legs(args):
+    """The rest of the metric beside the headline figure, measured in the same run: the product in the other
+    precision at the same size, and the MLP training step of configs[0] (recorded launch sequence).  A leg
+    that fails is reported as its error text and does not touch the headline figures."""
+    out = {}
+    other = "f32" if args.dtype == "f64" else "f64"
+    try:
+        ms, _, spot = gpu_leg(args.n, other, args.steps, args.warmup)
+        tf = 6.0 * args.n ** 3 / (ms / args.steps * 1e-3) / 1e12
+        out["matmul_fwd_bwd_" + other] = {"TFLOPs": tf, "frac_of_mfma_peak": tf / PEAK_TFLOPS[other], "n": args.n,
+                                          "ms_per_step": ms / args.steps, "spot_check_error": spot}
+    except Exception as e:  # noqa: BLE001 - reported, not hidden
+        out["matmul_fwd_bwd_" + other] = {"error": repr(e)}
+    for d in ("f64", "f32"):
+        try:
+            r = mlp_leg(d, 1000, 100, False)
+            out["mlp_train_steps_per_s_" + d] = {"value": 1e3 / r["recorded_ms_per_step"], "ms_per_step": r["recorded_ms_per_step"],
+                                                 "loss_after": r["loss_after"]}
+        except Exception as e:  # noqa: BLE001
+            out["mlp_train_steps_per_s_" + d] = {"error": repr(e)}
+    return out
 
 
 if __name__ == "__main__":
