@@ -212,6 +212,12 @@ int32_t prad_layernorm_bwd(prad_buf_t x, prad_buf_t mean, prad_buf_t stddev, pra
 /* Row-wise softmax, src/RMAD/SoftmaxOperation.cs:45-110 (backward: dx = J^T . dy per row). */
 int32_t prad_softmax_fwd(prad_buf_t x, prad_buf_t y);
 int32_t prad_softmax_bwd(prad_buf_t y, prad_buf_t dy, prad_buf_t dx);
+/* MatrixMultiplyScalarOperation followed by SoftmaxOperation in one pass, as attention scores take them
+ * (src/RMAD/MatrixMultiplyScalarOperation.cs, src/RMAD/SoftmaxOperation.cs:45-110): y = softmax(alpha * x) and,
+ * backward through both, dx = alpha * (J^T . dy).  Same values as prad_scale + prad_softmax_fwd and
+ * prad_softmax_bwd + prad_scale. */
+int32_t prad_softmax_scaled_fwd(prad_buf_t x, double alpha, prad_buf_t y);
+int32_t prad_softmax_scaled_bwd(prad_buf_t y, prad_buf_t dy, double alpha, prad_buf_t dx);
 /* Categorical cross-entropy, src/RMAD/Loss/CategoricalCrossEntropyLossOperation.cs:37-86:
  * loss (1 x 1) = sum(-t * log(p + 1e-15)) / rows ; dp = -(1/rows) * t / (p + 1e-15). */
 int32_t prad_cce_fwd(prad_buf_t p, prad_buf_t target, prad_buf_t loss);

@@ -88,6 +88,8 @@ SIGNATURES = {
     "prad_layernorm_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp]),
     "prad_softmax_fwd": (_i32, [_vp, _vp]),
     "prad_softmax_bwd": (_i32, [_vp, _vp, _vp]),
+    "prad_softmax_scaled_fwd": (_i32, [_vp, _f64, _vp]),
+    "prad_softmax_scaled_bwd": (_i32, [_vp, _vp, _f64, _vp]),
     "prad_cce_fwd": (_i32, [_vp, _vp, _vp]),
     "prad_cce_bwd": (_i32, [_vp, _vp, _vp]),
     "prad_mse_fwd": (_i32, [_vp, _vp, _vp]),

@@ -269,8 +269,8 @@ template <typename T> hipError_t launch_clip_adam(const TensorDesc<T>* host_desc
                                                   T min_value, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s);
 
 // softmax / categorical cross-entropy (csrc/loss.hip)
-template <typename T> hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s);
-template <typename T> hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, hipStream_t s);
+template <typename T> hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, T alpha, hipStream_t s);
+template <typename T> hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, T alpha, hipStream_t s);
 template <typename T> hipError_t launch_softmax_cce(const T* x, const T* t, T* y, T* dy, T* dx, T* loss, unsigned* counter, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_cce_fwd(const T* p, const T* t, T* loss, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t cols, hipStream_t s);

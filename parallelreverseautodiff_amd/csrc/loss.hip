@@ -38,16 +38,17 @@ __device__ __forceinline__ double short_exp(double x) { return exp(x); }
 
 // y[i][j] = exp(x[i][j] - max_i) / sum_j exp(x[i][j] - max_i)
 template <typename T>
-__global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols) {
+__global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols,
+                                                         T alpha) {
     const int64_t i = blockIdx.x;
     const T* __restrict__ xr = x + i * cols;
     T* __restrict__ yr = y + i * cols;
     double mx = -INFINITY;
-    for (int64_t j = threadIdx.x; j < cols; j += 64) mx = fmax(mx, (double)xr[j]);
+    for (int64_t j = threadIdx.x; j < cols; j += 64) mx = fmax(mx, (double)(xr[j] * alpha));
     const T m = (T)wave_max(mx);
     double sum = 0.0;
     for (int64_t j = threadIdx.x; j < cols; j += 64) {
-        const T e = dev_exp(xr[j] - m);
+        const T e = dev_exp(xr[j] * alpha - m);
         yr[j] = e;
         sum += (double)e;
     }
@@ -60,13 +61,14 @@ __global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x
 // leaves the memory system idle).  Each row is read once and written once.
 constexpr int SHORT_ROWS = 8;
 template <typename T>
-__global__ void __launch_bounds__(256) softmax_fwd_short_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols) {
+__global__ void __launch_bounds__(256) softmax_fwd_short_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols,
+                                                                T alpha) {
     const int64_t i0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * SHORT_ROWS;
     const int lane = threadIdx.x & 63;
     const bool on = lane < cols;
     T xv[SHORT_ROWS];
 #pragma unroll
-    for (int r = 0; r < SHORT_ROWS; ++r) xv[r] = (on && i0 + r < rows) ? x[(i0 + r) * cols + lane] : (T)0;
+    for (int r = 0; r < SHORT_ROWS; ++r) xv[r] = (on && i0 + r < rows) ? x[(i0 + r) * cols + lane] * alpha : (T)0;
 #pragma unroll
     for (int r = 0; r < SHORT_ROWS; ++r) {
         if (i0 + r >= rows) break;
@@ -78,7 +80,7 @@ __global__ void __launch_bounds__(256) softmax_fwd_short_kernel(const T* __restr
 }
 template <typename T>
 __global__ void __launch_bounds__(256) softmax_bwd_short_kernel(const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx,
-                                                                int64_t rows, int64_t cols) {
+                                                                int64_t rows, int64_t cols, T alpha) {
     const int64_t i0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * SHORT_ROWS;
     const int lane = threadIdx.x & 63;
     const bool on = lane < cols;
@@ -93,22 +95,57 @@ __global__ void __launch_bounds__(256) softmax_bwd_short_kernel(const T* __restr
     for (int r = 0; r < SHORT_ROWS; ++r) {
         if (i0 + r >= rows) break;
         const T dot = wave_sum_t(on ? gv[r] * yv[r] : (T)0);
-        if (on) dx[(i0 + r) * cols + lane] = yv[r] * (gv[r] - dot);
+        if (on) dx[(i0 + r) * cols + lane] = (yv[r] * (gv[r] - dot)) * alpha;
     }
+}
+
+// Many short rows (the attention scores of a windowed block: 150 528 rows of 49): a lane owns a whole row, so no
+// reduction crosses lanes and the sum runs over the columns in ascending order, as the reference's does.  The
+// workgroup's rows are contiguous in memory: they come in and go out as one coalesced block through LDS, where
+// the odd row pitch keeps the lanes' column-by-column walk free of bank conflicts.
+template <typename T> struct RowsPerGroup { static constexpr int N = sizeof(T) == 4 ? 256 : 128; };
+template <typename T>
+__global__ void __launch_bounds__(256) softmax_fwd_rows_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols,
+                                                               T alpha) {
+    constexpr int RPG = RowsPerGroup<T>::N;
+    extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
+    T* __restrict__ tile = reinterpret_cast<T*>(rows_lds);
+    const int pitch = (int)cols | 1;
+    const int64_t i0 = (int64_t)blockIdx.x * RPG;
+    const int nrows = (int)min((int64_t)RPG, rows - i0);
+    const int n = nrows * (int)cols;
+    const T* __restrict__ src = x + i0 * cols;
+    T* __restrict__ dst = y + i0 * cols;
+    for (int e = threadIdx.x; e < n; e += 256) tile[(e / (int)cols) * pitch + e % (int)cols] = src[e] * alpha;
+    __syncthreads();
+    if ((int)threadIdx.x < nrows) {
+        T* __restrict__ row = tile + threadIdx.x * pitch;
+        T m = row[0];
+        for (int j = 1; j < (int)cols; ++j) m = row[j] > m ? row[j] : m;
+        T sum = (T)0;
+        for (int j = 0; j < (int)cols; ++j) {
+            const T e = short_exp(row[j] - m);
+            row[j] = e;
+            sum = sum + e;
+        }
+        for (int j = 0; j < (int)cols; ++j) row[j] = row[j] / sum;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < n; e += 256) dst[e] = tile[(e / (int)cols) * pitch + e % (int)cols];
 }
 
 // The reference multiplies dy with the explicit Jacobian row by row (O(cols^2)):
 //   dx[j] = dy[j]*y[j]*(1-y[j]) - sum_{k != j} dy[k]*y[j]*y[k]  =  y[j] * (dy[j] - sum_k dy[k]*y[k]).
 template <typename T>
 __global__ void __launch_bounds__(64) softmax_bwd_kernel(const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dx,
-                                                         int64_t rows, int64_t cols) {
+                                                         int64_t rows, int64_t cols, T alpha) {
     const int64_t i = blockIdx.x;
     const T* __restrict__ yr = y + i * cols;
     const T* __restrict__ gr = dy + i * cols;
     double dot = 0.0;
     for (int64_t j = threadIdx.x; j < cols; j += 64) dot += (double)gr[j] * (double)yr[j];
     dot = wave_sum(dot);
-    for (int64_t j = threadIdx.x; j < cols; j += 64) dx[i * cols + j] = (T)((double)yr[j] * ((double)gr[j] - dot));
+    for (int64_t j = threadIdx.x; j < cols; j += 64) dx[i * cols + j] = (T)((double)yr[j] * ((double)gr[j] - dot)) * alpha;
 }
 
 // loss[0] = (sum_ij -t*log(p + 1e-15)) / rows ; one workgroup.
@@ -265,26 +302,34 @@ hipError_t launch_mse_bwd(const T* y, const T* t, T* dy, int64_t n, hipStream_t 
     return hipGetLastError();
 }
 
+// alpha: y = softmax(alpha * x) and dx = alpha * (J^T dy), the scaled scores of an attention block without a pass
+// of their own; alpha = 1 is the plain operation (a multiplication by one changes no value).
 template <typename T>
-hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, hipStream_t s) {
-    if (rows <= 0) return hipSuccess;
-    if (cols <= 64) {
-        hipLaunchKernelGGL((softmax_fwd_short_kernel<T>), dim3((unsigned)((rows + 4 * SHORT_ROWS - 1) / (4 * SHORT_ROWS))), dim3(256), 0, s, x, y,
-                           rows, cols);
+hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, T alpha, hipStream_t s) {
+    if (rows <= 0 || cols <= 0) return hipSuccess;
+    constexpr int RPG = RowsPerGroup<T>::N;
+    if (cols <= 64 && rows >= 16 * RPG) {  // enough rows to fill the chip a lane per row
+        const size_t lds = (size_t)RPG * ((size_t)cols | 1) * sizeof(T);
+        hipLaunchKernelGGL((softmax_fwd_rows_kernel<T>), dim3((unsigned)((rows + RPG - 1) / RPG)), dim3(256), lds, s, x, y, rows, cols, alpha);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL((softmax_fwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, x, y, rows, cols);
+    if (cols <= 64) {
+        hipLaunchKernelGGL((softmax_fwd_short_kernel<T>), dim3((unsigned)((rows + 4 * SHORT_ROWS - 1) / (4 * SHORT_ROWS))), dim3(256), 0, s, x, y,
+                           rows, cols, alpha);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL((softmax_fwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, x, y, rows, cols, alpha);
     return hipGetLastError();
 }
 template <typename T>
-hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, hipStream_t s) {
+hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, T alpha, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
     if (cols <= 64) {
         hipLaunchKernelGGL((softmax_bwd_short_kernel<T>), dim3((unsigned)((rows + 4 * SHORT_ROWS - 1) / (4 * SHORT_ROWS))), dim3(256), 0, s, y, dy,
-                           dx, rows, cols);
+                           dx, rows, cols, alpha);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, y, dy, dx, rows, cols);
+    hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3((unsigned)rows), dim3(64), 0, s, y, dy, dx, rows, cols, alpha);
     return hipGetLastError();
 }
 // counter: one unsigned in device memory that is zero between launches (not shared with a launch that may
@@ -312,8 +357,8 @@ hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t c
 }
 
 #define INSTANTIATE(T)                                                                              \
-    template hipError_t launch_softmax_fwd<T>(const T*, T*, int64_t, int64_t, hipStream_t);         \
-    template hipError_t launch_softmax_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t); \
+    template hipError_t launch_softmax_fwd<T>(const T*, T*, int64_t, int64_t, T, hipStream_t);         \
+    template hipError_t launch_softmax_bwd<T>(const T*, const T*, T*, int64_t, int64_t, T, hipStream_t); \
     template hipError_t launch_softmax_cce<T>(const T*, const T*, T*, T*, T*, T*, unsigned*, int64_t, int64_t, hipStream_t); \
     template hipError_t launch_cce_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
     template hipError_t launch_cce_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \

@@ -1112,28 +1112,33 @@ int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias) {
 }
 
 // ---------------------------------------------------------------------------------------------
-int32_t prad_softmax_fwd(prad_buf_t x, prad_buf_t y) {
+static int32_t softmax_fwd_scaled(prad_buf_t x, double alpha, prad_buf_t y) {
     REQUIRE_INIT();
     REQUIRE_BUF(x); REQUIRE_BUF(y);
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "softmax")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(x, launch_softmax_fwd<double>(D(x), D(y), x->depth * x->rows, x->cols, CUR_STREAM),
-             launch_softmax_fwd<float>(F(x), F(y), x->depth * x->rows, x->cols, CUR_STREAM));
+    DISPATCH(x, launch_softmax_fwd<double>(D(x), D(y), x->depth * x->rows, x->cols, alpha, CUR_STREAM),
+             launch_softmax_fwd<float>(F(x), F(y), x->depth * x->rows, x->cols, (float)alpha, CUR_STREAM));
     return PRAD_OK;
 }
 
-int32_t prad_softmax_bwd(prad_buf_t y, prad_buf_t dy, prad_buf_t dx) {
+static int32_t softmax_bwd_scaled(prad_buf_t y, prad_buf_t dy, double alpha, prad_buf_t dx) {
     REQUIRE_INIT();
     REQUIRE_BUF(y); REQUIRE_BUF(dy); REQUIRE_BUF(dx);
     if (int32_t st = same_dtype({y, dy, dx})) return st;
     if (int32_t st = same_shape(y, dy, "softmax backward")) return st;
     if (int32_t st = same_shape(y, dx, "softmax backward")) return st;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(y, launch_softmax_bwd<double>(D(y), D(dy), D(dx), y->depth * y->rows, y->cols, CUR_STREAM),
-             launch_softmax_bwd<float>(F(y), F(dy), F(dx), y->depth * y->rows, y->cols, CUR_STREAM));
+    DISPATCH(y, launch_softmax_bwd<double>(D(y), D(dy), D(dx), y->depth * y->rows, y->cols, alpha, CUR_STREAM),
+             launch_softmax_bwd<float>(F(y), F(dy), F(dx), y->depth * y->rows, y->cols, (float)alpha, CUR_STREAM));
     return PRAD_OK;
 }
+
+int32_t prad_softmax_fwd(prad_buf_t x, prad_buf_t y) { return softmax_fwd_scaled(x, 1.0, y); }
+int32_t prad_softmax_bwd(prad_buf_t y, prad_buf_t dy, prad_buf_t dx) { return softmax_bwd_scaled(y, dy, 1.0, dx); }
+int32_t prad_softmax_scaled_fwd(prad_buf_t x, double alpha, prad_buf_t y) { return softmax_fwd_scaled(x, alpha, y); }
+int32_t prad_softmax_scaled_bwd(prad_buf_t y, prad_buf_t dy, double alpha, prad_buf_t dx) { return softmax_bwd_scaled(y, dy, alpha, dx); }
 
 int32_t prad_cce_fwd(prad_buf_t p, prad_buf_t target, prad_buf_t loss) {
     REQUIRE_INIT();

@@ -85,8 +85,7 @@ class SwinBlock:
         hs = nw * wt * wt                 # scores are stored head-major: [head][window][wt][wt]
         # S = Q . K^T per window and head
         self._all_heads(0, 1, wt, wt, hd, self.QKV, 0, q3, wt * q3, hd, self.QKV, C, q3, wt * q3, hd, self.S, 0, wt, wt * wt, hs)
-        check(lib.prad_scale(self.S.handle, self.S.handle, self.scale))
-        check(lib.prad_softmax_fwd(self.S.handle, self.P.handle))
+        check(lib.prad_softmax_scaled_fwd(self.S.handle, self.scale, self.P.handle))   # P = softmax(S / sqrt(head dim))
         # O = P . V per window, written into each head's columns of O
         self._all_heads(0, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.QKV, 2 * C, q3, wt * q3, hd, self.O, 0, C, wt * C, hd)
         check(fused(self.O.handle, w["Wo"].handle, w["bo"].handle, None, self.Y1.handle, _lib.ACT_NONE, 0.0))
@@ -105,8 +104,7 @@ class SwinBlock:
         # dP = dO . V^T ; dV = P^T . dO
         self._all_heads(0, 1, wt, wt, hd, self.dO, 0, C, wt * C, hd, self.QKV, 2 * C, q3, wt * q3, hd, self.dP, 0, wt, wt * wt, hs)
         self._all_heads(1, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.dO, 0, C, wt * C, hd, self.dQKV, 2 * C, q3, wt * q3, hd)
-        check(lib.prad_softmax_bwd(self.P.handle, self.dP.handle, self.dS.handle))
-        check(lib.prad_scale(self.dS.handle, self.dS.handle, self.scale))
+        check(lib.prad_softmax_scaled_bwd(self.P.handle, self.dP.handle, self.scale, self.dS.handle))
         # dQ = dS . K ; dK = dS^T . Q
         self._all_heads(0, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, C, q3, wt * q3, hd, self.dQKV, 0, q3, wt * q3, hd)
         self._all_heads(1, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, 0, q3, wt * q3, hd, self.dQKV, C, q3, wt * q3, hd)

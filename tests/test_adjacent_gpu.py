@@ -102,3 +102,35 @@ def test_amplified_sigmoid_in_fused_product(gpu, oracle, dtype):
     rZ = oracle.add_broadcast_fwd(oracle.matmul_fwd(A, B), bias)
     assert_parity(Z.download(), rZ, dtype, "pre-activation")
     assert_parity(H.download(), oracle.amplified_sigmoid_fwd(rZ), dtype, "fused amplified sigmoid")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(37, 49), (5000, 49), (4100, 32), (4097, 64), (6000, 7), (2049, 1), (9, 200)])
+def test_scaled_softmax_forward_and_backward(gpu, oracle, dtype, shape):
+    """y = softmax(alpha x), dx = alpha J^T dy against the oracle's scale-then-softmax; few rows (a wavefront
+    per row), thousands of short rows (a lane per row, staged through LDS: even, odd and single-column pitches,
+    a last workgroup that is not full), rows wider than a wavefront; and bit for bit against the separate launches."""
+    lib = _lib.load()
+    rows, cols = shape
+    alpha = 1.0 / np.sqrt(32.0)
+    x = seeded.normal(31, 1, shape, 3.0, dtype)
+    dy = seeded.normal(31, 2, shape, 1.0, dtype)
+    X, Y, DY, DX = (DeviceBuffer.alloc(dtype, rows, cols) for _ in range(4))
+    X.upload(x); DY.upload(dy)
+    check(lib.prad_softmax_scaled_fwd(X.handle, alpha, Y.handle))
+    check(lib.prad_softmax_scaled_bwd(Y.handle, DY.handle, alpha, DX.handle))
+    y, dx = Y.download(), DX.download()
+    xs = x * dtype(alpha)                                  # MatrixMultiplyScalarOperation.Forward
+    ry = oracle.softmax_fwd(xs)
+    assert_parity(y, ry, dtype, "softmax(alpha x)")
+    assert np.all(np.abs(y.astype(np.float64).sum(axis=1) - 1.0) <= cols * np.finfo(dtype).eps * 4)
+    rdx = oracle.softmax_bwd(y, dy) * dtype(alpha)         # softmax backward, then the scalar's backward
+    assert_parity(dx, rdx, dtype, "alpha J^T dy")
+    # the separate launches
+    S, Y2, DX2 = (DeviceBuffer.alloc(dtype, rows, cols) for _ in range(3))
+    check(lib.prad_scale(X.handle, S.handle, alpha))
+    check(lib.prad_softmax_fwd(S.handle, Y2.handle))
+    assert np.array_equal(Y2.download(), y)
+    check(lib.prad_softmax_bwd(Y.handle, DY.handle, DX2.handle))
+    check(lib.prad_scale(DX2.handle, DX2.handle, alpha))
+    assert np.array_equal(DX2.download(), dx)
