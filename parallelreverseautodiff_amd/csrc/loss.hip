@@ -103,35 +103,87 @@ __global__ void __launch_bounds__(256) softmax_bwd_short_kernel(const T* __restr
 // reduction crosses lanes and the sum runs over the columns in ascending order, as the reference's does.  The
 // workgroup's rows are contiguous in memory: they come in and go out as one coalesced block through LDS, where
 // the odd row pitch keeps the lanes' column-by-column walk free of bank conflicts.
-template <typename T> struct RowsPerGroup { static constexpr int N = sizeof(T) == 4 ? 256 : 128; };
+template <typename T> struct RowsPerGroup { static constexpr int N = 1024 / sizeof(T); };  // 256 floats' rows, 128 doubles'
 template <typename T>
-__global__ void __launch_bounds__(256) softmax_fwd_rows_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols,
+__global__ void __launch_bounds__(256) softmax_fwd_rows_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols64,
                                                                T alpha) {
     constexpr int RPG = RowsPerGroup<T>::N;
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int U = RPG * 64 / VEC / 256;  // 16-byte vectors per thread that cover the largest block (64 columns)
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
     extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
     T* __restrict__ tile = reinterpret_cast<T*>(rows_lds);
-    const int pitch = (int)cols | 1;
+    const int cols = (int)cols64, pitch = cols | 1;
     const int64_t i0 = (int64_t)blockIdx.x * RPG;
     const int nrows = (int)min((int64_t)RPG, rows - i0);
-    const int n = nrows * (int)cols;
-    const T* __restrict__ src = x + i0 * cols;
+    const int n = nrows * cols, nvec = n / VEC;
+    const T* __restrict__ src = x + i0 * cols;   // 16-byte aligned: a block is RPG * cols elements, a multiple of 1 KiB
     T* __restrict__ dst = y + i0 * cols;
-    for (int e = threadIdx.x; e < n; e += 256) tile[(e / (int)cols) * pitch + e % (int)cols] = src[e] * alpha;
-    __syncthreads();
-    if ((int)threadIdx.x < nrows) {
-        T* __restrict__ row = tile + threadIdx.x * pitch;
-        T m = row[0];
-        for (int j = 1; j < (int)cols; ++j) m = row[j] > m ? row[j] : m;
-        T sum = (T)0;
-        for (int j = 0; j < (int)cols; ++j) {
-            const T e = short_exp(row[j] - m);
-            row[j] = e;
-            sum = sum + e;
+    // Element e of the block sits at row e / cols, column e % cols.  All of a thread's loads are issued before the
+    // first value is parked: taken a few at a time, the block would come in as a chain of memory latencies.
+    const int step = 256 * VEC, dr = step / cols, dc = step % cols;
+    const int e_first = (int)threadIdx.x * VEC;
+    {
+        Vec tmp[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if ((int)threadIdx.x + 256 * u < nvec) tmp[u] = *reinterpret_cast<const Vec*>(src + e_first + step * u);
+        int r = e_first / cols, c = e_first % cols;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if ((int)threadIdx.x + 256 * u < nvec) {
+                int rr = r, cc = c;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    tile[rr * pitch + cc] = tmp[u][k] * alpha;
+                    if (++cc == cols) { cc = 0; ++rr; }
+                }
+            }
+            r += dr; c += dc;
+            if (c >= cols) { c -= cols; ++r; }
         }
-        for (int j = 0; j < (int)cols; ++j) row[j] = row[j] / sum;
+        for (int e = nvec * VEC + threadIdx.x; e < n; e += 256) tile[(e / cols) * pitch + e % cols] = src[e] * alpha;  // ragged end
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < n; e += 256) dst[e] = tile[(e / (int)cols) * pitch + e % (int)cols];
+    if ((int)threadIdx.x < nrows) {
+        // the row lives in registers (rows here have at most 64 columns): independent LDS reads, one pass each way
+        T* __restrict__ row = tile + threadIdx.x * pitch;
+        T v[64];
+#pragma unroll
+        for (int j = 0; j < 64; ++j) v[j] = j < cols ? row[j] : (T)-INFINITY;
+        T m = v[0];
+#pragma unroll
+        for (int j = 1; j < 64; ++j) m = v[j] > m ? v[j] : m;
+        T sum = (T)0;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            v[j] = j < cols ? short_exp(v[j] - m) : (T)0;
+            sum = sum + v[j];  // columns in ascending order; the zeros past the row change nothing
+        }
+#pragma unroll
+        for (int j = 0; j < 64; ++j)
+            if (j < cols) row[j] = v[j] / sum;
+    }
+    __syncthreads();
+    {
+        int r = e_first / cols, c = e_first % cols;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if ((int)threadIdx.x + 256 * u < nvec) {
+                Vec out;
+                int rr = r, cc = c;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    out[k] = tile[rr * pitch + cc];
+                    if (++cc == cols) { cc = 0; ++rr; }
+                }
+                *reinterpret_cast<Vec*>(dst + e_first + step * u) = out;
+            }
+            r += dr; c += dc;
+            if (c >= cols) { c -= cols; ++r; }
+        }
+        for (int e = nvec * VEC + threadIdx.x; e < n; e += 256) dst[e] = tile[(e / cols) * pitch + e % cols];
+    }
 }
 
 // The reference multiplies dy with the explicit Jacobian row by row (O(cols^2)):
@@ -308,7 +360,8 @@ template <typename T>
 hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, T alpha, hipStream_t s) {
     if (rows <= 0 || cols <= 0) return hipSuccess;
     constexpr int RPG = RowsPerGroup<T>::N;
-    if (cols <= 64 && rows >= 16 * RPG) {  // enough rows to fill the chip a lane per row
+    const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    if (cols <= 64 && rows >= 16 * RPG && aligned) {  // enough rows to fill the chip a lane per row
         const size_t lds = (size_t)RPG * ((size_t)cols | 1) * sizeof(T);
         hipLaunchKernelGGL((softmax_fwd_rows_kernel<T>), dim3((unsigned)((rows + RPG - 1) / RPG)), dim3(256), lds, s, x, y, rows, cols, alpha);
         return hipGetLastError();
