@@ -511,3 +511,41 @@ def test_operand_larger_than_four_gib(gpu):
     # (40000 float terms per entry that add up coherently, block after block: the rounding of the running sums
     # is what the wider bar is for; a wrong tile base would be off by the size of the entries themselves)
     assert np.max(np.abs(dB.download() - ref_dB)) <= 1e-4 * np.max(np.abs(ref_dB))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(50176, 96, 288), (50001, 100, 96), (49160, 8, 128), (50176, 96, 384)])
+def test_tall_products_of_few_slabs(gpu, oracle, dtype, shape):
+    """A layer of about a hundred inputs applied to fifty thousand rows: hundreds of 128 x 128 tiles of one to
+    six K slabs, the shapes that the half-depth kernel takes (all three layouts, a ragged last row tile, a K that
+    ends inside a slab, plain and elementwise epilogues).  Held entry by entry against the product in double."""
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    M, K, N = shape
+    A = seeded.uniform(41, 1, (M, K), -1, 1, dtype)
+    B = seeded.uniform(41, 2, (K, N), -1, 1, dtype)
+    G = seeded.normal(41, 3, (M, N), 1.0, dtype)
+    dA_, dB_, dG_ = (DeviceBuffer.alloc(dtype, *x.shape) for x in (A, B, G))
+    dA_.upload(A); dB_.upload(B); dG_.upload(G)
+    C = DeviceBuffer.alloc(dtype, M, N)
+    check(lib.prad_gemm(0, 0, dA_.handle, dB_.handle, C.handle, 0))                      # A . B
+    assert_parity(C.download(), A.astype(np.float64) @ B.astype(np.float64), dtype, "A.B", bound=dot_bound(A, B, dtype))
+    dX = DeviceBuffer.alloc(dtype, M, K)
+    check(lib.prad_gemm(0, 1, dG_.handle, dB_.handle, dX.handle, 0))                     # G . B^T: K of this product is N
+    assert_parity(dX.download(), G.astype(np.float64) @ B.T.astype(np.float64), dtype, "G.B^T", bound=dot_bound(G, B.T, dtype))
+    # bias, pre-activation copy and GELU in the epilogue; then GELU' of the pre-activation on the way back
+    bias = seeded.normal(41, 4, (1, N), 0.5, dtype)
+    db = DeviceBuffer.alloc(dtype, 1, N); db.upload(bias)
+    Z, H = DeviceBuffer.alloc(dtype, M, N), DeviceBuffer.alloc(dtype, M, N)
+    check(lib.prad_matmul_fwd_fused(dA_.handle, dB_.handle, db.handle, Z.handle, H.handle, _lib.ACT_GELU, 0.0))
+    gZ = Z.download()
+    assert_parity(gZ, A.astype(np.float64) @ B.astype(np.float64) + bias.astype(np.float64), dtype, "Z",
+                  bound=dot_bound(A, B, dtype) + 4 * np.finfo(dtype).eps * (np.abs(gZ) + np.abs(bias)))
+    rows = slice(M - 300, M)                                                             # the oracle's elementwise part on the last rows
+    assert_parity(H.download()[rows], oracle.gelu_fwd(np.ascontiguousarray(gZ[rows])), dtype, "GELU(Z)")
+    src = seeded.normal(41, 5, (M, K), 1.0, dtype)
+    dS = DeviceBuffer.alloc(dtype, M, K); dS.upload(src)
+    dAct = DeviceBuffer.alloc(dtype, M, K)
+    check(lib.prad_matmul_bwd_fused(dG_.handle, dA_.handle, dB_.handle, dAct.handle, None, 0, _lib.ACT_GELU, dS.handle, 0.0))
+    plain = dX.download()[rows]
+    assert_parity(dAct.download()[rows], oracle.gelu_bwd(np.ascontiguousarray(src[rows]), np.ascontiguousarray(plain)), dtype, "GELU' (.) dX")
