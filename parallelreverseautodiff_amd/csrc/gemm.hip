@@ -763,15 +763,16 @@ static bool gemm_short_eligible(const GemmArgs<T>& a, int epi) {
 }
 
 // Products of very few K slabs on hundreds of 128 x 128 tiles (a layer of 96 inputs applied to tens of thousands of
-// rows) go to the half-depth kernel: measured on such layers 10 to 20 % faster per launch, while K = 256 on a
-// thousand tiles is 5 % slower on it.  PRAD_GEMM_THIN_MAX_K overrides the largest K that goes there (0 switches the
+// rows) go to the half-depth kernel in float: measured on such layers 4 to 25 % faster per launch (most with an
+// elementwise epilogue), while K = 256 on a thousand tiles is 5 % slower on it, and in double, where a slab is
+// half as deep to begin with, the same layers are 15 to 25 % slower on it.  PRAD_GEMM_THIN_MAX_K overrides the largest K that goes there (0 switches the
 // kernel off), PRAD_GEMM_THIN_MIN_TILES the smallest tile count: tuning aids.
 template <typename T>
 static bool gemm_thin_eligible(const GemmArgs<T>& a, bool edge, int epi, int64_t tiles) {
     static const int64_t max_k = [] { const char* e = getenv("PRAD_GEMM_THIN_MAX_K"); return e ? (int64_t)atoll(e) : (int64_t)128; }();
     static const int64_t min_tiles = [] { const char* e = getenv("PRAD_GEMM_THIN_MIN_TILES"); return e ? (int64_t)atoll(e) : (int64_t)384; }();
     if (edge || a.ksplit != 0 || a.colsum_dst != nullptr || a.K > max_k || tiles * a.batch < min_tiles) return false;
-    return epi == EPI_PLAIN || (epi == EPI_ELEMENTWISE && sizeof(T) == 4);
+    return epi == EPI_PLAIN || epi == EPI_ELEMENTWISE;
 }
 
 template <typename T, int WT, bool A_KC, bool B_KC>
@@ -781,11 +782,10 @@ static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStr
     const unsigned splits = a.ksplit > 0 ? (unsigned)((a.K + a.ksplit - 1) / a.ksplit) : 1u;
     const unsigned riders = a.colsum_dst != nullptr ? (unsigned)((a.colsum_cols + 63) / 64) : 0u;
     dim3 grid((unsigned)(tilesM * tilesN) + riders, (unsigned)a.batch, splits), block(GEMM_THREADS, 1, 1);
-    if constexpr (WT == 4) {
+    if constexpr (WT == 4 && sizeof(T) == 4) {
         if (gemm_thin_eligible<T>(a, edge, epi, (int64_t)tilesM * tilesN)) {
             if (epi == EPI_PLAIN) hipLaunchKernelGGL((gemm_thin_kernel<T, A_KC, B_KC, EPI_PLAIN>), grid, block, 0, stream, a, tilesM, tilesN);
-            else if constexpr (sizeof(T) == 4)
-                hipLaunchKernelGGL((gemm_thin_kernel<T, A_KC, B_KC, EPI_ELEMENTWISE>), grid, block, 0, stream, a, tilesM, tilesN);
+            else hipLaunchKernelGGL((gemm_thin_kernel<T, A_KC, B_KC, EPI_ELEMENTWISE>), grid, block, 0, stream, a, tilesM, tilesN);
             return hipGetLastError();
         }
     }
