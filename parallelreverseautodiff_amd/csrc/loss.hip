@@ -103,7 +103,7 @@ __global__ void __launch_bounds__(256) softmax_bwd_short_kernel(const T* __restr
 // reduction crosses lanes and the sum runs over the columns in ascending order, as the reference's does.  The
 // workgroup's rows are contiguous in memory: they come in and go out as one coalesced block through LDS, where
 // the odd row pitch keeps the lanes' column-by-column walk free of bank conflicts.
-template <typename T> struct RowsPerGroup { static constexpr int N = 1024 / sizeof(T); };  // 256 floats' rows, 128 doubles'
+template <typename T> struct RowsPerGroup { static constexpr int N = 128; };
 template <typename T>
 __global__ void __launch_bounds__(256) softmax_fwd_rows_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols64,
                                                                T alpha) {
