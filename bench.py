@@ -541,7 +541,8 @@ def main():
 
 def also_legs(args):
     """The rest of the metric beside the headline figure, measured in the same run: the product in the other
-    precision at the same size, and the MLP training step of configs[0] (recorded launch sequence).  A leg
+    precision at the same size, the MLP training step of configs[0] (recorded launch sequence; in double beside its CPU
+    restatement on the host cores) and the LSTM training step of configs[3].  A leg
     that fails is reported as its error text and does not touch the headline figures."""
     out = {}
     other = "f32" if args.dtype == "f64" else "f64"
@@ -554,11 +555,18 @@ def also_legs(args):
         out["matmul_fwd_bwd_" + other] = {"error": repr(e)}
     for d in ("f64", "f32"):
         try:
-            r = mlp_leg(d, 1000, 100, False)
-            out["mlp_train_steps_per_s_" + d] = {"value": 1e3 / r["recorded_ms_per_step"], "ms_per_step": r["recorded_ms_per_step"],
-                                                 "loss_after": r["loss_after"]}
+            r = mlp_leg(d, 1000, 100, d == "f64" and not args.no_cpu)
+            leg = {"value": 1e3 / r["recorded_ms_per_step"], "ms_per_step": r["recorded_ms_per_step"], "loss_after": r["loss_after"]}
+            if "cpu" in r:
+                leg["cpu_baseline"] = r["cpu"]
+            out["mlp_train_steps_per_s_" + d] = leg
         except Exception as e:  # noqa: BLE001
             out["mlp_train_steps_per_s_" + d] = {"error": repr(e)}
+    try:
+        r = lstm_leg("f32", 10, 2, False)
+        out["lstm_train_steps_per_s_f32"] = {"value": 1e3 / r["recorded_ms_per_step"], "ms_per_step": r["recorded_ms_per_step"]}
+    except Exception as e:  # noqa: BLE001
+        out["lstm_train_steps_per_s_f32"] = {"error": repr(e)}
     return out
 
 
