@@ -189,6 +189,14 @@ __device__ __forceinline__ void colsum_block(const T* __restrict__ dy, OUT* __re
     double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
     if (j < cols) {
         int64_t i = r0 + w;
+        // sixteen loads in flight where the rows allow; the additions keep the order of the four-at-a-time loop below
+        for (; i + 60 < r1; i += 64) {
+            double v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = (double)dy[(i + 4 * u) * cols + j];
+#pragma unroll
+            for (int u = 0; u < 16; u += 4) { acc0 += v[u]; acc1 += v[u + 1]; acc2 += v[u + 2]; acc3 += v[u + 3]; }
+        }
         for (; i + 12 < r1; i += 16) {
             const double a = (double)dy[i * cols + j], b = (double)dy[(i + 4) * cols + j];
             const double c = (double)dy[(i + 8) * cols + j], d = (double)dy[(i + 12) * cols + j];
