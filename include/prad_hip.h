@@ -227,6 +227,9 @@ int32_t prad_cce_bwd(prad_buf_t p, prad_buf_t target, prad_buf_t dp);
  * loss (1 x 1) = sum((y - t)^2) / (rows*cols) ; dy = (2 / (rows*cols)) * (y - t). */
 int32_t prad_mse_fwd(prad_buf_t y, prad_buf_t target, prad_buf_t loss);
 int32_t prad_mse_bwd(prad_buf_t y, prad_buf_t target, prad_buf_t dy);
+/* Forward and Backward of MeanSquaredErrorLossOperation in one pass over y and target (the loss of prad_mse_fwd
+ * and the gradient of prad_mse_bwd, value for value). */
+int32_t prad_mse(prad_buf_t y, prad_buf_t target, prad_buf_t loss, prad_buf_t dy);
 /* One LSTM time step's pointwise part, fused.  The reference builds it from separate nodes: three
  * SigmoidOperation and two TanhOperation forward (src/RMAD/SigmoidOperation.cs:46-62, TanhOperation.cs:42-57),
  * three HadamardProductOperation (HadamardProductOperation.cs:50-81) and a MatrixAddOperation (MatrixAddOperation.cs:29-45).

@@ -94,6 +94,7 @@ SIGNATURES = {
     "prad_cce_bwd": (_i32, [_vp, _vp, _vp]),
     "prad_mse_fwd": (_i32, [_vp, _vp, _vp]),
     "prad_mse_bwd": (_i32, [_vp, _vp, _vp]),
+    "prad_mse": (_i32, [_vp, _vp, _vp, _vp]),
     "prad_lstm_cell_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp]),
     "prad_lstm_cell_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_lstm_step_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -284,7 +284,9 @@ template <typename T> hipError_t launch_cce_fwd(const T* p, const T* t, T* loss,
 template <typename T> hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t cols, hipStream_t s);
 
 size_t mse_workspace_bytes();
-template <typename T> hipError_t launch_mse_fwd(const T* y, const T* t, T* loss, double* workspace, int64_t n, hipStream_t s);
+// dy != nullptr: the gradient is written in the same pass (the values of launch_mse_bwd).
+template <typename T> hipError_t launch_mse_fwd(const T* y, const T* t, T* loss, double* workspace, int64_t n, hipStream_t s,
+                                                T* dy = nullptr);
 template <typename T> hipError_t launch_mse_bwd(const T* y, const T* t, T* dy, int64_t n, hipStream_t s);
 
 // LSTM cell (csrc/lstm.hip)

@@ -307,13 +307,16 @@ __global__ void __launch_bounds__(256) softmax_cce_kernel(const T* __restrict__ 
 
 // MeanSquaredErrorLossOperation (src/RMAD/Loss/MeanSquaredErrorLossOperation.cs): loss = sum (y - t)^2 / (rows*cols),
 // dy = (2 / (rows*cols)) * (y - t).  The sum is taken in two levels (per workgroup, then by one thread).
-template <typename T>
+// WITH_DY: the same pass also writes the gradient, value for value what mse_bwd_kernel writes.
+template <typename T, bool WITH_DY>
 __global__ void __launch_bounds__(256) mse_partial_kernel(const T* __restrict__ y, const T* __restrict__ t, double* __restrict__ part,
-                                                          int64_t n) {
+                                                          T* __restrict__ dy, int64_t n) {
+    const T scale = (T)2 / (T)n;
     double s = 0.0;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
         const T d = y[i] - t[i];
         s += (double)(d * d);
+        if (WITH_DY) dy[i] = scale * d;
     }
     s = wave_sum(s);
     __shared__ double w[4];
@@ -337,11 +340,12 @@ __global__ void __launch_bounds__(256) mse_bwd_kernel(const T* __restrict__ y, c
 constexpr int MSE_PARTS = 1024;
 size_t mse_workspace_bytes() { return MSE_PARTS * sizeof(double); }
 template <typename T>
-hipError_t launch_mse_fwd(const T* y, const T* t, T* loss, double* workspace, int64_t n, hipStream_t s) {
+hipError_t launch_mse_fwd(const T* y, const T* t, T* loss, double* workspace, int64_t n, hipStream_t s, T* dy) {
     int64_t blocks = (n + 255) / 256;
     if (blocks > MSE_PARTS) blocks = MSE_PARTS;
     if (blocks < 1) blocks = 1;
-    hipLaunchKernelGGL((mse_partial_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, n);
+    if (dy != nullptr) hipLaunchKernelGGL((mse_partial_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, dy, n);
+    else hipLaunchKernelGGL((mse_partial_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, dy, n);
     hipLaunchKernelGGL((mse_final_kernel<T>), dim3(1), dim3(64), 0, s, workspace, (int)blocks, loss, n);
     return hipGetLastError();
 }
@@ -415,7 +419,7 @@ hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t c
     template hipError_t launch_softmax_cce<T>(const T*, const T*, T*, T*, T*, T*, unsigned*, int64_t, int64_t, hipStream_t); \
     template hipError_t launch_cce_fwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
     template hipError_t launch_cce_bwd<T>(const T*, const T*, T*, int64_t, int64_t, hipStream_t);   \
-    template hipError_t launch_mse_fwd<T>(const T*, const T*, T*, double*, int64_t, hipStream_t);   \
+    template hipError_t launch_mse_fwd<T>(const T*, const T*, T*, double*, int64_t, hipStream_t, T*);   \
     template hipError_t launch_mse_bwd<T>(const T*, const T*, T*, int64_t, hipStream_t);
 INSTANTIATE(double)
 INSTANTIATE(float)

@@ -1181,6 +1181,22 @@ int32_t prad_mse_fwd(prad_buf_t y, prad_buf_t target, prad_buf_t loss) {
     return PRAD_OK;
 }
 
+int32_t prad_mse(prad_buf_t y, prad_buf_t target, prad_buf_t loss, prad_buf_t dy) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(y); REQUIRE_BUF(target); REQUIRE_BUF(loss); REQUIRE_BUF(dy);
+    if (int32_t st = same_dtype({y, target, loss, dy})) return st;
+    if (y->depth != target->depth || y->rows != target->rows || y->cols != target->cols)
+        return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
+    if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
+    if (int32_t st = same_shape(y, dy, "mean squared error backward")) return st;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (int32_t st = ensure_workspace(mse_workspace_bytes())) return st;
+    double* w = static_cast<double*>(CUR_WORKSPACE);
+    DISPATCH(y, launch_mse_fwd<double>(D(y), D(target), D(loss), w, count(y), CUR_STREAM, D(dy)),
+             launch_mse_fwd<float>(F(y), F(target), F(loss), w, count(y), CUR_STREAM, F(dy)));
+    return PRAD_OK;
+}
+
 int32_t prad_mse_bwd(prad_buf_t y, prad_buf_t target, prad_buf_t dy) {
     REQUIRE_INIT();
     REQUIRE_BUF(y); REQUIRE_BUF(target); REQUIRE_BUF(dy);

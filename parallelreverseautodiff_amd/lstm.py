@@ -80,8 +80,7 @@ class LSTMLayer:
             check(lib.prad_gemm(0, 0, self.H_t[t].handle, self.Wh.handle, self.G_t[t].handle, 1))  # G_t += h_{t-1} . W_h
             check(lib.prad_lstm_cell_fwd(self.G_t[t].handle, self.C_t[t].handle, self.C_t[t + 1].handle, self.TC_t[t].handle,
                                          self.H_t[t + 1].handle))
-        check(lib.prad_mse_fwd(self.H_out.handle, self.Y.handle, self.loss.handle))
-        check(lib.prad_mse_bwd(self.H_out.handle, self.Y.handle, self.dHl.handle))
+        check(lib.prad_mse(self.H_out.handle, self.Y.handle, self.loss.handle, self.dHl.handle))   # loss and its gradient
         for t in range(T - 1, -1, -1):
             last = t == T - 1
             rec, dc_in, dc_out = self.dh[t % 2], self.dc[t % 2], self.dc[(t + 1) % 2]

@@ -91,9 +91,8 @@ class SwinBlock:
         check(fused(self.O.handle, w["Wo"].handle, w["bo"].handle, None, self.Y1.handle, _lib.ACT_NONE, 0.0))
         check(fused(self.Y1.handle, w["W1"].handle, w["b1"].handle, self.Z1.handle, self.H1.handle, _lib.ACT_GELU, 0.0))
         check(fused(self.H1.handle, w["W2"].handle, w["b2"].handle, None, self.Y2.handle, _lib.ACT_NONE, 0.0))
-        check(lib.prad_mse_fwd(self.Y2.handle, self.T.handle, self.loss.handle))
+        check(lib.prad_mse(self.Y2.handle, self.T.handle, self.loss.handle, self.dY2.handle))   # loss and its gradient
         # ---- backward ----
-        check(lib.prad_mse_bwd(self.Y2.handle, self.T.handle, self.dY2.handle))
         check(lib.prad_add_broadcast_bwd_bias(self.dY2.handle, g["b2"].handle))
         check(lib.prad_matmul_bwd_fused(self.dY2.handle, self.H1.handle, w["W2"].handle, self.dZ1.handle, g["W2"].handle, 0,
                                         _lib.ACT_GELU, self.Z1.handle, 0.0))

@@ -134,3 +134,26 @@ def test_scaled_softmax_forward_and_backward(gpu, oracle, dtype, shape):
     check(lib.prad_softmax_bwd(Y.handle, DY.handle, DX2.handle))
     check(lib.prad_scale(DX2.handle, DX2.handle, alpha))
     assert np.array_equal(DX2.download(), dx)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 1), (7, 13), (128, 512), (3000, 97)])
+def test_mean_squared_error_loss_and_gradient(gpu, oracle, dtype, shape):
+    """MeanSquaredErrorLossOperation Forward and Backward against the oracle, separately and in one pass
+    (prad_mse: the same values as the two launches, bit for bit)."""
+    lib = _lib.load()
+    y = seeded.normal(51, 1, shape, 1.0, dtype)
+    t = seeded.normal(51, 2, shape, 1.0, dtype)
+    Y, T, D1, D2 = (DeviceBuffer.alloc(dtype, *shape) for _ in range(4))
+    L1, L2 = DeviceBuffer.alloc(dtype, 1, 1), DeviceBuffer.alloc(dtype, 1, 1)
+    Y.upload(y); T.upload(t)
+    check(lib.prad_mse_fwd(Y.handle, T.handle, L1.handle))
+    check(lib.prad_mse_bwd(Y.handle, T.handle, D1.handle))
+    check(lib.prad_mse(Y.handle, T.handle, L2.handle, D2.handle))
+    loss = float(L1.download()[0, 0])
+    ref = oracle.mse_fwd(y, t)
+    assert abs(loss - ref) <= (1e-12 if dtype == np.float64 else 1e-5) * abs(ref)
+    assert_parity(D1.download(), oracle.mse_bwd(y, t), dtype, "mse backward")
+    assert np.array_equal(L2.download(), L1.download()) and np.array_equal(D2.download(), D1.download())
+    if shape != (1, 1):
+        assert lib.prad_mse(Y.handle, T.handle, D1.handle, D2.handle) == _lib.PRAD_ERR_ARG     # loss must be 1 x 1
