@@ -1,6 +1,7 @@
 """Compositions of the oracle's per-operation restatements into whole training steps, node by node as the
 reference's graph would run them.  TEST INFRASTRUCTURE ONLY (same rule as oracle.py): used by tests and by
-the benchmark's cpu_baseline leg."""
+the benchmark's cpu_baseline leg.  Both compositions are pinned by tests/test_oracle_compose.py: forward against an
+independent numpy statement, gradients against central differences of it, a hand-worked single step."""
 import numpy as np
 
 from . import oracle

@@ -19,7 +19,8 @@
 // each row separately like the reference does.
 //
 // Pinning status of each function (what independent fact checks it) is listed in
-// tests/test_oracle.py next to the test that does it; functions whose libm calls (exp, tanh,
+// tests/test_oracle.py next to the test that does it (the loss functions and the whole-step
+// compositions of oracle/compose.py: tests/test_oracle_compose.py); functions whose libm calls (exp, tanh,
 // pow) may differ from .NET's in the last ulp say so below.
 
 #include <cmath>

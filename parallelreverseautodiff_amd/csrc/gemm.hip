@@ -454,8 +454,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         // and counts its arrival; the one that arrives last adds the partial tiles in split order (its own
         // included, read back like the others, so that the sum does not depend on who arrives last) and goes on
         // to the epilogue.  No workgroup waits for another.  The partial tiles travel as device-coherent stores and
-        // loads (written through, read past the caches) whose completion the barriers wait for: a device-scope
-        // fence would write back and invalidate the whole L2 and evict the operand panels of every workgroup nearby.
+        // loads (written through to memory, read past the per-XCD caches): a device-scope fence would write back and
+        // invalidate the whole L2 and evict the operand panels of every workgroup nearby.  What orders them:
+        //   writer: every wavefront waits for its own parked stores to be acknowledged (vmcnt(0): a write-through
+        //           store is acknowledged once it is in memory), then the workgroup barrier, then thread 0's
+        //           device-scope atomic add on the tile's counter.  The workgroup barrier alone does not wait for
+        //           outstanding vector stores.
+        //   reader: the last arriver sees the count (the atomic's return value, through LDS and a barrier) before it
+        //           issues its device-coherent loads, which therefore find every other workgroup's tile in memory.
         const int64_t mn = p.M * p.N;
         const int splits = (int)g_.gz;
         T* __restrict__ mine = p.split_ws + ((int64_t)g_.bz * g_.gy + batch) * mn;
@@ -471,6 +477,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                     __hip_atomic_store(&mine[i * p.N + j], acc[x][y][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // compiler: the stores stay above the wait
+        __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0), other counters untouched
         __syncthreads();
         __shared__ unsigned arrived;
         if (tid == 0) {
