@@ -227,7 +227,7 @@ def lstm_leg(dtype_name, steps, warmup, with_cpu):
         return ms.value / steps
 
     eager_ms = timed(layer.step)
-    layer.record(adam_iteration=float(layer.iteration + 1))
+    layer.record()
     rec_ms = timed(layer.replay)
     layer.release()
     flops = layer.flops_per_step()
@@ -276,7 +276,7 @@ def swin_leg(dtype_name, steps, warmup, with_cpu):
         return ms.value / steps
 
     eager_ms = timed(blk.step)
-    blk.record(adam_iteration=float(blk.iteration + 1))
+    blk.record()
     rec_ms = timed(blk.replay)
     blk.release()
     flops = blk.flops_per_step()
@@ -360,7 +360,7 @@ def mlp_leg(dtype_name, steps, warmup, with_cpu):
         return ms.value / steps, wall * 1e3 / steps
 
     eager_ms, eager_wall = timed(net.step)
-    net.record(adam_iteration=float(net.iteration + 1))
+    net.record()
     graph_ms, graph_wall = timed(net.replay)
     loss = float(net.loss.download()[0, 0])
     net.release()

@@ -10,9 +10,17 @@
  *   - Matrices are dense row-major device buffers behind opaque handles (prad_buf_t).  A handle
  *     is valid on any host thread.  The reference's jagged Matrix (one array per row) is
  *     marshalled once with prad_buf_upload_rows and stays resident.
- *   - All work is enqueued, in call order, on one library stream; calls may come from any
- *     number of host threads (the reference runs Backward of different operations concurrently
- *     on pool threads).  Downloads and prad_stream_sync wait for the stream.
+ *   - All work is enqueued, in call order, on one library stream under one lock; calls may come from
+ *     any number of host threads (the reference runs Backward of different operations concurrently
+ *     on pool threads, src/RMAD/OperationNeuralNetworkVisitor.cs:303-306) and execute in the order in
+ *     which they took the lock.  Downloads and prad_stream_sync wait for the stream.  While one
+ *     thread records a launch sequence (prad_graph_begin .. prad_graph_end), calls from other threads
+ *     return PRAD_ERR_RECORDING and enqueue nothing.
+ *   - Kernels that need device scratch (products split along K, clip statistics, loss partial sums,
+ *     tall column sums) share one workspace that grows on demand.  A recorded launch sequence keeps
+ *     the workspace address it was recorded with: an outgrown workspace is kept alive until the last
+ *     recorded sequence is destroyed, and growing it during a recording fails (run the sequence once
+ *     eagerly first).
  *   - dtype: PRAD_F64 restates the PRAD (double) build, PRAD_F32 the PRADLite (float) build.
  *
  * Citations are to the reference tree (ameritusweb/ParallelReverseAutoDiff).
@@ -35,7 +43,9 @@ enum {
     PRAD_ERR_BAD_HANDLE = -5,
     PRAD_ERR_ARG = -6,             /* ArgumentException, src/RMAD/GpuMatrixMultiplyOperation.cs:177-180 */
     PRAD_ERR_NOT_RECTANGULAR = -7, /* InvalidOperationException("The given jagged array is not rectangular."), src/RMAD/GpuMatrixMultiplyOperation.cs:244-247 */
-    PRAD_ERR_DTYPE = -8
+    PRAD_ERR_DTYPE = -8,
+    PRAD_ERR_RECORDING = -9        /* refused because of an open recording (prad_graph_begin): the call came from another
+                                      thread, or it allocates, copies to or from the host or waits for the device */
 };
 
 enum { PRAD_F64 = 0, PRAD_F32 = 1 };
@@ -255,29 +265,25 @@ int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, 
  * stacked sequence).  The view must be freed before its parent. */
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out);
 
-/* ---- replay of a fixed launch sequence: everything enqueued by this thread between begin and end
+/* ---- replay of a fixed launch sequence: everything enqueued by the calling thread between begin and end
  *      is recorded instead of executed and can then be launched as one submission.  The forward loop
  *      of the reference walks the same operation list every step
  *      (examples/feedforward/ParallelReverseAutoDiff.FeedForwardExample/FeedForwardNeuralNetwork.cs:212-303);
- *      a recorded step replaces ~20 launches by one.  Only entry points that neither allocate nor
- *      copy to or from the host may be recorded. */
+ *      a recorded step replaces ~20 launches by one.  Entry points that allocate, free, copy to or from the
+ *      host or wait for the device return PRAD_ERR_RECORDING while a recording is open, and so does every
+ *      enqueueing call from a thread other than the recording one.
+ *      AdamIteration: the reference's caller advances it once per step (AdamOptimizer.cs:204-207, set from the
+ *      iteration count at FeedForwardNeuralNetwork.cs:165).  A recorded prad_adam_multi / prad_clip_adam_multi keeps
+ *      its bias-correction factors as launch arguments; prad_graph_launch replaces them before each launch so that
+ *      launch number k of a sequence recorded with AdamIteration t runs with t + k (k = 0, 1, ...), bit for bit what
+ *      the eager calls with those iterations give.  prad_graph_set_adam_iteration sets the value the next launch
+ *      uses (later launches continue from it). */
 int32_t prad_graph_begin(void);
 int32_t prad_graph_end(void** graph);
 int32_t prad_graph_launch(void* graph);
+int32_t prad_graph_set_adam_iteration(void* graph, double t);
 int32_t prad_graph_destroy(void* graph);
 
-/* ---- branches: the reference's backward visitor runs Backward of operations that do not depend on
- *      each other on pool threads (src/RMAD/OperationNeuralNetworkVisitor.cs:303-306).  Here such
- *      operations are enqueued on different branches and may execute side by side; in a recording they
- *      become parallel paths.  prad_fork(n) makes branches 1..n-1 start after everything enqueued on
- *      branch 0 so far (it may be called again to hand later results of branch 0 to the open branches,
- *      each branch keeps its own order); prad_branch(i) selects the branch that following calls enqueue
- *      on (0 = the library stream); prad_join() makes branch 0 wait for all open branches, closes them
- *      and selects branch 0.  The selection is library-wide: one thread submits while branches are open. */
-#define PRAD_MAX_BRANCHES 4
-int32_t prad_fork(int32_t branches);
-int32_t prad_branch(int32_t index);
-int32_t prad_join(void);
 /* Softmax.Forward (p), CategoricalCrossEntropy.Forward (loss, may be NULL) and .Backward (dp) and
  * Softmax.Backward (dx) of one batch; same arithmetic as prad_softmax_fwd + prad_cce_fwd + prad_cce_bwd +
  * prad_softmax_bwd (src/RMAD/SoftmaxOperation.cs:45-110,

@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libprad_hip.so")
+# PRAD_HIP_LIBRARY names another build of the library (a tuning aid: two builds measured side by side).
+LIB_PATH = os.environ.get("PRAD_HIP_LIBRARY") or os.path.join(_HERE, "libprad_hip.so")
 
 PRAD_OK = 0
 PRAD_ERR_NOT_INITIALIZED = -1
@@ -19,6 +20,7 @@ PRAD_ERR_BAD_HANDLE = -5
 PRAD_ERR_ARG = -6
 PRAD_ERR_NOT_RECTANGULAR = -7
 PRAD_ERR_DTYPE = -8
+PRAD_ERR_RECORDING = -9
 
 PRAD_F64 = 0
 PRAD_F32 = 1
@@ -100,13 +102,11 @@ SIGNATURES = {
     "prad_lstm_step_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_lstm_step_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_buf_view_rows": (_i32, [_vp, _i64, _i64, _vpp]),
-    "prad_fork": (_i32, [_i32]),
-    "prad_branch": (_i32, [_i32]),
-    "prad_join": (_i32, []),
     "prad_softmax_cce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_graph_begin": (_i32, []),
     "prad_graph_end": (_i32, [_vpp]),
     "prad_graph_launch": (_i32, [_vp]),
+    "prad_graph_set_adam_iteration": (_i32, [_vp, _f64]),
     "prad_graph_destroy": (_i32, [_vp]),
     "prad_clip": (_i32, [_vp, _f64, _f64]),
     "prad_adam": (_i32, [_vp, _vp, _vp, _vp, _f64, _f64, _f64, _f64, _f64]),

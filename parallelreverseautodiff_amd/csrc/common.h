@@ -270,11 +270,19 @@ struct TensorDesc {
 size_t clip_workspace_bytes(const int64_t* n, int ntensors);
 template <typename T> hipError_t launch_clip(const TensorDesc<T>* host_descs, int ntensors, void* workspace, T clip_value,
                                              T min_value, hipStream_t s);
+// Called after every launch of the Adam kernel with the stream it went to (a recording notes the graph node there).
+struct AdamLaunchObserver {
+    void (*fn)(void* ctx, hipStream_t s);
+    void* ctx;
+};
 // reverse: AdamOptimizer.ReverseAdamUpdate instead of UpdateWeightWithAdam
 template <typename T> hipError_t launch_adam(const TensorDesc<T>* host_descs, int ntensors, T lr, T beta1, T beta2, T eps, T c1,
-                                             T c2, bool reverse, hipStream_t s);
+                                             T c2, bool reverse, hipStream_t s, const AdamLaunchObserver* obs = nullptr);
 template <typename T> hipError_t launch_clip_adam(const TensorDesc<T>* host_descs, int ntensors, void* workspace, T clip_value,
-                                                  T min_value, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s);
+                                                  T min_value, T lr, T beta1, T beta2, T eps, T c1, T c2, hipStream_t s,
+                                                  const AdamLaunchObserver* obs = nullptr);
+// Replaces c1 and c2 in the launch arguments of a recorded Adam kernel node of an instantiated graph.
+template <typename T> hipError_t adam_node_set_bias_correction(hipGraphExec_t exec, hipGraphNode_t node, T c1, T c2);
 
 // softmax / categorical cross-entropy (csrc/loss.hip)
 template <typename T> hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, T alpha, hipStream_t s);

@@ -44,6 +44,9 @@ typedef double d4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef double d2_t __attribute__((ext_vector_type(2)));
 
+#ifndef PRAD_GEMM_FOLD_K
+#define PRAD_GEMM_FOLD_K 512  // float accumulators are folded into a second set every so many elements of K (0: never)
+#endif
 constexpr int GEMM_THREADS = 256;
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 8;
@@ -277,6 +280,37 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         for (int y = 0; y < WTN; ++y)
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[x][y][r] = (T)0;
+    // Float products of a long K: a single chain of MFMA accumulations rounds every step at the magnitude of the
+    // running sum, and at K of several thousand that noise reaches the 1e-5 parity bar by itself.  The accumulators
+    // are therefore folded into a second set every FOLD_K of the reduction (two-level summation: chains of at most
+    // FOLD_K / 4 steps, then one addition per fold).  Products of K <= FOLD_K give the bits they gave without it.
+    constexpr int FOLD_K = PRAD_GEMM_FOLD_K;
+    // (the single-stage and half-depth kernels only take K <= FOLD_K; the LSTM step kernels reduce at most 4 * hidden)
+    constexpr bool FOLD = FOLD_K > 0 && sizeof(T) == 4 && !SHORT && DIV == 1 && EPI != EPI_LSTM_FWD && EPI != EPI_LSTM_BWD;
+    constexpr int FOLD_SLABS = FOLD ? FOLD_K / BK : 2;
+    static_assert(!FOLD || (FOLD_SLABS >= 2 && (FOLD_SLABS & (FOLD_SLABS - 1)) == 0), "folds fall on even slab counts");
+    Acc acc2[FOLD ? WTM : 1][FOLD ? WTN : 1];
+    if (FOLD) {
+#pragma unroll
+        for (int x = 0; x < WTM; ++x)
+#pragma unroll
+            for (int y = 0; y < WTN; ++y)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc2[x][y][r] = (T)0;
+    }
+    auto fold = [&] {
+        if (FOLD) {
+#pragma unroll
+            for (int x = 0; x < WTM; ++x)
+#pragma unroll
+                for (int y = 0; y < WTN; ++y)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        acc2[x][y][r] = acc2[x][y][r] + acc[x][y][r];
+                        acc[x][y][r] = (T)0;
+                    }
+        }
+    };
 
     // Unguarded kernels run the whole slabs with vector loads and finish a ragged end of K (784 = 12 x 64 + 16)
     // with one guarded slab; guarded kernels treat every slab alike.
@@ -372,6 +406,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                 load_slab_fast<T>(ra1, ua + (kt + 3) * stepa, offa);
                 load_slab_fast<T>(rb1, ub + (kt + 3) * stepb, offb);
                 compute(smem[1]);
+                if (FOLD && ((kt + 2) & (FOLD_SLABS - 1)) == 0) fold();
                 store_slab<T, WT, A_KC, DIV>(smem[0], ra0, tid);
                 store_slab<T, WT, B_KC, DIV>(smem[0] + SA, rb0, tid);
                 __syncthreads();
@@ -419,6 +454,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                 load_slab_guarded<T, WT, B_KC, DIV>(rb, B, p.ldb, col0, p.N, (int64_t)(kt + 1) * BK, K, tid);
             }
             compute(smem[cur]);
+            if (FOLD && ((kt + 1) & (FOLD_SLABS - 1)) == 0) fold();
             if (more) {
                 store_slab<T, WT, A_KC, DIV>(smem[cur ^ 1], ra, tid);
                 store_slab<T, WT, B_KC, DIV>(smem[cur ^ 1] + SA, rb, tid);
@@ -426,6 +462,15 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
             __syncthreads();
             cur ^= 1;
         }
+    }
+
+    if (FOLD) {
+#pragma unroll
+        for (int x = 0; x < WTM; ++x)
+#pragma unroll
+            for (int y = 0; y < WTN; ++y)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[x][y][r] = acc2[x][y][r] + acc[x][y][r];
     }
 
     // ---- epilogue ------------------------------------------------------------------------
@@ -779,7 +824,7 @@ template <typename T>
 static bool gemm_thin_eligible(const GemmArgs<T>& a, bool edge, int epi, int64_t tiles) {
     static const int64_t max_k = [] { const char* e = getenv("PRAD_GEMM_THIN_MAX_K"); return e ? (int64_t)atoll(e) : (int64_t)128; }();
     static const int64_t min_tiles = [] { const char* e = getenv("PRAD_GEMM_THIN_MIN_TILES"); return e ? (int64_t)atoll(e) : (int64_t)384; }();
-    if (edge || a.ksplit != 0 || a.colsum_dst != nullptr || a.K > max_k || tiles * a.batch < min_tiles) return false;
+    if (edge || a.ksplit != 0 || a.colsum_dst != nullptr || a.K > max_k || (PRAD_GEMM_FOLD_K > 0 && a.K > PRAD_GEMM_FOLD_K) || tiles * a.batch < min_tiles) return false;  // (no fold on it)
     return epi == EPI_PLAIN || epi == EPI_ELEMENTWISE;
 }
 

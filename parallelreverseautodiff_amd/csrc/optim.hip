@@ -14,6 +14,8 @@
 // element (read for statistics, read + write for the clamp).
 #include "common.h"
 
+#include <cstring>
+
 namespace prad {
 
 constexpr int OPT_THREADS = 256;
@@ -400,7 +402,7 @@ size_t clip_workspace_bytes(const int64_t* n, int nt) {
 // One group of at most MAX_TABLE tensors: clip only (ADAM false), Adam only (CLIP false) or both in one pass.
 template <typename T, int CHUNK, bool CLIP, bool ADAM>
 static hipError_t launch_group(const TensorDesc<T>* host, int gn, void* workspace, T clip_value, T min_value,
-                               const AdamUpdate<T>& update, hipStream_t s) {
+                               const AdamUpdate<T>& update, hipStream_t s, const AdamLaunchObserver* obs) {
     TensorTable<T> tab;
     const int64_t chunks = build_table(host, gn, tab, CHUNK);
     if (chunks == 0) return hipSuccess;
@@ -420,10 +422,11 @@ static hipError_t launch_group(const TensorDesc<T>* host, int gn, void* workspac
         }
         partial = dpartial;
     }
-    if (ADAM)
+    if (ADAM) {
         hipLaunchKernelGGL((adam_kernel<T, CHUNK, CLIP>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, update, stats, partial,
                            clip_value, min_value);
-    else
+        if (obs != nullptr) obs->fn(obs->ctx, s);
+    } else
         hipLaunchKernelGGL((clip_apply_kernel<T, CHUNK>), dim3((unsigned)chunks), dim3(OPT_THREADS), 0, s, tab, stats, partial,
                            clip_value, min_value);
     return hipGetLastError();
@@ -431,14 +434,14 @@ static hipError_t launch_group(const TensorDesc<T>* host, int gn, void* workspac
 
 template <typename T, bool CLIP, bool ADAM>
 static hipError_t launch_groups(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value,
-                                const AdamUpdate<T>& update, hipStream_t s) {
+                                const AdamUpdate<T>& update, hipStream_t s, const AdamLaunchObserver* obs = nullptr) {
     for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
         const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
         int64_t total = 0;
         for (int i = 0; i < gn; ++i) total += host[g0 + i].n;
         const hipError_t e = (OPT_CHUNK_LARGE<T> != OPT_CHUNK_SMALL && total >= LARGE_CHUNK_FROM)
-                                 ? launch_group<T, OPT_CHUNK_LARGE<T>, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s)
-                                 : launch_group<T, OPT_CHUNK_SMALL, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s);
+                                 ? launch_group<T, OPT_CHUNK_LARGE<T>, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs)
+                                 : launch_group<T, OPT_CHUNK_SMALL, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -450,28 +453,54 @@ hipError_t launch_clip(const TensorDesc<T>* host, int nt, void* workspace, T cli
 }
 
 template <typename T>
-hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2, T eps, T c1, T c2, bool reverse, hipStream_t s) {
+hipError_t launch_adam(const TensorDesc<T>* host, int nt, T lr, T beta1, T beta2, T eps, T c1, T c2, bool reverse, hipStream_t s,
+                       const AdamLaunchObserver* obs) {
     const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps, reverse ? 1 : 0};
-    return launch_groups<T, false, true>(host, nt, nullptr, (T)0, (T)0, update, s);
+    return launch_groups<T, false, true>(host, nt, nullptr, (T)0, (T)0, update, s, obs);
 }
 
 // GradientClipper.Clip followed by AdamOptimizer.Optimize over the same tensors: statistics pass, then
 // one pass that clamps the gradient and updates w, m, v.
 template <typename T>
 hipError_t launch_clip_adam(const TensorDesc<T>* host, int nt, void* workspace, T clip_value, T min_value, T lr, T beta1, T beta2,
-                            T eps, T c1, T c2, hipStream_t s) {
+                            T eps, T c1, T c2, hipStream_t s, const AdamLaunchObserver* obs) {
     const AdamUpdate<T> update{lr, beta1, beta2, (T)1 - beta1, (T)1 - beta2, c1, c2, eps, 0};
-    return launch_groups<T, true, true>(host, nt, workspace, clip_value, min_value, update, s);
+    return launch_groups<T, true, true>(host, nt, workspace, clip_value, min_value, update, s, obs);
 }
+
+// The bias-correction factors are launch arguments of the Adam kernel (argument 1, an AdamUpdate<T>).  A recorded
+// launch sequence keeps the arguments it was recorded with; before a replay that stands for a later AdamIteration the
+// factors of its Adam kernel nodes are replaced here, every other argument staying as recorded.
+template <typename T>
+hipError_t adam_node_set_bias_correction(hipGraphExec_t exec, hipGraphNode_t node, T c1, T c2) {
+    hipKernelNodeParams kp;
+    memset(&kp, 0, sizeof(kp));
+    hipError_t e = hipGraphKernelNodeGetParams(node, &kp);
+    if (e != hipSuccess) return e;
+    if (kp.kernelParams == nullptr) return hipErrorInvalidValue;
+    constexpr int NARGS = 6;  // tab, update, stats, partial, clip_value, min_value
+    AdamUpdate<T> update = *static_cast<const AdamUpdate<T>*>(kp.kernelParams[1]);
+    update.c1 = c1;
+    update.c2 = c2;
+    void* args[NARGS];
+    for (int i = 0; i < NARGS; ++i) args[i] = kp.kernelParams[i];
+    args[1] = &update;
+    kp.kernelParams = args;
+    kp.extra = nullptr;
+    return hipGraphExecKernelNodeSetParams(exec, node, &kp);
+}
+template hipError_t adam_node_set_bias_correction<double>(hipGraphExec_t, hipGraphNode_t, double, double);
+template hipError_t adam_node_set_bias_correction<float>(hipGraphExec_t, hipGraphNode_t, float, float);
 
 template hipError_t launch_clip<double>(const TensorDesc<double>*, int, void*, double, double, hipStream_t);
 template hipError_t launch_clip<float>(const TensorDesc<float>*, int, void*, float, float, hipStream_t);
 template hipError_t launch_adam<double>(const TensorDesc<double>*, int, double, double, double, double, double, double, bool,
-                                        hipStream_t);
-template hipError_t launch_adam<float>(const TensorDesc<float>*, int, float, float, float, float, float, float, bool, hipStream_t);
+                                        hipStream_t, const AdamLaunchObserver*);
+template hipError_t launch_adam<float>(const TensorDesc<float>*, int, float, float, float, float, float, float, bool, hipStream_t,
+                                       const AdamLaunchObserver*);
 template hipError_t launch_clip_adam<double>(const TensorDesc<double>*, int, void*, double, double, double, double, double, double,
-                                             double, double, hipStream_t);
+                                             double, double, hipStream_t, const AdamLaunchObserver*);
 template hipError_t launch_clip_adam<float>(const TensorDesc<float>*, int, void*, float, float, float, float, float, float, float,
-                                            float, hipStream_t);
+                                            float, hipStream_t, const AdamLaunchObserver*);
 
 }  // namespace prad

@@ -16,6 +16,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 using namespace prad;
@@ -33,37 +34,31 @@ namespace {
 constexpr uint32_t BUF_MAGIC = 0x50524144u;  // "PRAD"
 constexpr size_t STAGING_CHUNK = (size_t)256 << 20;
 
-constexpr int MAX_BRANCHES = PRAD_MAX_BRANCHES;
-constexpr size_t COUNTER_BYTES = 4096;  // arrival counters of a branch: one per tile of a paired product, and a few
+constexpr size_t COUNTER_BYTES = 4096;  // arrival counters: one per tile of a split or paired product, and a few
 static_assert(COUNTER_BYTES >= GEMM_SPLIT_MAX_TILES * sizeof(unsigned), "a split product needs a counter per tile");
 
-// Branch 0 is the library stream; branches 1.. exist so that independent operations can overlap
-// (prad_fork / prad_branch / prad_join).  Each branch has its own kernel workspace, because two
-// kernels that run side by side cannot share partial-result storage.
-struct Branch {
-    hipStream_t stream = nullptr;
-    hipEvent_t done = nullptr;
-    void* workspace = nullptr;
-    size_t workspace_bytes = 0;
-    unsigned* counter = nullptr;  // arrival counter for kernels whose last workgroup finishes the job; zero between launches
-    bool open = false;
-};
-
+// One stream, one kernel workspace (partial results of split products, clip moments, loss partial sums, tall
+// column sums) and one block of arrival counters: everything is enqueued in lock order, so no two kernels
+// that use the workspace ever run side by side.
 struct Context {
     std::mutex mu;
     std::atomic<bool> initialized{false};
     int device = -1;
-    hipStream_t stream = nullptr;  // == branch[0].stream
-    Branch branch[MAX_BRANCHES];
-    int cur = 0;
-    hipEvent_t fork_event = nullptr;
+    hipStream_t stream = nullptr;
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
+    std::vector<void*> retired_workspaces;  // outgrown blocks that recorded launch sequences may still address
+    unsigned* counter = nullptr;            // zero between launches: the last workgroup to arrive resets its counter
     void* pinned = nullptr;
     size_t pinned_bytes = 0;
+    // A launch sequence is being recorded by `recorder`; calls from other threads are refused meanwhile.
+    bool recording = false;
+    std::thread::id recorder;
+    int live_graphs = 0;                    // recorded sequences not yet destroyed
 };
 Context g_ctx;
-inline Branch& cur_branch() { return g_ctx.branch[g_ctx.cur]; }
-#define CUR_STREAM (g_ctx.branch[g_ctx.cur].stream)
-#define CUR_WORKSPACE (g_ctx.branch[g_ctx.cur].workspace)
+#define CUR_STREAM (g_ctx.stream)
+#define CUR_WORKSPACE (g_ctx.workspace)
 thread_local std::string tl_error;
 
 int32_t fail(int32_t code, const char* fmt, ...) {
@@ -75,6 +70,20 @@ int32_t fail(int32_t code, const char* fmt, ...) {
     tl_error = buf;
     return code;
 }
+
+// Every entry point that enqueues takes the context lock through this: while a thread records a launch sequence,
+// calls from other threads are refused instead of being recorded into it.
+#define ENQUEUE_LOCK()                                                                                \
+    std::lock_guard<std::mutex> lock(g_ctx.mu);                                                       \
+    do {                                                                                              \
+        if (g_ctx.recording && g_ctx.recorder != std::this_thread::get_id())                          \
+            return fail(PRAD_ERR_RECORDING, "another thread is recording a launch sequence; call again after its prad_graph_end"); \
+    } while (0)
+// For entry points that allocate, copy to or from the host, or wait for the device (lock held).
+#define NOT_WHILE_RECORDING(what)                                                                     \
+    do {                                                                                              \
+        if (g_ctx.recording) return fail(PRAD_ERR_RECORDING, what " cannot be part of a recorded launch sequence"); \
+    } while (0)
 
 #define HIP_TRY(expr, code)                                                                           \
     do {                                                                                              \
@@ -98,17 +107,9 @@ inline int64_t count(prad_buf_t b) { return b->depth * b->rows * b->cols; }
         if (!valid(b)) return fail(PRAD_ERR_BAD_HANDLE, "%s is not a live buffer handle", #b);        \
     } while (0)
 
-// Lock must be held.
-// Waits for everything enqueued on the library stream and on every branch.
+// Lock must be held.  Waits for everything enqueued on the library stream.
 int32_t sync_all() {
-    for (int i = 0; i < MAX_BRANCHES; ++i)
-        if (g_ctx.branch[i].stream) HIP_TRY(hipStreamSynchronize(g_ctx.branch[i].stream), PRAD_ERR_LAUNCH);
-    return PRAD_OK;
-}
-// Copies run on the library stream; results that open branches still produce are waited for first.
-int32_t drain_open_branches() {
-    for (int i = 1; i < MAX_BRANCHES; ++i)
-        if (g_ctx.branch[i].open) HIP_TRY(hipStreamSynchronize(g_ctx.branch[i].stream), PRAD_ERR_LAUNCH);
+    if (g_ctx.stream) HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
 int32_t ensure_pinned(size_t bytes) {
@@ -121,19 +122,85 @@ int32_t ensure_pinned(size_t bytes) {
     g_ctx.pinned_bytes = bytes;
     return PRAD_OK;
 }
-// Grows the workspace of the branch that is selected (its stream is drained first; while a launch
-// sequence is being recorded that fails, which is why a recording follows an eager warm-up).
+void free_retired_workspaces() {
+    for (void* p : g_ctx.retired_workspaces) (void)hipFree(p);
+    g_ctx.retired_workspaces.clear();
+}
+// Grows the kernel workspace (lock held).  A recording cannot allocate: every shape is run once eagerly before it
+// is recorded, and a call that would have to grow the workspace during a recording fails.  Recorded launch
+// sequences keep the address of the workspace they were recorded with, so while any of them is alive an
+// outgrown block is not freed but retired (it is released when the last sequence is destroyed, or at
+// shutdown): a replay then still finds its own block, and replays and eager calls never run side by side.
 int32_t ensure_workspace(size_t bytes) {
-    Branch& b = cur_branch();
-    if (bytes <= b.workspace_bytes) return PRAD_OK;
-    HIP_TRY(hipStreamSynchronize(b.stream), PRAD_ERR_LAUNCH);
-    if (b.workspace) (void)hipFree(b.workspace);
-    b.workspace = nullptr;
-    b.workspace_bytes = 0;
+    if (bytes <= g_ctx.workspace_bytes) return PRAD_OK;
+    if (g_ctx.recording)
+        return fail(PRAD_ERR_RECORDING, "the workspace would have to grow during a recording: run the sequence once before recording it");
     bytes = (bytes + 4095) & ~(size_t)4095;
-    HIP_TRY(hipMalloc(&b.workspace, bytes), PRAD_ERR_ALLOC);
-    b.workspace_bytes = bytes;
+    void* fresh = nullptr;
+    HIP_TRY(hipMalloc(&fresh, bytes), PRAD_ERR_ALLOC);
+    if (g_ctx.workspace) {
+        if (g_ctx.live_graphs > 0) {
+            g_ctx.retired_workspaces.push_back(g_ctx.workspace);
+        } else {
+            if (int32_t st = sync_all()) { (void)hipFree(fresh); return st; }
+            (void)hipFree(g_ctx.workspace);
+        }
+    }
+    g_ctx.workspace = fresh;
+    g_ctx.workspace_bytes = bytes;
     return PRAD_OK;
+}
+
+// ---- recorded launch sequences ----------------------------------------------------------------------------
+constexpr uint32_t GRAPH_MAGIC = 0x50524147u;  // "PRAG"
+// An Adam kernel node of a recording: its bias-correction factors 1 / (1 - beta^t) are launch arguments, so every
+// replay that stands for a later AdamIteration gets them replaced (the reference's caller advances AdamIteration
+// once per step, src/RMAD/AdamOptimizer.cs:204-207).
+struct AdamNode {
+    hipGraphNode_t node;
+    int32_t dtype;
+    double beta1, beta2;
+    double t;        // AdamIteration the node was recorded with
+    double applied;  // AdamIteration its current arguments stand for
+};
+struct RecordedGraph {
+    uint32_t magic;
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    std::vector<AdamNode> adam;
+    double base_t;  // smallest recorded AdamIteration
+    double next_t;  // AdamIteration the next launch gives the nodes recorded with base_t
+};
+constexpr int MAX_ADAM_NODES = 64;
+AdamNode g_recording_adam[MAX_ADAM_NODES];  // nodes of the open recording (lock held whenever touched)
+int g_recording_adam_count = 0;
+bool g_recording_failed = false;
+
+struct PendingAdam { int32_t dtype; double beta1, beta2, t; };
+void note_adam_node(void* ctx, hipStream_t s) {
+    const PendingAdam* pa = static_cast<const PendingAdam*>(ctx);
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    hipGraph_t graph = nullptr;
+    const hipGraphNode_t* deps = nullptr;
+    size_t ndeps = 0;
+    if (hipStreamGetCaptureInfo_v2(s, &status, &id, &graph, &deps, &ndeps) != hipSuccess || status != hipStreamCaptureStatusActive ||
+        ndeps != 1 || g_recording_adam_count >= MAX_ADAM_NODES) {
+        g_recording_failed = true;  // reported by prad_graph_end
+        return;
+    }
+    g_recording_adam[g_recording_adam_count++] = AdamNode{deps[0], pa->dtype, pa->beta1, pa->beta2, pa->t, pa->t};
+}
+
+// 1 / (1 - Math.Pow(beta, AdamIteration)), src/RMAD/AdamOptimizer.cs:204-207; PRADLite: every parameter is a float and
+// PradMath.Pow(float, float) is (float)Math.Pow.
+inline void bias_correction(double beta1, double beta2, double t, double* c1, double* c2) {
+    *c1 = 1 / (1 - std::pow(beta1, t));
+    *c2 = 1 / (1 - std::pow(beta2, t));
+}
+inline void bias_correction(float b1, float b2, float tf, float* c1, float* c2) {
+    *c1 = 1 / (1 - (float)std::pow((double)b1, (double)tf));
+    *c2 = 1 / (1 - (float)std::pow((double)b2, (double)tf));
 }
 
 int32_t same_dtype(std::initializer_list<prad_buf_t> bufs) {
@@ -161,7 +228,7 @@ GemmArgs<T> plain_gemm(int transA, int transB, int64_t M, int64_t N, int64_t K, 
 }
 
 // Products split along K (in several passes, or as pairs of workgroups per tile) need room for their
-// partial results; the selected branch's workspace is grown here (lock held).
+// partial results; the workspace is grown here (lock held).
 template <typename T>
 int32_t attach_split_workspace(GemmArgs<T>& a) {
     const int splits = gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T));
@@ -169,7 +236,7 @@ int32_t attach_split_workspace(GemmArgs<T>& a) {
     if (splits <= 1 && !pairs) return PRAD_OK;
     if (int32_t st = ensure_workspace((size_t)(pairs ? 2 : splits) * a.batch * a.M * a.N * sizeof(T))) return st;
     a.split_ws = static_cast<T*>(CUR_WORKSPACE);
-    a.split_counters = cur_branch().counter;
+    a.split_counters = g_ctx.counter;
     return PRAD_OK;
 }
 
@@ -361,16 +428,11 @@ int32_t prad_init(int32_t device_id) {
     HIP_TRY(hipGetDeviceProperties(&prop, device_id), PRAD_ERR_NOT_INITIALIZED);
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(PRAD_ERR_NOT_INITIALIZED, "device %d is %s; this library is built for gfx950 only", device_id, prop.gcnArchName);
-    for (int i = 0; i < MAX_BRANCHES; ++i) {
-        HIP_TRY(hipStreamCreateWithFlags(&g_ctx.branch[i].stream, hipStreamNonBlocking), PRAD_ERR_NOT_INITIALIZED);
-        HIP_TRY(hipEventCreateWithFlags(&g_ctx.branch[i].done, hipEventDisableTiming), PRAD_ERR_NOT_INITIALIZED);
-        g_ctx.branch[i].open = false;
-        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.branch[i].counter), COUNTER_BYTES), PRAD_ERR_ALLOC);
-        HIP_TRY(hipMemset(g_ctx.branch[i].counter, 0, COUNTER_BYTES), PRAD_ERR_ALLOC);
-    }
-    HIP_TRY(hipEventCreateWithFlags(&g_ctx.fork_event, hipEventDisableTiming), PRAD_ERR_NOT_INITIALIZED);
-    g_ctx.stream = g_ctx.branch[0].stream;
-    g_ctx.cur = 0;
+    HIP_TRY(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking), PRAD_ERR_NOT_INITIALIZED);
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.counter), COUNTER_BYTES), PRAD_ERR_ALLOC);
+    HIP_TRY(hipMemset(g_ctx.counter, 0, COUNTER_BYTES), PRAD_ERR_ALLOC);
+    g_ctx.recording = false;
+    g_ctx.live_graphs = 0;
     g_ctx.device = device_id;
     g_ctx.initialized.store(true);
     return PRAD_OK;
@@ -382,18 +444,16 @@ int32_t prad_shutdown(void) {
     (void)hipSetDevice(g_ctx.device);
     (void)sync_all();
     if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
-    for (Branch& b : g_ctx.branch) {
-        if (b.workspace) (void)hipFree(b.workspace);
-        if (b.counter) (void)hipFree(b.counter);
-        if (b.done) (void)hipEventDestroy(b.done);
-        if (b.stream) (void)hipStreamDestroy(b.stream);
-        b = Branch{};
-    }
-    if (g_ctx.fork_event) (void)hipEventDestroy(g_ctx.fork_event);
-    g_ctx.fork_event = nullptr;
+    if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
+    free_retired_workspaces();
+    if (g_ctx.counter) (void)hipFree(g_ctx.counter);
+    if (g_ctx.stream) (void)hipStreamDestroy(g_ctx.stream);
+    g_ctx.workspace = nullptr; g_ctx.workspace_bytes = 0;
+    g_ctx.counter = nullptr;
     g_ctx.pinned = nullptr; g_ctx.pinned_bytes = 0;
     g_ctx.stream = nullptr;
-    g_ctx.cur = 0;
+    g_ctx.recording = false;
+    g_ctx.live_graphs = 0;
     g_ctx.device = -1;
     g_ctx.initialized.store(false);
     return PRAD_OK;
@@ -406,6 +466,8 @@ void* prad_stream(void) { return g_ctx.stream; }
 
 int32_t prad_stream_sync(void) {
     REQUIRE_INIT();
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("waiting for the device");
     return sync_all();
 }
 
@@ -418,9 +480,10 @@ int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t 
     if (depth <= 0 || rows <= 0 || cols <= 0) return fail(PRAD_ERR_ARG, "matrix dimensions must be positive");
     const size_t bytes = (size_t)depth * rows * cols * elem_size(dtype);
     void* p = nullptr;
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("an allocation");
     HIP_TRY(hipMalloc(&p, bytes), PRAD_ERR_ALLOC);
     {
-        std::lock_guard<std::mutex> lock(g_ctx.mu);
         hipError_t e = dtype == PRAD_F64 ? launch_fill_zero<double>(static_cast<double*>(p), depth * rows * cols, CUR_STREAM)
                                          : launch_fill_zero<float>(static_cast<float*>(p), depth * rows * cols, CUR_STREAM);
         if (e != hipSuccess) { (void)hipFree(p); return fail(PRAD_ERR_LAUNCH, "zero fill failed: %s", hipGetErrorString(e)); }
@@ -448,7 +511,8 @@ int32_t prad_buf_free(prad_buf_t b) {
     REQUIRE_BUF(b);
     if (b->owned) {
         REQUIRE_INIT();
-        std::lock_guard<std::mutex> lock(g_ctx.mu);
+        ENQUEUE_LOCK();
+        NOT_WHILE_RECORDING("freeing a buffer");
         // Work that still uses the buffer may be queued.
         if (int32_t st = sync_all()) return st;
         HIP_TRY(hipFree(b->ptr), PRAD_ERR_ALLOC);
@@ -472,7 +536,7 @@ void* prad_buf_device_ptr(prad_buf_t b) { return valid(b) ? b->ptr : nullptr; }
 int32_t prad_buf_zero(prad_buf_t b) {
     REQUIRE_INIT();
     REQUIRE_BUF(b);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     if (b->dtype == PRAD_F64) HIP_TRY(launch_fill_zero<double>(static_cast<double*>(b->ptr), count(b), CUR_STREAM), PRAD_ERR_LAUNCH);
     else HIP_TRY(launch_fill_zero<float>(static_cast<float*>(b->ptr), count(b), CUR_STREAM), PRAD_ERR_LAUNCH);
     return PRAD_OK;
@@ -489,8 +553,8 @@ int32_t prad_buf_upload_rows(prad_buf_t b, const void* const* row_ptrs, const in
     for (int64_t i = 0; i < nrows; ++i)
         if (row_ptrs[i] == nullptr) return fail(PRAD_ERR_NOT_RECTANGULAR, "The given jagged array is not rectangular.");
     const size_t row_bytes = (size_t)b->cols * elem_size(b->dtype);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (int32_t st = drain_open_branches()) return st;
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("a copy to or from the host");
     int64_t rows_per_chunk = (int64_t)(STAGING_CHUNK / row_bytes);
     if (rows_per_chunk < 1) rows_per_chunk = 1;
     if (rows_per_chunk > nrows) rows_per_chunk = nrows;
@@ -514,8 +578,8 @@ int32_t prad_buf_download_rows(prad_buf_t b, void* const* row_ptrs) {
     for (int64_t i = 0; i < nrows; ++i)
         if (row_ptrs[i] == nullptr) return fail(PRAD_ERR_NOT_RECTANGULAR, "The given jagged array is not rectangular.");
     const size_t row_bytes = (size_t)b->cols * elem_size(b->dtype);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (int32_t st = drain_open_branches()) return st;
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("a copy to or from the host");
     int64_t rows_per_chunk = (int64_t)(STAGING_CHUNK / row_bytes);
     if (rows_per_chunk < 1) rows_per_chunk = 1;
     if (rows_per_chunk > nrows) rows_per_chunk = nrows;
@@ -536,8 +600,8 @@ int32_t prad_buf_upload(prad_buf_t b, const void* src, int64_t ld) {
     REQUIRE_BUF(b);
     if (src == nullptr || ld < b->cols) return fail(PRAD_ERR_ARG, "bad source pointer or leading dimension");
     const size_t es = elem_size(b->dtype);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (int32_t st = drain_open_branches()) return st;
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("a copy to or from the host");
     HIP_TRY(hipMemcpy2DAsync(b->ptr, (size_t)b->cols * es, src, (size_t)ld * es, (size_t)b->cols * es,
                              (size_t)(b->depth * b->rows), hipMemcpyHostToDevice, g_ctx.stream), PRAD_ERR_LAUNCH);
     HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
@@ -549,8 +613,8 @@ int32_t prad_buf_download(prad_buf_t b, void* dst, int64_t ld) {
     REQUIRE_BUF(b);
     if (dst == nullptr || ld < b->cols) return fail(PRAD_ERR_ARG, "bad destination pointer or leading dimension");
     const size_t es = elem_size(b->dtype);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (int32_t st = drain_open_branches()) return st;
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("a copy to or from the host");
     HIP_TRY(hipMemcpy2DAsync(dst, (size_t)ld * es, b->ptr, (size_t)b->cols * es, (size_t)b->cols * es,
                              (size_t)(b->depth * b->rows), hipMemcpyDeviceToHost, g_ctx.stream), PRAD_ERR_LAUNCH);
     HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
@@ -562,7 +626,7 @@ int32_t prad_buf_copy(prad_buf_t dst, prad_buf_t src) {
     REQUIRE_BUF(dst); REQUIRE_BUF(src);
     if (int32_t st = same_dtype({dst, src})) return st;
     if (int32_t st = same_shape(dst, src, "copy")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     // A kernel rather than hipMemcpyAsync: it can be recorded into a captured graph and shows up in
     // kernel traces as a plain copy of known size.
     if (src->dtype == PRAD_F64)
@@ -577,19 +641,19 @@ int32_t prad_buf_copy(prad_buf_t dst, prad_buf_t src) {
 // ---------------------------------------------------------------------------------------------
 int32_t prad_gemm(int32_t transA, int32_t transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int32_t accumulate) {
     REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return enqueue_gemm(transA, transB, A, B, C, accumulate, Epilogue{}, false);
 }
 
 int32_t prad_gemm_batched(int32_t transA, int32_t transB, prad_buf_t A, prad_buf_t B, prad_buf_t C, int32_t accumulate) {
     REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return enqueue_gemm(transA, transB, A, B, C, accumulate, Epilogue{}, true);
 }
 
 int32_t prad_matmul_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t C) {
     REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return enqueue_gemm(0, 0, A, B, C, 0, Epilogue{}, false);
 }
 
@@ -599,7 +663,7 @@ int32_t prad_matmul_fwd_fused(prad_buf_t A, prad_buf_t B, prad_buf_t bias, prad_
     if (Z != nullptr) REQUIRE_BUF(Z);
     Epilogue ep;
     ep.bias = bias; ep.Z = Z; ep.act_fwd = act; ep.alpha = alpha;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return enqueue_gemm(0, 0, A, B, H, 0, ep, false);
 }
 
@@ -670,7 +734,7 @@ static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad
 int32_t prad_matmul_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf_t dA, prad_buf_t dB, int32_t accumulate_dA,
                         int32_t accumulate_dB) {
     REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return matmul_bwd_locked(dC, A, B, dA, dB, accumulate_dA, accumulate_dB, Epilogue{});
 }
 
@@ -679,7 +743,7 @@ int32_t prad_matmul_bwd_fused(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_bu
     REQUIRE_INIT();
     Epilogue ep;
     ep.act_bwd = act; ep.act_src = act_src; ep.alpha = alpha;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return matmul_bwd_locked(dC, A, B, dA, dB, 0, accumulate_dB, ep);
 }
 
@@ -694,7 +758,7 @@ int32_t prad_matmul_batch_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t bias, p
         return fail(PRAD_ERR_ARG, "output must be %lldx%lld", (long long)A->rows, (long long)B->cols);
     if (bias && (bias->rows != 1 || bias->cols != C->cols || bias->depth != 1))
         return fail(PRAD_ERR_ARG, "The length of the bias vector must be the same as the number of columns in the input matrix.");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return A->dtype == PRAD_F64 ? batch_sum_fwd_t<double>(A, B, bias, C) : batch_sum_fwd_t<float>(A, B, bias, C);
 }
 
@@ -706,7 +770,7 @@ int32_t prad_matmul_batch_sum_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, pra
     if (dC->depth != 1 || dC->rows != A->rows || dC->cols != B->cols)
         return fail(PRAD_ERR_ARG, "upstream gradient is %lldx%lld, the product is %lldx%lld", (long long)dC->rows,
                     (long long)dC->cols, (long long)A->rows, (long long)B->cols);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     if (dA != nullptr) {
         REQUIRE_BUF(dA);
         if (int32_t st = same_shape(A, dA, "gradient of the first operand")) return st;
@@ -726,7 +790,7 @@ int32_t prad_matmul_bias_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf
     REQUIRE_INIT();
     Epilogue ep;
     ep.act_bwd = act; ep.act_src = act_src; ep.alpha = alpha;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return matmul_bwd_locked(dC, A, B, dA, dB, 0, accumulate_dB, ep, dbias);
 }
 
@@ -740,7 +804,7 @@ int32_t prad_matmul_bias_bwd(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad_buf
             return fail(PRAD_ERR_ARG, "unsupported transpose combination (%d, %d)", transA, transB);                  \
         if (lda < (transA ? M : K) || ldb < (transB ? K : N) || ldc < N) return fail(PRAD_ERR_ARG, "leading dimension too small"); \
         GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                   \
-        std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                   \
+        ENQUEUE_LOCK();                                                                                               \
         if (int32_t st = attach_split_workspace(a)) return st;                                                        \
         HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);                                                    \
         return PRAD_OK;                                                                                               \
@@ -763,7 +827,7 @@ RAW_GEMM(f32, float)
         if (batch > 65535) return fail(PRAD_ERR_ARG, "at most 65535 products per call");                               \
         GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                    \
         a.batch = batch; a.strideA = strideA; a.strideB = strideB; a.strideC = strideC;                                \
-        std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                    \
+        ENQUEUE_LOCK();                                                                                                \
         HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);                                                     \
         return PRAD_OK;                                                                                                \
     }
@@ -787,7 +851,7 @@ RAW_BATCHED_GEMM(f32, float)
         GemmArgs<T> a = plain_gemm<T>(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, accumulate);                    \
         a.batch = batch_outer * batch_inner; a.strideA = strideA; a.strideB = strideB; a.strideC = strideC;            \
         a.batch_inner = batch_inner; a.istrideA = istrideA; a.istrideB = istrideB; a.istrideC = istrideC;              \
-        std::lock_guard<std::mutex> lock(g_ctx.mu);                                                                    \
+        ENQUEUE_LOCK();                                                                                                \
         HIP_TRY(launch_gemm<T>(a, CUR_STREAM), PRAD_ERR_LAUNCH);                                                     \
         return PRAD_OK;                                                                                                \
     }
@@ -888,7 +952,7 @@ int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out) {
     if (A->cols != B->rows) return fail(PRAD_ERR_SHAPE, "Matrix dimensions must be compatible for multiplication.");
     const int64_t P = B->depth;
     if (out->depth != 1 || out->rows != 1 || out->cols != P) return fail(PRAD_ERR_ARG, "output must be 1 x depth");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     const size_t ws = (size_t)P * gemm_tiles_per_product(A->rows, B->cols) * sizeof(double);
     if (int32_t st = ensure_workspace(ws)) return st;
     double* w = static_cast<double*>(CUR_WORKSPACE);
@@ -918,7 +982,7 @@ int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_bu
     }
     if (dB != nullptr && (dB->depth != P || dB->rows != K || dB->cols != M))
         return fail(PRAD_ERR_ARG, "dB must be depth x cols(A) x rows(A)");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     if (A->dtype == PRAD_F64)
         HIP_TRY(launch_matmul_sum_bwd<double>(static_cast<const double*>(A->ptr), static_cast<const double*>(B->ptr),
                                               static_cast<const double*>(dOut->ptr), dA ? static_cast<double*>(dA->ptr) : nullptr,
@@ -947,7 +1011,7 @@ int32_t prad_act_fwd(int32_t act, prad_buf_t x, prad_buf_t y, double alpha) {
     if (act < PRAD_ACT_LEAKYRELU || act > PRAD_ACT_AMPLIFIED_SIGMOID) return fail(PRAD_ERR_ARG, "unknown activation selector");
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "activation")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(x, launch_act_fwd<double>(act, D(x), D(y), count(x), alpha, CUR_STREAM),
              launch_act_fwd<float>(act, F(x), F(y), count(x), (float)alpha, CUR_STREAM));
     return PRAD_OK;
@@ -960,7 +1024,7 @@ int32_t prad_act_bwd(int32_t act, prad_buf_t src, prad_buf_t dy, prad_buf_t dx, 
     if (int32_t st = same_dtype({src, dy, dx})) return st;
     if (int32_t st = same_shape(src, dy, "activation backward")) return st;
     if (int32_t st = same_shape(src, dx, "activation backward")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(src, launch_act_bwd<double>(act, D(src), D(dy), D(dx), count(src), alpha, CUR_STREAM),
              launch_act_bwd<float>(act, F(src), F(dy), F(dx), count(src), (float)alpha, CUR_STREAM));
     return PRAD_OK;
@@ -972,7 +1036,7 @@ int32_t prad_hadamard_fwd(prad_buf_t a, prad_buf_t b, prad_buf_t y) {
     if (int32_t st = same_dtype({a, b, y})) return st;
     if (int32_t st = same_shape(a, b, "Hadamard product")) return st;
     if (int32_t st = same_shape(a, y, "Hadamard product")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(a, launch_hadamard_fwd<double>(D(a), D(b), D(y), count(a), CUR_STREAM),
              launch_hadamard_fwd<float>(F(a), F(b), F(y), count(a), CUR_STREAM));
     return PRAD_OK;
@@ -984,7 +1048,7 @@ int32_t prad_hadamard_bwd(prad_buf_t a, prad_buf_t b, prad_buf_t dy, prad_buf_t 
     if (int32_t st = same_dtype({a, b, dy, da, db})) return st;
     for (prad_buf_t o : {b, dy, da, db})
         if (int32_t st = same_shape(a, o, "Hadamard product")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(a, launch_hadamard_bwd<double>(D(a), D(b), D(dy), D(da), D(db), count(a), CUR_STREAM),
              launch_hadamard_bwd<float>(F(a), F(b), F(dy), F(da), F(db), count(a), CUR_STREAM));
     return PRAD_OK;
@@ -995,7 +1059,7 @@ int32_t prad_scale(prad_buf_t x, prad_buf_t y, double scalar) {
     REQUIRE_BUF(x); REQUIRE_BUF(y);
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "multiply by scalar")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(x, launch_scale<double>(D(y), D(x), count(x), scalar, CUR_STREAM),
              launch_scale<float>(F(y), F(x), count(x), (float)scalar, CUR_STREAM));
     return PRAD_OK;
@@ -1006,7 +1070,7 @@ int32_t prad_accumulate(prad_buf_t dest, prad_buf_t grad) {
     REQUIRE_BUF(dest); REQUIRE_BUF(grad);
     if (int32_t st = same_dtype({dest, grad})) return st;
     if (int32_t st = same_shape(dest, grad, "accumulate")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(dest, launch_accumulate<double>(D(dest), D(grad), count(dest), CUR_STREAM),
              launch_accumulate<float>(F(dest), F(grad), count(dest), CUR_STREAM));
     return PRAD_OK;
@@ -1018,7 +1082,7 @@ int32_t prad_add(prad_buf_t a, prad_buf_t b, prad_buf_t y) {
     if (int32_t st = same_dtype({a, b, y})) return st;
     if (int32_t st = same_shape(a, b, "add")) return st;
     if (int32_t st = same_shape(a, y, "add")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(a, launch_add<double>(D(a), D(b), D(y), count(a), CUR_STREAM), launch_add<float>(F(a), F(b), F(y), count(a), CUR_STREAM));
     return PRAD_OK;
 }
@@ -1029,7 +1093,7 @@ int32_t prad_add_three(prad_buf_t a, prad_buf_t b, prad_buf_t c, prad_buf_t y) {
     if (int32_t st = same_dtype({a, b, c, y})) return st;
     for (prad_buf_t o : {b, c, y})
         if (int32_t st = same_shape(a, o, "add three")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(a, launch_add_three<double>(D(a), D(b), D(c), D(y), count(a), CUR_STREAM),
              launch_add_three<float>(F(a), F(b), F(c), F(y), count(a), CUR_STREAM));
     return PRAD_OK;
@@ -1043,7 +1107,7 @@ int32_t prad_transpose(prad_buf_t x, prad_buf_t y) {
         return fail(PRAD_ERR_ARG, "the transpose of a %lldx%lld matrix is %lldx%lld", (long long)x->rows, (long long)x->cols,
                     (long long)x->cols, (long long)x->rows);
     if (x->ptr == y->ptr) return fail(PRAD_ERR_ARG, "transpose in place is not supported");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(x, launch_transpose<double>(D(x), D(y), x->rows, x->cols, CUR_STREAM),
              launch_transpose<float>(F(x), F(y), x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
@@ -1062,7 +1126,7 @@ int32_t prad_layernorm_fwd(prad_buf_t x, prad_buf_t y, prad_buf_t mean, prad_buf
     if (int32_t st = same_dtype({x, y, mean, stddev})) return st;
     if (int32_t st = same_shape(x, y, "layer normalization")) return st;
     if (int32_t st = layernorm_shapes(x, mean, stddev)) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(x, launch_layernorm_fwd<double>(D(x), D(y), D(mean), D(stddev), x->rows, x->cols, CUR_STREAM),
              launch_layernorm_fwd<float>(F(x), F(y), F(mean), F(stddev), x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
@@ -1075,7 +1139,7 @@ int32_t prad_layernorm_bwd(prad_buf_t x, prad_buf_t mean, prad_buf_t stddev, pra
     if (int32_t st = same_shape(x, dy, "layer normalization backward")) return st;
     if (int32_t st = same_shape(x, dx, "layer normalization backward")) return st;
     if (int32_t st = layernorm_shapes(x, mean, stddev)) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(x, launch_layernorm_bwd<double>(D(x), D(mean), D(stddev), D(dy), D(dx), x->rows, x->cols, CUR_STREAM),
              launch_layernorm_bwd<float>(F(x), F(mean), F(stddev), F(dy), F(dx), x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
@@ -1088,7 +1152,7 @@ int32_t prad_add_broadcast_fwd(prad_buf_t x, prad_buf_t bias, prad_buf_t y) {
     if (bias->cols != x->cols || bias->rows != 1 || bias->depth != 1)
         return fail(PRAD_ERR_ARG, "The length of the bias vector must be the same as the number of columns in the input matrix.");
     if (int32_t st = same_shape(x, y, "add broadcasting")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(x, launch_add_broadcast_fwd<double>(D(x), D(bias), D(y), x->depth * x->rows, x->cols, CUR_STREAM),
              launch_add_broadcast_fwd<float>(F(x), F(bias), F(y), x->depth * x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
@@ -1100,7 +1164,7 @@ int32_t prad_add_broadcast_bwd_bias(prad_buf_t dy, prad_buf_t dbias) {
     if (int32_t st = same_dtype({dy, dbias})) return st;
     if (dbias->cols != dy->cols || dbias->rows != 1 || dbias->depth != 1 || dy->depth != 1)
         return fail(PRAD_ERR_ARG, "bias gradient must be 1 x cols");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     double* ws = nullptr;
     if (colsum_chunks(dy->rows) > 1) {
         if (int32_t st = ensure_workspace((size_t)colsum_chunks(dy->rows) * dy->cols * sizeof(double))) return st;
@@ -1117,7 +1181,7 @@ static int32_t softmax_fwd_scaled(prad_buf_t x, double alpha, prad_buf_t y) {
     REQUIRE_BUF(x); REQUIRE_BUF(y);
     if (int32_t st = same_dtype({x, y})) return st;
     if (int32_t st = same_shape(x, y, "softmax")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(x, launch_softmax_fwd<double>(D(x), D(y), x->depth * x->rows, x->cols, alpha, CUR_STREAM),
              launch_softmax_fwd<float>(F(x), F(y), x->depth * x->rows, x->cols, (float)alpha, CUR_STREAM));
     return PRAD_OK;
@@ -1129,7 +1193,7 @@ static int32_t softmax_bwd_scaled(prad_buf_t y, prad_buf_t dy, double alpha, pra
     if (int32_t st = same_dtype({y, dy, dx})) return st;
     if (int32_t st = same_shape(y, dy, "softmax backward")) return st;
     if (int32_t st = same_shape(y, dx, "softmax backward")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(y, launch_softmax_bwd<double>(D(y), D(dy), D(dx), y->depth * y->rows, y->cols, alpha, CUR_STREAM),
              launch_softmax_bwd<float>(F(y), F(dy), F(dx), y->depth * y->rows, y->cols, (float)alpha, CUR_STREAM));
     return PRAD_OK;
@@ -1147,7 +1211,7 @@ int32_t prad_cce_fwd(prad_buf_t p, prad_buf_t target, prad_buf_t loss) {
     if (p->depth != 1 || p->rows != target->rows || p->cols != target->cols || target->depth != 1)
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(p, launch_cce_fwd<double>(D(p), D(target), D(loss), p->rows, p->cols, CUR_STREAM),
              launch_cce_fwd<float>(F(p), F(target), F(loss), p->rows, p->cols, CUR_STREAM));
     return PRAD_OK;
@@ -1160,7 +1224,7 @@ int32_t prad_cce_bwd(prad_buf_t p, prad_buf_t target, prad_buf_t dp) {
     if (p->depth != 1 || p->rows != target->rows || p->cols != target->cols || target->depth != 1)
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (int32_t st = same_shape(p, dp, "cross-entropy backward")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(p, launch_cce_bwd<double>(D(p), D(target), D(dp), p->rows, p->cols, CUR_STREAM),
              launch_cce_bwd<float>(F(p), F(target), F(dp), p->rows, p->cols, CUR_STREAM));
     return PRAD_OK;
@@ -1173,7 +1237,7 @@ int32_t prad_mse_fwd(prad_buf_t y, prad_buf_t target, prad_buf_t loss) {
     if (y->depth != target->depth || y->rows != target->rows || y->cols != target->cols)
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     if (int32_t st = ensure_workspace(mse_workspace_bytes())) return st;
     double* w = static_cast<double*>(CUR_WORKSPACE);
     DISPATCH(y, launch_mse_fwd<double>(D(y), D(target), D(loss), w, count(y), CUR_STREAM),
@@ -1189,7 +1253,7 @@ int32_t prad_mse(prad_buf_t y, prad_buf_t target, prad_buf_t loss, prad_buf_t dy
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (loss->depth != 1 || loss->rows != 1 || loss->cols != 1) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
     if (int32_t st = same_shape(y, dy, "mean squared error backward")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     if (int32_t st = ensure_workspace(mse_workspace_bytes())) return st;
     double* w = static_cast<double*>(CUR_WORKSPACE);
     DISPATCH(y, launch_mse_fwd<double>(D(y), D(target), D(loss), w, count(y), CUR_STREAM, D(dy)),
@@ -1204,7 +1268,7 @@ int32_t prad_mse_bwd(prad_buf_t y, prad_buf_t target, prad_buf_t dy) {
     if (y->depth != target->depth || y->rows != target->rows || y->cols != target->cols)
         return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
     if (int32_t st = same_shape(y, dy, "mean squared error backward")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(y, launch_mse_bwd<double>(D(y), D(target), D(dy), count(y), CUR_STREAM),
              launch_mse_bwd<float>(F(y), F(target), F(dy), count(y), CUR_STREAM));
     return PRAD_OK;
@@ -1219,7 +1283,7 @@ int32_t prad_lstm_cell_fwd(prad_buf_t G, prad_buf_t c_prev, prad_buf_t c, prad_b
         return fail(PRAD_ERR_ARG, "gate pre-activations must be rows x 4*hidden");
     for (prad_buf_t o : {c_prev, tanh_c, h})
         if (int32_t st = same_shape(c, o, "LSTM cell")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(c, launch_lstm_cell_fwd<double>(D(G), D(c_prev), D(c), D(tanh_c), D(h), rows, hidden, CUR_STREAM),
              launch_lstm_cell_fwd<float>(F(G), F(c_prev), F(c), F(tanh_c), F(h), rows, hidden, CUR_STREAM));
     return PRAD_OK;
@@ -1239,7 +1303,7 @@ int32_t prad_lstm_cell_bwd(prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_
     for (prad_buf_t o : {tanh_c, dh_a, dh_b, dc_in, dc_prev})
         if (o != nullptr)
             if (int32_t st = same_shape(c_prev, o, "LSTM cell backward")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     DISPATCH(c_prev,
              launch_lstm_cell_bwd<double>(D(gates), D(c_prev), D(tanh_c), D(dh_a), dh_b ? D(dh_b) : nullptr, dc_in ? D(dc_in) : nullptr,
                                           D(dG), D(dc_prev), rows, hidden, CUR_STREAM),
@@ -1259,7 +1323,7 @@ int32_t prad_lstm_step_fwd(prad_buf_t h_prev, prad_buf_t Wh, prad_buf_t G, prad_
     if (Wh->depth != 1 || Wh->rows != hidden || Wh->cols != 4 * hidden) return fail(PRAD_ERR_SHAPE, "recurrent weight must be hidden x 4*hidden");
     for (prad_buf_t o : {h_prev, c_prev, tanh_c, h})
         if (int32_t st = same_shape(c, o, "LSTM step")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return G->dtype == PRAD_F64 ? lstm_step_fwd_t<double>(h_prev, Wh, G, c_prev, c, tanh_c, h)
                                 : lstm_step_fwd_t<float>(h_prev, Wh, G, c_prev, c, tanh_c, h);
 }
@@ -1280,7 +1344,7 @@ int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, 
     for (prad_buf_t o : {tanh_c, dh_loss, dc_in, dc_prev, dh_scratch})
         if (o != nullptr)
             if (int32_t st = same_shape(c_prev, o, "LSTM step backward")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     return gates->dtype == PRAD_F64
                ? lstm_step_bwd_t<double>(dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch)
                : lstm_step_bwd_t<float>(dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch);
@@ -1297,84 +1361,107 @@ int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_b
 }
 
 // ---------------------------------------------------------------------------------------------
-// Recording holds the context lock's place in line only per call: other threads must not enqueue
-// while a recording is open (their work would be recorded too), which the caller guarantees.
+// Recording.  The stream is captured in thread-local mode and the context remembers which thread records:
+// every enqueueing entry point called from another thread while a recording is open returns
+// PRAD_ERR_RECORDING instead of slipping its work into the recorded sequence (the reference calls Backward of
+// independent operations from pool threads, src/RMAD/OperationNeuralNetworkVisitor.cs:303-306).
 int32_t prad_graph_begin(void) {
     REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
+    if (g_ctx.recording) return fail(PRAD_ERR_RECORDING, "a launch sequence is already being recorded");
     HIP_TRY(hipStreamBeginCapture(g_ctx.stream, hipStreamCaptureModeThreadLocal), PRAD_ERR_LAUNCH);
+    g_ctx.recording = true;
+    g_ctx.recorder = std::this_thread::get_id();
+    g_recording_adam_count = 0;
+    g_recording_failed = false;
     return PRAD_OK;
 }
 
 int32_t prad_graph_end(void** graph) {
     REQUIRE_INIT();
     if (graph == nullptr) return fail(PRAD_ERR_ARG, "graph is NULL");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    for (int i = 1; i < MAX_BRANCHES; ++i)
-        if (g_ctx.branch[i].open) return fail(PRAD_ERR_ARG, "prad_join must close the open branches before prad_graph_end");
+    *graph = nullptr;
+    ENQUEUE_LOCK();
+    if (!g_ctx.recording) return fail(PRAD_ERR_ARG, "prad_graph_end without prad_graph_begin");
+    g_ctx.recording = false;
     hipGraph_t g = nullptr;
     HIP_TRY(hipStreamEndCapture(g_ctx.stream, &g), PRAD_ERR_LAUNCH);
+    if (g_recording_failed) {
+        (void)hipGraphDestroy(g);
+        return fail(PRAD_ERR_LAUNCH, "the recording lost track of an Adam kernel node");
+    }
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
-    (void)hipGraphDestroy(g);
-    if (e != hipSuccess) return fail(PRAD_ERR_LAUNCH, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
-    *graph = exec;
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        return fail(PRAD_ERR_LAUNCH, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    RecordedGraph* rg = new RecordedGraph{GRAPH_MAGIC, g, exec,
+                                          std::vector<AdamNode>(g_recording_adam, g_recording_adam + g_recording_adam_count), 0.0, 0.0};
+    g_recording_adam_count = 0;
+    if (!rg->adam.empty()) {
+        rg->base_t = rg->adam[0].t;
+        for (const AdamNode& n : rg->adam) rg->base_t = n.t < rg->base_t ? n.t : rg->base_t;
+        rg->next_t = rg->base_t;
+    }
+    ++g_ctx.live_graphs;
+    *graph = rg;
+    return PRAD_OK;
+}
+
+static RecordedGraph* recorded(void* graph) {
+    RecordedGraph* rg = static_cast<RecordedGraph*>(graph);
+    return (rg != nullptr && rg->magic == GRAPH_MAGIC) ? rg : nullptr;
+}
+
+int32_t prad_graph_set_adam_iteration(void* graph, double t) {
+    REQUIRE_INIT();
+    ENQUEUE_LOCK();
+    RecordedGraph* rg = recorded(graph);
+    if (rg == nullptr) return fail(PRAD_ERR_BAD_HANDLE, "not a recorded launch sequence");
+    if (!(t >= 1.0)) return fail(PRAD_ERR_ARG, "AdamIteration starts at 1");
+    rg->next_t = t;
     return PRAD_OK;
 }
 
 int32_t prad_graph_launch(void* graph) {
     REQUIRE_INIT();
-    if (graph == nullptr) return fail(PRAD_ERR_ARG, "graph is NULL");
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), g_ctx.stream), PRAD_ERR_LAUNCH);
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("launching a recorded sequence");
+    RecordedGraph* rg = recorded(graph);
+    if (rg == nullptr) return fail(PRAD_ERR_BAD_HANDLE, "not a recorded launch sequence");
+    for (AdamNode& n : rg->adam) {
+        const double t = rg->next_t + (n.t - rg->base_t);
+        if (t == n.applied) continue;
+        if (n.dtype == PRAD_F64) {
+            double c1, c2;
+            bias_correction(n.beta1, n.beta2, t, &c1, &c2);
+            HIP_TRY(adam_node_set_bias_correction<double>(rg->exec, n.node, c1, c2), PRAD_ERR_LAUNCH);
+        } else {
+            float c1, c2;
+            bias_correction((float)n.beta1, (float)n.beta2, (float)t, &c1, &c2);
+            HIP_TRY(adam_node_set_bias_correction<float>(rg->exec, n.node, c1, c2), PRAD_ERR_LAUNCH);
+        }
+        n.applied = t;
+    }
+    HIP_TRY(hipGraphLaunch(rg->exec, g_ctx.stream), PRAD_ERR_LAUNCH);
+    rg->next_t += 1.0;
     return PRAD_OK;
 }
 
 int32_t prad_graph_destroy(void* graph) {
     REQUIRE_INIT();
     if (graph == nullptr) return PRAD_OK;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("destroying a recorded sequence");
+    RecordedGraph* rg = recorded(graph);
+    if (rg == nullptr) return fail(PRAD_ERR_BAD_HANDLE, "not a recorded launch sequence");
     if (int32_t st = sync_all()) return st;
-    HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)), PRAD_ERR_ARG);
-    return PRAD_OK;
-}
-
-// ---------------------------------------------------------------------------------------------
-// Branches: operations that do not depend on each other (the reference's visitor runs their
-// Backward on pool threads, src/RMAD/OperationNeuralNetworkVisitor.cs:303-306) are enqueued on
-// different branches and may run side by side; recorded, they become parallel paths of the graph.
-int32_t prad_fork(int32_t branches) {
-    REQUIRE_INIT();
-    if (branches < 2 || branches > MAX_BRANCHES) return fail(PRAD_ERR_ARG, "branches must be 2..%d", MAX_BRANCHES);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    HIP_TRY(hipEventRecord(g_ctx.fork_event, g_ctx.stream), PRAD_ERR_LAUNCH);
-    for (int i = 1; i < branches; ++i) {
-        HIP_TRY(hipStreamWaitEvent(g_ctx.branch[i].stream, g_ctx.fork_event, 0), PRAD_ERR_LAUNCH);
-        g_ctx.branch[i].open = true;
-    }
-    return PRAD_OK;
-}
-
-int32_t prad_branch(int32_t index) {
-    REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (index < 0 || index >= MAX_BRANCHES) return fail(PRAD_ERR_ARG, "branch %d out of range", index);
-    if (index > 0 && !g_ctx.branch[index].open) return fail(PRAD_ERR_ARG, "branch %d was not opened by prad_fork", index);
-    g_ctx.cur = index;
-    return PRAD_OK;
-}
-
-int32_t prad_join(void) {
-    REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    g_ctx.cur = 0;
-    for (int i = 1; i < MAX_BRANCHES; ++i) {
-        Branch& b = g_ctx.branch[i];
-        if (!b.open) continue;
-        b.open = false;
-        HIP_TRY(hipEventRecord(b.done, b.stream), PRAD_ERR_LAUNCH);
-        HIP_TRY(hipStreamWaitEvent(g_ctx.stream, b.done, 0), PRAD_ERR_LAUNCH);
-    }
+    (void)hipGraphExecDestroy(rg->exec);
+    (void)hipGraphDestroy(rg->graph);
+    rg->magic = 0;
+    delete rg;
+    if (g_ctx.live_graphs > 0 && --g_ctx.live_graphs == 0) free_retired_workspaces();
     return PRAD_OK;
 }
 
@@ -1389,9 +1476,9 @@ int32_t prad_softmax_cce(prad_buf_t x, prad_buf_t target, prad_buf_t p, prad_buf
     if (loss != nullptr && (loss->depth != 1 || loss->rows != 1 || loss->cols != 1)) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
     for (prad_buf_t o : {p, dp, dx})
         if (int32_t st = same_shape(x, o, "softmax + cross-entropy")) return st;
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
-    DISPATCH(x, launch_softmax_cce<double>(D(x), D(target), D(p), D(dp), D(dx), loss ? D(loss) : nullptr, cur_branch().counter, x->rows, x->cols, CUR_STREAM),
-             launch_softmax_cce<float>(F(x), F(target), F(p), F(dp), F(dx), loss ? F(loss) : nullptr, cur_branch().counter, x->rows, x->cols, CUR_STREAM));
+    ENQUEUE_LOCK();
+    DISPATCH(x, launch_softmax_cce<double>(D(x), D(target), D(p), D(dp), D(dx), loss ? D(loss) : nullptr, g_ctx.counter, x->rows, x->cols, CUR_STREAM),
+             launch_softmax_cce<float>(F(x), F(target), F(p), F(dp), F(dx), loss ? F(loss) : nullptr, g_ctx.counter, x->rows, x->cols, CUR_STREAM));
     return PRAD_OK;
 }
 
@@ -1406,7 +1493,7 @@ int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, doubl
     }
     std::vector<int64_t> sizes((size_t)n);
     for (int i = 0; i < n; ++i) sizes[i] = count(g[i]);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     if (int32_t st = ensure_workspace(clip_workspace_bytes(sizes.data(), n))) return st;
     if (g[0]->dtype == PRAD_F64) {
         std::vector<TensorDesc<double>> d((size_t)n);
@@ -1438,32 +1525,34 @@ static int32_t adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_b
     }
     std::vector<int64_t> sizes((size_t)n);
     for (int i = 0; i < n; ++i) sizes[i] = count(w[i]);
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     if (clip)
         if (int32_t st = ensure_workspace(clip_workspace_bytes(sizes.data(), n))) return st;
+    PendingAdam pending{w[0]->dtype, beta1, beta2, t};
+    const AdamLaunchObserver observer{note_adam_node, &pending};
+    const AdamLaunchObserver* obs = (g_ctx.recording && !reverse) ? &observer : nullptr;
     if (w[0]->dtype == PRAD_F64) {
-        // 1 / (1 - Math.Pow(beta, AdamIteration)), src/RMAD/AdamOptimizer.cs:204-207
-        const double c1 = 1 / (1 - std::pow(beta1, t)), c2 = 1 / (1 - std::pow(beta2, t));
+        double c1, c2;
+        bias_correction(beta1, beta2, t, &c1, &c2);
         std::vector<TensorDesc<double>> d((size_t)n);
         for (int i = 0; i < n; ++i) d[i] = TensorDesc<double>{D(g[i]), D(w[i]), D(m[i]), D(v[i]), sizes[i]};
         if (clip)
-            HIP_TRY(launch_clip_adam<double>(d.data(), n, CUR_WORKSPACE, clip_value, min_value, lr, beta1, beta2, eps, c1, c2, CUR_STREAM),
+            HIP_TRY(launch_clip_adam<double>(d.data(), n, CUR_WORKSPACE, clip_value, min_value, lr, beta1, beta2, eps, c1, c2, CUR_STREAM, obs),
                     PRAD_ERR_LAUNCH);
         else
-            HIP_TRY(launch_adam<double>(d.data(), n, lr, beta1, beta2, eps, c1, c2, reverse, CUR_STREAM), PRAD_ERR_LAUNCH);
+            HIP_TRY(launch_adam<double>(d.data(), n, lr, beta1, beta2, eps, c1, c2, reverse, CUR_STREAM, obs), PRAD_ERR_LAUNCH);
     } else {
-        // PRADLite: every parameter is a float and PradMath.Pow(float, float) is (float)Math.Pow.
-        const float b1 = (float)beta1, b2 = (float)beta2, tf = (float)t;
-        const float c1 = 1 / (1 - (float)std::pow((double)b1, (double)tf));
-        const float c2 = 1 / (1 - (float)std::pow((double)b2, (double)tf));
+        const float b1 = (float)beta1, b2 = (float)beta2;
+        float c1, c2;
+        bias_correction(b1, b2, (float)t, &c1, &c2);
         std::vector<TensorDesc<float>> d((size_t)n);
         for (int i = 0; i < n; ++i) d[i] = TensorDesc<float>{F(g[i]), F(w[i]), F(m[i]), F(v[i]), sizes[i]};
         if (clip)
             HIP_TRY(launch_clip_adam<float>(d.data(), n, CUR_WORKSPACE, (float)clip_value, (float)min_value, (float)lr, b1, b2,
-                                            (float)eps, c1, c2, CUR_STREAM),
+                                            (float)eps, c1, c2, CUR_STREAM, obs),
                     PRAD_ERR_LAUNCH);
         else
-            HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, reverse, CUR_STREAM), PRAD_ERR_LAUNCH);
+            HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, reverse, CUR_STREAM, obs), PRAD_ERR_LAUNCH);
     }
     return PRAD_OK;
 }
@@ -1504,7 +1593,7 @@ int32_t prad_event_destroy(void* ev) {
 }
 int32_t prad_event_record(void* ev) {
     REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    ENQUEUE_LOCK();
     HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(ev), g_ctx.stream), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }

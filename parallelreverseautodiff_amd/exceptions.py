@@ -32,6 +32,7 @@ _BY_CODE = {
     _lib.PRAD_ERR_ARG: ArgumentException,
     _lib.PRAD_ERR_NOT_RECTANGULAR: InvalidOperationException,
     _lib.PRAD_ERR_DTYPE: ArgumentException,
+    _lib.PRAD_ERR_RECORDING: InvalidOperationException,
 }
 
 

@@ -9,10 +9,8 @@ Per layer the product, the bias add and the activation are one launch (fused epi
 activation's Backward is the epilogue of the next layer's dA product.  A step of this size costs what
 its chain of dependent launches costs, so fused=True (the default) uses the entry points that cover
 several reference operations per launch (softmax + cross-entropy forward and backward; the bias gradient
-next to the weight gradient; clip + Adam);
-overlap=True puts gradients that do not depend on each other on separate branches, as the reference's
-visitor hands independent Backward calls to pool threads.  The arithmetic of every operation is the
-same in all variants and the results are bit for bit equal.
+next to the weight gradient; clip + Adam).  The arithmetic of every operation is the same in both variants
+and the results are bit for bit equal.
 """
 import ctypes
 
@@ -26,7 +24,7 @@ from .optim import NeuralNetworkParameters
 
 
 class FeedForwardNetwork:
-    def __init__(self, sizes=(784, 256, 128, 10), batch=64, dtype=np.float64, seed=seeded.DEFAULT_SEED, parameters=None, fused=True, overlap=False):
+    def __init__(self, sizes=(784, 256, 128, 10), batch=64, dtype=np.float64, seed=seeded.DEFAULT_SEED, parameters=None, fused=True):
         _ensure_initialized()
         self.lib = _lib.load()
         self.dtype = np.dtype(dtype)
@@ -56,7 +54,6 @@ class FeedForwardNetwork:
         self.dZ = [alloc(batch, sizes[l + 1]) for l in range(L)]
         self.dX = alloc(batch, sizes[0])
         self.iteration = 0
-        self.overlap = overlap
         self.fused = fused
         self._graph = None
         self._weights = self.W + self.b
@@ -81,8 +78,6 @@ class FeedForwardNetwork:
             a = out
 
     def _enqueue_forward_backward(self):
-        if self.overlap:
-            return self._enqueue_forward_backward_overlapped()
         lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
         self._enqueue_forward()
         if self.fused:
@@ -109,33 +104,6 @@ class FeedForwardNetwork:
                 check(lib.prad_matmul_bwd_fused(self.dZ[l].handle, inp.handle, self.W[l].handle, dA.handle,
                                                 self.dW[l].handle, 0, act, src, alpha))
 
-    def _enqueue_forward_backward_overlapped(self):
-        """Branch 0 carries the chain forward -> loss gradient -> dA of every layer; branch 1 the weight
-        gradients, branch 2 the bias gradients and the loss value, branch 3 the input gradient."""
-        lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
-        self._enqueue_forward()
-        check(lib.prad_softmax_cce(self.Z[-1].handle, self.T.handle, self.P.handle, None, self.dP.handle, self.dZ[-1].handle))
-        try:
-            for l in range(L - 1, -1, -1):
-                inp = self.X if l == 0 else self.H[l - 1]
-                check(lib.prad_fork(4))                      # dZ[l] (and P) are ready for the side branches
-                check(lib.prad_branch(2))
-                if l == L - 1:
-                    check(lib.prad_cce_fwd(self.P.handle, self.T.handle, self.loss.handle))
-                check(lib.prad_add_broadcast_bwd_bias(self.dZ[l].handle, self.db[l].handle))
-                check(lib.prad_branch(1))
-                check(lib.prad_matmul_bwd(self.dZ[l].handle, inp.handle, self.W[l].handle, None, self.dW[l].handle, 0, 0))
-                if l == 0:
-                    check(lib.prad_branch(3))
-                    check(lib.prad_matmul_bwd(self.dZ[0].handle, inp.handle, self.W[0].handle, self.dX.handle, None, 0, 0))
-                    check(lib.prad_branch(0))
-                else:
-                    check(lib.prad_branch(0))
-                    check(lib.prad_matmul_bwd_fused(self.dZ[l].handle, inp.handle, self.W[l].handle, self.dZ[l - 1].handle,
-                                                    None, 0, _lib.ACT_LEAKYRELU, self.Z[l - 1].handle, alpha))
-        finally:
-            check(lib.prad_join())
-
     def _enqueue_update(self, t):
         p = self.params
         n = len(self._grads)
@@ -157,14 +125,17 @@ class FeedForwardNetwork:
         self._enqueue_update(self.iteration)
 
     # ---- one step as a recorded launch sequence ------------------------------------------------
-    def record(self, adam_iteration=1.0):
-        """Records one step with a fixed AdamIteration (the bias-correction factors are launch arguments);
-        one eager step must have run before so that shared workspace is already sized."""
+    def record(self, adam_iteration=None):
+        """Records one step; one eager step must have run before so that the shared workspace is already sized.
+        The recording stands for the step after the last one taken (AdamIteration = iteration + 1) unless
+        `adam_iteration` says otherwise; every replay advances AdamIteration by one, as step() does."""
         lib = self.lib
+        self._recorded_from = float(self.iteration + 1 if adam_iteration is None else adam_iteration)
+        self.iteration = int(self._recorded_from) - 1
         check(lib.prad_graph_begin())
         try:
             self._enqueue_forward_backward()
-            self._enqueue_update(adam_iteration)
+            self._enqueue_update(self._recorded_from)
         finally:
             g = ctypes.c_void_p()
             check(lib.prad_graph_end(ctypes.byref(g)))
@@ -172,7 +143,9 @@ class FeedForwardNetwork:
         return g
 
     def replay(self):
+        """One recorded step; AdamIteration advances by one per replay."""
         check(self.lib.prad_graph_launch(self._graph))
+        self.iteration += 1
 
     def release(self):
         if self._graph is not None:

@@ -116,18 +116,22 @@ class LSTMLayer:
         if update:
             self._enqueue_update(self.iteration)
 
-    def record(self, adam_iteration=1.0):
+    def record(self, adam_iteration=None):
+        self._recorded_from = float(self.iteration + 1 if adam_iteration is None else adam_iteration)
+        self.iteration = int(self._recorded_from) - 1
         check(self.lib.prad_graph_begin())
         try:
             self._enqueue_forward_backward()
-            self._enqueue_update(adam_iteration)
+            self._enqueue_update(self._recorded_from)
         finally:
             g = ctypes.c_void_p()
             check(self.lib.prad_graph_end(ctypes.byref(g)))
         self._graph = g
 
     def replay(self):
+        """One recorded step; AdamIteration advances by one per replay."""
         check(self.lib.prad_graph_launch(self._graph))
+        self.iteration += 1
 
     def release(self):
         if self._graph is not None:

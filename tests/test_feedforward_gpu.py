@@ -78,12 +78,11 @@ def test_recorded_step_equals_eager_step(gpu):
     eager, rec = FeedForwardNetwork(), FeedForwardNetwork()
     for net in (eager, rec):
         net.set_batch(X, T)
-    # warm-up step on both (sizes shared workspace), then record with the iteration the replays will use
+    # warm-up step on both (sizes shared workspace), then record the next step; AdamIteration advances on both sides
     eager.step(); rec.step()
-    rec.record(adam_iteration=2.0)
+    rec.record()
     for replay in range(4):
-        eager.iteration = 1
-        eager.step()  # t = 2 again on the eager side
+        eager.step()
         rec.replay()
         gpu.Synchronize()
         junk = FeedForwardNetwork(sizes=(32, 16, 4), batch=8)  # unrelated eager work between replays
@@ -114,55 +113,138 @@ def test_softmax_and_cross_entropy_operations(gpu, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_overlapped_step_equals_sequential_step(gpu, dtype):
-    """Independent gradients on separate branches (and the fused softmax + cross-entropy launch) must give
-    bit for bit what the one-branch, operation-by-operation step gives; also when recorded and replayed."""
+def test_recorded_steps_equal_eager_steps_with_advancing_adam_iteration(gpu, dtype):
+    """N replays of a recorded step give, bit for bit, what N eager steps with AdamIteration 2, 3, ... give (the
+    reference's caller advances AdamIteration every step, src/RMAD/AdamOptimizer.cs:204-207); the fused launches give
+    the bits of the operation-by-operation step throughout.  Eager work runs between the replays."""
     X = seeded.uniform(7, 1, (64, 784), 0.0, 1.0, dtype)
     T = seeded.one_hot_labels(7, 2, 64, 10, dtype)
-    seq = FeedForwardNetwork(dtype=dtype, fused=False, overlap=False)   # one reference operation per launch
-    fus = FeedForwardNetwork(dtype=dtype, fused=True, overlap=False)
-    par, rec = (FeedForwardNetwork(dtype=dtype, overlap=True) for _ in range(2))
-    for net in (seq, fus, par, rec):
+    seq = FeedForwardNetwork(dtype=dtype, fused=False)   # one reference operation per launch
+    fus = FeedForwardNetwork(dtype=dtype, fused=True)
+    rec = FeedForwardNetwork(dtype=dtype, fused=True)
+    for net in (seq, fus, rec):
         net.set_batch(X, T)
         net.step()
-    rec.record(adam_iteration=2.0)
-    for replay in range(3):
-        for net in (seq, fus, par):
-            net.iteration = 1
+    rec.record()
+    assert rec.iteration == 1
+    for replay in range(4):
+        for net in (seq, fus):
             net.step()
         rec.replay()
         gpu.Synchronize()
+        assert seq.iteration == fus.iteration == rec.iteration == replay + 2
         for name in ("_weights", "_grads", "_m", "_v"):
-            for a, f, b2, c in zip(getattr(seq, name), getattr(fus, name), getattr(par, name), getattr(rec, name)):
+            for a, f, c in zip(getattr(seq, name), getattr(fus, name), getattr(rec, name)):
                 ref = a.download()
                 assert np.array_equal(ref, f.download()), "%s differs (fused launches, pass %d)" % (name, replay)
-                assert np.array_equal(ref, b2.download()), "%s differs (eager branches, pass %d)" % (name, replay)
-                assert np.array_equal(ref, c.download()), "%s differs (recorded branches, pass %d)" % (name, replay)
-        for other in (fus, par, rec):
+                assert np.array_equal(ref, c.download()), "%s differs (recorded step, pass %d)" % (name, replay)
+        for other in (fus, rec):
             assert np.array_equal(seq.loss.download(), other.loss.download())
-        assert np.array_equal(seq.dX.download(), par.dX.download())
+    # a replay can be told which AdamIteration it stands for
+    from parallelreverseautodiff_amd.exceptions import check
+    check(rec.lib.prad_graph_set_adam_iteration(rec._graph, 9.0))
+    rec.iteration = 8
+    fus.iteration = 8
+    fus.step(); rec.replay()
+    gpu.Synchronize()
+    for a, c in zip(fus._weights, rec._weights):
+        assert np.array_equal(a.download(), c.download())
     rec.release()
 
 
-def test_branch_protocol_errors(gpu):
+def test_recording_refuses_other_threads_and_host_traffic(gpu):
+    """While one thread records, an enqueueing call from another thread is refused instead of being recorded
+    (the reference calls Backward from pool threads, src/RMAD/OperationNeuralNetworkVisitor.cs:303-306), and the
+    recording thread itself cannot allocate, free, copy to or from the host or wait for the device."""
+    import ctypes
+    import threading
     from parallelreverseautodiff_amd import _lib
-    from parallelreverseautodiff_amd.exceptions import ArgumentException, check
+    from parallelreverseautodiff_amd.exceptions import InvalidOperationException, check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
     lib = _lib.load()
-    with pytest.raises(ArgumentException):
-        check(lib.prad_fork(1))
-    with pytest.raises(ArgumentException):
-        check(lib.prad_fork(5))
-    with pytest.raises(ArgumentException):
-        check(lib.prad_branch(2))          # not opened
-    check(lib.prad_fork(2))
-    check(lib.prad_branch(1))
-    with pytest.raises(ArgumentException):
-        check(lib.prad_branch(2))          # only branch 1 is open
-    check(lib.prad_join())
-    with pytest.raises(ArgumentException):
-        check(lib.prad_branch(1))          # closed again
-    check(lib.prad_join())                 # joining with nothing open is a no-op
-    check(lib.prad_branch(0))
+    a, b, c = (DeviceBuffer.alloc(np.float64, 32, 32) for _ in range(3))
+    a.upload(np.ones((32, 32))); b.upload(np.full((32, 32), 2.0))
+    check(lib.prad_matmul_fwd(a.handle, b.handle, c.handle))          # eager once
+    check(lib.prad_graph_begin())
+    status = {}
+    try:
+        def other():
+            status["matmul"] = lib.prad_matmul_fwd(a.handle, b.handle, c.handle)
+            status["message"] = lib.prad_last_error().decode()
+            status["end"] = lib.prad_graph_end(ctypes.byref(ctypes.c_void_p()))
+        th = threading.Thread(target=other)
+        th.start(); th.join()
+        assert status["matmul"] == _lib.PRAD_ERR_RECORDING and "another thread" in status["message"]
+        assert status["end"] == _lib.PRAD_ERR_RECORDING
+        extra = ctypes.c_void_p()
+        assert lib.prad_buf_alloc(_lib.PRAD_F64, 4, 4, ctypes.byref(extra)) == _lib.PRAD_ERR_RECORDING
+        host = np.zeros((32, 32))
+        assert lib.prad_buf_download(c.handle, host.ctypes.data_as(ctypes.c_void_p), 32) == _lib.PRAD_ERR_RECORDING
+        assert lib.prad_stream_sync() == _lib.PRAD_ERR_RECORDING
+        assert lib.prad_graph_begin() == _lib.PRAD_ERR_RECORDING
+        with pytest.raises(InvalidOperationException):
+            check(lib.prad_buf_upload(c.handle, host.ctypes.data_as(ctypes.c_void_p), 32))
+        check(lib.prad_matmul_fwd(a.handle, b.handle, c.handle))      # the recording thread records
+    finally:
+        g = ctypes.c_void_p()
+        check(lib.prad_graph_end(ctypes.byref(g)))
+    check(lib.prad_buf_zero(c.handle))
+    check(lib.prad_graph_launch(g))
+    assert np.array_equal(c.download(), np.full((32, 32), 64.0))      # exactly one product was recorded
+    assert lib.prad_graph_launch(ctypes.c_void_p(a.handle.value)) == _lib.PRAD_ERR_BAD_HANDLE
+    check(lib.prad_graph_destroy(g))
+
+
+def test_workspace_growth_while_a_recorded_sequence_is_alive(gpu, oracle):
+    """A recorded split product keeps the workspace address it was recorded with.  An eager call that needs a larger
+    workspace afterwards must not free that block under it: the replay still gives the recorded product's bits, and
+    growing the workspace during a recording is refused."""
+    import ctypes
+    from parallelreverseautodiff_amd import _lib
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    dtype = np.float64
+    M, K, N = 64, 4096, 64                      # few tiles, long K: runs split along K through the workspace
+    A = seeded.uniform(3, 1, (M, K), -1, 1, dtype)
+    B = seeded.uniform(3, 2, (K, N), -1, 1, dtype)
+    a, b, c = DeviceBuffer.alloc(dtype, M, K), DeviceBuffer.alloc(dtype, K, N), DeviceBuffer.alloc(dtype, M, N)
+    a.upload(A); b.upload(B)
+    check(lib.prad_matmul_fwd(a.handle, b.handle, c.handle))
+    eager = c.download()
+    check(lib.prad_graph_begin())
+    try:
+        check(lib.prad_matmul_fwd(a.handle, b.handle, c.handle))
+    finally:
+        g = ctypes.c_void_p()
+        check(lib.prad_graph_end(ctypes.byref(g)))
+    # eager work that outgrows the workspace: a taller split product (same kernels, 16x the partial tiles)
+    M2 = 1024
+    a2, c2 = DeviceBuffer.alloc(dtype, M2, K), DeviceBuffer.alloc(dtype, M2, N)
+    a2.upload(seeded.uniform(3, 4, (M2, K), -1, 1, dtype))
+    check(lib.prad_matmul_fwd(a2.handle, b.handle, c2.handle))
+    check(lib.prad_buf_zero(c.handle))
+    for _ in range(3):
+        check(lib.prad_graph_launch(g))
+        check(lib.prad_matmul_fwd(a2.handle, b.handle, c2.handle))   # eager work in between, on the new workspace
+        gpu.Synchronize()
+        assert np.array_equal(c.download(), eager)
+    check(lib.prad_graph_destroy(g))
+    # growth during a recording is refused with a message that says what to do: a sum of 16 products whose partial
+    # results (16 x 512 x 512 doubles = 32 MiB) outgrow everything above
+    P, m, k, n = 16, 512, 64, 512
+    da, db, dc = DeviceBuffer.alloc(dtype, m, k, depth=P), DeviceBuffer.alloc(dtype, k, n, depth=P), DeviceBuffer.alloc(dtype, m, n)
+    check(lib.prad_graph_begin())
+    try:
+        st = lib.prad_matmul_batch_sum_fwd(da.handle, db.handle, None, dc.handle)
+        msg = lib.prad_last_error().decode()
+    finally:
+        g = ctypes.c_void_p()
+        check(lib.prad_graph_end(ctypes.byref(g)))
+    assert st == _lib.PRAD_ERR_RECORDING and "once before recording" in msg
+    check(lib.prad_graph_destroy(g))
+    check(lib.prad_matmul_batch_sum_fwd(da.handle, db.handle, None, dc.handle))   # eagerly it grows and runs
+    gpu.Synchronize()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -4,7 +4,7 @@ HadamardProduct, MatrixAdd, MeanSquaredError, and their Backward methods in reve
 import numpy as np
 import pytest
 
-from conftest import assert_parity
+from conftest import assert_long_sum_parity, assert_parity, norm_err, strict_err
 from oracle import compose
 from parallelreverseautodiff_amd.lstm import LSTMLayer
 
@@ -26,12 +26,32 @@ def test_lstm_step_matches_node_by_node_oracle(gpu, oracle, dtype, cfg):
     assert_parity(layer.dX.download(), dX, dtype, "dX")
 
 
+def test_lstm_benchmark_configuration_full_size(gpu, oracle):
+    """The configuration the benchmark times, at its full size: input 256, hidden 512, batch 128, 64 time steps,
+    float.  The node-by-node composition takes some seconds on the host cores.  The weight gradient is a sum over
+    64 x 128 = 8192 rows (the reference adds 64 per-step products, the device runs one product): see
+    assert_long_sum_parity."""
+    I, H, B, T = 256, 512, 128, 64
+    layer = LSTMLayer(I, H, B, T, dtype=np.float32)
+    layer.step(update=False)
+    zero_b = np.zeros((1, 4 * H), np.float32)
+    loss, Hout, dW, db, dX = compose.lstm_forward_backward(layer.host_W, zero_b, layer.host_X, layer.host_Y, I, H, B, T, threads=16)
+    assert abs(float(layer.loss.download()[0, 0]) - loss) <= 1e-5 * abs(loss)
+    for what, got, ref in (("hidden states", layer.H_out, Hout), ("db", layer.db, db), ("dX", layer.dX, dX)):
+        g = got.download()
+        err = assert_parity(g, ref, np.float32, what)
+        print("LSTM 256/512/128/64 float %s: relative %.2e, normwise %.2e, floor 1e-3 rms %.2e" % (what, err, norm_err(g, ref), strict_err(g, ref)))
+    XH = np.concatenate([layer.host_X, layer.Hs.download()[:T * B]], axis=1)      # [X | H_prev] over all time steps
+    errs = assert_long_sum_parity(layer.dW.download(), dW, XH, layer.dG.download(), np.float32, "dW")
+    print("LSTM 256/512/128/64 float dW (K = 8192): against the reference %.2e; against the double product: device %.2e, "
+          "reference arithmetic %.2e" % errs)
+
+
 def test_lstm_recorded_step_equals_eager(gpu):
     a, b = LSTMLayer(16, 32, 8, 6, dtype=np.float64), LSTMLayer(16, 32, 8, 6, dtype=np.float64)
     a.step(); b.step()
-    b.record(adam_iteration=2.0)
+    b.record()                       # stands for step 2; every replay advances AdamIteration like step() does
     for _ in range(3):
-        a.iteration = 1
         a.step()
         b.replay()
         gpu.Synchronize()

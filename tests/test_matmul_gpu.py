@@ -149,8 +149,8 @@ def test_full_size_properties_fp64(gpu, n):
     assert abs(float(np.sum(dB * B)) - lhs) <= 1e-11 * abs(lhs)
 
 
-def test_full_size_properties_fp32(gpu):
-    n = 2048
+@pytest.mark.parametrize("n", [2048, 4096])
+def test_full_size_properties_fp32(gpu, n):
     A, B, dC = inputs(np.float32, n, n, n)
     C, dA, dB = run_op(GpuMatrixMultiplyOperation, A, B, dC)
     rng = np.random.default_rng(5)
@@ -160,6 +160,40 @@ def test_full_size_properties_fp32(gpu):
         assert abs(C[i, j] - math.fsum(A64[i, :] * B64[:, j])) <= 1e-5 * math.sqrt(n / 3.0)
         assert abs(dA[i, j] - math.fsum(G64[i, :] * B64[j, :])) <= 1e-5 * math.sqrt(n)
         assert abs(dB[i, j] - math.fsum(A64[:, i] * G64[:, j])) <= 1e-5 * math.sqrt(n)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [2048, 4096])
+def test_full_size_whole_matrix_identities(gpu, dtype, n):
+    """Every tile of every output is touched for O(N^2) host work: a product applied to the all-ones vector
+    equals the chain of matrix-vector products, C.1 = A.(B.1) and 1^T.C = (1^T.A).B, and likewise for
+    dA = dC.B^T and dB = A^T.dC.  The right-hand sides are evaluated in double.  The worst-case rounding bound of
+    the sums an entry stands for is 8 sqrt(K) eps (|X|.|Y|.1)_i; rounding errors of different entries cancel, and the
+    sums measured on the device stay below 1e-4 of it, so the bar is 1e-3 of that bound: one wrong entry of typical
+    magnitude in a row (let alone a misplaced, dropped or doubled tile) exceeds it."""
+    A, B, dC = inputs(dtype, n, n, n)
+    C, dA, dB = run_op(GpuMatrixMultiplyOperation, A, B, dC)
+    f = lambda x: x.astype(np.float64)
+    A64, B64, G64 = f(A), f(B), f(dC)
+    one = np.ones(n)
+    eps = float(np.finfo(dtype).eps)
+    factor = 8.0 * math.sqrt(n) * eps
+    worst = 0.0
+
+    def check_pair(out, X, Y, what):
+        # out = X . Y (already oriented): rows against X.(Y.1), columns against (1^T.X).Y
+        nonlocal worst
+        out64 = f(out)
+        for got, ref, bound in ((out64 @ one, X @ (Y @ one), np.abs(X) @ (np.abs(Y) @ one)),
+                                (one @ out64, (one @ X) @ Y, (one @ np.abs(X)) @ np.abs(Y))):
+            excess = np.abs(got - ref) / (factor * bound)
+            worst = max(worst, float(excess.max()))
+            assert excess.max() <= 1e-3, "%s: a row or column sum is off by %.2e x its rounding bound" % (what, excess.max())
+
+    check_pair(C, A64, B64, "C")
+    check_pair(dA, G64, B64.T, "dA")
+    check_pair(dB, A64.T, G64, "dB")
+    print("whole-matrix identities %s n=%d: worst sum at %.2e of its bound" % (np.dtype(dtype).name, n, worst))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from conftest import assert_parity
+from conftest import assert_long_sum_parity, assert_parity, norm_err, strict_err
 from oracle import compose
 from parallelreverseautodiff_amd import _lib, seeded
 from parallelreverseautodiff_amd.matrix import DeviceBuffer
@@ -27,6 +27,27 @@ def test_swin_block_matches_node_by_node_oracle(gpu, oracle, dtype, cfg):
     for k in blk.names:
         assert_parity(blk.g[k].download(), g[k], dtype, "gradient of " + k)
     assert_parity(blk.dX.download(), dX, dtype, "dX")
+
+
+def test_swin_benchmark_configuration_full_size(gpu, oracle):
+    """The configuration the benchmark times, at its full size: 16 images of 56 x 56 tokens in 7 x 7 windows, embed 96,
+    3 heads, float (50 176 token rows, 1024 windows).  The four weight gradients are sums over all 50 176 rows: see
+    assert_long_sum_parity (the reference's k-ascending float loop is the less accurate side there)."""
+    blk = SwinBlock(images=16, side=56, embed=96, heads=3, dtype=np.float32)
+    assert blk.nw == 1024 and blk.wt == 49
+    blk.step(update=False)
+    params = {k: blk.host[k] for k in blk.names}
+    loss, Y2, g, dX = compose.swin_block_forward_backward(params, blk.host["X"], blk.host["T"], blk.nw, blk.wt, 3, threads=16)
+    assert abs(float(blk.loss.download()[0, 0]) - loss) <= 1e-5 * abs(loss)
+    for what, got, ref in [("block output", blk.Y2, Y2), ("dX", blk.dX, dX)] + [("gradient of " + k, blk.g[k], g[k]) for k in blk.names if k.startswith("b")]:
+        x = got.download()
+        err = assert_parity(x, ref, np.float32, what)
+        print("Swin 16/56/96/3 float %s: relative %.2e, normwise %.2e, floor 1e-3 rms %.2e" % (what, err, norm_err(x, ref), strict_err(x, ref)))
+    operands = {"W2": (blk.H1, blk.dY2), "W1": (blk.Y1, blk.dZ1), "Wo": (blk.O, blk.dY1), "Wqkv": (blk.X, blk.dQKV)}
+    for k, (lhs, rhs) in operands.items():
+        errs = assert_long_sum_parity(blk.g[k].download(), g[k], lhs.download(), rhs.download(), np.float32, "gradient of " + k)
+        print("Swin 16/56/96/3 float gradient of %s (K = 50176): against the reference %.2e; against the double product: device %.2e, "
+              "reference arithmetic %.2e" % ((k,) + errs))
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
