@@ -316,6 +316,18 @@ int32_t prad_clip_adam_multi(const prad_buf_t* w, const prad_buf_t* m, const pra
                              double clip_value, double min_value, double lr, double beta1, double beta2, double eps,
                              double t);
 
+/* ---- allocation-free form of prad_clip_adam_multi.  No counterpart in the reference: it is for callers that cannot
+ *      allocate at the point of the call (a launch sequence being captured, a tight serving or training loop, a
+ *      harness that forbids hipMalloc).  Same arguments, same results (clamped g, w, m, v) bit for bit.  It never calls
+ *      hipMalloc / hipFree and uses no host heap: the clip statistics go to a static device array of 1 MiB inside the
+ *      library (one per GPU, held until the process ends) instead of the growable workspace.  Limits: at most 64
+ *      tensors per call and at most about 43 000 chunks of 4096 elements in all (roughly 1.7e8 elements); beyond them
+ *      it returns PRAD_ERR_ARG and enqueues nothing.  Every call on a GPU shares that array: calls that overlapped on
+ *      one GPU would race, which the single library stream rules out for calls made through this library. */
+int32_t prad_clip_adam_multi_noalloc(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
+                                     double clip_value, double min_value, double lr, double beta1, double beta2, double eps,
+                                     double t);
+
 /* ---- timing helpers for harnesses: events recorded on the library stream ------------------ */
 int32_t prad_event_create(void** ev);
 int32_t prad_event_destroy(void* ev);

@@ -114,6 +114,7 @@ SIGNATURES = {
     "prad_adam_multi": (_i32, [_vpp, _vpp, _vpp, _vpp, _i32, _f64, _f64, _f64, _f64, _f64]),
     "prad_adam_revert_multi": (_i32, [_vpp, _vpp, _vpp, _vpp, _i32, _f64, _f64, _f64, _f64, _f64]),
     "prad_clip_adam_multi": (_i32, [_vpp, _vpp, _vpp, _vpp, _i32, _f64, _f64, _f64, _f64, _f64, _f64, _f64]),
+    "prad_clip_adam_multi_noalloc": (_i32, [_vpp, _vpp, _vpp, _vpp, _i32, _f64, _f64, _f64, _f64, _f64, _f64, _f64]),
     "prad_event_create": (_i32, [_vpp]),
     "prad_event_destroy": (_i32, [_vp]),
     "prad_event_record": (_i32, [_vp]),

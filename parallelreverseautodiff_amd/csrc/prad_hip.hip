@@ -29,6 +29,13 @@ struct prad_buf {
     bool owned;
 };
 
+// Scratch of the allocation-free entry point (prad_clip_adam_multi_noalloc): device memory that exists from the
+// moment the code object is loaded, one copy per GPU, held until the process ends.  In host code the name is only
+// a stand-in for the symbol: its device address is asked for once per device (init_static_scratch) and every
+// kernel argument uses that address.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)1 << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
 namespace {
 
 constexpr uint32_t BUF_MAGIC = 0x50524144u;  // "PRAD"
@@ -148,6 +155,20 @@ int32_t ensure_workspace(size_t bytes) {
     }
     g_ctx.workspace = fresh;
     g_ctx.workspace_bytes = bytes;
+    return PRAD_OK;
+}
+
+// ---- the static scratch of the allocation-free entry point ----------------------------------------------
+constexpr int MAX_DEVICES = 64;
+void* g_scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each GPU this process has initialised
+// Lock held, `device` current.
+int32_t init_static_scratch(int device) {
+    if (device < 0 || device >= MAX_DEVICES) return fail(PRAD_ERR_ARG, "device %d beyond the %d this library keeps scratch for", device, MAX_DEVICES);
+    if (g_scratch_ptr[device] != nullptr) return PRAD_OK;
+    void* ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), PRAD_ERR_NOT_INITIALIZED);
+    if (ptr == nullptr) return fail(PRAD_ERR_NOT_INITIALIZED, "hipGetSymbolAddress returned no address for the static scratch");
+    g_scratch_ptr[device] = ptr;
     return PRAD_OK;
 }
 
@@ -431,6 +452,7 @@ int32_t prad_init(int32_t device_id) {
     HIP_TRY(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking), PRAD_ERR_NOT_INITIALIZED);
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.counter), COUNTER_BYTES), PRAD_ERR_ALLOC);
     HIP_TRY(hipMemset(g_ctx.counter, 0, COUNTER_BYTES), PRAD_ERR_ALLOC);
+    if (int32_t st = init_static_scratch(device_id)) return st;
     g_ctx.recording = false;
     g_ctx.live_graphs = 0;
     g_ctx.device = device_id;
@@ -1553,6 +1575,56 @@ static int32_t adam_multi(const prad_buf_t* w, const prad_buf_t* m, const prad_b
                     PRAD_ERR_LAUNCH);
         else
             HIP_TRY(launch_adam<float>(d.data(), n, (float)lr, b1, b2, (float)eps, c1, c2, reverse, CUR_STREAM, obs), PRAD_ERR_LAUNCH);
+    }
+    return PRAD_OK;
+}
+
+// The allocation-free form of prad_clip_adam_multi: no hipMalloc, no hipFree, no host heap.  The chunk moments of the
+// clip statistics go to the static device array `scratch` (through the address looked up at prad_init) instead of the
+// growable workspace.  Every call on a device shares that array, so calls must not overlap on a device: here they
+// cannot, because every call is enqueued on the one library stream.  Nothing in it needs to start at zero (the statistics
+// pass writes every slot that the later passes read), so a call after a larger one is not disturbed by what that left.
+int32_t prad_clip_adam_multi_noalloc(const prad_buf_t* w, const prad_buf_t* m, const prad_buf_t* v, const prad_buf_t* g, int32_t n,
+                                     double clip_value, double min_value, double lr, double beta1, double beta2, double eps,
+                                     double t) {
+    REQUIRE_INIT();
+    constexpr int MAX_TENSORS = 64;
+    if (n < 0 || (n > 0 && (w == nullptr || m == nullptr || v == nullptr || g == nullptr))) return fail(PRAD_ERR_ARG, "bad tensor list");
+    if (n == 0) return PRAD_OK;
+    if (n > MAX_TENSORS) return fail(PRAD_ERR_ARG, "the allocation-free form takes at most %d tensors per call (got %d)", MAX_TENSORS, n);
+    int64_t sizes[MAX_TENSORS];
+    for (int i = 0; i < n; ++i) {
+        REQUIRE_BUF(w[i]); REQUIRE_BUF(m[i]); REQUIRE_BUF(v[i]); REQUIRE_BUF(g[i]);
+        for (prad_buf_t o : {w[i], m[i], v[i], g[i]})
+            if (o->dtype != w[0]->dtype) return fail(PRAD_ERR_DTYPE, "buffers of different element types in one call");
+        for (prad_buf_t o : {m[i], v[i], g[i]})
+            if (int32_t st = same_shape(w[i], o, "Adam")) return st;
+        sizes[i] = count(w[i]);
+    }
+    const size_t need = clip_workspace_bytes(sizes, n);
+    if (need > STATIC_SCRATCH_BYTES)
+        return fail(PRAD_ERR_ARG, "the tensors need %zu bytes of clip statistics, the static scratch holds %zu (about %lld elements in all); "
+                    "use prad_clip_adam_multi", need, STATIC_SCRATCH_BYTES, (long long)(STATIC_SCRATCH_BYTES / 24 * 4096));
+    ENQUEUE_LOCK();
+    void* const ptr = g_scratch_ptr[g_ctx.device];
+    if (ptr == nullptr) return fail(PRAD_ERR_NOT_INITIALIZED, "the static scratch has no address on device %d", g_ctx.device);
+    PendingAdam pending{w[0]->dtype, beta1, beta2, t};
+    const AdamLaunchObserver observer{note_adam_node, &pending};
+    const AdamLaunchObserver* obs = g_ctx.recording ? &observer : nullptr;
+    if (w[0]->dtype == PRAD_F64) {
+        double c1, c2;
+        bias_correction(beta1, beta2, t, &c1, &c2);
+        TensorDesc<double> d[MAX_TENSORS];
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<double>{D(g[i]), D(w[i]), D(m[i]), D(v[i]), sizes[i]};
+        HIP_TRY(launch_clip_adam<double>(d, n, ptr, clip_value, min_value, lr, beta1, beta2, eps, c1, c2, CUR_STREAM, obs), PRAD_ERR_LAUNCH);
+    } else {
+        const float b1 = (float)beta1, b2 = (float)beta2;
+        float c1, c2;
+        bias_correction(b1, b2, (float)t, &c1, &c2);
+        TensorDesc<float> d[MAX_TENSORS];
+        for (int i = 0; i < n; ++i) d[i] = TensorDesc<float>{F(g[i]), F(w[i]), F(m[i]), F(v[i]), sizes[i]};
+        HIP_TRY(launch_clip_adam<float>(d, n, ptr, (float)clip_value, (float)min_value, (float)lr, b1, b2, (float)eps, c1, c2,
+                                        CUR_STREAM, obs), PRAD_ERR_LAUNCH);
     }
     return PRAD_OK;
 }
