@@ -78,6 +78,7 @@ void* prad_stream(void);           /* getter: the library's hipStream_t, for cal
 int32_t prad_buf_alloc(int32_t dtype, int64_t rows, int64_t cols, prad_buf_t* out); /* zero-filled, like new Matrix(rows, cols) */
 int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out); /* DeepMatrix: depth contiguous slices; src/RMAD/DeepMatrix.cs:22 */
 int32_t prad_buf_wrap(int32_t dtype, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out); /* borrow caller-owned device memory */
+int32_t prad_buf_wrap_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out); /* the same for depth contiguous slices (a tensor of more than two dimensions: Tensor.Shape, src/PRAD/Tensor.cs) */
 int32_t prad_buf_free(prad_buf_t b);
 int32_t prad_buf_shape(prad_buf_t b, int64_t* depth, int64_t* rows, int64_t* cols, int32_t* dtype);
 void* prad_buf_device_ptr(prad_buf_t b); /* getter: NULL for a bad handle */
@@ -176,11 +177,14 @@ int32_t prad_tensor_matmul_reverse_host(int32_t dtype, const void* dc, const voi
                                         int64_t m, int64_t k, int64_t n);
 
 /* ---- MatrixMultiplyAndSumOperation / GpuMatrixMultiplyAndSumOperation,
- *      src/RMAD/MatrixMultiplyAndSumOperation.cs:50-89, GpuMatrixMultiplyAndSumOperation.cs:114-154 */
-/* out[0][q] = sum_ij (A . B[q])_ij ; A is M x K, B is deep (P, K, N), out is 1 x P. */
+ *      src/RMAD/MatrixMultiplyAndSumOperation.cs:50-89, GpuMatrixMultiplyAndSumOperation.cs:114-154, and their per-sample
+ *      wrappers BatchMatrixMultiplyAndSumOperation / BatchGpuMatrixMultiplyAndSumOperation
+ *      (src/RMAD/BatchGpuMatrixMultiplyAndSumOperation.cs:51-74): A of depth S holds one M x K matrix per sample, the P
+ *      slices of B (K x N) are shared by all samples; S = 1 is the single operation. */
+/* out[i][0][q] = sum over all entries of A[i] . B[q]; out is deep (S, 1, P).  One launch over all S * P products. */
 int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out);
-/* As written in the reference: dB[q] = A^T * dOut[0][q] (deep (P, K, M)); dA = sum_q B[q]^T * dOut[0][q]
- * (needs N == M). */
+/* As written in the reference, per sample i: dB[i * P + q] = A[i]^T * dOut[i][0][q] (dB deep (S * P, K, M));
+ * dA[i] = sum_q B[q]^T * dOut[i][0][q] (dA deep (S, M, K); needs N == M).  dA or dB may be NULL.  One launch. */
 int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_buf_t dA, prad_buf_t dB);
 /* Independent products summed into one output plus a broadcast bias: C = sum_q A[q].B[q] + bias, A deep
  * (P, M, K), B deep (P, K, N), bias 1 x N or NULL, C M x N.  The reference has no single operation of this

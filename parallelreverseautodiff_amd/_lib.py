@@ -45,6 +45,7 @@ SIGNATURES = {
     "prad_buf_alloc": (_i32, [_i32, _i64, _i64, _vpp]),
     "prad_buf_alloc_deep": (_i32, [_i32, _i64, _i64, _i64, _vpp]),
     "prad_buf_wrap": (_i32, [_i32, _i64, _i64, _vp, _vpp]),
+    "prad_buf_wrap_deep": (_i32, [_i32, _i64, _i64, _i64, _vp, _vpp]),
     "prad_buf_free": (_i32, [_vp]),
     "prad_buf_shape": (_i32, [_vp, _i64p, _i64p, _i64p, _i32p]),
     "prad_buf_device_ptr": (_vp, [_vp]),

@@ -304,9 +304,10 @@ template <typename T> hipError_t launch_lstm_cell_bwd(const T* gates, const T* c
                                                       const T* dc_in, T* dG, T* dc_prev, int64_t rows, int64_t hidden, hipStream_t s);
 
 // MatrixMultiplyAndSum
+// S = samples of a batch (each with its own A, out, dOut, dA and P slices of dB; the P slices of B are shared).
 template <typename T> hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K,
-                                                       int64_t N, int64_t P, hipStream_t s);
+                                                       int64_t N, int64_t P, int64_t S, hipStream_t s);
 template <typename T> hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T* dB, int64_t M, int64_t K,
-                                                       int64_t N, int64_t P, hipStream_t s);
+                                                       int64_t N, int64_t P, int64_t S, hipStream_t s);
 
 }  // namespace prad

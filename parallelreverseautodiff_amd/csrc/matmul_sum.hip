@@ -24,23 +24,32 @@ __global__ void __launch_bounds__(64) sum_tiles_kernel(const double* __restrict_
     out[q] = (T)s;
 }
 
+// S samples (BatchMatrixMultiplyAndSumOperation / BatchGpuMatrixMultiplyAndSumOperation,
+// src/RMAD/BatchGpuMatrixMultiplyAndSumOperation.cs:51-74: sample i multiplies its own A[i] with the shared slices B[q]):
+// all S x P products are one two-level batch, sample-major like the output (S, 1, P).
 template <typename T>
 hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K, int64_t N, int64_t P,
-                                 hipStream_t s) {
-    if (P <= 0) return hipSuccess;
+                                 int64_t S, hipStream_t s) {
+    if (P <= 0 || S <= 0) return hipSuccess;
+    if (S * P > 65535) return hipErrorInvalidValue;
     GemmArgs<T> g{};
     g.transA = 0; g.transB = 0;
     g.M = M; g.N = N; g.K = K;
     g.A = A; g.lda = K;
     g.B = B; g.ldb = N;
     g.C = nullptr; g.ldc = N;
-    g.batch = (int)P;
+    g.batch = (int)(S * P);
     g.strideA = 0; g.strideB = K * N; g.strideC = 0;
+    if (S > 1) {
+        g.batch_inner = (int)P;            // product (sample, slice) = batch index sample * P + slice
+        g.strideA = M * K; g.istrideA = 0;
+        g.strideB = 0; g.istrideB = K * N;
+    }
     g.tile_sums = workspace;
     hipError_t e = launch_gemm<T>(g, s);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((sum_tiles_kernel<T>), dim3((unsigned)((P + 63) / 64)), dim3(64), 0, s, workspace, out,
-                       gemm_tiles_per_product(M, N), P);
+    hipLaunchKernelGGL((sum_tiles_kernel<T>), dim3((unsigned)((S * P + 63) / 64)), dim3(64), 0, s, workspace, out,
+                       gemm_tiles_per_product(M, N), S * P);
     return hipGetLastError();
 }
 
@@ -223,6 +232,12 @@ __global__ void __launch_bounds__(256) sum_bwd_kernel(const T* __restrict__ A, c
                                                       T* __restrict__ dA, T* __restrict__ dB, int64_t M, int64_t K, int64_t N,
                                                       int64_t P, int64_t da_blocks, int64_t da_bm, int64_t bm, int64_t db_by) {
     __shared__ T tile[TS][TS + 1];
+    // blockIdx.y is the sample of a batch (its own A, dOut, dA and dB slices; B is shared by all samples)
+    const int64_t sample = blockIdx.y;
+    A += sample * M * K;
+    dOut += sample * P;
+    if (dA != nullptr) dA += sample * M * K;
+    if (dB != nullptr) dB += sample * P * K * M;
     int64_t id = blockIdx.x;
     if (id < da_blocks) {
         if (VECTOR) sum_bwd_da_block_vec<T>(tile, B, dOut, dA, M, K, N, P, id % da_bm, id / da_bm);
@@ -236,8 +251,9 @@ __global__ void __launch_bounds__(256) sum_bwd_kernel(const T* __restrict__ A, c
 
 template <typename T>
 hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T* dB, int64_t M, int64_t K, int64_t N, int64_t P,
-                                 hipStream_t s) {
-    if (M <= 0 || K <= 0) return hipSuccess;
+                                 int64_t S, hipStream_t s) {
+    if (M <= 0 || K <= 0 || S <= 0) return hipSuccess;
+    if (S > 65535) return hipErrorInvalidValue;
     constexpr int VEC = SumVec<T>::N;
     auto aligned = [](const void* p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     const bool vec = M % VEC == 0 && K % VEC == 0 && N % VEC == 0 && aligned(A) && aligned(B) && aligned(dA) && aligned(dB);
@@ -247,7 +263,7 @@ hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T
     const int64_t db_blocks = (dB != nullptr && P > 0) ? bm * db_by * ((P + qpw - 1) / qpw) : 0;
     if (da_blocks + db_blocks == 0) return hipSuccess;
     if (da_blocks + db_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)(da_blocks + db_blocks)), block(256);
+    const dim3 grid((unsigned)(da_blocks + db_blocks), (unsigned)S), block(256);
     if (vec)
         hipLaunchKernelGGL((sum_bwd_kernel<T, true>), grid, block, 0, s, A, B, dOut, dA, dB, M, K, N, P, da_blocks, da_bm, bm, db_by);
     else
@@ -256,12 +272,12 @@ hipError_t launch_matmul_sum_bwd(const T* A, const T* B, const T* dOut, T* dA, T
 }
 
 template hipError_t launch_matmul_sum_fwd<double>(const double*, const double*, double*, double*, int64_t, int64_t, int64_t,
-                                                  int64_t, hipStream_t);
-template hipError_t launch_matmul_sum_fwd<float>(const float*, const float*, float*, double*, int64_t, int64_t, int64_t, int64_t,
-                                                 hipStream_t);
-template hipError_t launch_matmul_sum_bwd<double>(const double*, const double*, const double*, double*, double*, int64_t, int64_t,
                                                   int64_t, int64_t, hipStream_t);
+template hipError_t launch_matmul_sum_fwd<float>(const float*, const float*, float*, double*, int64_t, int64_t, int64_t, int64_t,
+                                                 int64_t, hipStream_t);
+template hipError_t launch_matmul_sum_bwd<double>(const double*, const double*, const double*, double*, double*, int64_t, int64_t,
+                                                  int64_t, int64_t, int64_t, hipStream_t);
 template hipError_t launch_matmul_sum_bwd<float>(const float*, const float*, const float*, float*, float*, int64_t, int64_t,
-                                                 int64_t, int64_t, hipStream_t);
+                                                 int64_t, int64_t, int64_t, hipStream_t);
 
 }  // namespace prad

@@ -519,13 +519,17 @@ int32_t prad_buf_alloc(int32_t dtype, int64_t rows, int64_t cols, prad_buf_t* ou
     return prad_buf_alloc_deep(dtype, 1, rows, cols, out);
 }
 
-int32_t prad_buf_wrap(int32_t dtype, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out) {
+int32_t prad_buf_wrap_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out) {
     REQUIRE_INIT();
     if (out == nullptr || device_ptr == nullptr) return fail(PRAD_ERR_ARG, "NULL argument");
     if (dtype != PRAD_F64 && dtype != PRAD_F32) return fail(PRAD_ERR_DTYPE, "unknown dtype %d", dtype);
-    if (rows <= 0 || cols <= 0) return fail(PRAD_ERR_ARG, "matrix dimensions must be positive");
-    *out = new prad_buf{BUF_MAGIC, dtype, 1, rows, cols, device_ptr, false};
+    if (depth <= 0 || rows <= 0 || cols <= 0) return fail(PRAD_ERR_ARG, "matrix dimensions must be positive");
+    *out = new prad_buf{BUF_MAGIC, dtype, depth, rows, cols, device_ptr, false};
     return PRAD_OK;
+}
+
+int32_t prad_buf_wrap(int32_t dtype, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out) {
+    return prad_buf_wrap_deep(dtype, 1, rows, cols, device_ptr, out);
 }
 
 int32_t prad_buf_free(prad_buf_t b) {
@@ -970,21 +974,22 @@ int32_t prad_matmul_sum_fwd(prad_buf_t A, prad_buf_t B, prad_buf_t out) {
     REQUIRE_INIT();
     REQUIRE_BUF(A); REQUIRE_BUF(B); REQUIRE_BUF(out);
     if (int32_t st = same_dtype({A, B, out})) return st;
-    if (A->depth != 1) return fail(PRAD_ERR_SHAPE, "first operand must be a single matrix");
     if (A->cols != B->rows) return fail(PRAD_ERR_SHAPE, "Matrix dimensions must be compatible for multiplication.");
-    const int64_t P = B->depth;
-    if (out->depth != 1 || out->rows != 1 || out->cols != P) return fail(PRAD_ERR_ARG, "output must be 1 x depth");
+    const int64_t P = B->depth, S = A->depth;
+    if (out->depth != S || out->rows != 1 || out->cols != P)
+        return fail(PRAD_ERR_ARG, "output must be 1 x depth(B) for each of the depth(A) samples");
+    if (S * P > 65535) return fail(PRAD_ERR_ARG, "at most 65535 products per call");
     ENQUEUE_LOCK();
-    const size_t ws = (size_t)P * gemm_tiles_per_product(A->rows, B->cols) * sizeof(double);
+    const size_t ws = (size_t)S * P * gemm_tiles_per_product(A->rows, B->cols) * sizeof(double);
     if (int32_t st = ensure_workspace(ws)) return st;
     double* w = static_cast<double*>(CUR_WORKSPACE);
     if (A->dtype == PRAD_F64)
         HIP_TRY(launch_matmul_sum_fwd<double>(static_cast<const double*>(A->ptr), static_cast<const double*>(B->ptr),
-                                              static_cast<double*>(out->ptr), w, A->rows, A->cols, B->cols, P, CUR_STREAM),
+                                              static_cast<double*>(out->ptr), w, A->rows, A->cols, B->cols, P, S, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     else
         HIP_TRY(launch_matmul_sum_fwd<float>(static_cast<const float*>(A->ptr), static_cast<const float*>(B->ptr),
-                                             static_cast<float*>(out->ptr), w, A->rows, A->cols, B->cols, P, CUR_STREAM),
+                                             static_cast<float*>(out->ptr), w, A->rows, A->cols, B->cols, P, S, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -995,25 +1000,27 @@ int32_t prad_matmul_sum_bwd(prad_buf_t A, prad_buf_t B, prad_buf_t dOut, prad_bu
     if (dA != nullptr) REQUIRE_BUF(dA);
     if (dB != nullptr) REQUIRE_BUF(dB);
     if (int32_t st = same_dtype({A, B, dOut, dA, dB})) return st;
-    const int64_t M = A->rows, K = A->cols, N = B->cols, P = B->depth;
-    if (A->depth != 1 || B->rows != K) return fail(PRAD_ERR_SHAPE, "Matrix dimensions must be compatible for multiplication.");
-    if (dOut->depth != 1 || dOut->rows != 1 || dOut->cols != P) return fail(PRAD_ERR_ARG, "upstream gradient must be 1 x depth");
+    const int64_t M = A->rows, K = A->cols, N = B->cols, P = B->depth, S = A->depth;
+    if (B->rows != K) return fail(PRAD_ERR_SHAPE, "Matrix dimensions must be compatible for multiplication.");
+    if (dOut->depth != S || dOut->rows != 1 || dOut->cols != P)
+        return fail(PRAD_ERR_ARG, "upstream gradient must be 1 x depth(B) for each of the depth(A) samples");
+    if (S > 65535) return fail(PRAD_ERR_ARG, "at most 65535 samples per call");
     if (dA != nullptr) {
         if (N != M) return fail(PRAD_ERR_SHAPE, "transpose(B[q]) must have the shape of A (the reference adds them elementwise)");
-        if (dA->depth != 1 || dA->rows != M || dA->cols != K) return fail(PRAD_ERR_ARG, "dA must have the shape of A");
+        if (dA->depth != S || dA->rows != M || dA->cols != K) return fail(PRAD_ERR_ARG, "dA must have the shape of A");
     }
-    if (dB != nullptr && (dB->depth != P || dB->rows != K || dB->cols != M))
-        return fail(PRAD_ERR_ARG, "dB must be depth x cols(A) x rows(A)");
+    if (dB != nullptr && (dB->depth != S * P || dB->rows != K || dB->cols != M))
+        return fail(PRAD_ERR_ARG, "dB must be (samples * depth) x cols(A) x rows(A)");
     ENQUEUE_LOCK();
     if (A->dtype == PRAD_F64)
         HIP_TRY(launch_matmul_sum_bwd<double>(static_cast<const double*>(A->ptr), static_cast<const double*>(B->ptr),
                                               static_cast<const double*>(dOut->ptr), dA ? static_cast<double*>(dA->ptr) : nullptr,
-                                              dB ? static_cast<double*>(dB->ptr) : nullptr, M, K, N, P, CUR_STREAM),
+                                              dB ? static_cast<double*>(dB->ptr) : nullptr, M, K, N, P, S, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     else
         HIP_TRY(launch_matmul_sum_bwd<float>(static_cast<const float*>(A->ptr), static_cast<const float*>(B->ptr),
                                              static_cast<const float*>(dOut->ptr), dA ? static_cast<float*>(dA->ptr) : nullptr,
-                                             dB ? static_cast<float*>(dB->ptr) : nullptr, M, K, N, P, CUR_STREAM),
+                                             dB ? static_cast<float*>(dB->ptr) : nullptr, M, K, N, P, S, CUR_STREAM),
                 PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }

@@ -125,8 +125,7 @@ class Matrix:
                 raise ArgumentException("matrix needs at least one row")
             first = np.asarray(given[0])
             self.dtype = np.dtype(first.dtype if first.dtype in (np.float32, np.float64) else dtype)
-            self._rows = [r if isinstance(r, np.ndarray) and r.dtype == self.dtype and r.ndim == 1
-                          else np.array(r, dtype=self.dtype).reshape(-1) for r in given]
+            self._rows = [self._adopt_row(r) for r in given]
             self._nrows, self._ncols = len(self._rows), self._rows[0].shape[0]
         else:
             if rows <= 0 or cols <= 0:
@@ -136,6 +135,14 @@ class Matrix:
             self._nrows, self._ncols = int(rows), int(cols)
             self._rows = [np.zeros(self._ncols, dtype=self.dtype) for _ in range(self._nrows)]  # one array per row
         self._host_valid = True
+
+    def _adopt_row(self, r):
+        """A row array as the device copies read it: one-dimensional, contiguous, of this matrix's element type.  An
+        array that already is (the usual case) is adopted as it is and stays live, like a row of the reference's
+        double[][]; a strided view or an array of another type is copied."""
+        if isinstance(r, np.ndarray) and r.dtype == self.dtype and r.ndim == 1 and r.flags["C_CONTIGUOUS"]:
+            return r
+        return np.ascontiguousarray(np.asarray(r, dtype=self.dtype).reshape(-1))
 
     # ---- construction helpers -------------------------------------------------------------
     @classmethod
@@ -196,7 +203,7 @@ class Matrix:
             i, j = index
             rows[i][j] = value
         else:
-            rows[index] = np.asarray(value, dtype=self.dtype)  # row replacement, as GradientClearer does
+            rows[index] = self._adopt_row(value)  # row replacement, as GradientClearer does
 
     def __iter__(self):
         return iter(self._host())
@@ -205,7 +212,7 @@ class Matrix:
         return self._host()
 
     def Replace(self, rows):
-        self._rows = list(rows)
+        self._rows = [self._adopt_row(r) for r in rows]
         self._nrows, self._ncols = len(self._rows), self._rows[0].shape[0]
         self._host_valid, self._dev_valid = True, False
         if self._dev is not None and (self._dev.rows != self._nrows or self._dev.cols != self._ncols):
@@ -213,7 +220,9 @@ class Matrix:
 
     # ---- device side ------------------------------------------------------------------------
     def device(self):
-        """Device buffer holding the current values (uploads the jagged rows when needed)."""
+        """Device buffer holding the current values (uploads the jagged rows when needed).  Row arrays handed out
+        before this call stay live on the host only: fetch them again (m[i], ToArray()) before writing, which marks
+        the device copy stale."""
         if self._dev is None:
             self._dev = DeviceBuffer.alloc(self.dtype, self._nrows, self._ncols)
             self._dev_valid = False

@@ -306,6 +306,75 @@ class GpuMatrixMultiplyAndSumOperation(MatrixMultiplyAndSumOperation):
         return GpuMatrixMultiplyAndSumOperation()
 
 
+class _BatchMatrixMultiplyAndSumBase(Operation):
+    """MatrixMultiplyAndSum per sample of a batch (src/RMAD/BatchGpuMatrixMultiplyAndSumOperation.cs:51-74,
+    src/RMAD/BatchMatrixMultiplyAndSumOperation.cs:51-74): Forward(input1 deep of S samples, input2 deep of P slices)
+    returns a DeepMatrix of S matrices 1 x P, sample i being MatrixMultiplyAndSum(input1[i], input2); Backward(dOutput
+    deep of S matrices 1 x P) returns one BackwardResult per sample, [dA_i, dB_i[0], ..., dB_i[P-1]] as the single
+    operation builds it.  The reference loops over the samples (Parallel.For in Backward); here every sample and
+    slice shares one launch each way."""
+
+    _needs_init = True
+
+    def __init__(self):
+        super().__init__()
+        self.DeepOutput = None
+        self._in1 = None
+        self._in2 = None
+
+    def GetDeepOutput(self):
+        return self.DeepOutput
+
+    def _intermediates(self):
+        return [self._in1, self._in2]
+
+    def _restore_from(self, items):
+        self._in1, self._in2 = items
+
+    def Forward(self, input1, input2):
+        if self._needs_init:
+            _require_initialized()
+        else:
+            _ensure_initialized()
+        if not isinstance(input1, DeepMatrix) or not isinstance(input2, DeepMatrix):
+            raise ArgumentException("both inputs must be DeepMatrix")
+        if input1.Cols != input2.Rows:
+            raise InvalidOperationException("Matrix dimensions must be compatible for multiplication.")
+        self._in1, self._in2 = input1, input2
+        out = DeviceBuffer.alloc(input1.dtype, 1, input2.Depth, depth=input1.Depth)
+        check(_lib.load().prad_matmul_sum_fwd(input1.device().handle, input2.device().handle, out.handle))
+        self.DeepOutput = DeepMatrix._from_device(out)
+        return self.DeepOutput
+
+    def Backward(self, dOutput):
+        if self._needs_init:
+            _require_initialized()
+        a, b = self._in1, self._in2
+        S, P = a.Depth, b.Depth
+        if dOutput.Depth != S:
+            raise ArgumentException("upstream gradient must hold one matrix per sample")
+        d_a = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols, depth=S)
+        d_b = DeviceBuffer.alloc(a.dtype, a.Cols, a.Rows, depth=S * P)
+        check(_lib.load().prad_matmul_sum_bwd(a.device().handle, b.device().handle, dOutput.device().handle, d_a.handle, d_b.handle))
+        m_a, m_b = DeepMatrix._from_device(d_a), DeepMatrix._from_device(d_b)
+        return [BackwardResultBuilder().AddInputGradient(m_a[i]).AddInputGradientArray([m_b[i * P + q] for q in range(P)]).Build()
+                for i in range(S)]
+
+
+class BatchMatrixMultiplyAndSumOperation(_BatchMatrixMultiplyAndSumBase):
+    _needs_init = False
+
+    @staticmethod
+    def Instantiate(net):
+        return BatchMatrixMultiplyAndSumOperation()
+
+
+class BatchGpuMatrixMultiplyAndSumOperation(_BatchMatrixMultiplyAndSumBase):
+    @staticmethod
+    def Instantiate(net):
+        return BatchGpuMatrixMultiplyAndSumOperation()
+
+
 class BatchMatrixMultiplySumOperation(Operation):
     """Independent products summed into one output plus a broadcast bias: C = sum_q A[q].B[q] + bias.
     No operation of the reference has this form; it is the composition of MatrixMultiplyOperation.Forward

@@ -31,6 +31,23 @@ def test_matrix_ids_are_unique_and_adopted_rows_are_live():
     assert f.dtype == np.float32
 
 
+def test_matrix_rows_are_contiguous_and_of_the_matrix_type():
+    """What the device copies read from a row is cols contiguous elements of the matrix's type: a strided view or a
+    row of another type is copied on adoption (also through Replace and row assignment) instead of being read past."""
+    base = np.arange(12.0).reshape(3, 4)
+    m = Matrix([base[:, 0], base[:, 1]])                     # column views: stride of 32 bytes
+    assert all(r.flags["C_CONTIGUOUS"] and r.dtype == np.float64 for r in m.ToArray())
+    assert np.array_equal(m.to_numpy(), base[:, :2].T)
+    m.Replace([np.arange(3, dtype=np.float32), base[0, ::2][:3] if False else np.array([7, 8, 9])])
+    assert all(r.dtype == np.float64 and r.flags["C_CONTIGUOUS"] for r in m.ToArray()) and m.Cols == 3
+    m[1] = base[:, 3]
+    assert m.ToArray()[1].flags["C_CONTIGUOUS"] and np.array_equal(m.ToArray()[1], [3.0, 7.0, 11.0])
+    live = np.zeros(3)
+    m[0] = live                                              # a conforming array is adopted, not copied
+    live[2] = 5.0
+    assert m[0, 2] == 5.0
+
+
 def test_matrix_rejects_bad_arguments():
     with pytest.raises(exceptions.ArgumentException):
         Matrix(0, 3)

@@ -6,7 +6,8 @@ from conftest import TOL, assert_parity
 from parallelreverseautodiff_amd import seeded
 from parallelreverseautodiff_amd.exceptions import InvalidOperationException
 from parallelreverseautodiff_amd.matrix import DeepMatrix, Matrix
-from parallelreverseautodiff_amd.operations import GpuMatrixMultiplyAndSumOperation, MatrixMultiplyAndSumOperation
+from parallelreverseautodiff_amd.operations import (BatchGpuMatrixMultiplyAndSumOperation, BatchMatrixMultiplyAndSumOperation,
+                                                   GpuMatrixMultiplyAndSumOperation, MatrixMultiplyAndSumOperation)
 
 pytestmark = pytest.mark.gpu
 DTYPES = [np.float64, np.float32]
@@ -57,6 +58,53 @@ def test_benchmark_configuration_shape_fp32(gpu, oracle):
     assert np.array_equal(res.Item1.to_numpy(), rdA)
     for q in (0, 13, 31):
         assert np.array_equal(res.Results[1 + q].to_numpy(), rdB[q])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cls", [BatchGpuMatrixMultiplyAndSumOperation, BatchMatrixMultiplyAndSumOperation])
+@pytest.mark.parametrize("shape", [(3, 6, 9, 4), (8, 64, 96, 5), (5, 130, 70, 3), (2, 100, 36, 1), (1, 32, 48, 7)])
+def test_per_sample_wrappers(gpu, oracle, dtype, cls, shape):
+    """BatchMatrixMultiplyAndSumOperation / BatchGpuMatrixMultiplyAndSumOperation
+    (src/RMAD/BatchGpuMatrixMultiplyAndSumOperation.cs:51-74): sample i is MatrixMultiplyAndSum(input1[i], input2); the
+    results per sample are those of the single operation (backward bit for bit)."""
+    S, M, K, P = shape
+    A = seeded.normal(83, 1, (S, M, K), 1.0, dtype)
+    B = seeded.normal(83, 2, (P, K, M), 1.0, dtype)
+    dOut = seeded.normal(83, 3, (S, 1, P), 1.0, dtype)
+    op = cls.Instantiate(None)
+    out = op.Forward(DeepMatrix.from_numpy(A), DeepMatrix.from_numpy(B))
+    assert op.GetDeepOutput() is out and out.Depth == S and (out.Rows, out.Cols) == (1, P)
+    for i in range(S):
+        check_forward(out[i].to_numpy(), A[i], B, oracle.matmul_sum_fwd(A[i], B), dtype)
+    results = op.Backward(DeepMatrix.from_numpy(dOut))
+    assert len(results) == S
+    for i, res in enumerate(results):
+        assert res.HasMultipleInputs and len(res.Results) == 1 + P
+        rdA, rdB = oracle.matmul_sum_bwd(A[i], B, dOut[i])
+        assert np.array_equal(res.Item1.to_numpy(), rdA), "dA of sample %d" % i
+        for q in range(P):
+            assert np.array_equal(res.Results[1 + q].to_numpy(), rdB[q]), "dB[%d] of sample %d" % (q, i)
+    # the single operation on one sample gives the bits of that sample in the batch
+    single = GpuMatrixMultiplyAndSumOperation.Instantiate(None)
+    assert np.array_equal(single.Forward(Matrix.from_numpy(A[S - 1]), DeepMatrix.from_numpy(B)).to_numpy(), out[S - 1].to_numpy())
+    # Store / Restore keep the per-sample inputs (IOperationBase.Store, src/RMAD/IOperationBase.cs:188-194)
+    op.Store("a")
+    op.Forward(DeepMatrix.from_numpy(A[::-1].copy()), DeepMatrix.from_numpy(B))
+    op.Restore("a")
+    again = op.Backward(DeepMatrix.from_numpy(dOut))
+    assert np.array_equal(again[0].Item1.to_numpy(), results[0].Item1.to_numpy())
+
+
+def test_per_sample_wrapper_errors(gpu):
+    op = BatchGpuMatrixMultiplyAndSumOperation.Instantiate(None)
+    with pytest.raises(InvalidOperationException, match="compatible for multiplication"):
+        op.Forward(DeepMatrix(3, 4, 5), DeepMatrix(2, 6, 4))
+    from parallelreverseautodiff_amd.exceptions import ArgumentException
+    with pytest.raises(ArgumentException):
+        op.Forward(Matrix(4, 5), DeepMatrix(2, 5, 4))
+    op.Forward(DeepMatrix(3, 4, 5), DeepMatrix(2, 5, 4))
+    with pytest.raises(ArgumentException):
+        op.Backward(DeepMatrix(2, 1, 2))          # one upstream matrix per sample
 
 
 def test_ones_closed_form_and_cpu_name(gpu):
