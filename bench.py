@@ -23,7 +23,52 @@ PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3}  # MI355X dense matrix-core peaks
 METRIC = "fp64/fp32 matmul fwd+bwd TFLOP/s (% MFMA peak); MLP train steps/sec"
 
 
-def gpu_leg(n, dtype_name, steps, warmup):
+def error_metrics(x, ref):
+    """The two error figures of a result against the reference's arithmetic: normwise max|x - ref| / max|ref|, and
+    elementwise max |x - ref| / max(|ref|, 1e-3 rms(ref)); beside them the measure the parity tests hold to the bar,
+    elementwise against max(|ref|, rms(ref))."""
+    x, ref = np.asarray(x, np.float64), np.asarray(ref, np.float64)
+    diff = np.abs(x - ref)
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    tiny = np.finfo(np.float64).tiny
+    return {"normwise": float(diff.max() / max(float(np.abs(ref).max()), tiny)),
+            "elementwise_floor_1e-3_rms": float(np.max(diff / np.maximum(np.abs(ref), max(1e-3 * rms, tiny)))),
+            "elementwise_floor_rms": float(np.max(diff / np.maximum(np.abs(ref), max(rms, tiny))))}
+
+
+def worst_metrics(items):
+    out = {}
+    for m in items:
+        for k, v in m.items():
+            out[k] = max(out.get(k, 0.0), v)
+    return out
+
+
+def gemm_sample_errors(A, B, dC, C, dA, dB, dtype, rows=48):
+    """Error of the timed buffers against the CPU restatement of MatrixMultiplyOperation (same element type, k-ascending
+    sums) on a sample of `rows` rows of each of C, dA and dB; for float also against the products evaluated in double,
+    since at K in the thousands the reference's own float loop is further from the exact product than the bar."""
+    from oracle import oracle
+    n = A.shape[0]
+    rng = np.random.default_rng(1)
+    idx = np.sort(rng.choice(n, size=min(rows, n), replace=False))
+    threads = min(16, oracle.hardware_threads() or 1)
+    cont = np.ascontiguousarray
+    refs = [(C[idx], oracle.matmul_fwd(cont(A[idx]), B, threads=threads)),                       # C = A.B
+            (dA[idx], oracle.matmul_fwd(cont(dC[idx]), cont(B.T), threads=threads)),            # dA = dC.B^T
+            (dB[idx], oracle.matmul_fwd(cont(A[:, idx].T), dC, threads=threads))]               # dB = A^T.dC
+    out = {"against_reference_arithmetic": worst_metrics(error_metrics(x, r) for x, r in refs), "sampled_rows_per_output": int(len(idx))}
+    if dtype == np.float32:
+        f = lambda z: np.asarray(z, np.float64)
+        exact = [f(A[idx]) @ f(B), f(dC[idx]) @ f(B).T, f(A[:, idx]).T @ f(dC)]
+        out["device_against_double"] = worst_metrics(error_metrics(x, e) for (x, _), e in zip(refs, exact))
+        out["reference_arithmetic_against_double"] = worst_metrics(error_metrics(r, e) for (_, r), e in zip(refs, exact))
+    return out
+
+
+def gpu_leg(n, dtype_name, steps, warmup, with_errors=True):
+    """cfg2: MatrixMultiplyOperation forward + backward on device-resident n x n operands; returns the time of `steps`
+    steps (HIP events on the library stream), the wall time, a spot check and the sampled error figures."""
     from parallelreverseautodiff_amd import _lib, seeded
     from parallelreverseautodiff_amd.cudablas import CudaBlas
     from parallelreverseautodiff_amd.exceptions import check
@@ -71,7 +116,8 @@ def gpu_leg(n, dtype_name, steps, warmup):
     tol = 1e-12 if dtype_name == "f64" else 1e-5
     if not worst <= tol:
         raise SystemExit("benchmark output failed its spot check: %.3e" % worst)
-    return float(ms.value), wall_ms, worst
+    errors = gemm_sample_errors(A, B, dC, C, bufs["dA"].download(), bufs["dB"].download(), dtype) if with_errors else None
+    return {"ms": float(ms.value), "wall_ms": wall_ms, "spot": worst, "errors": errors}
 
 
 def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
@@ -226,6 +272,12 @@ def lstm_leg(dtype_name, steps, warmup, with_cpu):
         check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
         return ms.value / steps
 
+    first = None
+    if with_cpu:  # forward + backward from the initial weights, kept for the error figures
+        layer.step(update=False)
+        layer.iteration = 0
+        first = {"loss": float(layer.loss.download()[0, 0]), "hidden states": layer.H_out.download(), "dW": layer.dW.download(),
+                 "db": layer.db.download(), "dX": layer.dX.download()}
     eager_ms = timed(layer.step)
     layer.record()
     rec_ms = timed(layer.replay)
@@ -238,10 +290,14 @@ def lstm_leg(dtype_name, steps, warmup, with_cpu):
         threads = min(16, oracle.hardware_threads() or 1)
         I, H, B, T = layer.input_dim, layer.hidden, layer.batch, layer.steps
         t0 = time.perf_counter()
-        compose.lstm_forward_backward(layer.host_W, np.zeros((1, 4 * H), dtype), layer.host_X, layer.host_Y, I, H, B, T, threads=threads)
+        loss, Hout, dW, db, dX = compose.lstm_forward_backward(layer.host_W, np.zeros((1, 4 * H), dtype), layer.host_X, layer.host_Y,
+                                                               I, H, B, T, threads=threads)
         secs = time.perf_counter() - t0
         out["cpu"] = {"steps_per_s": 1.0 / secs, "ms_per_step": secs * 1e3, "cores": threads, "steps_timed": 1, "kind": "port",
                       "note": "forward + backward only (no clip/Adam), node-by-node composition of the oracle's operations"}
+        out["errors"] = {"against_reference_arithmetic": worst_metrics(
+            error_metrics(first[k], r) for k, r in (("hidden states", Hout), ("dW", dW), ("db", db), ("dX", dX))),
+            "loss_relative": abs(first["loss"] - loss) / abs(loss)}
     return out
 
 
@@ -275,6 +331,14 @@ def swin_leg(dtype_name, steps, warmup, with_cpu):
         check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
         return ms.value / steps
 
+    first = None
+    if with_cpu:  # forward + backward from the initial weights, kept for the error figures
+        blk.step(update=False)
+        blk.iteration = 0
+        first = {"loss": float(blk.loss.download()[0, 0]), "Y2": blk.Y2.download(), "dX": blk.dX.download()}
+        first.update({k: blk.g[k].download() for k in blk.names})
+        operands = {"W2": (blk.H1, blk.dY2), "W1": (blk.Y1, blk.dZ1), "Wo": (blk.O, blk.dY1), "Wqkv": (blk.X, blk.dQKV)}
+        exact = {k: lhs.download().astype(np.float64).T @ rhs.download().astype(np.float64) for k, (lhs, rhs) in operands.items()}
     eager_ms = timed(blk.step)
     blk.record()
     rec_ms = timed(blk.replay)
@@ -286,11 +350,18 @@ def swin_leg(dtype_name, steps, warmup, with_cpu):
         from oracle import compose, oracle
         threads = min(16, oracle.hardware_threads() or 1)
         t0 = time.perf_counter()
-        compose.swin_block_forward_backward({k: blk.host[k] for k in blk.names}, blk.host["X"], blk.host["T"], blk.nw, blk.wt,
-                                            blk.heads, threads=threads)
+        loss, Y2, g, dX = compose.swin_block_forward_backward({k: blk.host[k] for k in blk.names}, blk.host["X"], blk.host["T"],
+                                                              blk.nw, blk.wt, blk.heads, threads=threads)
         secs = time.perf_counter() - t0
         out["cpu"] = {"steps_per_s": 1.0 / secs, "ms_per_step": secs * 1e3, "cores": threads, "steps_timed": 1, "kind": "port",
                       "note": "forward + backward only, node-by-node composition of the oracle's operations (per-window loop in Python)"}
+        pairs = [("Y2", Y2), ("dX", dX)] + [(k, g[k]) for k in blk.names]
+        out["errors"] = {"against_reference_arithmetic": worst_metrics(error_metrics(first[k], r) for k, r in pairs),
+                         "loss_relative": abs(first["loss"] - loss) / abs(loss),
+                         # the weight gradients are sums over all 50 176 token rows: there the reference's k-ascending
+                         # float loop is the less accurate side, so both are also measured against the double product
+                         "weight_gradients_device_against_double": worst_metrics(error_metrics(first[k], exact[k]) for k in exact),
+                         "weight_gradients_reference_arithmetic_against_double": worst_metrics(error_metrics(g[k], exact[k]) for k in exact)}
     return out
 
 
@@ -359,6 +430,13 @@ def mlp_leg(dtype_name, steps, warmup, with_cpu):
         check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
         return ms.value / steps, wall * 1e3 / steps
 
+    first = None
+    if with_cpu:  # the first step from the initial weights, kept for the error figures
+        net.step()
+        first = {"loss": float(net.loss.download()[0, 0]), "grads": [g.download() for g in net._grads],
+                 "weights": [w.download() for w in net._weights]}
+        net = FeedForwardNetwork(dtype=dtype)
+        net.set_batch(X, T)
     eager_ms, eager_wall = timed(net.step)
     net.record()
     graph_ms, graph_wall = timed(net.replay)
@@ -368,7 +446,13 @@ def mlp_leg(dtype_name, steps, warmup, with_cpu):
            "recorded_wall_ms_per_step": graph_wall, "loss_after": loss, "flop_per_step": net.flops_per_step(),
            "parameters": net.parameter_count()}
     if with_cpu:
-        out["cpu"] = mlp_cpu_leg(net.host_W, X, T, net.params, dtype)
+        out["cpu"], ref = mlp_cpu_leg(net.host_W, X, T, net.params, dtype)
+        # clipped gradients of the first step, and in double also the weights after it (in float a gradient entry at
+        # rounding-noise level changes sign between two correct summation orders, and the first Adam step moves its
+        # weight by the learning rate either way: the float weights are compared operation by operation in the tests)
+        pairs = list(zip(first["grads"], ref["grads"])) + (list(zip(first["weights"], ref["weights"])) if dtype_name == "f64" else [])
+        out["errors"] = {"against_reference_arithmetic": worst_metrics(error_metrics(x, r) for x, r in pairs),
+                         "loss_relative": abs(first["loss"] - ref["loss"]) / abs(ref["loss"])}
     return out
 
 
@@ -392,7 +476,7 @@ def mlp_cpu_leg(W0, X, T, params, dtype, budget_s=15.0):
             a = z if l == L - 1 else oracle.leakyrelu_fwd(z, alpha)
             H.append(a)
         P = oracle.softmax_fwd(Z[-1])
-        oracle.cce_fwd(P, T)
+        loss = oracle.cce_fwd(P, T)
         dz = oracle.softmax_bwd(P, oracle.cce_bwd(P, T))
         dW, db = [None] * L, [None] * L
         for l in range(L - 1, -1, -1):
@@ -405,14 +489,15 @@ def mlp_cpu_leg(W0, X, T, params, dtype, budget_s=15.0):
                for w, mm, vv, g in zip(W + b, m, v, grads)]
         W, b = [n[0] for n in new[:L]], [n[0] for n in new[L:]]
         m, v = [n[1] for n in new], [n[2] for n in new]
+        return {"loss": loss, "grads": grads, "weights": W + b}
 
-    step(1)
+    first = step(1)
     n, t0 = 0, time.perf_counter()
     while n < 200 and time.perf_counter() - t0 < budget_s:
         step(n + 2)
         n += 1
     secs = (time.perf_counter() - t0) / n
-    return {"steps_per_s": 1.0 / secs, "ms_per_step": secs * 1e3, "cores": threads, "steps_timed": n, "kind": "port"}
+    return {"steps_per_s": 1.0 / secs, "ms_per_step": secs * 1e3, "cores": threads, "steps_timed": n, "kind": "port"}, first
 
 
 def cpu_leg(budget_s=40.0):
@@ -428,7 +513,7 @@ def cpu_leg(budget_s=40.0):
         n = bigger
         secs = oracle.time_matmul_fwdbwd(n, np.float64, threads=threads, iters=1)
     flops = 6.0 * n ** 3
-    return {"value": flops / secs / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+    return {"value": flops / secs / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port", "n": n, "secs": secs,
             "sample": "fp64 MatrixMultiplyOperation forward+backward at N=%d (%.1f GFLOP, 1 pass, %.2f s), "
                       "C++ restatement of the reference's Parallel.For loops on jagged rows, -O2, no FMA" % (n, flops / 1e9, secs)}
 
@@ -512,7 +597,8 @@ def main():
                           "kernels": res}))
         return
 
-    ms, wall_ms, spot = gpu_leg(args.n, args.dtype, args.steps, args.warmup)
+    head = gpu_leg(args.n, args.dtype, args.steps, args.warmup, with_errors=not args.no_cpu)
+    ms, wall_ms, spot = head["ms"], head["wall_ms"], head["spot"]
     flops_per_step = 6.0 * args.n ** 3
     ms_per_step = ms / args.steps
     tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
@@ -532,41 +618,136 @@ def main():
                      ("double" if args.dtype == "f64" else "float"), "launch_ms": launch_ms},
         "wall_ms_per_step": wall_ms / args.steps, "spot_check_error": spot,
     }
+    if head["errors"] is not None:
+        line["errors"] = head["errors"]
+    cpu = None if args.no_cpu else cpu_leg()
+    table = [gemm_row(args.n, args.dtype, ms_per_step, head["errors"], cpu)]
     if not args.no_also:
-        line["also"] = also_legs(args)
-    if not args.no_cpu:
-        line["cpu_baseline"] = cpu_leg()
+        line["also"] = also_legs(args, table)
+    if cpu is not None:
+        line["cpu_baseline"] = cpu
+    line["table"] = table
     print(json.dumps(line))
 
 
-def also_legs(args):
-    """The rest of the metric beside the headline figure, measured in the same run: the product in the other
-    precision at the same size, the MLP training step of configs[0] (recorded launch sequence; in double beside its CPU
-    restatement on the host cores) and the LSTM training step of configs[3].  A leg
-    that fails is reported as its error text and does not touch the headline figures."""
+def mfma_roofline(flops, ms, dtype_name, kernel):
+    achieved = flops / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS[dtype_name], "unit": "TFLOP/s",
+            "frac": achieved / PEAK_TFLOPS[dtype_name], "traffic": None, "kernel": kernel}
+
+
+def hbm_roofline(nbytes, ms, kernel):
+    achieved = nbytes / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s", "frac": achieved / 8000.0, "traffic": None, "kernel": kernel}
+
+
+def flat_errors(errors):
+    """The two error columns of a table row from an `errors` block (None where the leg had no CPU side)."""
+    if not errors:
+        return {"err_normwise": None, "err_elementwise_floor_1e-3_rms": None}
+    m = errors["against_reference_arithmetic"]
+    return {"err_normwise": m["normwise"], "err_elementwise_floor_1e-3_rms": m["elementwise_floor_1e-3_rms"],
+            "err_elementwise_floor_rms": m["elementwise_floor_rms"]}
+
+
+def gemm_row(n, dtype_name, ms_per_step, errors, cpu):
+    """Table row of the square product; the CPU columns are filled where the CPU sample ran at this very size."""
+    tf = 6.0 * n ** 3 / (ms_per_step * 1e-3) / 1e12
+    row = {"config": "configs[1] MatrixMultiply fwd+bwd N=%d" % n, "precision": dtype_name, "gpu_ms": ms_per_step, "rate": tf,
+           "unit": "TFLOP/s", "bound": "mfma", "frac_of_peak": tf / PEAK_TFLOPS[dtype_name], "cpu_ms": None, "cpu_cores": None, "speedup": None}
+    if cpu is not None and dtype_name == "f64" and cpu.get("n") == n:
+        row.update({"cpu_ms": cpu["secs"] * 1e3, "cpu_cores": cpu["cores"], "speedup": cpu["secs"] * 1e3 / ms_per_step})
+    row.update(flat_errors(errors))
+    return row
+
+
+def step_row(config, dtype_name, r):
+    """Table row of a training step (MLP, LSTM, attention block) from its leg's result."""
+    ms = r["recorded_ms_per_step"]
+    tf = r["flop_per_step"] / (ms * 1e-3) / 1e12
+    row = {"config": config, "precision": dtype_name, "gpu_ms": ms, "rate": 1e3 / ms, "unit": "steps/s", "bound": "mfma",
+           "frac_of_peak": tf / PEAK_TFLOPS[dtype_name], "cpu_ms": None, "cpu_cores": None, "speedup": None}
+    if "cpu" in r:
+        row.update({"cpu_ms": r["cpu"]["ms_per_step"], "cpu_cores": r["cpu"]["cores"], "speedup": r["cpu"]["ms_per_step"] / ms})
+    row.update(flat_errors(r.get("errors")))
+    return row
+
+
+def also_legs(args, table):
+    """The rest of the metric beside the headline figure, measured in the same run, each with the roofline that bounds
+    it: the product in the other precision at the same size and both precisions at the smaller sizes of the
+    configuration, the MLP training step (recorded launch sequence; beside its CPU restatement on the host cores), the
+    LSTM and attention-block steps, MatrixMultiplyAndSum, and the bandwidth-bound gradient kernels on 64 Mi elements.
+    Every leg also adds its row to `table`.  A leg that fails is reported as its error text and does not touch the
+    headline figures."""
     out = {}
+    with_cpu = not args.no_cpu
     other = "f32" if args.dtype == "f64" else "f64"
-    try:
-        ms, _, spot = gpu_leg(args.n, other, args.steps, args.warmup)
-        tf = 6.0 * args.n ** 3 / (ms / args.steps * 1e-3) / 1e12
-        out["matmul_fwd_bwd_" + other] = {"TFLOPs": tf, "frac_of_mfma_peak": tf / PEAK_TFLOPS[other], "n": args.n,
-                                          "ms_per_step": ms / args.steps, "spot_check_error": spot}
-    except Exception as e:  # noqa: BLE001 - reported, not hidden
-        out["matmul_fwd_bwd_" + other] = {"error": repr(e)}
+    for n, d, steps in [(args.n, other, args.steps)] + [(m, dt, 60) for m in (2048, 1024, 512) if m < args.n for dt in ("f64", "f32")]:
+        key = "matmul_fwd_bwd_%s_n%d" % (d, n)
+        try:
+            r = gpu_leg(n, d, steps, args.warmup, with_errors=with_cpu)
+            per = r["ms"] / steps
+            out[key] = {"TFLOPs": 6.0 * n ** 3 / (per * 1e-3) / 1e12, "n": n, "ms_per_step": per, "spot_check_error": r["spot"],
+                        "roofline": mfma_roofline(2.0 * n ** 3, per / 3, d, "prad::gemm_kernel<%s>" % ("double" if d == "f64" else "float")),
+                        "errors": r["errors"]}
+            table.append(gemm_row(n, d, per, r["errors"], None))
+        except Exception as e:  # noqa: BLE001 - reported, not hidden
+            out[key] = {"error": repr(e)}
     for d in ("f64", "f32"):
         try:
-            r = mlp_leg(d, 1000, 100, d == "f64" and not args.no_cpu)
-            leg = {"value": 1e3 / r["recorded_ms_per_step"], "ms_per_step": r["recorded_ms_per_step"], "loss_after": r["loss_after"]}
+            r = mlp_leg(d, 1000, 100, with_cpu)
+            leg = {"value": 1e3 / r["recorded_ms_per_step"], "unit": "steps/s", "ms_per_step": r["recorded_ms_per_step"],
+                   "loss_after": r["loss_after"], "errors": r.get("errors"),
+                   "roofline": mfma_roofline(r["flop_per_step"], r["recorded_ms_per_step"], d,
+                                             "whole step: 9 dependent launches (products on 32x32 tiles, softmax + cross-entropy, clip + Adam)")}
             if "cpu" in r:
                 leg["cpu_baseline"] = r["cpu"]
             out["mlp_train_steps_per_s_" + d] = leg
+            table.append(step_row("configs[0] MLP 784-256-128-10 batch 64 step", d, r))
         except Exception as e:  # noqa: BLE001
             out["mlp_train_steps_per_s_" + d] = {"error": repr(e)}
+    for name, fn, config, kernel in (
+            ("lstm_train_steps_per_s_f32", lstm_leg, "configs[3] LSTM 256->512 batch 128 T=64 step",
+             "whole step: 2 x 64 recurrent launches + 5 large products"),
+            ("swin_block_train_steps_per_s_f32", swin_leg, "configs[4] windowed attention block 16x56x56 embed 96 step",
+             "whole step: 12 dense products, 6 batched window products, softmax, column sums")):
+        try:
+            r = fn("f32", 10, 2, with_cpu)
+            leg = {"value": 1e3 / r["recorded_ms_per_step"], "unit": "steps/s", "ms_per_step": r["recorded_ms_per_step"],
+                   "errors": r.get("errors"), "roofline": mfma_roofline(r["flop_per_step"], r["recorded_ms_per_step"], "f32", kernel)}
+            if "cpu" in r:
+                leg["cpu_baseline"] = r["cpu"]
+            out[name] = leg
+            table.append(step_row(config, "f32", r))
+        except Exception as e:  # noqa: BLE001
+            out[name] = {"error": repr(e)}
     try:
-        r = lstm_leg("f32", 10, 2, False)
-        out["lstm_train_steps_per_s_f32"] = {"value": 1e3 / r["recorded_ms_per_step"], "ms_per_step": r["recorded_ms_per_step"]}
+        r = matmul_sum_leg("f32", 100, 10)
+        out["matmul_and_sum_f32"] = {
+            "forward": {"ms": r["fwd_ms"], "roofline": mfma_roofline(r["fwd_flop"], r["fwd_ms"], "f32", "prad::gemm_kernel<float> with the per-tile sum epilogue")},
+            "backward": {"ms": r["bwd_ms"], "roofline": hbm_roofline(r["bwd_bytes"], r["bwd_ms"], "prad::sum_bwd_kernel<float>")}}
+        table.append({"config": "configs[2] MatrixMultiplyAndSum forward 512x768 x 32 slices", "precision": "f32", "gpu_ms": r["fwd_ms"],
+                      "rate": r["fwd_TFLOPs"], "unit": "TFLOP/s", "bound": "mfma", "frac_of_peak": r["fwd_frac_of_mfma_peak"],
+                      "cpu_ms": None, "cpu_cores": None, "speedup": None, "err_normwise": None, "err_elementwise_floor_1e-3_rms": None})
+        table.append({"config": "configs[2] MatrixMultiplyAndSum backward (as the reference writes it)", "precision": "f32", "gpu_ms": r["bwd_ms"],
+                      "rate": r["bwd_GBps"], "unit": "GB/s", "bound": "hbm", "frac_of_peak": r["bwd_frac_of_8TBps"],
+                      "cpu_ms": None, "cpu_cores": None, "speedup": None, "err_normwise": 0.0, "err_elementwise_floor_1e-3_rms": 0.0})
     except Exception as e:  # noqa: BLE001
-        out["lstm_train_steps_per_s_f32"] = {"error": repr(e)}
+        out["matmul_and_sum_f32"] = {"error": repr(e)}
+    for d in ("f64", "f32"):
+        try:
+            res, n = bandwidth_leg(64 * 1024 * 1024, d, 10, 2,
+                                   ["leakyrelu_bwd", "sigmoid_bwd", "tanh_bwd", "gelu_bwd", "hadamard_bwd", "accumulate", "clip", "adam"])
+            es = 8 if d == "f64" else 4
+            out["gradient_kernels_64Mi_" + d] = {
+                k: {"ms": v["ms"], "roofline": hbm_roofline(v["bytes_per_element"] * n, v["ms"], k)} for k, v in res.items()}
+            for k, v in res.items():
+                table.append({"config": "%s on 64 Mi elements" % k, "precision": d, "gpu_ms": v["ms"], "rate": v["GB/s"], "unit": "GB/s",
+                              "bound": "hbm", "frac_of_peak": v["frac_of_8TBps"], "cpu_ms": None, "cpu_cores": None, "speedup": None,
+                              "err_normwise": None, "err_elementwise_floor_1e-3_rms": None})
+        except Exception as e:  # noqa: BLE001
+            out["gradient_kernels_64Mi_" + d] = {"error": repr(e)}
     return out
 
 

@@ -327,37 +327,38 @@ __global__ void __launch_bounds__(OPT_THREADS) adam_kernel(const TensorTable<T> 
     if (vector_chunk<T, CHUNK>(t.w, t.m, t.v, t.g, begin, end)) {
         typedef typename OptVec<T>::type V;
         constexpr int VN = OptVec<T>::N;
-        constexpr int HALF = PER / VN / 2;  // two passes keep the register footprint moderate
+        constexpr int NV = PER / VN;  // 16-byte vectors per thread and tensor
         V* __restrict__ wv = reinterpret_cast<V*>(t.w + begin);
         V* __restrict__ mv = reinterpret_cast<V*>(t.m + begin);
         V* __restrict__ vv = reinterpret_cast<V*>(t.v + begin);
         V* __restrict__ gv = reinterpret_cast<V*>(t.g + begin);
+        // All loads of the chunk are issued before the first update: the arithmetic of a vector (a division and a
+        // square root per element) then runs while the later vectors are still on their way, and the stores go out
+        // as the updates finish.  Measured against two half-chunk passes: 68.0 -> 69.3 % of 8 TB/s in double,
+        // 73.5 -> 74.5 % in float; plain instead of non-temporal loads or stores cost 4 to 6 points.
+        V w[NV], m[NV], v[NV], g[NV];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            V w[HALF], m[HALF], v[HALF], g[HALF];
+        for (int e = 0; e < NV; ++e) {
+            const int iv = e * OPT_THREADS + threadIdx.x;
+            w[e] = __builtin_nontemporal_load(wv + iv);
+            m[e] = __builtin_nontemporal_load(mv + iv);
+            v[e] = __builtin_nontemporal_load(vv + iv);
+            g[e] = __builtin_nontemporal_load(gv + iv);
+        }
 #pragma unroll
-            for (int e = 0; e < HALF; ++e) {
-                const int iv = (h * HALF + e) * OPT_THREADS + threadIdx.x;
-                w[e] = __builtin_nontemporal_load(wv + iv);
-                m[e] = __builtin_nontemporal_load(mv + iv);
-                v[e] = __builtin_nontemporal_load(vv + iv);
-                g[e] = __builtin_nontemporal_load(gv + iv);
+        for (int e = 0; e < NV; ++e) {
+            const int iv = e * OPT_THREADS + threadIdx.x;
+#pragma unroll
+            for (int c = 0; c < VN; ++c) {
+                T wi = w[e][c], mi = m[e][c], vi = v[e][c];
+                if (CLIP) g[e][c] = clamp(g[e][c]);
+                update(wi, mi, vi, g[e][c]);
+                w[e][c] = wi; m[e][c] = mi; v[e][c] = vi;
             }
-#pragma unroll
-            for (int e = 0; e < HALF; ++e) {
-                const int iv = (h * HALF + e) * OPT_THREADS + threadIdx.x;
-#pragma unroll
-                for (int c = 0; c < VN; ++c) {
-                    T wi = w[e][c], mi = m[e][c], vi = v[e][c];
-                    if (CLIP) g[e][c] = clamp(g[e][c]);
-                    update(wi, mi, vi, g[e][c]);
-                    w[e][c] = wi; m[e][c] = mi; v[e][c] = vi;
-                }
-                if (CLIP) __builtin_nontemporal_store(g[e], gv + iv);
-                __builtin_nontemporal_store(w[e], wv + iv);
-                __builtin_nontemporal_store(m[e], mv + iv);
-                __builtin_nontemporal_store(v[e], vv + iv);
-            }
+            if (CLIP) __builtin_nontemporal_store(g[e], gv + iv);
+            __builtin_nontemporal_store(w[e], wv + iv);
+            __builtin_nontemporal_store(m[e], mv + iv);
+            __builtin_nontemporal_store(v[e], vv + iv);
         }
         return;
     }
