@@ -160,6 +160,10 @@ struct GemmArgs {
     // last at a tile's counter adds the partial tiles; without it, a several-way split takes a second launch
     // and a product that would run as pairs runs unsplit.
     unsigned* split_counters;
+    // Set by launch_gemm: the first shared_tiles tiles of the launch are each shared by shared_splits workgroups, a K
+    // range each, while the tiles after them run unsplit in the same launch (see gemm_shared_tiles_plan).  Their
+    // partial tiles lie compactly in split_ws, tile by tile.  0 = none.
+    int shared_tiles, shared_splits;
     // LSTM step epilogues (launch_lstm_step_fwd / _bwd; see there).  All matrices are rows x lstm_hidden with
     // leading dimension lstm_hidden, except gates / dG (rows x 4 * lstm_hidden, blocks [i | f | g | o]).
     int64_t lstm_hidden;
@@ -217,6 +221,11 @@ int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size)
 // Whether launch_gemm would run the product as pairs of workgroups per tile (needs GemmArgs::split_counters and
 // split_ws: 2 * batch * M * N elements).  In-kernel reduction uses at most GEMM_SPLIT_MAX_TILES counters.
 bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size);
+// A product on 128 x 128 tiles whose tile count leaves a poorly filled last round of workgroups (576 tiles over 512
+// workgroup slots: 64 tiles would run alone on 64 compute units while 192 sit idle) splits that many tiles along K
+// so that they fill the chip too.  Returns how many ways (0: none) and, through shared_tiles, how many tiles;
+// split_ws must then hold shared_tiles * ways * 128 * 128 elements and split_counters be set.
+int gemm_shared_tiles_plan(int64_t M, int64_t N, int64_t K, int batch, int elem_size, int* shared_tiles);
 constexpr int GEMM_SPLIT_MAX_TILES = 384;
 
 // Number of 128 x 128 output tiles of one product (the tile_sums layout).

@@ -20,7 +20,10 @@
 //       S[mn][k], row pitch BK elements + 16 bytes, chosen so that the 16 bytes of two neighbouring k
 //       of 16 consecutive mn fall into distinct 16-byte bank groups (an XOR-swizzled unpadded
 //       layout was measured too: same speed in double, 6 % slower in float because the compiler
-//       can no longer merge neighbouring LDS reads);
+//       can no longer merge neighbouring LDS reads; a pitch of one element (double) / two (float) past the
+//       power of two, which takes the two-way conflicts that SQ_LDS_BANK_CONFLICT shows for this placement out of
+//       the fragment reads but lets the slab be written in 8-byte halves only, was measured as well: nothing at
+//       N <= 2048 in double, -2 % at N >= 2048 in float - the conflicts are not what the small tiles wait for);
 //   stored with mn contiguous ("MC": B of the forward, both operands of dB)
 //       S[k][mn], row pitch MN + 16 elements for the 128 tile; the smaller tiles keep the pitch at MN and
 //       rotate row k instead (Slab::mc_shift), so that two of their workgroups fit on a compute unit.
@@ -229,8 +232,16 @@ struct GridPos {
 // K = 32 or 49).  Software pipelining has nothing to work with there, so the kernel keeps one LDS stage instead
 // of two and no prefetch registers: more workgroups share a compute unit and overlap one another's loads,
 // products and stores.  It multiplies only the k steps that the last slab has.
+// LDS of one workgroup of gemm_tile: the slab stages ([stage][A slab | B slab]), reused by the epilogues.
+template <typename T, int WT, bool A_KC, bool B_KC, bool SHORT = false, int DIV = 1>
+constexpr int gemm_lds_elems() {
+    return (SHORT ? 1 : 2) * (Slab<T, WT, DIV>::template elems<A_KC>() + Slab<T, WT, DIV>::template elems<B_KC>());
+}
+
+// `lds`: gemm_lds_elems<...>() elements of 16-byte aligned LDS that the kernel provides (a kernel that holds two
+// products gives both the same block).
 template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI, bool SHORT = false, int DIV = 1>
-__device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM, const int tilesN, const GridPos g_) {
+__device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM, const int tilesN, const GridPos g_, T* __restrict__ lds) {
     typedef Mfma<T> MF;
     typedef Slab<T, WT, DIV> S;
     typedef typename MF::Acc Acc;
@@ -242,7 +253,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     constexpr int SA = S::template elems<A_KC>(), SB = S::template elems<B_KC>();
 
     static_assert(!SHORT || (EDGE && EPI == EPI_PLAIN), "the single-stage kernel is guarded and stores plainly");
-    __shared__ __attribute__((aligned(16))) T smem[SHORT ? 1 : 2][SA + SB];  // [stage][A slab | B slab]
+    T (*smem)[SA + SB] = reinterpret_cast<T (*)[SA + SB]>(lds);  // [stage][A slab | B slab]
 
     // Workgroups beyond the tiles carry a column sum that rides along with this launch.
     if (g_.bx >= (unsigned)(tilesM * tilesN)) {
@@ -261,7 +272,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     const T* __restrict__ B = p.B + b_outer * p.strideB + b_inner * p.istrideB;
     // A product split along K: this workgroup reduces [kb, kb + K) and writes its own M x N partial result.
     int64_t K = p.K;
-    if (p.ksplit > 0) {
+    if (g_.gz > 1) {
         const int64_t kb = (int64_t)g_.bz * p.ksplit;
         K = min(p.ksplit, p.K - kb);
         A += (int64_t)g_.bz * p.zstrideA;
@@ -494,7 +505,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         return;
     }
 
-    if (EPI != EPI_TILE_SUM && p.split_counters != nullptr) {
+    if (EPI != EPI_TILE_SUM && p.split_counters != nullptr && g_.gz > 1) {
         // Several workgroups share this tile, a K range each.  Every one parks its partial tile in the workspace
         // and counts its arrival; the one that arrives last adds the partial tiles in split order (its own
         // included, read back like the others, so that the sum does not depend on who arrives last) and goes on
@@ -566,6 +577,22 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                 }
             }
         }
+    }
+
+    if (WT == 4 && EPI != EPI_TILE_SUM && p.shared_splits > 1 && g_.gz > 1) {
+        // One of the workgroups that share a tile of an otherwise unsplit launch: its partial tile goes to the workspace
+        // as a plain 128 x 128 row-major block (tile by tile, split by split); shared_reduce_kernel adds the blocks of a
+        // tile in split order and applies the epilogue.
+        T* __restrict__ mine = p.split_ws + ((int64_t)g_.bx * g_.gz + g_.bz) * (BM * BN);
+#pragma unroll
+        for (int x = 0; x < WTM; ++x)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int il = wm * WS + x * 16 + MF::row(r, g);
+#pragma unroll
+                for (int y = 0; y < WTN; ++y) mine[il * BN + wn * WS + y * 16 + li] = acc[x][y][r];
+            }
+        return;
     }
 
     if (EPI == EPI_LSTM_FWD) {
@@ -649,7 +676,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     }
 
     T* __restrict__ C = p.C + b_outer * p.strideC + b_inner * p.istrideC +
-                        ((p.ksplit > 0 && p.split_counters == nullptr) ? (int64_t)g_.bz * g_.gy * p.strideC : 0);
+                        ((g_.gz > 1 && p.split_counters == nullptr) ? (int64_t)g_.bz * g_.gy * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
         // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
         // row-major: the elementwise arithmetic (which includes exp/tanh code) then sits in one runtime loop
@@ -775,20 +802,36 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
 template <typename T, int WT, bool A_KC, bool B_KC, bool EDGE, int EPI>
 __global__ void __launch_bounds__(GEMM_THREADS, min_blocks(WT)) gemm_kernel(const GemmArgs<T> p, const int tilesM,
                                                                             const int tilesN) {
-    gemm_tile<T, WT, A_KC, B_KC, EDGE, EPI>(p, tilesM, tilesN, GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z});
+    GridPos g{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z};
+    if (WT == 4 && p.shared_splits > 1) {
+        // The first workgroups of the launch share the first tiles, shared_splits consecutive workgroups per tile;
+        // the rest take one unsplit tile each.
+        const unsigned head = (unsigned)p.shared_tiles * (unsigned)p.shared_splits;
+        if (blockIdx.x < head) {
+            g.bx = blockIdx.x / (unsigned)p.shared_splits;
+            g.bz = blockIdx.x % (unsigned)p.shared_splits;
+            g.gz = (unsigned)p.shared_splits;
+        } else {
+            g.bx = (unsigned)p.shared_tiles + (blockIdx.x - head);
+        }
+    }
+    __shared__ __attribute__((aligned(16))) T lds[gemm_lds_elems<T, WT, A_KC, B_KC>()];
+    gemm_tile<T, WT, A_KC, B_KC, EDGE, EPI>(p, tilesM, tilesN, g, lds);
 }
 
 // 128 x 128 tiles on slabs of half the depth, three workgroups to a compute unit.
 template <typename T, bool A_KC, bool B_KC, int EPI>
 __global__ void __launch_bounds__(GEMM_THREADS, 3) gemm_thin_kernel(const GemmArgs<T> p, const int tilesM, const int tilesN) {
+    __shared__ __attribute__((aligned(16))) T lds[gemm_lds_elems<T, 4, A_KC, B_KC, false, 2>()];
     gemm_tile<T, 4, A_KC, B_KC, false, EPI, false, 2>(p, tilesM, tilesN,
-                                                      GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z});
+                                                      GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z}, lds);
 }
 
 template <typename T, int WT, bool A_KC, bool B_KC>
 __global__ void __launch_bounds__(GEMM_THREADS, 4) gemm_short_kernel(const GemmArgs<T> p, const int tilesM, const int tilesN) {
+    __shared__ __attribute__((aligned(16))) T lds[gemm_lds_elems<T, WT, A_KC, B_KC, true>()];
     gemm_tile<T, WT, A_KC, B_KC, true, EPI_PLAIN, true>(p, tilesM, tilesN,
-                                                        GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z});
+                                                        GridPos{blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y, gridDim.z}, lds);
 }
 
 // The two gradient products of a layer, dA = dC . B^T (both operands k-contiguous; the upstream activation's
@@ -796,13 +839,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, 4) gemm_short_kernel(const GemmA
 // in one launch on 32 x 32 tiles: small layers cost what their chain of dependent launches costs.  Workgroups
 // [0, first) belong to the first product, the rest to the second.  Neither product is split or batched.
 template <typename T, bool EDGE1, int EPI1, bool EDGE2>
-__global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_pair_kernel(const GemmArgs<T> p1, const int tilesM1, const int tilesN1,
+__global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_pair_kernel(const GemmArgs<T> p1, const int tilesM1, const int tilesN1,
                                                                      const GemmArgs<T> p2, const int tilesM2, const int tilesN2,
                                                                      const unsigned first) {
-    // (each product's slab stages are LDS of their own: 133 KB together, one workgroup per compute unit, which is
-    // all such small products put there anyway)
-    if (blockIdx.x < first) gemm_tile<T, 1, true, true, EDGE1, EPI1>(p1, tilesM1, tilesN1, GridPos{blockIdx.x, 0u, 0u, 1u, 1u});
-    else gemm_tile<T, 1, false, false, EDGE2, EPI_PLAIN>(p2, tilesM2, tilesN2, GridPos{blockIdx.x - first, 0u, 0u, 1u, 1u});
+    // (one block of LDS serves whichever product the workgroup belongs to, so two workgroups fit on a compute unit)
+    constexpr int LDS1 = gemm_lds_elems<T, 1, true, true>(), LDS2 = gemm_lds_elems<T, 1, false, false>();
+    __shared__ __attribute__((aligned(16))) T lds[LDS1 > LDS2 ? LDS1 : LDS2];
+    if (blockIdx.x < first) gemm_tile<T, 1, true, true, EDGE1, EPI1>(p1, tilesM1, tilesN1, GridPos{blockIdx.x, 0u, 0u, 1u, 1u}, lds);
+    else gemm_tile<T, 1, false, false, EDGE2, EPI_PLAIN>(p2, tilesM2, tilesN2, GridPos{blockIdx.x - first, 0u, 0u, 1u, 1u}, lds);
 }
 
 // Which products go to the single-stage kernel (PRAD_GEMM_SHORT=0 switches it off: tuning aid): batches of small
@@ -824,7 +868,7 @@ template <typename T>
 static bool gemm_thin_eligible(const GemmArgs<T>& a, bool edge, int epi, int64_t tiles) {
     static const int64_t max_k = [] { const char* e = getenv("PRAD_GEMM_THIN_MAX_K"); return e ? (int64_t)atoll(e) : (int64_t)128; }();
     static const int64_t min_tiles = [] { const char* e = getenv("PRAD_GEMM_THIN_MIN_TILES"); return e ? (int64_t)atoll(e) : (int64_t)384; }();
-    if (edge || a.ksplit != 0 || a.colsum_dst != nullptr || a.K > max_k || (PRAD_GEMM_FOLD_K > 0 && a.K > PRAD_GEMM_FOLD_K) || tiles * a.batch < min_tiles) return false;  // (no fold on it)
+    if (edge || a.ksplit != 0 || a.shared_splits > 1 || a.colsum_dst != nullptr || a.K > max_k || (PRAD_GEMM_FOLD_K > 0 && a.K > PRAD_GEMM_FOLD_K) || tiles * a.batch < min_tiles) return false;  // (no fold on it)
     return epi == EPI_PLAIN || epi == EPI_ELEMENTWISE;
 }
 
@@ -832,9 +876,10 @@ template <typename T, int WT, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const GemmArgs<T>& a, bool edge, int epi, hipStream_t stream) {
     constexpr int BM = 32 * WT;
     const int tilesM = (int)((a.M + BM - 1) / BM), tilesN = (int)((a.N + BM - 1) / BM);
-    const unsigned splits = a.ksplit > 0 ? (unsigned)((a.K + a.ksplit - 1) / a.ksplit) : 1u;
+    const unsigned splits = (a.ksplit > 0 && a.shared_splits <= 1) ? (unsigned)((a.K + a.ksplit - 1) / a.ksplit) : 1u;
     const unsigned riders = a.colsum_dst != nullptr ? (unsigned)((a.colsum_cols + 63) / 64) : 0u;
     dim3 grid((unsigned)(tilesM * tilesN) + riders, (unsigned)a.batch, splits), block(GEMM_THREADS, 1, 1);
+    if (WT == 4 && a.shared_splits > 1) grid.x = (unsigned)(tilesM * tilesN) + (unsigned)a.shared_tiles * (unsigned)(a.shared_splits - 1);
     if constexpr (WT == 4 && sizeof(T) == 4) {
         if (gemm_thin_eligible<T>(a, edge, epi, (int64_t)tilesM * tilesN)) {
             if (epi == EPI_PLAIN) hipLaunchKernelGGL((gemm_thin_kernel<T, A_KC, B_KC, EPI_PLAIN>), grid, block, 0, stream, a, tilesM, tilesN);
@@ -969,6 +1014,27 @@ bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
     return t != TILE_128x128 && wgs >= 128 && wgs <= GEMM_SPLIT_MAX_TILES && K >= 32 * slab_depth(t, elem_size);
 }
 
+int gemm_shared_tiles_plan(int64_t M, int64_t N, int64_t K, int batch, int elem_size, int* shared_tiles) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_SHARED"); return !(e && e[0] == '0'); }();  // tuning aid
+    *shared_tiles = 0;
+    if (!enabled || batch != 1 || choose_tile(M, N, batch, false) != TILE_128x128) return 0;
+    if (gemm_split_factor(M, N, K, batch, elem_size) > 1) return 0;
+    constexpr int64_t SLOTS = 512;  // two workgroups of the 128 x 128 kernels per compute unit
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    // (fewer tiles than slots - 256 tiles, one per compute unit - were measured with every tile shared two ways: +2 %,
+    // the partial tiles' round trip eats what the second workgroup per compute unit gains; not done)
+    const int64_t rest = tiles % SLOTS;
+    if (tiles < SLOTS || rest == 0 || rest > SLOTS / 2) return 0;  // a last round that is at least half full is left alone
+    const int64_t bk = slab_depth(TILE_128x128, elem_size);
+    static const int64_t max_ways = [] { const char* e = getenv("PRAD_GEMM_SHARED_MAX_WAYS"); const int x = e ? atoi(e) : 0; return (int64_t)(x > 1 ? x : 4); }();
+    int64_t ways = SLOTS / rest;
+    if (ways > max_ways) ways = max_ways;
+    if (ways > K / (8 * bk)) ways = K / (8 * bk);  // at least eight slabs per workgroup
+    if (ways < 2) return 0;
+    *shared_tiles = (int)rest;
+    return (int)ways;
+}
+
 // Adds the partial results of a split product in split order and applies the epilogue.
 template <typename T>
 __global__ void __launch_bounds__(256) split_reduce_kernel(const GemmArgs<T> p, const T* __restrict__ ws, int splits) {
@@ -984,6 +1050,43 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const GemmArgs<T> p, 
         T* c = p.C + b * p.strideC + i * p.ldc + j;
         if (p.accumulate) v = *c + v;
         *c = v;
+    }
+}
+
+// Adds the partial blocks of the shared tiles of a launch (see gemm_shared_tiles_plan) in split order and applies the
+// epilogue.  One workgroup takes 16 rows of one tile, a thread one 16-byte vector of eight rows of them.
+template <typename T>
+__global__ void __launch_bounds__(256) shared_reduce_kernel(const GemmArgs<T> p, const int tilesM, const int tilesN) {
+    typedef typename Mfma<T>::Vec Vec;
+    constexpr int VEC = Mfma<T>::VEC, BM = 128, BN = 128, VPR = BN / VEC;  // vectors per tile row
+    const int tile = blockIdx.x / (BM / 16), strip = blockIdx.x % (BM / 16);
+    int tm, tn;
+    tile_of_workgroup(tile, tilesM, tilesN, tm, tn);
+    const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+    const int splits = p.shared_splits;
+    const T* __restrict__ ws = p.split_ws + (int64_t)tile * splits * (BM * BN);
+    for (int e = threadIdx.x; e < 16 * VPR; e += 256) {
+        const int il = strip * 16 + e / VPR, jl = (e % VPR) * VEC;
+        const int64_t i = row0 + il, j = col0 + jl;
+        if (i >= p.M || j >= p.N) continue;
+        Vec v = *reinterpret_cast<const Vec*>(ws + il * BN + jl);
+        for (int z = 1; z < splits; ++z) {
+            const Vec o = *reinterpret_cast<const Vec*>(ws + (int64_t)z * (BM * BN) + il * BN + jl);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) v[c] = v[c] + o[c];
+        }
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            if (j + c >= p.N) break;
+            T x = v[c];
+            if (p.bias != nullptr) x = x + p.bias[j + c];
+            if (p.Z != nullptr) p.Z[i * p.ldz + j + c] = x;
+            if (p.act_fwd != ACT_NONE) x = act_forward<T>(p.act_fwd, x, p.alpha);
+            if (p.act_bwd != ACT_NONE) x = x * act_derivative<T>(p.act_bwd, p.act_src[i * p.ld_act + j + c], p.alpha);
+            T* out = p.C + i * p.ldc + j + c;
+            if (p.accumulate) x = *out + x;
+            *out = x;
+        }
     }
 }
 
@@ -1049,7 +1152,21 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         return hipGetLastError();
     }
     const TileShape tile = choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr);
-    if (a.split_counters != nullptr && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
+    a.shared_tiles = 0; a.shared_splits = 0;
+    int shared_tiles = 0;
+    const int shared_ways = (tile == TILE_128x128 && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
+                             a.batch_inner <= 1 && a.colsum_dst == nullptr)
+                                ? gemm_shared_tiles_plan(a.M, a.N, a.K, a.batch, (int)sizeof(T), &shared_tiles) : 0;
+    if (shared_ways > 1) {
+        const int64_t bk = slab_depth(tile, (int)sizeof(T));
+        a.ksplit = ((a.K + shared_ways - 1) / shared_ways + bk - 1) / bk * bk;
+        a.shared_splits = (int)((a.K + a.ksplit - 1) / a.ksplit);
+        a.shared_tiles = shared_tiles;
+        a.zstrideA = a.transA ? a.ksplit * a.lda : a.ksplit;
+        a.zstrideB = a.transB ? a.ksplit : a.ksplit * a.ldb;
+        a.split_counters = nullptr;  // the shared tiles are reduced by a launch of their own
+        if (a.shared_splits < 2) { a.shared_splits = 0; a.shared_tiles = 0; a.ksplit = 0; }
+    } else if (a.split_counters != nullptr && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
         gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T))) {
         const int64_t bk = slab_depth(tile, (int)sizeof(T));
         a.ksplit = ((a.K + 1) / 2 + bk - 1) / bk * bk;
@@ -1059,7 +1176,13 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         a.split_counters = nullptr;
     }
     switch (tile) {
-        case TILE_128x128: return launch_tile<T, 4>(a, epi, stream);
+        case TILE_128x128: {
+            const hipError_t e = launch_tile<T, 4>(a, epi, stream);
+            if (e != hipSuccess || a.shared_splits <= 1) return e;
+            hipLaunchKernelGGL((shared_reduce_kernel<T>), dim3((unsigned)a.shared_tiles * 8u), dim3(256), 0, stream, a,
+                               (int)((a.M + 127) / 128), (int)((a.N + 127) / 128));
+            return hipGetLastError();
+        }
         case TILE_64x64: return launch_tile<T, 2>(a, epi, stream);
         default: return launch_tile<T, 1>(a, epi, stream);
     }
@@ -1090,7 +1213,8 @@ hipError_t launch_gemm_pair(const GemmArgs<T>& first_in, const GemmArgs<T>& seco
     const unsigned first = (unsigned)(tilesM1 * tilesN1);
     const unsigned riders = p2.colsum_dst != nullptr ? (unsigned)((p2.colsum_cols + 63) / 64) : 0u;
     const unsigned total = first + (unsigned)(tilesM2 * tilesN2) + riders;
-    if (total > 256u) return hipErrorNotSupported;
+    static const unsigned max_total = [] { const char* e = getenv("PRAD_GEMM_DUAL_MAX"); const int x = e ? atoi(e) : 0; return (unsigned)(x > 0 ? x : 512); }();  // tuning aid
+    if (total > max_total) return hipErrorNotSupported;
     const int epi1 = epilogue(p1);
     const bool edge1 = !vector_loads_ok(p1, epi1, 32), edge2 = !vector_loads_ok(p2, EPI_PLAIN, 32);
     const dim3 grid(total), block(GEMM_THREADS);

@@ -254,8 +254,12 @@ template <typename T>
 int32_t attach_split_workspace(GemmArgs<T>& a) {
     const int splits = gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T));
     const bool pairs = splits <= 1 && gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T));
-    if (splits <= 1 && !pairs) return PRAD_OK;
-    if (int32_t st = ensure_workspace((size_t)(pairs ? 2 : splits) * a.batch * a.M * a.N * sizeof(T))) return st;
+    int shared_tiles = 0;
+    const int shared = (splits <= 1 && !pairs) ? gemm_shared_tiles_plan(a.M, a.N, a.K, a.batch, (int)sizeof(T), &shared_tiles) : 0;
+    if (splits <= 1 && !pairs && shared <= 1) return PRAD_OK;
+    const size_t bytes = shared > 1 ? (size_t)shared_tiles * shared * 128 * 128 * sizeof(T)
+                                  : (size_t)(pairs ? 2 : splits) * a.batch * a.M * a.N * sizeof(T);
+    if (int32_t st = ensure_workspace(bytes)) return st;
     a.split_ws = static_cast<T*>(CUR_WORKSPACE);
     a.split_counters = g_ctx.counter;
     return PRAD_OK;

@@ -197,6 +197,36 @@ def test_full_size_whole_matrix_identities(gpu, dtype, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("trans", [(0, 0), (0, 1), (1, 0)])
+def test_shared_tiles_of_a_poorly_filled_last_round(gpu, oracle, dtype, trans):
+    """An output of 20 x 26 = 520 tiles of 128 x 128 over 512 workgroup slots: 8 tiles are split along K (several
+    workgroups per tile, reduced by the last to arrive) inside the same launch as the 512 unsplit ones.  Every entry is
+    held to its order-independent rounding bound against the product in double, rows sampled from every tile row
+    (split tiles and tiles that hang over the ragged edge included) to the parity bar against the oracle, and a second
+    launch into the same buffer adds onto the first (accumulate)."""
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    tA, tB = trans
+    M, K, N = 2500, 1056, 3300
+    X = seeded.uniform(17, 1, (K, M) if tA else (M, K), -1, 1, dtype)      # op(X) is M x K
+    Y = seeded.uniform(17, 2, (N, K) if tB else (K, N), -1, 1, dtype)      # op(Y) is K x N
+    bx, by, bc = DeviceBuffer.alloc(dtype, *X.shape), DeviceBuffer.alloc(dtype, *Y.shape), DeviceBuffer.alloc(dtype, M, N)
+    bx.upload(X); by.upload(Y)
+    check(lib.prad_gemm(tA, tB, bx.handle, by.handle, bc.handle, 0))
+    C = bc.download()
+    opX = np.ascontiguousarray(X.T) if tA else X
+    opY = np.ascontiguousarray(Y.T) if tB else Y
+    exact = opX.astype(np.float64) @ opY.astype(np.float64)
+    assert float(np.max(np.abs(C - exact) - dot_bound(opX, opY, dtype))) <= 0.0
+    rows = np.unique(np.concatenate([np.arange(3, M, 128), np.arange(M - 40, M, 7)]))
+    assert_parity(C[rows], oracle.matmul_fwd(np.ascontiguousarray(opX[rows]), opY, threads=16), dtype, "sampled rows")
+    check(lib.prad_gemm(tA, tB, bx.handle, by.handle, bc.handle, 1))
+    assert np.array_equal(bc.download(), C + C)
+    check(lib.prad_gemm(tA, tB, bx.handle, by.handle, bc.handle, 0))       # same bits on every run
+    assert np.array_equal(bc.download(), C)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_accumulating_backward(gpu, oracle, dtype):
     """dW += A^T.dC written by the product's own epilogue equals OperationBase.AccumulateGradient after Backward."""
     lib = _lib.load()
