@@ -265,6 +265,26 @@ int32_t prad_lstm_step_fwd(prad_buf_t h_prev, prad_buf_t Wh, prad_buf_t G, prad_
                            prad_buf_t h);
 int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, prad_buf_t c_prev, prad_buf_t tanh_c,
                            prad_buf_t dh_loss, prad_buf_t dc_in, prad_buf_t dG, prad_buf_t dc_prev, prad_buf_t dh_scratch);
+/* All time steps of a sequence in one launch each way.  The reference unrolls a sequence into one set of operation
+ * nodes per time step (src/RMAD/ComputationGraph.cs:808-849), each step's recurrent product being a
+ * MatrixMultiplyOperation (src/RMAD/MatrixMultiplyOperation.cs:50-126) that needs the step before it; these two run
+ * that loop inside one kernel, with the recurrent weight held in registers for the whole sequence and the time
+ * steps ordered by flags between the workgroups of a group of 16 batch rows.  Same values as `steps` calls of
+ * prad_lstm_step_fwd / prad_lstm_step_bwd up to the order of the sums along hidden (forward) and 4*hidden (backward).
+ *   forward:  G (steps*batch x 4*hidden) holds x_t . W_x + b for every step and becomes the activated gates;
+ *             C and Hs ((steps+1)*batch x hidden) hold c_0 / h_0 in their first batch rows and receive c_t / h_t in
+ *             the following blocks; tanh_c (steps*batch x hidden) receives tanh(c_t).
+ *   backward: dh_loss (steps*batch x hidden) is the loss gradient with respect to every h_t; dG receives the gradient of
+ *             the pre-activations of every step.  (dh_{-1} and dc_{-1}, which nothing consumes, are not formed.)
+ * Shapes: float only, batch a multiple of 16, hidden a multiple of 64 up to 512, and (batch/16)*(hidden/16) workgroups
+ * must fit the device at once (one per compute unit): prad_lstm_sequence_supported says 1 or 0 for a shape, and the
+ * two calls return PRAD_ERR_ARG for others.  Every wait inside the kernels is bounded (PRAD_LSTM_SPIN_LIMIT polls,
+ * default 2^22): if the device did not run the whole grid at once - other work held compute units for seconds -
+ * the kernels end early and the next call that waits for the stream returns PRAD_ERR_LAUNCH. */
+int32_t prad_lstm_sequence_supported(int32_t dtype, int64_t batch, int64_t hidden, int64_t steps);
+int32_t prad_lstm_sequence_fwd(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_buf_t Hs, prad_buf_t tanh_c, int64_t steps);
+int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, prad_buf_t tanh_c, prad_buf_t dh_loss, prad_buf_t dG,
+                               int64_t steps);
 /* Borrowed view of rows [row0, row0 + rows) of a 2-D buffer (a block of a fused weight, a time step of a
  * stacked sequence).  The view must be freed before its parent. */
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out);

@@ -102,6 +102,9 @@ SIGNATURES = {
     "prad_lstm_cell_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_lstm_step_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_lstm_step_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "prad_lstm_sequence_supported": (_i32, [_i32, _i64, _i64, _i64]),
+    "prad_lstm_sequence_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64]),
+    "prad_lstm_sequence_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64]),
     "prad_buf_view_rows": (_i32, [_vp, _i64, _i64, _vpp]),
     "prad_softmax_cce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "prad_graph_begin": (_i32, []),

@@ -312,6 +312,25 @@ template <typename T> hipError_t launch_lstm_cell_fwd(T* G, const T* c_prev, T* 
 template <typename T> hipError_t launch_lstm_cell_bwd(const T* gates, const T* c_prev, const T* tanh_c, const T* dh_a, const T* dh_b,
                                                       const T* dc_in, T* dG, T* dc_prev, int64_t rows, int64_t hidden, hipStream_t s);
 
+// A whole LSTM sequence in one launch each way (csrc/lstm_seq.hip; float).
+struct LstmSeqArgs {
+    const float* Wh;   // hidden x 4*hidden, gate blocks [i | f | g | o]
+    float* G;          // steps*batch x 4*hidden: pre-activations in, activated gates out (forward); gates in (backward)
+    float* C;          // (steps+1)*batch x hidden, block 0 = c_0
+    float* Hs;         // (steps+1)*batch x hidden, block 0 = h_0
+    float* TC;         // steps*batch x hidden: tanh(c_t)
+    const float* dHl;  // steps*batch x hidden: loss gradient with respect to h_t (backward)
+    float* dG;         // steps*batch x 4*hidden (backward)
+    float* partial;    // backward: lstm_seq_partial_bytes() of scratch
+    unsigned* flags;   // (batch/16) * (hidden/16) words
+    unsigned* abort_word;  // host-visible; a workgroup that gives up waiting writes 1
+    int batch, hidden, steps;
+    int spin_limit;
+};
+bool lstm_seq_eligible(int64_t batch, int64_t hidden, int64_t steps, int compute_units);
+size_t lstm_seq_partial_bytes(int64_t batch, int64_t hidden);
+hipError_t launch_lstm_seq(const LstmSeqArgs& a, bool backward, hipStream_t s);
+
 // MatrixMultiplyAndSum
 // S = samples of a batch (each with its own A, out, dOut, dA and P slices of dB; the P slices of B are shared).
 template <typename T> hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K,

@@ -1,0 +1,293 @@
+// A whole LSTM sequence in one launch each way (float): the recurrent product h_{t-1} . W_h of every time step
+// with the cell arithmetic, forward, and dh_t = dG_{t+1} . W_h^T with the cell's backward, in reverse.  The reference
+// unrolls a sequence into one MatrixMultiplyOperation (src/RMAD/MatrixMultiplyOperation.cs:50-126) plus Sigmoid / Tanh /
+// HadamardProduct / MatrixAdd nodes per time step (src/RMAD/ComputationGraph.cs:808-849); run as one launch per time step
+// and direction, the recurrence costs what 2 x T dependent launches cost (9 to 11 us each for 0.27 GFLOP), about 17 % of
+// the matrix cores.  Here the time loop is inside the kernel:
+//
+//   * the batch rows are cut into groups of 16 and the hidden units into blocks of 16; workgroup (r, c) owns rows
+//     [16 r, 16 r + 16) x units [16 c, 16 c + 16) for the whole sequence, one workgroup per compute unit;
+//   * its slice of W_h - the 64 columns [gate q][16 c .. 16 c + 16) forward, the same 64 columns as rows of W_h^T
+//     backward - is 128 KB for hidden = 512 and lives in the registers of its four wavefronts (128 per lane) for
+//     the whole sequence: W_h is read from memory once per launch instead of once per time step;
+//   * a time step depends on the other workgroups of its row group only (rows are independent): forward each
+//     workgroup publishes its 16 x 16 block of h_t and gathers the group's whole 16 x hidden block; backward each
+//     multiplies its own 16 x 64 block of dG_{t+1} by its rows of W_h^T into a partial dh for all hidden units,
+//     publishes it cut by consumer, and every workgroup adds the partial blocks meant for it in producer order
+//     (deterministic).  The exchange is per-producer flags, no atomics and no device-wide barrier: a producer writes
+//     its block with device-scope stores, waits for them (vmcnt(0)), then writes its flag; a consumer polls the flags
+//     of its group (one lane per producer) and then reads with device-scope loads.  One exchange round trip was
+//     measured at 3 us among 32 workgroups, against 9 to 11 us for a launch per step.
+//
+// Every wait is bounded: a workgroup that polls `spin_limit` times in vain (the grid is not co-resident, or
+// a peer gave up) writes the abort word, which the host checks at its next synchronisation, and leaves; every
+// other workgroup then leaves at its next wait.  The arithmetic per element is that of lstm_cell_fwd_kernel /
+// lstm_cell_bwd_kernel, statement for statement; only the order of the sums along K differs from the per-step kernels.
+#include "common.h"
+
+namespace prad {
+
+typedef float f4v __attribute__((ext_vector_type(4)));
+
+constexpr int SEQ_THREADS = 256;
+constexpr int SEQ_MAX_J = 32;  // hidden / 16 at most: hidden <= 512 (the slice of W_h must fit the registers)
+// More than half a compute unit's LDS per workgroup, so that no two workgroups of a grid share a compute unit while
+// another stands empty: the step time is that of the slowest workgroup.
+constexpr int SEQ_LDS_FLOATS = 21 * 1024;
+constexpr int SEQ_STAGE = 16 * (16 * SEQ_MAX_J / 4) / SEQ_THREADS;  // 16-byte vectors of a 16 x hidden block per thread, at most
+static_assert(16 * SEQ_MAX_J / 4 * 17 * 4 <= SEQ_LDS_FLOATS, "the staged block (rows padded to 17 vectors) must fit");
+
+// Keeps an LDS array the kernel does not otherwise need in the allocation.
+__device__ __forceinline__ void keep_allocated(float* lds) { asm volatile("" : : "v"(lds) : "memory"); }
+
+
+// 16 bytes at `base + byte_offset` with a device-scope load; `base` must be uniform over the wavefront (it becomes the
+// buffer descriptor; a descriptor that differs per lane would be executed lane by lane).
+__device__ __forceinline__ f4v coherent_load4(const float* base, int byte_offset) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, -1, 0x00020000);
+    return __builtin_bit_cast(f4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 16 /* sc1: device scope */));
+}
+__device__ __forceinline__ float coherent_load(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// All of this wavefront's stores so far are acknowledged (a device-scope store is written through).
+__device__ __forceinline__ void wait_for_stores() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+}
+
+// Waits until the `blocks` flags at `flags` have all reached `want` (called by every thread of the workgroup; the
+// first wavefront polls, one lane per flag).  Returns false - for the whole workgroup - when it gave up.
+__device__ __forceinline__ bool wait_for_group(const unsigned* flags, int blocks, unsigned want, unsigned* abort_word, int spin_limit,
+                                               int* verdict /* LDS */) {
+    if (threadIdx.x < 64) {
+        bool done = (int)threadIdx.x >= blocks;
+        int spins = 0;
+        bool ok = true;
+        while (true) {
+            if (!done) done = __hip_atomic_load(flags + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= want;
+            if (__all(done)) break;
+            ++spins;
+            if (spins > spin_limit || ((spins & 1023) == 0 && __hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0u)) {
+                ok = false;
+                break;
+            }
+        }
+        if (threadIdx.x == 0) {
+            if (!ok) __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            *verdict = ok ? 1 : 0;
+        }
+    }
+    __syncthreads();
+    return *verdict != 0;
+}
+
+// ---- forward ----------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_fwd_kernel(const LstmSeqArgs p) {
+    const int H = p.hidden, B = p.batch, NJ = H / 16, groups = B / 16, blocks = H / 16;
+    const int r = blockIdx.x % groups, c = blockIdx.x / groups;
+    const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;  // wavefront q multiplies for gate q
+    const int n = lane & 15, g = lane >> 4;
+    const int row = tid >> 4, u = tid & 15;                      // the element this thread finishes: (row, unit u)
+    __shared__ __attribute__((aligned(16))) float hblock[SEQ_LDS_FLOATS];  // h_{t-1} rows of the group, as MFMA fragments (16 x hidden used)
+    __shared__ float exch[4 * 16 * 16];                              // the four gates' products, [gate][row][unit]
+    __shared__ int verdict;
+    keep_allocated(hblock);
+
+    // W_h slice of this wavefront in registers: vector j of lane (n, g) = W_h[16 j + 4 g + i][q H + 16 c + n], i = 0..3
+    f4v w[SEQ_MAX_J];
+#pragma unroll
+    for (int j = 0; j < SEQ_MAX_J; ++j) {
+        if (j < NJ) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[j][i] = p.Wh[(int64_t)(16 * j + 4 * g + i) * 4 * H + q * H + 16 * c + n];
+        }
+    }
+    const int64_t own = (int64_t)(16 * r + row) * H + 16 * c + u;  // offset of (row, u) inside a batch x hidden block
+    float c_prev = p.C[own];
+    // the vectors of the group's 16 x hidden block this thread stages every step: where from (bytes) and where to (floats)
+    int stage_src[SEQ_STAGE], stage_dst[SEQ_STAGE];
+#pragma unroll
+    for (int e = 0; e < SEQ_STAGE; ++e) {
+        const int v = e * SEQ_THREADS + tid, vecs_per_row = H / 4;
+        const int m = v / vecs_per_row, kv = v % vecs_per_row;  // kv = 4 j + g'
+        stage_src[e] = v < 16 * vecs_per_row ? (m * H + kv * 4) * 4 : -1;
+        stage_dst[e] = (kv * 17 + m) * 4;
+    }
+    unsigned* my_flag = p.flags + r * blocks + c;
+    const unsigned* group_flags = p.flags + r * blocks;
+
+    for (int t = 0; t < p.steps; ++t) {
+        // pre-activations of this thread's four gates (x_t . W_x + b, from the launch before this one)
+        float* grow = p.G + (int64_t)(t * B + 16 * r + row) * 4 * H + 16 * c + u;
+        float pre[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) pre[k] = grow[k * H];
+        if (t > 0 && !wait_for_group(group_flags, blocks, (unsigned)t, p.abort_word, p.spin_limit, &verdict)) return;
+        // h_{t-1} rows of the group -> LDS in fragment order: vector (j, g') of row m = h[m][16 j + 4 g' .. + 3] at slot (4 j + g') * 17 + m
+        const float* hsrc = p.Hs + (int64_t)(t * B + 16 * r) * H;
+        f4v hv[SEQ_STAGE];
+#pragma unroll
+        for (int e = 0; e < SEQ_STAGE; ++e)
+            if (stage_src[e] >= 0) hv[e] = coherent_load4(hsrc, stage_src[e]);
+#pragma unroll
+        for (int e = 0; e < SEQ_STAGE; ++e)
+            if (stage_src[e] >= 0) *reinterpret_cast<f4v*>(&hblock[stage_dst[e]]) = hv[e];
+        __syncthreads();
+        f4v acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < SEQ_MAX_J; j += 2) {
+            if (j < NJ) {
+                const f4v a0 = *reinterpret_cast<const f4v*>(&hblock[((4 * j + g) * 17 + n) * 4]);
+                const f4v a1 = *reinterpret_cast<const f4v*>(&hblock[((4 * (j + 1) + g) * 17 + n) * 4]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[i], w[j][i], acc0, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[i], w[j + 1][i], acc1, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) exch[(q * 16 + 4 * g + rr) * 16 + n] = acc0[rr] + acc1[rr];
+        __syncthreads();
+        // the cell, as lstm_cell_fwd_kernel writes it
+        const float i_ = act_forward<float>(ACT_SIGMOID, pre[0] + exch[(0 * 16 + row) * 16 + u], 0.f);
+        const float f_ = act_forward<float>(ACT_SIGMOID, pre[1] + exch[(1 * 16 + row) * 16 + u], 0.f);
+        const float g_ = act_forward<float>(ACT_TANH, pre[2] + exch[(2 * 16 + row) * 16 + u], 0.f);
+        const float o_ = act_forward<float>(ACT_SIGMOID, pre[3] + exch[(3 * 16 + row) * 16 + u], 0.f);
+        grow[0] = i_; grow[H] = f_; grow[2 * H] = g_; grow[3 * H] = o_;
+        const float cn = (f_ * c_prev) + (i_ * g_);
+        const float tc = act_forward<float>(ACT_TANH, cn, 0.f);
+        const int64_t blk = (int64_t)B * H;
+        p.C[(t + 1) * blk + own] = cn;
+        p.TC[t * blk + own] = tc;
+        coherent_store(p.Hs + (t + 1) * blk + own, o_ * tc);
+        c_prev = cn;
+        wait_for_stores();
+        __syncthreads();  // every wavefront's h is in memory; also: hblock and exch are free again
+        if (tid == 0) __hip_atomic_store(my_flag, (unsigned)(t + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// ---- backward ---------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_bwd_kernel(const LstmSeqArgs p) {
+    const int H = p.hidden, B = p.batch, groups = B / 16, blocks = H / 16;
+    const int r = blockIdx.x % groups, c = blockIdx.x / groups;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int row = tid >> 4, u = tid & 15;
+    __shared__ __attribute__((aligned(16))) float dgblock[SEQ_LDS_FLOATS];  // this workgroup's dG block as fragments: vector (q, g', m) (16 x 64 used)
+    keep_allocated(dgblock);
+    __shared__ int verdict;
+
+    // Rows of W_h^T for this workgroup's 64 gate columns, spread over the wavefronts by output unit: wavefront wv
+    // produces partial dh for units [tile * 16, tile * 16 + 16), tile = wv + 4 y (y < blocks / 4); vector (y, q) of lane
+    // (n, g) = W_h[16 tile + n][q H + 16 c + 4 g + i], i = 0..3.
+    constexpr int MAX_Y = SEQ_MAX_J / 4;
+    const int NY = blocks / 4;
+    f4v w[MAX_Y][4];
+#pragma unroll
+    for (int y = 0; y < MAX_Y; ++y) {
+        if (y < NY) {
+            const int unit = 16 * (wv + 4 * y) + n;
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq) w[y][qq] = *reinterpret_cast<const f4v*>(p.Wh + (int64_t)unit * 4 * H + qq * H + 16 * c + 4 * g);
+        }
+    }
+    const int64_t own = (int64_t)(16 * r + row) * H + 16 * c + u;
+    const int64_t blk = (int64_t)B * H;
+    unsigned* my_flag = p.flags + r * blocks + c;
+    const unsigned* group_flags = p.flags + r * blocks;
+    float dc_next = 0.f;  // gradient of c_t arriving from step t + 1
+    float rec = 0.f;      // recurrent part of dh_t: sum over producers of their partial products
+
+    // what the cell's backward of one time step reads, loaded one step ahead (before the wait for the peers)
+    struct StepInputs { float i_, f_, g_, o_, tc, dhl, cp; };
+    auto load_step = [&](int t) {
+        const float* grow = p.G + (int64_t)(t * B + 16 * r + row) * 4 * H + 16 * c + u;
+        return StepInputs{grow[0], grow[H], grow[2 * H], grow[3 * H], p.TC[t * blk + own], p.dHl[t * blk + own], p.C[t * blk + own]};
+    };
+    StepInputs in = load_step(p.steps - 1);
+
+    for (int t = p.steps - 1, s = 0; t >= 0; --t, ++s) {
+        const float i_ = in.i_, f_ = in.f_, g_ = in.g_, o_ = in.o_, tc = in.tc, dhl = in.dhl, cp = in.cp;
+        // the cell's backward, as lstm_cell_bwd_kernel writes it (the last time step has no recurrent part and no dc_in)
+        const float dh = s == 0 ? dhl : dhl + rec;
+        const float d_o = dh * tc;
+        float dc = (dh * o_) * act_derivative<float>(ACT_TANH, tc, 0.f);
+        if (s > 0) dc = dc + dc_next;
+        const float d_i = dc * g_, d_g = dc * i_, d_f = dc * cp;
+        dc_next = dc * f_;
+        float dz[4];
+        dz[0] = d_i * act_derivative<float>(ACT_SIGMOID, i_, 0.f);
+        dz[1] = d_f * act_derivative<float>(ACT_SIGMOID, f_, 0.f);
+        dz[2] = d_g * act_derivative<float>(ACT_TANH, g_, 0.f);
+        dz[3] = d_o * act_derivative<float>(ACT_SIGMOID, o_, 0.f);
+        float* dgrow = p.dG + (int64_t)(t * B + 16 * r + row) * 4 * H + 16 * c + u;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) dgrow[k * H] = dz[k];
+        if (t == 0) break;
+        // this block of dG as the A operand: k = 16 q + u; lane (m, g') reads vector (q, g') = k in [16 q + 4 g', + 4)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) dgblock[((k * 4 + (u >> 2)) * 16 + row) * 4 + (u & 3)] = dz[k];
+        __syncthreads();
+        f4v a[4];
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq) a[qq] = *reinterpret_cast<const f4v*>(&dgblock[((qq * 4 + g) * 16 + n) * 4]);
+        // partial dh_{t-1}[rows][units of tile] = dG block . (W_h rows of the tile)^T, K = 64
+        float* pbase = p.partial + (int64_t)(s & 1) * groups * blocks * blocks * 256;
+#pragma unroll
+        for (int y = 0; y < MAX_Y; ++y) {
+            if (y < NY) {
+                f4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[qq][i], w[y][qq][i], acc, 0, 0, 0);
+                // consumer = the workgroup that owns the tile's units; blocks are laid out [group][consumer][producer][row][unit]
+                float* dst = pbase + ((int64_t)((r * blocks + (wv + 4 * y)) * blocks + c) * 16) * 16;
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) coherent_store(dst + (4 * g + rr) * 16 + n, acc[rr]);
+            }
+        }
+        wait_for_stores();
+        __syncthreads();  // (also: dgblock is free again)
+        if (tid == 0) __hip_atomic_store(my_flag, (unsigned)(s + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        in = load_step(t - 1);
+        if (!wait_for_group(group_flags, blocks, (unsigned)(s + 1), p.abort_word, p.spin_limit, &verdict)) return;
+        // the blocks meant for this workgroup, added in producer order
+        const float* src = pbase + ((int64_t)(r * blocks + c) * blocks * 16) * 16 + row * 16 + u;
+        float part[SEQ_MAX_J];
+#pragma unroll
+        for (int pr = 0; pr < SEQ_MAX_J; ++pr)
+            if (pr < blocks) part[pr] = coherent_load(src + pr * 256);
+        rec = 0.f;
+#pragma unroll
+        for (int pr = 0; pr < SEQ_MAX_J; ++pr)
+            if (pr < blocks) rec = rec + part[pr];
+    }
+}
+
+// Shapes the sequence kernels take: float, hidden a multiple of 64 up to 512 (the slice of W_h in registers, the
+// backward tiles four wavefronts wide), batch a multiple of 16, one workgroup per compute unit for the whole grid.
+bool lstm_seq_eligible(int64_t batch, int64_t hidden, int64_t steps, int compute_units) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_LSTM_SEQUENCE"); return !(e && e[0] == '0'); }();  // tuning aid
+    if (!enabled || steps < 1 || batch < 16 || batch % 16 != 0 || hidden < 64 || hidden % 64 != 0 || hidden > 16 * SEQ_MAX_J) return false;
+    return (batch / 16) * (hidden / 16) <= compute_units;
+}
+size_t lstm_seq_partial_bytes(int64_t batch, int64_t hidden) {
+    return (size_t)2 * (batch / 16) * (hidden / 16) * (hidden / 16) * 256 * sizeof(float);
+}
+
+hipError_t launch_lstm_seq(const LstmSeqArgs& a, bool backward, hipStream_t s) {
+    const unsigned grid = (unsigned)((a.batch / 16) * (a.hidden / 16));
+    hipError_t e = launch_fill_zero<float>(reinterpret_cast<float*>(a.flags), grid, s);  // unsigned zero == float zero bits
+    if (e != hipSuccess) return e;
+    if (backward) hipLaunchKernelGGL(lstm_seq_bwd_kernel, dim3(grid), dim3(SEQ_THREADS), 0, s, a);
+    else hipLaunchKernelGGL(lstm_seq_fwd_kernel, dim3(grid), dim3(SEQ_THREADS), 0, s, a);
+    return hipGetLastError();
+}
+
+}  // namespace prad

@@ -42,6 +42,7 @@ constexpr uint32_t BUF_MAGIC = 0x50524144u;  // "PRAD"
 constexpr size_t STAGING_CHUNK = (size_t)256 << 20;
 
 constexpr size_t COUNTER_BYTES = 4096;  // arrival counters: one per tile of a split or paired product, and a few
+constexpr size_t SEQ_FLAG_BYTES = 4096;  // one progress word per workgroup of an LSTM sequence kernel
 static_assert(COUNTER_BYTES >= GEMM_SPLIT_MAX_TILES * sizeof(unsigned), "a split product needs a counter per tile");
 
 // One stream, one kernel workspace (partial results of split products, clip moments, loss partial sums, tall
@@ -62,6 +63,11 @@ struct Context {
     bool recording = false;
     std::thread::id recorder;
     int live_graphs = 0;                    // recorded sequences not yet destroyed
+    // LSTM sequence kernels: the workgroups' progress flags, and a word in host memory that a workgroup writes
+    // when it gives up waiting for its peers (checked after every wait for the stream).
+    unsigned* seq_flags = nullptr;
+    unsigned* seq_abort = nullptr;          // hipHostMalloc'ed, also the address the kernels use
+    int compute_units = 0;
 };
 Context g_ctx;
 #define CUR_STREAM (g_ctx.stream)
@@ -117,6 +123,11 @@ inline int64_t count(prad_buf_t b) { return b->depth * b->rows * b->cols; }
 // Lock must be held.  Waits for everything enqueued on the library stream.
 int32_t sync_all() {
     if (g_ctx.stream) HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    if (g_ctx.seq_abort != nullptr && *static_cast<volatile unsigned*>(g_ctx.seq_abort) != 0u) {
+        *static_cast<volatile unsigned*>(g_ctx.seq_abort) = 0u;
+        return fail(PRAD_ERR_LAUNCH, "an LSTM sequence kernel gave up waiting for its peer workgroups (the device did not run its whole "
+                                     "grid at once); the buffers it was writing hold partial results");
+    }
     return PRAD_OK;
 }
 int32_t ensure_pinned(size_t bytes) {
@@ -457,6 +468,10 @@ int32_t prad_init(int32_t device_id) {
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.counter), COUNTER_BYTES), PRAD_ERR_ALLOC);
     HIP_TRY(hipMemset(g_ctx.counter, 0, COUNTER_BYTES), PRAD_ERR_ALLOC);
     if (int32_t st = init_static_scratch(device_id)) return st;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.seq_flags), SEQ_FLAG_BYTES), PRAD_ERR_ALLOC);
+    HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&g_ctx.seq_abort), 64, hipHostMallocDefault), PRAD_ERR_ALLOC);
+    *g_ctx.seq_abort = 0u;
+    g_ctx.compute_units = std::min<int>(prop.multiProcessorCount, (int)(SEQ_FLAG_BYTES / sizeof(unsigned)));
     g_ctx.recording = false;
     g_ctx.live_graphs = 0;
     g_ctx.device = device_id;
@@ -473,6 +488,9 @@ int32_t prad_shutdown(void) {
     if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
     free_retired_workspaces();
     if (g_ctx.counter) (void)hipFree(g_ctx.counter);
+    if (g_ctx.seq_flags) (void)hipFree(g_ctx.seq_flags);
+    if (g_ctx.seq_abort) (void)hipHostFree(g_ctx.seq_abort);
+    g_ctx.seq_flags = nullptr; g_ctx.seq_abort = nullptr;
     if (g_ctx.stream) (void)hipStreamDestroy(g_ctx.stream);
     g_ctx.workspace = nullptr; g_ctx.workspace_bytes = 0;
     g_ctx.counter = nullptr;
@@ -1381,6 +1399,73 @@ int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, 
     return gates->dtype == PRAD_F64
                ? lstm_step_bwd_t<double>(dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch)
                : lstm_step_bwd_t<float>(dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch);
+}
+
+// Whole-sequence kernels: shape checks shared by both directions.  `gates` is steps*batch x 4*hidden.
+static int32_t lstm_sequence_check(prad_buf_t Wh, prad_buf_t gates, int64_t steps, int64_t* batch, int64_t* hidden) {
+    if (steps < 1 || gates->depth != 1 || gates->rows % steps != 0 || gates->cols % 4 != 0)
+        return fail(PRAD_ERR_ARG, "gates must be steps*batch x 4*hidden");
+    *batch = gates->rows / steps;
+    *hidden = gates->cols / 4;
+    if (Wh->depth != 1 || Wh->rows != *hidden || Wh->cols != 4 * *hidden) return fail(PRAD_ERR_SHAPE, "recurrent weight must be hidden x 4*hidden");
+    if (gates->dtype != PRAD_F32 || !lstm_seq_eligible(*batch, *hidden, steps, g_ctx.compute_units))
+        return fail(PRAD_ERR_ARG, "the sequence kernels take float, batch a multiple of 16, hidden a multiple of 64 up to 512 and "
+                                  "(batch/16)*(hidden/16) <= %d workgroups; ask prad_lstm_sequence_supported first", g_ctx.compute_units);
+    return PRAD_OK;
+}
+static int lstm_spin_limit() {
+    const char* e = getenv("PRAD_LSTM_SPIN_LIMIT");  // polls of a peer's flag before a workgroup gives up
+    const long v = e ? atol(e) : 0;
+    return v > 0 ? (int)std::min<long>(v, 1L << 30) : (1 << 22);
+}
+static int32_t expect_rows(prad_buf_t b, int64_t rows, int64_t cols, const char* what) {
+    if (b->depth != 1 || b->rows != rows || b->cols != cols) return fail(PRAD_ERR_ARG, "%s must be %lld x %lld", what, (long long)rows, (long long)cols);
+    return PRAD_OK;
+}
+
+int32_t prad_lstm_sequence_supported(int32_t dtype, int64_t batch, int64_t hidden, int64_t steps) {
+    if (!g_ctx.initialized.load()) return 0;
+    return dtype == PRAD_F32 && lstm_seq_eligible(batch, hidden, steps, g_ctx.compute_units) ? 1 : 0;
+}
+
+int32_t prad_lstm_sequence_fwd(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_buf_t Hs, prad_buf_t tanh_c, int64_t steps) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(Wh); REQUIRE_BUF(G); REQUIRE_BUF(C); REQUIRE_BUF(Hs); REQUIRE_BUF(tanh_c);
+    if (int32_t st = same_dtype({Wh, G, C, Hs, tanh_c})) return st;
+    int64_t batch = 0, hidden = 0;
+    if (int32_t st = lstm_sequence_check(Wh, G, steps, &batch, &hidden)) return st;
+    if (int32_t st = expect_rows(C, (steps + 1) * batch, hidden, "C")) return st;
+    if (int32_t st = expect_rows(Hs, (steps + 1) * batch, hidden, "Hs")) return st;
+    if (int32_t st = expect_rows(tanh_c, steps * batch, hidden, "tanh_c")) return st;
+    ENQUEUE_LOCK();
+    LstmSeqArgs a{};
+    a.Wh = F(Wh); a.G = F(G); a.C = F(C); a.Hs = F(Hs); a.TC = F(tanh_c);
+    a.flags = g_ctx.seq_flags; a.abort_word = g_ctx.seq_abort;
+    a.batch = (int)batch; a.hidden = (int)hidden; a.steps = (int)steps; a.spin_limit = lstm_spin_limit();
+    HIP_TRY(launch_lstm_seq(a, false, CUR_STREAM), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
+int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, prad_buf_t tanh_c, prad_buf_t dh_loss, prad_buf_t dG,
+                               int64_t steps) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(Wh); REQUIRE_BUF(gates); REQUIRE_BUF(C); REQUIRE_BUF(tanh_c); REQUIRE_BUF(dh_loss); REQUIRE_BUF(dG);
+    if (int32_t st = same_dtype({Wh, gates, C, tanh_c, dh_loss, dG})) return st;
+    int64_t batch = 0, hidden = 0;
+    if (int32_t st = lstm_sequence_check(Wh, gates, steps, &batch, &hidden)) return st;
+    if (int32_t st = expect_rows(C, (steps + 1) * batch, hidden, "C")) return st;
+    if (int32_t st = expect_rows(tanh_c, steps * batch, hidden, "tanh_c")) return st;
+    if (int32_t st = expect_rows(dh_loss, steps * batch, hidden, "dh_loss")) return st;
+    if (int32_t st = expect_rows(dG, steps * batch, 4 * hidden, "dG")) return st;
+    ENQUEUE_LOCK();
+    if (int32_t st = ensure_workspace(lstm_seq_partial_bytes(batch, hidden))) return st;
+    LstmSeqArgs a{};
+    a.Wh = F(Wh); a.G = F(gates); a.C = F(C); a.TC = F(tanh_c); a.dHl = F(dh_loss); a.dG = F(dG);
+    a.partial = static_cast<float*>(CUR_WORKSPACE);
+    a.flags = g_ctx.seq_flags; a.abort_word = g_ctx.seq_abort;
+    a.batch = (int)batch; a.hidden = (int)hidden; a.steps = (int)steps; a.spin_limit = lstm_spin_limit();
+    HIP_TRY(launch_lstm_seq(a, true, CUR_STREAM), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
 }
 
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out) {

@@ -11,6 +11,10 @@ MatrixAdd nodes (examples/lstm/.../architecture/SelfAttentionMultiLayerLSTMArchi
   * backward keeps only dh_{t-1} = dG_t . W_h^T in the loop; dW = [X_all | H_prev_all]^T . dG_all, the bias
     gradient and dX_all are three large products / one column sum after it.
 
+  * where the shape allows it (float, batch a multiple of 16, hidden a multiple of 64 up to 512, one workgroup per
+    compute unit) the time loop itself runs inside one kernel each way (prad_lstm_sequence_fwd / _bwd), the recurrent
+    weight staying in registers for the whole sequence; otherwise one launch per time step each way.
+
 Every value equals the node-by-node evaluation up to the order of the floating-point sums.
 W is steps-independent: (input + hidden) x 4*hidden, gate blocks [i | f | g | o].
 """
@@ -19,7 +23,7 @@ import ctypes
 import numpy as np
 
 from . import _lib, seeded
-from .exceptions import check
+from .exceptions import ArgumentException, check
 from .matrix import DeviceBuffer
 from .operations import _ensure_initialized, handle_array
 from .optim import NeuralNetworkParameters
@@ -27,7 +31,7 @@ from .optim import NeuralNetworkParameters
 
 class LSTMLayer:
     def __init__(self, input_dim=256, hidden=512, batch=128, steps=64, dtype=np.float32, seed=seeded.DEFAULT_SEED,
-                 parameters=None, fused=True):
+                 parameters=None, fused=True, sequence=None):
         _ensure_initialized()
         self.lib = _lib.load()
         self.dtype = np.dtype(dtype)
@@ -68,11 +72,18 @@ class LSTMLayer:
         self.iteration = 0
         self._graph = None
         self.fused = fused   # one launch per time step each way (cell arithmetic as the recurrent product's epilogue)
+        # the whole time loop in one launch each way where the shape allows it (sequence=False: never; True: required)
+        supported = bool(self.lib.prad_lstm_sequence_supported(_lib.PRAD_F32 if self.dtype == np.float32 else _lib.PRAD_F64, B, H, T))
+        if sequence and not supported:
+            raise ArgumentException("the sequence kernels do not take this shape (float, batch % 16 == 0, hidden % 64 == 0, hidden <= 512)")
+        self.sequence = supported and fused if sequence is None else bool(sequence)
 
     def _enqueue_forward_backward(self):
         lib, T = self.lib, self.steps
         check(lib.prad_matmul_fwd_fused(self.X.handle, self.Wx.handle, self.b.handle, None, self.G.handle, _lib.ACT_NONE, 0.0))
-        for t in range(T):
+        if self.sequence:
+            check(lib.prad_lstm_sequence_fwd(self.Wh.handle, self.G.handle, self.C.handle, self.Hs.handle, self.TC.handle, T))
+        for t in range(0 if self.sequence else T):
             if self.fused:
                 check(lib.prad_lstm_step_fwd(self.H_t[t].handle, self.Wh.handle, self.G_t[t].handle, self.C_t[t].handle,
                                              self.C_t[t + 1].handle, self.TC_t[t].handle, self.H_t[t + 1].handle))
@@ -81,7 +92,9 @@ class LSTMLayer:
             check(lib.prad_lstm_cell_fwd(self.G_t[t].handle, self.C_t[t].handle, self.C_t[t + 1].handle, self.TC_t[t].handle,
                                          self.H_t[t + 1].handle))
         check(lib.prad_mse(self.H_out.handle, self.Y.handle, self.loss.handle, self.dHl.handle))   # loss and its gradient
-        for t in range(T - 1, -1, -1):
+        if self.sequence:
+            check(lib.prad_lstm_sequence_bwd(self.Wh.handle, self.G.handle, self.C.handle, self.TC.handle, self.dHl.handle, self.dG.handle, T))
+        for t in range(-1 if self.sequence else T - 1, -1, -1):
             last = t == T - 1
             rec, dc_in, dc_out = self.dh[t % 2], self.dc[t % 2], self.dc[(t + 1) % 2]
             if self.fused and not last:
@@ -96,7 +109,7 @@ class LSTMLayer:
             if not self.fused:
                 # dh_{t-1} = dG_t . W_h^T (formed for t = 0 too: MatrixMultiplyOperation.Backward always returns both gradients)
                 check(lib.prad_gemm(0, 1, self.dG_t[t].handle, self.Wh.handle, self.dh[(t + 1) % 2].handle, 0))
-        if self.fused:
+        if self.fused or self.sequence:
             check(lib.prad_gemm(0, 1, self.dG_t[0].handle, self.Wh.handle, self.dh[1].handle, 0))   # dh_{-1}, as above
         check(lib.prad_gemm(1, 0, self.X.handle, self.dG.handle, self.dWx.handle, 0))
         check(lib.prad_gemm(1, 0, self.H_prev_all.handle, self.dG.handle, self.dWh.handle, 0))

@@ -1,11 +1,14 @@
 """LSTM layer step (fused 4-gate weight, BPTT, MSE) against the oracle's node-by-node composition of the
 reference operations: MatrixMultiply on the concatenated [x_t | h_{t-1}], MatrixAddBroadcasting, Sigmoid, Tanh,
 HadamardProduct, MatrixAdd, MeanSquaredError, and their Backward methods in reverse order."""
+import os
+
 import numpy as np
 import pytest
 
 from conftest import assert_long_sum_parity, assert_parity, norm_err, strict_err
 from oracle import compose
+from parallelreverseautodiff_amd.exceptions import ArgumentException, InvalidOperationException
 from parallelreverseautodiff_amd.lstm import LSTMLayer
 
 pytestmark = pytest.mark.gpu
@@ -67,9 +70,67 @@ def test_one_launch_per_time_step_equals_product_plus_cell_kernels(gpu, dtype, c
     backward: on the product split along K) gives the bits of the product followed by the cell kernel; row counts
     that do not fill the tiles and a hidden size that takes the two-launch path (32) included."""
     I, H, B, T = cfg
-    a, b = LSTMLayer(I, H, B, T, dtype=dtype, fused=True), LSTMLayer(I, H, B, T, dtype=dtype, fused=False)
+    a, b = LSTMLayer(I, H, B, T, dtype=dtype, fused=True, sequence=False), LSTMLayer(I, H, B, T, dtype=dtype, fused=False, sequence=False)
     for step in range(2):
         a.step(); b.step()
         for name in ("G", "C", "Hs", "TC", "dG", "dX", "dW", "db", "W", "b", "loss"):
             assert np.array_equal(getattr(a, name).download(), getattr(b, name).download()), (name, step)
         assert np.array_equal(a.dh[1].download(), b.dh[1].download())
+
+
+@pytest.mark.parametrize("cfg", [(256, 512, 128, 5), (32, 64, 16, 6), (16, 256, 48, 4), (16, 128, 32, 1), (24, 448, 64, 3)])
+def test_whole_sequence_in_one_launch_matches_one_launch_per_time_step(gpu, cfg):
+    """The time loop inside one kernel each way (recurrent weight in registers, time steps ordered by flags between
+    workgroups) against one launch per time step: the same arithmetic per element, another order of the sums along
+    hidden (forward) and 4 * hidden (backward), so the float parity bar rather than bits.  One row group and several, a
+    single time step, hidden sizes that fill the register slice fully (512) and partly."""
+    I, H, B, T = cfg
+    a, b = LSTMLayer(I, H, B, T, dtype=np.float32, sequence=True), LSTMLayer(I, H, B, T, dtype=np.float32, sequence=False)
+    assert a.sequence and not b.sequence
+    # gradients are compared before clipping (which is discontinuous at the minimum clip value)
+    a.step(update=False); b.step(update=False)
+    for name in ("G", "C", "Hs", "TC", "dG", "dX", "dW", "db"):
+        assert_parity(getattr(a, name).download(), getattr(b, name).download(), np.float32, name)
+    assert abs(float(a.loss.download()[0, 0]) - float(b.loss.download()[0, 0])) <= 1e-5 * abs(float(b.loss.download()[0, 0]))
+    assert_parity(a.dh[1].download(), b.dh[1].download(), np.float32, "dh before the first step")
+
+
+def test_whole_sequence_kernels_are_deterministic_and_replay(gpu):
+    """Partial products are added in producer order, so two runs give the same bits, and so does a recorded step."""
+    I, H, B, T = 64, 256, 64, 8
+    a, b = LSTMLayer(I, H, B, T, dtype=np.float32, sequence=True), LSTMLayer(I, H, B, T, dtype=np.float32, sequence=True)
+    a.step(); b.step()
+    b.record()
+    for _ in range(3):
+        a.step()
+        b.replay()
+        gpu.Synchronize()
+        for x, y in ((a.W, b.W), (a.dW, b.dW), (a.dG, b.dG), (a.Hs, b.Hs), (a.loss, b.loss)):
+            assert np.array_equal(x.download(), y.download())
+    b.release()
+
+
+def test_whole_sequence_shapes_it_does_not_take(gpu):
+    assert not LSTMLayer(16, 32, 8, 4, dtype=np.float32).sequence       # batch and hidden too small: per-step launches
+    assert not LSTMLayer(16, 64, 16, 4, dtype=np.float64).sequence      # double: the weight slice does not fit the registers
+    with pytest.raises(ArgumentException):
+        LSTMLayer(16, 64, 24, 4, dtype=np.float32, sequence=True)       # batch not a multiple of 16
+    layer = LSTMLayer(16, 64, 16, 4, dtype=np.float32, sequence=False)
+    assert layer.lib.prad_lstm_sequence_fwd(layer.Wh.handle, layer.G.handle, layer.C.handle, layer.Hs.handle, layer.TC.handle, 3) != 0   # rows % steps
+
+
+def test_whole_sequence_kernel_gives_up_instead_of_waiting_forever(gpu):
+    """Every wait on a peer workgroup is bounded.  With a limit of one poll some workgroup gives up at once; all the
+    others then leave at their next wait, the kernels end normally, and the next wait for the stream reports it.  The
+    step after, with the default limit, is unaffected."""
+    layer, ref = LSTMLayer(64, 512, 128, 16, dtype=np.float32, sequence=True), LSTMLayer(64, 512, 128, 16, dtype=np.float32, sequence=True)
+    os.environ["PRAD_LSTM_SPIN_LIMIT"] = "1"
+    try:
+        layer.step(update=False)
+        with pytest.raises(InvalidOperationException, match="gave up waiting"):
+            gpu.Synchronize()
+    finally:
+        del os.environ["PRAD_LSTM_SPIN_LIMIT"]
+    layer.step(update=False); ref.step(update=False)
+    gpu.Synchronize()
+    assert np.array_equal(layer.dW.download(), ref.dW.download())
