@@ -39,6 +39,7 @@
 #include "common.h"
 
 #include <cstdlib>
+#include <type_traits>
 #include <cstring>
 
 namespace prad {
@@ -47,6 +48,9 @@ typedef double d4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef double d2_t __attribute__((ext_vector_type(2)));
 
+#ifndef PRAD_GEMM_MIX_WT
+#define PRAD_GEMM_MIX_WT 4  // largest tile (edge / 32) whose main loop issues its transfers between its MFMAs
+#endif
 #ifndef PRAD_GEMM_FOLD_K
 #define PRAD_GEMM_FOLD_K 512  // float accumulators are folded into a second set every so many elements of K (0: never)
 #endif
@@ -184,6 +188,25 @@ __device__ __forceinline__ void store_slab(T* __restrict__ s, const typename Mfm
             const int col = ((tid % S::TPR_MC) * VEC + S::mc_shift(k)) & (S::ROTATE_MC ? S::MN - 1 : ~0);
             *reinterpret_cast<Vec*>(s + k * S::LDM + col) = r[p];
         }
+    }
+}
+
+// The same transfers one 16-byte vector at a time (the main loop issues them between its MFMAs).
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::Vec load_vec_fast(const T* __restrict__ ubase, unsigned off) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ubase), 0, -1, 0x00020000);
+    return __builtin_bit_cast(typename Mfma<T>::Vec, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+}
+template <typename T, int WT, bool KC, int DIV = 1>
+__device__ __forceinline__ void store_vec(T* __restrict__ s, const typename Mfma<T>::Vec& r, int p, int tid) {
+    typedef Slab<T, WT, DIV> S;
+    typedef typename Mfma<T>::Vec Vec;
+    constexpr int VEC = Mfma<T>::VEC;
+    if (KC) *reinterpret_cast<Vec*>(s + (tid / S::TPR_KC + S::ROWS_KC * p) * S::LDK + (tid % S::TPR_KC) * VEC) = r;
+    else {
+        const int k = tid / S::TPR_MC + S::ROWS_MC * p;
+        const int col = ((tid % S::TPR_MC) * VEC + S::mc_shift(k)) & (S::ROTATE_MC ? S::MN - 1 : ~0);
+        *reinterpret_cast<Vec*>(s + k * S::LDM + col) = r;
     }
 }
 
@@ -350,6 +373,48 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         __builtin_amdgcn_s_setprio(0);
     };
 
+    // The same slab of MFMAs with the workgroup's other work issued in their shadow.  A wavefront that issues an MFMA
+    // is free to issue other instructions while the matrix core works on it (16 to 64 cycles), but the next MFMA has
+    // to wait for the core; so every MFMA is followed by at most a few of: the LDS reads of the next k step's
+    // fragments (read one step ahead into a second set of registers), and `op(o)`, o in [0, NOPS) - the caller's
+    // transfers for the slabs ahead (one 16-byte vector each: registers -> the other LDS stage, memory -> registers).
+    // Issued as blocks before and after the MFMAs of a slab, those transfers and the wait for the first fragments
+    // left the matrix core idle for a third of the time of a workgroup that has its compute unit to itself.
+    // The MFMAs run in the same order on the same operands as in `compute`: same bits.
+    constexpr int NM = WTM * WTN, NR = WTM + WTN, KSTEPS = BK / 4, SLOTS = KSTEPS * NM;
+    auto compute_mix = [&](const T* __restrict__ st, auto&& op, auto nops_) {
+        constexpr int NOPS = decltype(nops_)::value;
+        const T* __restrict__ sA = st;
+        const T* __restrict__ sB = st + SA;
+        T a[2][WTM], b[2][WTN];
+        auto read = [&](int s, int r) {
+            const int k = 4 * s + g;
+            if (r < WTM) a[s & 1][r] = slab_at<T, WT, A_KC, DIV>(sA, wm * WS + r * 16 + li, k);
+            else b[s & 1][r - WTM] = slab_at<T, WT, B_KC, DIV>(sB, wn * WS + (r - WTM) * 16 + li, k);
+        };
+#pragma unroll
+        for (int r = 0; r < NR; ++r) read(0, r);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                const int x = m / WTN, y = m % WTN;
+                acc[x][y] = MF::run(a[s & 1][x], b[s & 1][y], acc[x][y]);
+                if (s + 1 < KSTEPS) {
+#pragma unroll
+                    for (int r = m * NR / NM; r < (m + 1) * NR / NM; ++r) read(s + 1, r);
+                }
+                const int q = s * NM + m;
+#pragma unroll
+                for (int o = q * NOPS / SLOTS; o < (q + 1) * NOPS / SLOTS; ++o) op(o);
+                __builtin_amdgcn_sched_barrier(0);  // (the scheduler would gather the transfers into blocks again)
+            }
+        }
+        __builtin_amdgcn_s_setprio(0);
+    };
+
     if (SHORT) {
         // One LDS stage and no prefetch: the loads of a slab are hidden by the other workgroups of the compute unit.
         Vec ra[S::NVEC], rb[S::NVEC];
@@ -406,8 +471,32 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
             store_slab<T, WT, B_KC, DIV>(smem[0] + SA, rb0, tid);
             __syncthreads();
             int kt = 0;
+            constexpr int NV_ = S::NVEC;
+            constexpr bool MIX = WT <= PRAD_GEMM_MIX_WT;
+            constexpr bool MIX_DRAIN = MIX && WT <= 2;  // (the 128 x 128 kernels have no registers to spare for the extra code paths: hundreds of spills)
             for (; kt + 3 < ntiles; kt += 2) {
                 // LDS stage 0 holds slab kt, set 1 holds slab kt+1 (in flight), set 0 is free.
+                if (MIX) {
+                    // even o: vector o/2 of slab kt+1, registers -> stage 1 (free since the barrier); odd o: vector o/2 of slab kt+2, memory -> set 0
+                    const T* __restrict__ na = ua + (kt + 2) * stepa;
+                    const T* __restrict__ nb = ub + (kt + 2) * stepb;
+                    compute_mix(smem[0], [&](int o) {
+                        const int j = o >> 1;
+                        if (o & 1) { if (j < NV_) ra0[j] = load_vec_fast<T>(na, offa[j]); else rb0[j - NV_] = load_vec_fast<T>(nb, offb[j - NV_]); }
+                        else { if (j < NV_) store_vec<T, WT, A_KC, DIV>(smem[1], ra1[j], j, tid); else store_vec<T, WT, B_KC, DIV>(smem[1] + SA, rb1[j - NV_], j - NV_, tid); }
+                    }, std::integral_constant<int, 4 * NV_>{});
+                    __syncthreads();
+                    const T* __restrict__ ma = ua + (kt + 3) * stepa;
+                    const T* __restrict__ mb = ub + (kt + 3) * stepb;
+                    compute_mix(smem[1], [&](int o) {
+                        const int j = o >> 1;
+                        if (o & 1) { if (j < NV_) ra1[j] = load_vec_fast<T>(ma, offa[j]); else rb1[j - NV_] = load_vec_fast<T>(mb, offb[j - NV_]); }
+                        else { if (j < NV_) store_vec<T, WT, A_KC, DIV>(smem[0], ra0[j], j, tid); else store_vec<T, WT, B_KC, DIV>(smem[0] + SA, rb0[j - NV_], j - NV_, tid); }
+                    }, std::integral_constant<int, 4 * NV_>{});
+                    if (FOLD && ((kt + 2) & (FOLD_SLABS - 1)) == 0) fold();
+                    __syncthreads();
+                    continue;
+                }
                 load_slab_fast<T>(ra0, ua + (kt + 2) * stepa, offa);
                 load_slab_fast<T>(rb0, ub + (kt + 2) * stepb, offb);
                 compute(smem[0]);
@@ -423,6 +512,30 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                 __syncthreads();
             }
             // left: slab kt in stage 0, slab kt+1 (if any) in set 1, slab kt+2 (if any) still to be fetched
+            if (MIX_DRAIN && kt + 1 < ntiles) {
+                auto stores_1 = [&](int j) {  // slab kt+1: set 1 -> stage 1
+                    if (j < NV_) store_vec<T, WT, A_KC, DIV>(smem[1], ra1[j], j, tid); else store_vec<T, WT, B_KC, DIV>(smem[1] + SA, rb1[j - NV_], j - NV_, tid);
+                };
+                if (kt + 2 < ntiles) {
+                    const T* __restrict__ na = ua + (kt + 2) * stepa;
+                    const T* __restrict__ nb = ub + (kt + 2) * stepb;
+                    compute_mix(smem[0], [&](int o) {
+                        const int j = o >> 1;
+                        if (o & 1) { if (j < NV_) ra0[j] = load_vec_fast<T>(na, offa[j]); else rb0[j - NV_] = load_vec_fast<T>(nb, offb[j - NV_]); }
+                        else stores_1(j);
+                    }, std::integral_constant<int, 4 * NV_>{});
+                    __syncthreads();
+                    compute_mix(smem[1], [&](int j) {  // slab kt+2: set 0 -> stage 0
+                        if (j < NV_) store_vec<T, WT, A_KC, DIV>(smem[0], ra0[j], j, tid); else store_vec<T, WT, B_KC, DIV>(smem[0] + SA, rb0[j - NV_], j - NV_, tid);
+                    }, std::integral_constant<int, 2 * NV_>{});
+                    __syncthreads();
+                    compute_mix(smem[0], [](int) {}, std::integral_constant<int, 0>{});
+                } else {
+                    compute_mix(smem[0], stores_1, std::integral_constant<int, 2 * NV_>{});
+                    __syncthreads();
+                    compute_mix(smem[1], [](int) {}, std::integral_constant<int, 0>{});
+                }
+            } else {
             if (kt + 2 < ntiles) {
                 load_slab_fast<T>(ra0, ua + (kt + 2) * stepa, offa);
                 load_slab_fast<T>(rb0, ub + (kt + 2) * stepb, offb);
@@ -439,6 +552,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
                 store_slab<T, WT, B_KC, DIV>(smem[0] + SA, rb0, tid);
                 __syncthreads();
                 compute(smem[0]);
+            }
             }
         }
         if ((int64_t)ntiles * BK < K) {    // ragged end of K: one guarded slab through stage 1
@@ -999,14 +1113,14 @@ static int64_t slab_depth(TileShape t, int elem_size) {
 }
 
 // A product whose chosen tile yields between half and one and a half workgroups per compute unit leaves
-// workgroup slots empty (two fit per compute unit).  On the 64 x 64 and 32 x 32 tiles a lone workgroup has too
-// few MFMAs per fragment read to keep its compute unit busy, so with a K of 32 slabs or more such a product runs
-// as pairs of workgroups per tile (measured +4 to +20 %; at 16 slabs the exchange of the partial tiles costs
-// more than the pairing gains: -3 %).  The 128 x 128 tile keeps a compute unit busy on its own and only pays for
-// the exchange (-5 % at N = 2048 in double, -16 % on a 1024 x 4096 output): it never pairs.
-// PRAD_GEMM_PAIRS=0 switches pairing off.
+// workgroup slots empty (two fit per compute unit).  Such a product on the 64 x 64 or 32 x 32 tile, with a K of 32
+// slabs or more, can run as pairs of workgroups per tile, half of K each.  That paid (+4 to +20 %) as long as a lone
+// workgroup left the matrix core idle while it moved its slabs; since the main loop issues those transfers between its
+// MFMAs a lone workgroup is the faster one everywhere it was measured (N = 1024 in double: 40 us against 45 us paired;
+// 1536 x 1024 x 1024: 67 against 70), so pairing is off unless PRAD_GEMM_PAIRS=1 asks for it (a tuning aid; the
+// exchange is the one of the products split along K).  The 128 x 128 tile never pairs.
 bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
-    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_PAIRS"); return !(e && e[0] == '0'); }();
+    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_PAIRS"); return e && e[0] == '1'; }();
     if (!enabled || gemm_split_factor(M, N, K, batch, elem_size) > 1) return false;
     const TileShape t = choose_tile(M, N, batch, false);
     const int64_t e = t == TILE_128x128 ? 128 : t == TILE_64x64 ? 64 : 32;
