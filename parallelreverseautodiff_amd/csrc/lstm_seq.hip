@@ -98,12 +98,19 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_fwd_kernel(const Lstm
     keep_allocated(hblock);
 
     // W_h slice of this wavefront in registers: vector j of lane (n, g) = W_h[16 j + 4 g + i][q H + 16 c + n], i = 0..3
+    // (buffer loads: the lane's part of the address is one register for all 128 of them, the (j, i) part a scalar;
+    // with per-lane 64-bit addresses every load costs a dozen dependent instructions of a wavefront that runs alone)
     f4v w[SEQ_MAX_J];
+    {
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.Wh), 0, -1, 0x00020000);
+        const int lane_off = 4 * (4 * g * 4 * H + q * H + 16 * c + n);
 #pragma unroll
-    for (int j = 0; j < SEQ_MAX_J; ++j) {
-        if (j < NJ) {
+        for (int j = 0; j < SEQ_MAX_J; ++j) {
+            if (j < NJ) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) w[j][i] = p.Wh[(int64_t)(16 * j + 4 * g + i) * 4 * H + q * H + 16 * c + n];
+                for (int i = 0; i < 4; ++i)
+                    w[j][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_off, 4 * (16 * j + i) * 4 * H, 0));
+            }
         }
     }
     const int64_t own = (int64_t)(16 * r + row) * H + 16 * c + u;  // offset of (row, u) inside a batch x hidden block

@@ -613,3 +613,53 @@ def test_tall_products_of_few_slabs(gpu, oracle, dtype, shape):
     check(lib.prad_matmul_bwd_fused(dG_.handle, dA_.handle, dB_.handle, dAct.handle, None, 0, _lib.ACT_GELU, dS.handle, 0.0))
     plain = dX.download()[rows]
     assert_parity(dAct.download()[rows], oracle.gelu_bwd(np.ascontiguousarray(src[rows]), np.ascontiguousarray(plain)), dtype, "GELU' (.) dX")
+
+
+@pytest.mark.parametrize("shape", [(16384, 96, 288), (9000, 96, 96), (8200, 384, 96), (12001, 288, 96), (8192, 64, 384), (10000, 20, 48)])
+def test_rows_of_a_tall_product_do_not_depend_on_how_many_rows_there_are(gpu, oracle, shape):
+    """Row i of a product depends on row i of A only, and every kernel adds along K in the same order, whatever tile
+    the sizes select (a tall product runs on 128 x 128 tiles or the half-depth kernel, its first 4096 rows alone on
+    smaller ones): the first 4096 rows of the tall product equal the product of the first 4096 rows bit for bit - for
+    every epilogue (bias, pre-activation copy, activation, the upstream activation's derivative, accumulation), both
+    layouts of B, and a ragged last tile."""
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    dtype = np.float32
+    M, K, N = shape
+    head = 4096
+    A = seeded.uniform(43, 1, (M, K), -1, 1, dtype)
+    B = seeded.uniform(43, 2, (K, N), -1, 1, dtype)
+    Bt = np.ascontiguousarray(B.T)                                  # N x K: the operand of dC . W^T
+    bias = seeded.normal(43, 3, (1, N), 0.5, dtype)
+    src = seeded.normal(43, 4, (M, N), 1.0, dtype)
+    old = seeded.normal(43, 5, (M, N), 1.0, dtype)
+    up = lambda a: (lambda b: (b.upload(a), b)[1])(DeviceBuffer.alloc(dtype, *a.shape))
+    bA, bB, bBt, bbias, bsrc = up(A), up(B), up(Bt), up(bias), up(src)
+    hA, hsrc = bA.view_rows(0, head), bsrc.view_rows(0, head)
+
+    def both(call):
+        """Runs `call(A, act_src, out buffers...)` on all rows and on the first `head` rows; returns the downloads."""
+        full = [DeviceBuffer.alloc(dtype, M, N) for _ in range(2)]
+        part = [DeviceBuffer.alloc(dtype, head, N) for _ in range(2)]
+        full[1].upload(old); part[1].upload(old[:head])
+        call(bA, bsrc, *full)
+        call(hA, hsrc, *part)
+        return [f.download() for f in full], [q.download() for q in part]
+
+    # plain store, and accumulation into C
+    f, q = both(lambda a, s, c0, c1: (check(lib.prad_gemm(0, 0, a.handle, bB.handle, c0.handle, 0)),
+                                      check(lib.prad_gemm(0, 0, a.handle, bB.handle, c1.handle, 1))))
+    assert np.array_equal(f[0][:head], q[0]) and np.array_equal(f[1][:head], q[1])
+    assert_parity(f[0], A.astype(np.float64) @ B.astype(np.float64), dtype, "A.B", bound=dot_bound(A, B, dtype))
+    assert_parity(f[1], old + A.astype(np.float64) @ B.astype(np.float64), dtype, "C += A.B")
+    # B stored N x K (the layout of dA = dC . W^T)
+    f, q = both(lambda a, s, c0, c1: check(lib.prad_gemm(0, 1, a.handle, bBt.handle, c0.handle, 0)))
+    assert np.array_equal(f[0][:head], q[0])
+    assert_parity(f[0], A.astype(np.float64) @ B.astype(np.float64), dtype, "A.(B^T)^T", bound=dot_bound(A, B, dtype))
+    # bias, pre-activation copy, activation
+    f, q = both(lambda a, s, c0, c1: check(lib.prad_matmul_fwd_fused(a.handle, bB.handle, bbias.handle, c1.handle, c0.handle, _lib.ACT_TANH, 0.0)))
+    assert np.array_equal(f[0][:head], q[0]) and np.array_equal(f[1][:head], q[1])
+    assert_parity(f[0][-200:], oracle.tanh_fwd(np.ascontiguousarray(f[1][-200:])), dtype, "tanh(Z), last rows")
+    # the upstream activation's derivative on the way out (dA = (dC . W^T) (.) act'(src)): here "dC" = A, "W" = B^T
+    f, q = both(lambda a, s, c0, c1: check(lib.prad_matmul_bwd_fused(a.handle, s.handle, bBt.handle, c0.handle, None, 0, _lib.ACT_SIGMOID, s.handle, 0.0)))
+    assert np.array_equal(f[0][:head], q[0])
