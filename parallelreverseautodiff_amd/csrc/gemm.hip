@@ -302,10 +302,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         B += (int64_t)g_.bz * p.zstrideB;
     }
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int li = lane & 15, g = lane >> 4;
+    // (not const: they are formed again after the K loop, see there)
+    int tid = threadIdx.x;
+    int lane = tid & 63, wave = tid >> 6;
+    int wm = wave >> 1, wn = wave & 1;
+    int li = lane & 15, g = lane >> 4;
 
     Acc acc[WTM][WTN];
 #pragma unroll
@@ -589,6 +590,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         }
     }
 
+    // The epilogues use the thread's coordinates again.  Kept alive across the K loop, where every register is taken,
+    // they were spilled before it (five dwords per lane, 5 MiB of scratch writes per launch of the 128 x 128 kernel in
+    // double); formed anew from a thread index the compiler cannot tie to the one above, they cost a few instructions.
+    {
+        int t = threadIdx.x;
+        asm volatile("" : "+v"(t));
+        tid = t; lane = tid & 63; wave = tid >> 6; wm = wave >> 1; wn = wave & 1; li = lane & 15; g = lane >> 4;
+    }
     if (FOLD) {
 #pragma unroll
         for (int x = 0; x < WTM; ++x)

@@ -497,12 +497,13 @@ def test_both_gradients_in_one_launch(gpu, dtype, accumulate, shape):
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("shape", [(512, 2048, 512), (1024, 1024, 1024), (384, 2100, 500), (512, 4096, 512)])
-def test_products_run_as_workgroup_pairs(gpu, oracle, dtype, shape):
+def test_products_of_few_tiles_and_long_k(gpu, oracle, dtype, shape):
     """Shapes whose 64 x 64 or 32 x 32 tiles fill between half and one and a half of the chip's workgroup slots and
-    whose K holds at least 32 slabs (which of these shapes do depends on the element type) run with two workgroups
-    per tile (half of K each; the later one adds the other's partial tile):
-    parity with the oracle for the forward and both backward layouts, fused epilogue included, and the same
-    bits on every run, whichever workgroup of a pair arrives last."""
+    whose K holds at least 32 slabs (which of these shapes do depends on the element type): parity with the oracle
+    for the forward and both backward layouts, fused epilogue included, and the same bits on every run.  With
+    PRAD_GEMM_PAIRS=1 in the environment (test_workgroup_pairs_when_switched_on runs this test that way) they run
+    with two workgroups per tile, half of K each, the later one adding the other's partial tile: the same bits then
+    whichever workgroup of a pair arrives last."""
     from parallelreverseautodiff_amd.exceptions import check
     from parallelreverseautodiff_amd.matrix import DeviceBuffer
     lib = _lib.load()
@@ -663,3 +664,16 @@ def test_rows_of_a_tall_product_do_not_depend_on_how_many_rows_there_are(gpu, or
     # the upstream activation's derivative on the way out (dA = (dC . W^T) (.) act'(src)): here "dC" = A, "W" = B^T
     f, q = both(lambda a, s, c0, c1: check(lib.prad_matmul_bwd_fused(a.handle, s.handle, bBt.handle, c0.handle, None, 0, _lib.ACT_SIGMOID, s.handle, 0.0)))
     assert np.array_equal(f[0][:head], q[0])
+
+
+def test_workgroup_pairs_when_switched_on(gpu):
+    """Pairs of workgroups per tile are a tuning aid that is off by default (the library reads PRAD_GEMM_PAIRS once):
+    the test above runs again in a process of its own with the switch on."""
+    import os, subprocess, sys
+    env = dict(os.environ, PRAD_GEMM_PAIRS="1")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(root, "tests", "test_matmul_gpu.py"), "-q", "-x", "-m", "gpu",
+                        "-k", "test_products_of_few_tiles_and_long_k", "-p", "no:cacheprovider"],
+                       cwd=root, env=env, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
+    assert "8 passed" in r.stdout, r.stdout[-2000:]
