@@ -221,6 +221,11 @@ int gemm_split_factor(int64_t M, int64_t N, int64_t K, int batch, int elem_size)
 // Whether launch_gemm would run the product as pairs of workgroups per tile (needs GemmArgs::split_counters and
 // split_ws: 2 * batch * M * N elements).  In-kernel reduction uses at most GEMM_SPLIT_MAX_TILES counters.
 bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size);
+// A^T . B with a very long K and a small output, float: one pass over both operands (csrc/gemm_skinny.hip).  The launch
+// needs gemm_skinny_workspace_bytes() of split_ws (0: not such a product) and returns hipErrorNotSupported otherwise.
+bool gemm_skinny_eligible(const GemmArgs<float>& a);
+size_t gemm_skinny_workspace_bytes(const GemmArgs<float>& a);
+hipError_t launch_gemm_skinny(const GemmArgs<float>& a, hipStream_t stream);
 // A product on 128 x 128 tiles whose tile count leaves a poorly filled last round of workgroups (576 tiles over 512
 // workgroup slots: 64 tiles would run alone on 64 compute units while 192 sit idle) splits that many tiles along K
 // so that they fill the chip too.  Returns how many ways (0: none) and, through shared_tiles, how many tiles;

@@ -1222,6 +1222,12 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
     const int epi = a.tile_sums != nullptr ? EPI_TILE_SUM
                     : (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) ? EPI_ELEMENTWISE
                                                                                                              : EPI_PLAIN;
+    if constexpr (sizeof(T) == 4) {
+        if (epi == EPI_PLAIN) {
+            const hipError_t e = launch_gemm_skinny(a, stream);
+            if (e != hipErrorNotSupported) return e;
+        }
+    }
     if (a.nseg > 1) {
         // Sum of nseg products: one operand pair per split, partial results added in pair order.
         if (a.split_ws == nullptr || a.batch != 1 || epi == EPI_TILE_SUM) return hipErrorInvalidValue;

@@ -263,6 +263,14 @@ GemmArgs<T> plain_gemm(int transA, int transB, int64_t M, int64_t N, int64_t K, 
 // partial results; the workspace is grown here (lock held).
 template <typename T>
 int32_t attach_split_workspace(GemmArgs<T>& a) {
+    if constexpr (sizeof(T) == 4) {
+        if (const size_t bytes = gemm_skinny_workspace_bytes(a)) {  // one pass over both operands, partial outputs per workgroup
+            if (int32_t st = ensure_workspace(bytes)) return st;
+            a.split_ws = static_cast<T*>(CUR_WORKSPACE);
+            a.split_counters = g_ctx.counter;
+            return PRAD_OK;
+        }
+    }
     const int splits = gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T));
     const bool pairs = splits <= 1 && gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T));
     int shared_tiles = 0;
@@ -750,6 +758,12 @@ static int32_t matmul_bwd_locked(prad_buf_t dC, prad_buf_t A, prad_buf_t B, prad
                     (long long)dC->cols, (long long)A->rows, (long long)B->cols);
     Epilogue rider;
     if (dB != nullptr && dbias != nullptr && dC->rows < COLSUM_CHUNK_ROWS) { rider.colsum_src = dC; rider.colsum_dst = dbias; }
+    if (dB != nullptr && dbias != nullptr && rider.colsum_dst == nullptr && dC->dtype == PRAD_F32 && valid(dB) && valid(dbias)) {
+        // a tall dC whose weight gradient runs as one pass over A and dC: the column sums are taken in that pass
+        Epilogue tall;
+        tall.colsum_src = dC; tall.colsum_dst = dbias;
+        if (gemm_skinny_eligible(gemm_args_of<float>(1, 0, A, dC, dB, acc_dB, tall, false))) rider = tall;
+    }
     bool paired = false;
     // (one launch only if the first product's output is not an operand of the second: launched one after the other,
     // the second would read what the first wrote)

@@ -93,13 +93,14 @@ class SwinBlock:
         check(fused(self.H1.handle, w["W2"].handle, w["b2"].handle, None, self.Y2.handle, _lib.ACT_NONE, 0.0))
         check(lib.prad_mse(self.Y2.handle, self.T.handle, self.loss.handle, self.dY2.handle))   # loss and its gradient
         # ---- backward ----
-        check(lib.prad_add_broadcast_bwd_bias(self.dY2.handle, g["b2"].handle))
-        check(lib.prad_matmul_bwd_fused(self.dY2.handle, self.H1.handle, w["W2"].handle, self.dZ1.handle, g["W2"].handle, 0,
-                                        _lib.ACT_GELU, self.Z1.handle, 0.0))
-        check(lib.prad_add_broadcast_bwd_bias(self.dZ1.handle, g["b1"].handle))
-        check(lib.prad_matmul_bwd(self.dZ1.handle, self.Y1.handle, w["W1"].handle, self.dY1.handle, g["W1"].handle, 0, 0))
-        check(lib.prad_add_broadcast_bwd_bias(self.dY1.handle, g["bo"].handle))
-        check(lib.prad_matmul_bwd(self.dY1.handle, self.O.handle, w["Wo"].handle, self.dO.handle, g["Wo"].handle, 0, 0))
+        # (a layer's input, weight and bias gradients in one call: in float the weight gradient of these tall batches is
+        # one pass over the layer's input and dZ, and the bias gradient - the column sums of dZ - is taken in that pass)
+        check(lib.prad_matmul_bias_bwd(self.dY2.handle, self.H1.handle, w["W2"].handle, self.dZ1.handle, g["W2"].handle, g["b2"].handle, 0,
+                                       _lib.ACT_GELU, self.Z1.handle, 0.0))
+        check(lib.prad_matmul_bias_bwd(self.dZ1.handle, self.Y1.handle, w["W1"].handle, self.dY1.handle, g["W1"].handle, g["b1"].handle, 0,
+                                       _lib.ACT_NONE, None, 0.0))
+        check(lib.prad_matmul_bias_bwd(self.dY1.handle, self.O.handle, w["Wo"].handle, self.dO.handle, g["Wo"].handle, g["bo"].handle, 0,
+                                       _lib.ACT_NONE, None, 0.0))
         # dP = dO . V^T ; dV = P^T . dO
         self._all_heads(0, 1, wt, wt, hd, self.dO, 0, C, wt * C, hd, self.QKV, 2 * C, q3, wt * q3, hd, self.dP, 0, wt, wt * wt, hs)
         self._all_heads(1, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.dO, 0, C, wt * C, hd, self.dQKV, 2 * C, q3, wt * q3, hd)
@@ -107,8 +108,8 @@ class SwinBlock:
         # dQ = dS . K ; dK = dS^T . Q
         self._all_heads(0, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, C, q3, wt * q3, hd, self.dQKV, 0, q3, wt * q3, hd)
         self._all_heads(1, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, 0, q3, wt * q3, hd, self.dQKV, C, q3, wt * q3, hd)
-        check(lib.prad_add_broadcast_bwd_bias(self.dQKV.handle, g["bqkv"].handle))
-        check(lib.prad_matmul_bwd(self.dQKV.handle, self.X.handle, w["Wqkv"].handle, self.dX.handle, g["Wqkv"].handle, 0, 0))
+        check(lib.prad_matmul_bias_bwd(self.dQKV.handle, self.X.handle, w["Wqkv"].handle, self.dX.handle, g["Wqkv"].handle, g["bqkv"].handle, 0,
+                                       _lib.ACT_NONE, None, 0.0))
 
     def _enqueue_update(self, t):
         p, n = self.params, len(self.names)

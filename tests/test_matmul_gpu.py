@@ -677,3 +677,42 @@ def test_workgroup_pairs_when_switched_on(gpu):
                        cwd=root, env=env, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
     assert "8 passed" in r.stdout, r.stdout[-2000:]
+
+
+@pytest.mark.parametrize("shape", [(50176, 96, 288), (8192, 96, 96), (16384, 384, 96), (12288, 96, 384), (4096, 64, 320), (20000, 32, 48)])
+def test_weight_gradient_of_a_tall_batch_in_one_pass(gpu, oracle, shape):
+    """dB = A^T . dC in float for thousands of rows and a small output runs as one pass over A and dC (every workgroup
+    multiplies a range of rows into the whole output, a second launch adds the partial outputs in order), and the bias
+    gradient - the column sums of dC - is taken in the same pass when prad_matmul_bias_bwd asks for both.  Held against
+    the product and the sums in double, with and without accumulation into dB; the same bits on every run; the bias
+    gradient equal to the one of the call that asks for it alone."""
+    lib = _lib.load()
+    from parallelreverseautodiff_amd.exceptions import check
+    dtype = np.float32
+    K, M, N = shape                                   # K rows of the batch, M inputs, N outputs of the layer
+    A = seeded.uniform(47, 1, (K, M), -1, 1, dtype)
+    dC = seeded.normal(47, 2, (K, N), 1.0, dtype)
+    W = seeded.normal(47, 3, (M, N), 1.0, dtype)
+    old = seeded.normal(47, 4, (M, N), 1.0, dtype)
+    up = lambda a: (lambda b: (b.upload(a), b)[1])(DeviceBuffer.alloc(dtype, *a.shape))
+    bA, bdC, bW = up(A), up(dC), up(W)
+    ref = A.astype(np.float64).T @ dC.astype(np.float64)
+    ref_db = dC.astype(np.float64).sum(axis=0, keepdims=True)
+    first = None
+    for run in range(3):
+        dB, dBacc, db, db_alone = DeviceBuffer.alloc(dtype, M, N), up(old), DeviceBuffer.alloc(dtype, 1, N), DeviceBuffer.alloc(dtype, 1, N)
+        check(lib.prad_matmul_bias_bwd(bdC.handle, bA.handle, bW.handle, None, dB.handle, db.handle, 0, _lib.ACT_NONE, None, 0.0))
+        check(lib.prad_matmul_bwd(bdC.handle, bA.handle, bW.handle, None, dBacc.handle, 0, 1))
+        check(lib.prad_add_broadcast_bwd_bias(bdC.handle, db_alone.handle))
+        got = [x.download() for x in (dB, dBacc, db, db_alone)]
+        if first is None:
+            first = got
+        else:
+            for a, b in zip(first, got):
+                assert np.array_equal(a, b), "run %d differs from run 0" % run
+    # (thousands of float terms per entry: the bar of the long sums, see assert_long_sum_parity)
+    scale = np.sqrt(np.mean(ref ** 2))
+    assert np.max(np.abs(first[0] - ref)) <= 2e-5 * max(scale, np.max(np.abs(ref)) * 1e-3) + 1e-5 * np.max(np.abs(ref)), "dB"
+    assert np.max(np.abs(first[1] - (old + ref))) <= 2e-5 * np.max(np.abs(ref)), "dB accumulated"
+    assert_parity(first[2], ref_db.astype(dtype), dtype, "bias gradient")
+    assert np.array_equal(first[2], first[3])
