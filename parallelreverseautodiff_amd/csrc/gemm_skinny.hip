@@ -172,9 +172,10 @@ __global__ void __launch_bounds__(64 * WR * WC, WR * WC == 4 ? 2 : 1) gemm_skinn
 #pragma unroll
         for (int o = 0; o < NOPS; o += 2) transfer(o, c0, lds, c0, 0);  // set 0 -> stage 0
         __syncthreads();
-        // (every workgroup has an even number of slabs - see sk_plan - so the loop body holds no branch: a branch around
-        // a slab's MFMAs sends all accumulators through copies at every iteration)
-        for (int s = 0; s < nsl; s += 2) {
+        // (no branch inside the loop body: a branch around a slab's MFMAs sends all accumulators through copies at every
+        // iteration; an odd last slab is multiplied after the loop)
+        int s = 0;
+        for (; s + 1 < nsl; s += 2) {
             // stage 0 holds slab s, set 1 slab s+1; slab s+2 goes into set 0
             colsum(lds);
             compute(lds, [&](int o) { transfer(o, c1, lds + S::STAGE, c0, s + 2); });
@@ -183,6 +184,10 @@ __global__ void __launch_bounds__(64 * WR * WC, WR * WC == 4 ? 2 : 1) gemm_skinn
             colsum(lds + S::STAGE);
             compute(lds + S::STAGE, [&](int o) { transfer(o, c0, lds, c1, s + 3); });
             __syncthreads();
+        }
+        if (s < nsl) {
+            colsum(lds);
+            compute(lds, [](int) {});
         }
     }
     // this workgroup's partial output and column sums
@@ -207,51 +212,63 @@ __global__ void __launch_bounds__(64 * WR * WC, WR * WC == 4 ? 2 : 1) gemm_skinn
     }
 }
 
-// Adds the workgroups' partial outputs (and column sums) in a fixed order: eight threads per element each add every
-// eighth partial, in ascending order, eight loads in flight at a time, and their sums are added in thread order (one
+// Adds the workgroups' partial outputs (and column sums) in a fixed order: sixteen threads per element each add every
+// sixteenth partial, in ascending order, sixteen loads in flight at a time, and their sums are added in thread order (one
 // thread walking all partials of an element was a chain of some 250 dependent loads: 110 us).
-constexpr int SKR_WAYS = 8;
+constexpr int SKR_WAYS = 16, SKR_ELEMS = 256 / SKR_WAYS;
 __global__ void __launch_bounds__(256) skinny_reduce_kernel(const float* __restrict__ partial, const double* __restrict__ colsum_partial,
                                                             float* __restrict__ C, int64_t ldc, float* __restrict__ colsum_dst, int M, int N,
                                                             int parts, int accumulate) {
     __shared__ double red[256];
-    const int64_t total = (int64_t)M * N;
-    const int q = threadIdx.x / 32, e = threadIdx.x % 32;  // way, element of the block
-    const int64_t blocks_c = (total + 31) / 32;
+    const int64_t total = (int64_t)M * N;                                // (a multiple of 4: N is)
+    const int q = threadIdx.x / SKR_ELEMS, e = threadIdx.x % SKR_ELEMS;  // way; element of the block (four consecutive outputs)
+    const int64_t blocks_c = (total / 4 + SKR_ELEMS - 1) / SKR_ELEMS;
     if ((int64_t)blockIdx.x < blocks_c) {
-        const int64_t idx = (int64_t)blockIdx.x * 32 + e;
-        float v = 0.f;
+        const int64_t idx = ((int64_t)blockIdx.x * SKR_ELEMS + e) * 4;
+        f4s v = {0.f, 0.f, 0.f, 0.f};
         if (idx < total) {
-            int w = q;
-            for (; w + 7 * SKR_WAYS < parts; w += 8 * SKR_WAYS) {
-                float t[8];
+            for (int w = q; w < parts; w += 16 * SKR_WAYS) {
+                f4s t[16];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) t[u] = partial[(int64_t)(w + u * SKR_WAYS) * total + idx];
+                for (int u = 0; u < 16; ++u)
+                    t[u] = w + u * SKR_WAYS < parts ? *reinterpret_cast<const f4s*>(partial + (int64_t)(w + u * SKR_WAYS) * total + idx) : f4s{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int u = 0; u < 8; ++u) v = v + t[u];
+                for (int u = 0; u < 16; ++u)
+                    if (w + u * SKR_WAYS < parts) v = v + t[u];
             }
-            for (; w < parts; w += SKR_WAYS) v = v + partial[(int64_t)w * total + idx];
         }
-        red[threadIdx.x] = (double)v;
+        __shared__ f4s red4[256];
+        red4[threadIdx.x] = v;
         __syncthreads();
         if (q == 0 && idx < total) {
-            float sum = (float)red[e];
+            f4s sum = red4[e];
 #pragma unroll
-            for (int u = 1; u < SKR_WAYS; ++u) sum = sum + (float)red[u * 32 + e];
-            float* c = C + (idx / N) * ldc + idx % N;
-            *c = accumulate ? *c + sum : sum;
+            for (int u = 1; u < SKR_WAYS; ++u) sum = sum + red4[u * SKR_ELEMS + e];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float* c = C + ((idx + i) / N) * ldc + (idx + i) % N;
+                *c = accumulate ? *c + sum[i] : sum[i];
+            }
         }
     } else if (colsum_dst != nullptr) {
-        const int64_t j = ((int64_t)blockIdx.x - blocks_c) * 32 + e;
+        const int64_t j = ((int64_t)blockIdx.x - blocks_c) * SKR_ELEMS + e;
         double v = 0.0;
-        if (j < N)
-            for (int w = q; w < parts; w += SKR_WAYS) v += colsum_partial[(int64_t)w * N + j];
+        if (j < N) {
+            for (int w = q; w < parts; w += 16 * SKR_WAYS) {  // (sixteen loads in flight, added in ascending order)
+                double t[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) t[u] = w + u * SKR_WAYS < parts ? colsum_partial[(int64_t)(w + u * SKR_WAYS) * N + j] : 0.0;
+#pragma unroll
+                for (int u = 0; u < 16; ++u)
+                    if (w + u * SKR_WAYS < parts) v += t[u];
+            }
+        }
         red[threadIdx.x] = v;
         __syncthreads();
         if (q == 0 && j < N) {
             double sum = red[e];
 #pragma unroll
-            for (int u = 1; u < SKR_WAYS; ++u) sum += red[u * 32 + e];
+            for (int u = 1; u < SKR_WAYS; ++u) sum += red[u * SKR_ELEMS + e];
             colsum_dst[j] = (float)sum;
         }
     }
@@ -276,18 +293,17 @@ int sk_compute_units() {
     }();
     return v;
 }
-// Slabs per workgroup (an even number; K is a multiple of two slabs, so the last workgroup's share is even too) and workgroups.
+// Slabs per workgroup and workgroups.
 void sk_plan(int64_t K, int* slabs_per_wg, int* wgs) {
     const int64_t slabs = K / SK_KB;
-    int64_t per = (slabs + sk_compute_units() - 1) / sk_compute_units();
-    per += per & 1;
+    const int64_t per = (slabs + sk_compute_units() - 1) / sk_compute_units();
     *slabs_per_wg = (int)per;
     *wgs = (int)((slabs + per - 1) / per);
 }
 
 }  // namespace
 
-// Shapes that go to the kernel above: float, A^T . B with both operands row-major K x M and K x N, K a multiple of 32 and
+// Shapes that go to the kernel above: float, A^T . B with both operands row-major K x M and K x N, K a multiple of 16 and
 // at least 4096 rows, the output at most 96 x 384 or 384 x 96, every row 16-byte aligned, no epilogue but accumulation.
 // A column sum may ride along if it is that of the second operand.  PRAD_GEMM_SKINNY=0 switches it off (tuning aid).
 bool gemm_skinny_eligible(const GemmArgs<float>& a) {
@@ -295,7 +311,7 @@ bool gemm_skinny_eligible(const GemmArgs<float>& a) {
     static const int64_t min_k = [] { const char* e = getenv("PRAD_GEMM_SKINNY_MIN_K"); return e ? (int64_t)atoll(e) : (int64_t)4096; }();
     if (!enabled || !a.transA || a.transB || a.batch != 1 || a.batch_inner > 1 || a.nseg > 1 || a.tile_sums != nullptr) return false;
     if (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) return false;
-    if (a.K < min_k || a.K % (2 * SK_KB) != 0 || a.M < 16 || a.N < 16 || a.M % 4 != 0 || a.N % 4 != 0 || sk_class_of(a.M, a.N) < 0) return false;
+    if (a.K < min_k || a.K % SK_KB != 0 || a.M < 16 || a.N < 16 || a.M % 4 != 0 || a.N % 4 != 0 || sk_class_of(a.M, a.N) < 0) return false;
     if (a.lda % 4 != 0 || a.ldb % 4 != 0 || reinterpret_cast<uintptr_t>(a.A) % 16 != 0 || reinterpret_cast<uintptr_t>(a.B) % 16 != 0) return false;
     if (a.lda >= (1 << 20) || a.ldb >= (1 << 20)) return false;  // (byte offsets inside a slab are kept in 32 bits)
     if (a.colsum_dst != nullptr && (a.colsum_src != a.B || a.colsum_rows != a.K || a.colsum_cols != a.N)) return false;
@@ -328,7 +344,7 @@ hipError_t launch_gemm_skinny(const GemmArgs<float>& a, hipStream_t stream) {
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int64_t blocks = ((int64_t)a.M * a.N + 31) / 32 + (a.colsum_dst != nullptr ? (a.N + 31) / 32 : 0);
+    const int64_t blocks = ((int64_t)a.M * a.N / 4 + SKR_ELEMS - 1) / SKR_ELEMS + (a.colsum_dst != nullptr ? (a.N + SKR_ELEMS - 1) / SKR_ELEMS : 0);
     hipLaunchKernelGGL(skinny_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, k.partial, k.colsum_partial, a.C, a.ldc,
                        a.colsum_dst, (int)a.M, (int)a.N, wgs, a.accumulate);
     return hipGetLastError();
