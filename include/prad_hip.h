@@ -285,6 +285,17 @@ int32_t prad_lstm_sequence_supported(int32_t dtype, int64_t batch, int64_t hidde
 int32_t prad_lstm_sequence_fwd(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_buf_t Hs, prad_buf_t tanh_c, int64_t steps);
 int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, prad_buf_t tanh_c, prad_buf_t dh_loss, prad_buf_t dG,
                                int64_t steps);
+/* Windowed self-attention of a block, forward, in one launch: per window w and head h,
+ * S = Q_wh . K_wh^T * scale, P = softmax rows(S), O_wh = P . V_wh - the nodes MatrixMultiply, MatrixMultiplyScalar, Softmax,
+ * MatrixMultiply of examples/swin/SwinExample/SwinTransformerTools.cs:348-399 (src/RMAD/MatrixMultiplyOperation.cs:50-86,
+ * src/RMAD/SoftmaxOperation.cs:45-110).  QKV is (windows*tokens) x (3*heads*head_dim), rows window-major, columns
+ * [Q | K | V] with a head's head_dim columns inside each; P (heads*windows*tokens x tokens, head-major: what the backward
+ * pass reads) and O ((windows*tokens) x (heads*head_dim)) are written; the scores themselves never reach memory.  Same
+ * values as prad_gemm_strided_batched_2d_f32 + prad_softmax_scaled_fwd + prad_gemm_strided_batched_2d_f32 up to the order
+ * of the sums along head_dim.  Float, head_dim 32, at most 64 tokens per window: prad_window_attention_supported says
+ * 1 or 0, the call returns PRAD_ERR_ARG for other shapes. */
+int32_t prad_window_attention_supported(int32_t dtype, int64_t tokens, int64_t head_dim);
+int32_t prad_window_attention_fwd(prad_buf_t QKV, prad_buf_t P, prad_buf_t O, int64_t windows, int64_t heads, int64_t tokens, double scale);
 /* Borrowed view of rows [row0, row0 + rows) of a 2-D buffer (a block of a fused weight, a time step of a
  * stacked sequence).  The view must be freed before its parent. */
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out);

@@ -1,0 +1,176 @@
+// Windowed self-attention of one block, forward, per window and head in one launch (float, head dimension 32, up to 64
+// tokens per window): S = Q . K^T (MatrixMultiplyOperation, src/RMAD/MatrixMultiplyOperation.cs:50-86), scaled
+// (MatrixMultiplyScalarOperation), P = softmax rows (src/RMAD/SoftmaxOperation.cs:45-110), O = P . V - the node sequence
+// of examples/swin/SwinExample/SwinTransformerTools.cs:348-399.  As separate launches the 49 x 49 scores of 9216
+// windows x heads go to memory and back twice (two products of K = 32 and 49 at 26 us each and a softmax pass at 25 us,
+// all bound by that traffic).  Here one wavefront takes one (window, head): the scores stay in its accumulators and its
+// LDS tile, only P - which the backward pass needs - is written, and Q, K, V are read once.
+//
+//   * Q and K fragments come straight from memory: lane (i, g) of a 16 x 16 x 4 MFMA holds k = 8 g .. 8 g + 7 of its
+//     row (two 16-byte loads; MFMA step s multiplies the k's {8 g + s}: a permutation of the sum along k, the same for
+//     both operands), so a row's 128 bytes are read whole by four lanes;
+//   * the 4 x 4 tiles of S are parked in an LDS tile (pitch 65), lane r < tokens takes row r through the softmax exactly
+//     as softmax_fwd_rows_kernel does (scale, maximum, exp, sum in ascending column order, divide), columns past the
+//     window become zeros;
+//   * P leaves as the contiguous tokens x tokens block it is in memory, and feeds the second product as the A operand
+//     from the same tile; V fragments were fetched at the start.
+#include "common.h"
+
+#include <cstdlib>
+
+namespace prad {
+
+namespace {
+
+typedef float f4a __attribute__((ext_vector_type(4)));
+constexpr int ATT_HD = 32;      // head dimension
+constexpr int ATT_PITCH = 65;   // LDS tile pitch (odd: a lane walking its row and 16 lanes reading a column meet no conflicts)
+constexpr int ATT_WAVES = 4;
+
+struct AttArgs {
+    const float* QKV;  // tokens_total x (3 * heads * 32): [Q | K | V], a head's 32 columns inside each
+    float* P;          // [head][window][tokens][tokens]
+    float* O;          // tokens_total x (heads * 32)
+    int windows, heads, tokens;
+    float scale;
+};
+
+__device__ __forceinline__ float att_exp(float x) { return __expf(x); }
+
+__global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel(const AttArgs p) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int li = lane & 15, g = lane >> 4;
+    const int64_t pair = (int64_t)blockIdx.x * ATT_WAVES + wave;  // (window, head), heads innermost
+    __shared__ float tiles[ATT_WAVES][64 * ATT_PITCH];
+    if (pair >= (int64_t)p.windows * p.heads) return;
+    const int w = (int)(pair / p.heads), h = (int)(pair % p.heads);
+    const int wt = p.tokens, C = p.heads * ATT_HD, ld = 3 * C;
+    float* __restrict__ tile = tiles[wave];
+    const float* __restrict__ Q = p.QKV + (int64_t)w * wt * ld + h * ATT_HD;
+    const float* __restrict__ K = Q + C;
+    const float* __restrict__ V = Q + 2 * C;
+
+    // fragments of Q and K: row 16 x + li (rows past the window: the last row again, never stored), k = 8 g .. 8 g + 7
+    f4a qf[4][2], kf[4][2];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        const int row = min(16 * x + li, wt - 1);
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            qf[x][v] = *reinterpret_cast<const f4a*>(Q + (int64_t)row * ld + 8 * g + 4 * v);
+            kf[x][v] = *reinterpret_cast<const f4a*>(K + (int64_t)row * ld + 8 * g + 4 * v);
+        }
+    }
+    // fragments of V for the second product: token 4 s + g (clamped: P is zero there), column 16 y + li
+    constexpr int MAX_STEPS = 16;
+    float vf[MAX_STEPS][2];
+#pragma unroll
+    for (int s = 0; s < MAX_STEPS; ++s) {
+        const int tok = min(4 * s + g, wt - 1);
+#pragma unroll
+        for (int y = 0; y < 2; ++y) vf[s][y] = V[(int64_t)tok * ld + 16 * y + li];
+    }
+
+    // S = Q . K^T
+    f4a acc[4][4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int y = 0; y < 4; ++y) acc[x][y] = f4a{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 4; ++y) acc[x][y] = __builtin_amdgcn_mfma_f32_16x16x4f32(qf[x][s >> 2][s & 3], kf[y][s >> 2][s & 3], acc[x][y], 0, 0, 0);
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int y = 0; y < 4; ++y)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tile[(16 * x + 4 * g + r) * ATT_PITCH + 16 * y + li] = acc[x][y][r];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // softmax of row `lane` (the arithmetic of softmax_fwd_rows_kernel); the columns past the window become zeros
+    {
+        float* __restrict__ row = tile + lane * ATT_PITCH;
+        float v[64];
+#pragma unroll
+        for (int j = 0; j < 64; ++j) v[j] = j < wt ? row[j] * p.scale : -INFINITY;
+        float m = v[0];
+#pragma unroll
+        for (int j = 1; j < 64; ++j) m = v[j] > m ? v[j] : m;
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            v[j] = j < wt ? att_exp(v[j] - m) : 0.f;
+            sum = sum + v[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 64; ++j) row[j] = j < wt ? v[j] / sum : 0.f;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // P leaves as one contiguous block
+    {
+        float* __restrict__ dst = p.P + ((int64_t)h * p.windows + w) * wt * wt;
+        int r = lane / wt, c = lane % wt;  // element lane + 64 i
+        const int dr = 64 / wt, dc = 64 % wt;
+        for (int e = lane; e < wt * wt; e += 64) {
+            dst[e] = tile[r * ATT_PITCH + c];
+            r += dr; c += dc;
+            if (c >= wt) { c -= wt; ++r; }
+        }
+    }
+
+    // O = P . V: rows 16 x + li of P from the tile, k = token
+    f4a out[4][2];
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int y = 0; y < 2; ++y) out[x][y] = f4a{0.f, 0.f, 0.f, 0.f};
+    // (all 16 steps whatever the window: P is zero past it, and a branch per step would send the accumulators through copies)
+#pragma unroll
+    for (int s = 0; s < MAX_STEPS; ++s) {
+        float a[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) a[x] = tile[(16 * x + li) * ATT_PITCH + 4 * s + g];
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 2; ++y) out[x][y] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[x], vf[s][y], out[x][y], 0, 0, 0);
+    }
+    float* __restrict__ O = p.O + (int64_t)w * wt * C + h * ATT_HD;
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 16 * x + 4 * g + r;
+            if (row < wt) {
+#pragma unroll
+                for (int y = 0; y < 2; ++y) O[(int64_t)row * C + 16 * y + li] = out[x][y][r];
+            }
+        }
+}
+
+}  // namespace
+
+bool window_attention_supported(int64_t tokens, int64_t head_dim) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_ATTENTION_FUSED"); return !(e && e[0] == '0'); }();  // tuning aid
+    return enabled && head_dim == ATT_HD && tokens >= 1 && tokens <= 64;
+}
+
+hipError_t launch_window_attention_fwd(const float* QKV, float* P, float* O, int64_t windows, int64_t heads, int64_t tokens, float scale,
+                                       hipStream_t stream) {
+    if (!window_attention_supported(tokens, ATT_HD) || reinterpret_cast<uintptr_t>(QKV) % 16 != 0) return hipErrorNotSupported;
+    AttArgs a{QKV, P, O, (int)windows, (int)heads, (int)tokens, scale};
+    const int64_t pairs = windows * heads;
+    hipLaunchKernelGGL(window_attention_fwd_kernel, dim3((unsigned)((pairs + ATT_WAVES - 1) / ATT_WAVES)), dim3(64 * ATT_WAVES), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace prad

@@ -336,6 +336,11 @@ bool lstm_seq_eligible(int64_t batch, int64_t hidden, int64_t steps, int compute
 size_t lstm_seq_partial_bytes(int64_t batch, int64_t hidden);
 hipError_t launch_lstm_seq(const LstmSeqArgs& a, bool backward, hipStream_t s);
 
+// Windowed self-attention, forward, one launch (csrc/attention.hip; float, head dimension 32, <= 64 tokens per window)
+bool window_attention_supported(int64_t tokens, int64_t head_dim);
+hipError_t launch_window_attention_fwd(const float* QKV, float* P, float* O, int64_t windows, int64_t heads, int64_t tokens, float scale,
+                                       hipStream_t stream);
+
 // MatrixMultiplyAndSum
 // S = samples of a batch (each with its own A, out, dOut, dA and P slices of dB; the P slices of B are shared).
 template <typename T> hipError_t launch_matmul_sum_fwd(const T* A, const T* B, T* out, double* workspace, int64_t M, int64_t K,

@@ -1482,6 +1482,27 @@ int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, pr
     return PRAD_OK;
 }
 
+int32_t prad_window_attention_supported(int32_t dtype, int64_t tokens, int64_t head_dim) {
+    return dtype == PRAD_F32 && window_attention_supported(tokens, head_dim) ? 1 : 0;
+}
+
+int32_t prad_window_attention_fwd(prad_buf_t QKV, prad_buf_t P, prad_buf_t O, int64_t windows, int64_t heads, int64_t tokens, double scale) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(QKV); REQUIRE_BUF(P); REQUIRE_BUF(O);
+    if (int32_t st = same_dtype({QKV, P, O})) return st;
+    if (windows < 1 || heads < 1 || tokens < 1 || QKV->depth != 1 || QKV->rows != windows * tokens || QKV->cols % (3 * heads) != 0)
+        return fail(PRAD_ERR_ARG, "QKV must be (windows*tokens) x (3*heads*head_dim)");
+    const int64_t head_dim = QKV->cols / (3 * heads);
+    if (QKV->dtype != PRAD_F32 || !window_attention_supported(tokens, head_dim))
+        return fail(PRAD_ERR_ARG, "the one-launch attention takes float, head dimension 32 and at most 64 tokens per window; ask "
+                                  "prad_window_attention_supported first");
+    if (int32_t st = expect_rows(P, heads * windows * tokens, tokens, "P")) return st;
+    if (int32_t st = expect_rows(O, windows * tokens, heads * head_dim, "O")) return st;
+    ENQUEUE_LOCK();
+    HIP_TRY(launch_window_attention_fwd(F(QKV), F(P), F(O), windows, heads, tokens, (float)scale, CUR_STREAM), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out) {
     REQUIRE_INIT();
     REQUIRE_BUF(parent);

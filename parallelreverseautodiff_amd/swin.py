@@ -25,7 +25,7 @@ from .optim import NeuralNetworkParameters
 
 class SwinBlock:
     def __init__(self, images=16, side=56, window=7, embed=96, heads=3, mlp_ratio=4, dtype=np.float32,
-                 seed=seeded.DEFAULT_SEED, parameters=None):
+                 seed=seeded.DEFAULT_SEED, parameters=None, fused_attention=None):
         _ensure_initialized()
         self.lib = _lib.load()
         self.dtype = np.dtype(dtype)
@@ -65,6 +65,8 @@ class SwinBlock:
         self.scale = 1.0 / float(np.sqrt(self.hd))
         self.iteration = 0
         self._graph = None
+        supported = bool(self.lib.prad_window_attention_supported(_lib.PRAD_F32 if self.dtype == np.float32 else _lib.PRAD_F64, self.wt, self.hd))
+        self.fused_attention = supported if fused_attention is None else bool(fused_attention) and supported
         self._batched = (self.lib.prad_gemm_strided_batched_2d_f64 if self.dtype == np.float64
                          else self.lib.prad_gemm_strided_batched_2d_f32)
 
@@ -83,11 +85,15 @@ class SwinBlock:
         fused = lib.prad_matmul_fwd_fused
         check(fused(self.X.handle, w["Wqkv"].handle, w["bqkv"].handle, None, self.QKV.handle, _lib.ACT_NONE, 0.0))
         hs = nw * wt * wt                 # scores are stored head-major: [head][window][wt][wt]
-        # S = Q . K^T per window and head
-        self._all_heads(0, 1, wt, wt, hd, self.QKV, 0, q3, wt * q3, hd, self.QKV, C, q3, wt * q3, hd, self.S, 0, wt, wt * wt, hs)
-        check(lib.prad_softmax_scaled_fwd(self.S.handle, self.scale, self.P.handle))   # P = softmax(S / sqrt(head dim))
-        # O = P . V per window, written into each head's columns of O
-        self._all_heads(0, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.QKV, 2 * C, q3, wt * q3, hd, self.O, 0, C, wt * C, hd)
+        if self.fused_attention:
+            # scores, softmax and P . V of every window and head in one launch; the scores never reach memory
+            check(lib.prad_window_attention_fwd(self.QKV.handle, self.P.handle, self.O.handle, nw, self.heads, wt, self.scale))
+        else:
+            # S = Q . K^T per window and head
+            self._all_heads(0, 1, wt, wt, hd, self.QKV, 0, q3, wt * q3, hd, self.QKV, C, q3, wt * q3, hd, self.S, 0, wt, wt * wt, hs)
+            check(lib.prad_softmax_scaled_fwd(self.S.handle, self.scale, self.P.handle))   # P = softmax(S / sqrt(head dim))
+            # O = P . V per window, written into each head's columns of O
+            self._all_heads(0, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.QKV, 2 * C, q3, wt * q3, hd, self.O, 0, C, wt * C, hd)
         check(fused(self.O.handle, w["Wo"].handle, w["bo"].handle, None, self.Y1.handle, _lib.ACT_NONE, 0.0))
         check(fused(self.Y1.handle, w["W1"].handle, w["b1"].handle, self.Z1.handle, self.H1.handle, _lib.ACT_GELU, 0.0))
         check(fused(self.H1.handle, w["W2"].handle, w["b2"].handle, None, self.Y2.handle, _lib.ACT_NONE, 0.0))

@@ -79,3 +79,46 @@ def test_strided_batched_products_on_column_blocks(gpu, oracle, dtype):
     assert not out[:, :32].any() and not out[:, 64:].any()  # neighbouring column blocks untouched
     assert fn(0, 0, m, k, m, ctypes.c_void_p(S.ptr), m, m * m, ctypes.c_void_p(dB.ptr), ld, m * ld, ctypes.c_void_p(O.ptr), ld, 10, nb, 0) \
         == _lib.PRAD_ERR_ARG  # overlapping outputs
+
+
+@pytest.mark.parametrize("cfg", [(64, 3, 49), (5, 2, 64), (7, 4, 16), (33, 1, 33), (3, 3, 1)])
+def test_attention_of_all_windows_and_heads_in_one_launch(gpu, oracle, cfg):
+    """Scores, scaling, softmax and P . V per window and head in one launch (float, head dimension 32): P and O against
+    the three launches they stand for (strided-batched products and the scaled softmax) and against numpy in double;
+    windows that fill the 64-token tile, the 49 of the benchmark, small and odd ones."""
+    import ctypes
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.exceptions import ArgumentException, check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    nw, heads, wt = cfg
+    hd, dtype = 32, np.float32
+    C = heads * hd
+    assert lib.prad_window_attention_supported(_lib.PRAD_F32, wt, hd) == 1
+    assert lib.prad_window_attention_supported(_lib.PRAD_F64, wt, hd) == 0 and lib.prad_window_attention_supported(_lib.PRAD_F32, 65, hd) == 0
+    QKV = seeded.normal(77, 1, (nw * wt, 3 * C), 1.0, dtype)
+    scale = 1.0 / np.sqrt(hd)
+    bQKV = DeviceBuffer.alloc(dtype, *QKV.shape); bQKV.upload(QKV)
+    P1, O1 = DeviceBuffer.alloc(dtype, heads * nw * wt, wt), DeviceBuffer.alloc(dtype, nw * wt, C)
+    check(lib.prad_window_attention_fwd(bQKV.handle, P1.handle, O1.handle, nw, heads, wt, scale))
+    # the three launches
+    S, P2, O2 = DeviceBuffer.alloc(dtype, heads * nw * wt, wt), DeviceBuffer.alloc(dtype, heads * nw * wt, wt), DeviceBuffer.alloc(dtype, nw * wt, C)
+    ptr = lambda b, off: ctypes.c_void_p(b.ptr + off * 4)
+    q3, hs = 3 * C, nw * wt * wt
+    check(lib.prad_gemm_strided_batched_2d_f32(0, 1, wt, wt, hd, ptr(bQKV, 0), q3, wt * q3, hd, ptr(bQKV, C), q3, wt * q3, hd,
+                                               ptr(S, 0), wt, wt * wt, hs, nw, heads, 0))
+    check(lib.prad_softmax_scaled_fwd(S.handle, scale, P2.handle))
+    check(lib.prad_gemm_strided_batched_2d_f32(0, 0, wt, hd, wt, ptr(P2, 0), wt, wt * wt, hs, ptr(bQKV, 2 * C), q3, wt * q3, hd,
+                                               ptr(O2, 0), C, wt * C, hd, nw, heads, 0))
+    gP, gO = P1.download(), O1.download()
+    assert_parity(gP, P2.download(), dtype, "P against the separate launches")
+    assert_parity(gO, O2.download(), dtype, "O against the separate launches")
+    # numpy in double
+    X = QKV.astype(np.float64).reshape(nw, wt, 3, heads, hd)
+    Sd = np.einsum("wihd,wjhd->hwij", X[:, :, 0], X[:, :, 1]) * scale
+    Pd = np.exp(Sd - Sd.max(axis=-1, keepdims=True)); Pd /= Pd.sum(axis=-1, keepdims=True)
+    Od = np.einsum("hwij,wjhd->wihd", Pd, X[:, :, 2]).reshape(nw * wt, C)
+    assert_parity(gP, Pd.reshape(heads * nw * wt, wt).astype(dtype), dtype, "P against numpy")
+    assert_parity(gO, Od.astype(dtype), dtype, "O against numpy")
+    with pytest.raises(ArgumentException):
+        check(lib.prad_window_attention_fwd(bQKV.handle, P1.handle, O1.handle, nw, heads, wt + 1, scale))   # rows do not match
