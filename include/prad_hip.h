@@ -296,6 +296,13 @@ int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, pr
  * 1 or 0, the call returns PRAD_ERR_ARG for other shapes. */
 int32_t prad_window_attention_supported(int32_t dtype, int64_t tokens, int64_t head_dim);
 int32_t prad_window_attention_fwd(prad_buf_t QKV, prad_buf_t P, prad_buf_t O, int64_t windows, int64_t heads, int64_t tokens, double scale);
+/* Backward of the same nodes in one launch: from dO (the gradient of O) and the forward's P,
+ * dP = dO . V^T, dV = P^T . dO, dS = P (.) (dP - rowsum(dP (.) P)) * scale (src/RMAD/SoftmaxOperation.cs:75-110 and the
+ * scalar product's backward), dQ = dS . K, dK = dS^T . Q (src/RMAD/MatrixMultiplyOperation.cs:88-143); dQKV
+ * ((windows*tokens) x (3*heads*head_dim), columns [dQ | dK | dV]) is written whole, dP and dS never reach memory.  Same
+ * values as the five separate calls up to the order of the sums.  Shapes as for the forward call. */
+int32_t prad_window_attention_bwd(prad_buf_t QKV, prad_buf_t P, prad_buf_t dO, prad_buf_t dQKV, int64_t windows, int64_t heads, int64_t tokens,
+                                  double scale);
 /* Borrowed view of rows [row0, row0 + rows) of a 2-D buffer (a block of a fused weight, a time step of a
  * stacked sequence).  The view must be freed before its parent. */
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out);

@@ -157,6 +157,199 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel
         }
 }
 
+// Backward of the same nodes for one (window, head) per wavefront: with dO the gradient of O,
+//   dP = dO . V^T ;  dV = P^T . dO ;  dS = P (.) (dP - rowsum(dP (.) P)) * scale  (SoftmaxOperation.Backward followed by the
+//   scalar product's, src/RMAD/SoftmaxOperation.cs:75-110) ;  dQ = dS . K ;  dK = dS^T . Q
+// - five launches and four trips of the 49 x 49 blocks through memory when taken one by one.  P comes into the
+// wavefront's LDS tile once (zeros past the window), serves dV as the A operand read across, and the softmax's backward
+// in the accumulators' own layout; dS then takes the tile's place for the last two products.  KS = k steps of the three
+// products whose reduction runs over the tokens (13 for windows of 49 to 52 tokens, else 16).
+struct AttBwdArgs {
+    const float* QKV; const float* P; const float* dO; float* dQKV;
+    int windows, heads, tokens;
+    float scale;
+};
+
+template <int KS>
+__global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_bwd_kernel(const AttBwdArgs p) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int li = lane & 15, g = lane >> 4;
+    const int64_t pair = (int64_t)blockIdx.x * ATT_WAVES + wave;
+    __shared__ float tiles[ATT_WAVES][64 * ATT_PITCH];
+    if (pair >= (int64_t)p.windows * p.heads) return;
+    const int w = (int)(pair / p.heads), h = (int)(pair % p.heads);
+    const int wt = p.tokens, C = p.heads * ATT_HD, ld = 3 * C;
+    float* __restrict__ tile = tiles[wave];
+    const float* __restrict__ Q = p.QKV + (int64_t)w * wt * ld + h * ATT_HD;
+    const float* __restrict__ K = Q + C;
+    const float* __restrict__ V = Q + 2 * C;
+    const float* __restrict__ dO = p.dO + (int64_t)w * wt * C + h * ATT_HD;
+    const float* __restrict__ P = p.P + ((int64_t)h * p.windows + w) * wt * wt;
+
+    // token-major fragments of an operand whose rows are tokens: element [token 4 s + g][16 y + li] (tokens past the window: the last one;
+    // they meet zeros of P or dS)
+    auto token_frags = [&](const float* __restrict__ base, int64_t pitch, float (&f)[KS][2]) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const int tok = min(4 * s + g, wt - 1);
+#pragma unroll
+            for (int y = 0; y < 2; ++y) f[s][y] = base[(int64_t)tok * pitch + 16 * y + li];
+        }
+    };
+    // every operand that comes from memory is asked for before the first product, the ones used last, last
+    f4a af[4][2], bf[4][2];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        const int row = min(16 * x + li, wt - 1);
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            af[x][v] = *reinterpret_cast<const f4a*>(dO + (int64_t)row * C + 8 * g + 4 * v);
+            bf[x][v] = *reinterpret_cast<const f4a*>(V + (int64_t)row * ld + 8 * g + 4 * v);
+        }
+    }
+    // P -> tile, zeros past the window; sixteen loads in flight per lane
+    for (int e = lane; e < 64 * ATT_PITCH / 4; e += 64) reinterpret_cast<f4a*>(tile)[e] = f4a{0.f, 0.f, 0.f, 0.f};
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    {
+        int r = lane / wt, c = lane % wt;
+        const int dr = 64 / wt, dc = 64 % wt, n = wt * wt;
+        for (int e0 = lane; e0 < n; e0 += 64 * 16) {
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = P[min(e0 + 64 * u, n - 1)];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                if (e0 + 64 * u < n) tile[r * ATT_PITCH + c] = v[u];
+                r += dr; c += dc;
+                if (c >= wt) { c -= wt; ++r; }
+            }
+        }
+    }
+    float dof[KS][2], kf[KS][2], qf[KS][2];
+    token_frags(dO, C, dof);
+    token_frags(K, ld, kf);
+    token_frags(Q, ld, qf);
+    // dP = dO . V^T: rows of dO and V as k-contiguous fragments (k = 8 g .. 8 g + 7, as in the forward kernel)
+    f4a acc[4][4];
+    {
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 4; ++y) acc[x][y] = f4a{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int y = 0; y < 4; ++y) acc[x][y] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[x][s >> 2][s & 3], bf[y][s >> 2][s & 3], acc[x][y], 0, 0, 0);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    auto store_block = [&](float* __restrict__ dst, const f4a (&o)[4][2]) {  // rows = tokens, 32 columns of this head
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = 16 * x + 4 * g + r;
+                if (row < wt) {
+#pragma unroll
+                    for (int y = 0; y < 2; ++y) dst[(int64_t)row * ld + 16 * y + li] = o[x][y][r];
+                }
+            }
+    };
+    float* __restrict__ dQ = p.dQKV + (int64_t)w * wt * ld + h * ATT_HD;
+
+    // dV = P^T . dO: A = P read across (row j of P^T = column j of P), k = token i
+    {
+        auto& bfr = dof;
+        f4a o[4][2];
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 2; ++y) o[x][y] = f4a{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            float a[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) a[x] = tile[(4 * s + g) * ATT_PITCH + 16 * x + li];
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int y = 0; y < 2; ++y) o[x][y] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[x], bfr[s][y], o[x][y], 0, 0, 0);
+        }
+        store_block(dQ + 2 * C, o);
+    }
+    // dS = P (.) (dP - rowsum(dP (.) P)) * scale in the accumulators' layout: acc[x][y][r] is (row 16 x + 4 g + r, column 16 y + li)
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float pv[4], dot = 0.f;
+#pragma unroll
+            for (int y = 0; y < 4; ++y) {
+                pv[y] = tile[(16 * x + 4 * g + r) * ATT_PITCH + 16 * y + li];
+                dot += acc[x][y][r] * pv[y];
+            }
+#pragma unroll
+            for (int m = 1; m < 16; m <<= 1) dot += __shfl_xor(dot, m, 64);  // over the 16 lanes that share the row
+#pragma unroll
+            for (int y = 0; y < 4; ++y) acc[x][y][r] = (pv[y] * (acc[x][y][r] - dot)) * p.scale;
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();  // every lane has read its part of P
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int y = 0; y < 4; ++y)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tile[(16 * x + 4 * g + r) * ATT_PITCH + 16 * y + li] = acc[x][y][r];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // dQ = dS . K (A = dS rows) and dK = dS^T . Q (A = dS read across)
+    {
+        auto& bfr = kf;
+        f4a o[4][2];
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 2; ++y) o[x][y] = f4a{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            float a[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) a[x] = tile[(16 * x + li) * ATT_PITCH + 4 * s + g];
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int y = 0; y < 2; ++y) o[x][y] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[x], bfr[s][y], o[x][y], 0, 0, 0);
+        }
+        store_block(dQ, o);
+    }
+    {
+        auto& bfr = qf;
+        f4a o[4][2];
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 2; ++y) o[x][y] = f4a{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            float a[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) a[x] = tile[(4 * s + g) * ATT_PITCH + 16 * x + li];
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int y = 0; y < 2; ++y) o[x][y] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[x], bfr[s][y], o[x][y], 0, 0, 0);
+        }
+        store_block(dQ + C, o);
+    }
+}
+
 }  // namespace
 
 bool window_attention_supported(int64_t tokens, int64_t head_dim) {
@@ -170,6 +363,18 @@ hipError_t launch_window_attention_fwd(const float* QKV, float* P, float* O, int
     AttArgs a{QKV, P, O, (int)windows, (int)heads, (int)tokens, scale};
     const int64_t pairs = windows * heads;
     hipLaunchKernelGGL(window_attention_fwd_kernel, dim3((unsigned)((pairs + ATT_WAVES - 1) / ATT_WAVES)), dim3(64 * ATT_WAVES), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_window_attention_bwd(const float* QKV, const float* P, const float* dO, float* dQKV, int64_t windows, int64_t heads,
+                                       int64_t tokens, float scale, hipStream_t stream) {
+    if (!window_attention_supported(tokens, ATT_HD) || reinterpret_cast<uintptr_t>(QKV) % 16 != 0 || reinterpret_cast<uintptr_t>(dO) % 16 != 0)
+        return hipErrorNotSupported;
+    AttBwdArgs a{QKV, P, dO, dQKV, (int)windows, (int)heads, (int)tokens, scale};
+    const int64_t pairs = windows * heads;
+    const dim3 grid((unsigned)((pairs + ATT_WAVES - 1) / ATT_WAVES)), block(64 * ATT_WAVES);
+    if (tokens > 48 && tokens <= 52) hipLaunchKernelGGL(window_attention_bwd_kernel<13>, grid, block, 0, stream, a);
+    else hipLaunchKernelGGL(window_attention_bwd_kernel<16>, grid, block, 0, stream, a);
     return hipGetLastError();
 }
 

@@ -340,6 +340,8 @@ hipError_t launch_lstm_seq(const LstmSeqArgs& a, bool backward, hipStream_t s);
 bool window_attention_supported(int64_t tokens, int64_t head_dim);
 hipError_t launch_window_attention_fwd(const float* QKV, float* P, float* O, int64_t windows, int64_t heads, int64_t tokens, float scale,
                                        hipStream_t stream);
+hipError_t launch_window_attention_bwd(const float* QKV, const float* P, const float* dO, float* dQKV, int64_t windows, int64_t heads,
+                                       int64_t tokens, float scale, hipStream_t stream);
 
 // MatrixMultiplyAndSum
 // S = samples of a batch (each with its own A, out, dOut, dA and P slices of dB; the P slices of B are shared).

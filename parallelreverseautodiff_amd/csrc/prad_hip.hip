@@ -1503,6 +1503,26 @@ int32_t prad_window_attention_fwd(prad_buf_t QKV, prad_buf_t P, prad_buf_t O, in
     return PRAD_OK;
 }
 
+int32_t prad_window_attention_bwd(prad_buf_t QKV, prad_buf_t P, prad_buf_t dO, prad_buf_t dQKV, int64_t windows, int64_t heads, int64_t tokens,
+                                  double scale) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(QKV); REQUIRE_BUF(P); REQUIRE_BUF(dO); REQUIRE_BUF(dQKV);
+    if (int32_t st = same_dtype({QKV, P, dO, dQKV})) return st;
+    if (windows < 1 || heads < 1 || tokens < 1 || QKV->depth != 1 || QKV->rows != windows * tokens || QKV->cols % (3 * heads) != 0)
+        return fail(PRAD_ERR_ARG, "QKV must be (windows*tokens) x (3*heads*head_dim)");
+    const int64_t head_dim = QKV->cols / (3 * heads);
+    if (QKV->dtype != PRAD_F32 || !window_attention_supported(tokens, head_dim))
+        return fail(PRAD_ERR_ARG, "the one-launch attention takes float, head dimension 32 and at most 64 tokens per window; ask "
+                                  "prad_window_attention_supported first");
+    if (int32_t st = expect_rows(P, heads * windows * tokens, tokens, "P")) return st;
+    if (int32_t st = expect_rows(dO, windows * tokens, heads * head_dim, "dO")) return st;
+    if (int32_t st = expect_rows(dQKV, windows * tokens, 3 * heads * head_dim, "dQKV")) return st;
+    if (dQKV->ptr == QKV->ptr || dQKV->ptr == dO->ptr) return fail(PRAD_ERR_ARG, "dQKV must not alias an input");
+    ENQUEUE_LOCK();
+    HIP_TRY(launch_window_attention_bwd(F(QKV), F(P), F(dO), F(dQKV), windows, heads, tokens, (float)scale, CUR_STREAM), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
 int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_buf_t* out) {
     REQUIRE_INIT();
     REQUIRE_BUF(parent);

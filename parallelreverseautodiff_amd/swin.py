@@ -107,13 +107,17 @@ class SwinBlock:
                                        _lib.ACT_NONE, None, 0.0))
         check(lib.prad_matmul_bias_bwd(self.dY1.handle, self.O.handle, w["Wo"].handle, self.dO.handle, g["Wo"].handle, g["bo"].handle, 0,
                                        _lib.ACT_NONE, None, 0.0))
-        # dP = dO . V^T ; dV = P^T . dO
-        self._all_heads(0, 1, wt, wt, hd, self.dO, 0, C, wt * C, hd, self.QKV, 2 * C, q3, wt * q3, hd, self.dP, 0, wt, wt * wt, hs)
-        self._all_heads(1, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.dO, 0, C, wt * C, hd, self.dQKV, 2 * C, q3, wt * q3, hd)
-        check(lib.prad_softmax_scaled_bwd(self.P.handle, self.dP.handle, self.scale, self.dS.handle))
-        # dQ = dS . K ; dK = dS^T . Q
-        self._all_heads(0, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, C, q3, wt * q3, hd, self.dQKV, 0, q3, wt * q3, hd)
-        self._all_heads(1, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, 0, q3, wt * q3, hd, self.dQKV, C, q3, wt * q3, hd)
+        if self.fused_attention:
+            # dP, dV, the softmax's backward, dQ and dK of every window and head in one launch; dP and dS never reach memory
+            check(lib.prad_window_attention_bwd(self.QKV.handle, self.P.handle, self.dO.handle, self.dQKV.handle, nw, self.heads, wt, self.scale))
+        else:
+            # dP = dO . V^T ; dV = P^T . dO
+            self._all_heads(0, 1, wt, wt, hd, self.dO, 0, C, wt * C, hd, self.QKV, 2 * C, q3, wt * q3, hd, self.dP, 0, wt, wt * wt, hs)
+            self._all_heads(1, 0, wt, hd, wt, self.P, 0, wt, wt * wt, hs, self.dO, 0, C, wt * C, hd, self.dQKV, 2 * C, q3, wt * q3, hd)
+            check(lib.prad_softmax_scaled_bwd(self.P.handle, self.dP.handle, self.scale, self.dS.handle))
+            # dQ = dS . K ; dK = dS^T . Q
+            self._all_heads(0, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, C, q3, wt * q3, hd, self.dQKV, 0, q3, wt * q3, hd)
+            self._all_heads(1, 0, wt, hd, wt, self.dS, 0, wt, wt * wt, hs, self.QKV, 0, q3, wt * q3, hd, self.dQKV, C, q3, wt * q3, hd)
         check(lib.prad_matmul_bias_bwd(self.dQKV.handle, self.X.handle, w["Wqkv"].handle, self.dX.handle, g["Wqkv"].handle, g["bqkv"].handle, 0,
                                        _lib.ACT_NONE, None, 0.0))
 

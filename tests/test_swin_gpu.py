@@ -122,3 +122,57 @@ def test_attention_of_all_windows_and_heads_in_one_launch(gpu, oracle, cfg):
     assert_parity(gO, Od.astype(dtype), dtype, "O against numpy")
     with pytest.raises(ArgumentException):
         check(lib.prad_window_attention_fwd(bQKV.handle, P1.handle, O1.handle, nw, heads, wt + 1, scale))   # rows do not match
+
+
+@pytest.mark.parametrize("cfg", [(64, 3, 49), (5, 2, 64), (7, 4, 16), (33, 1, 33), (3, 3, 1), (9, 2, 52)])
+def test_attention_backward_of_all_windows_and_heads_in_one_launch(gpu, oracle, cfg):
+    """dQ, dK and dV of every window and head from dO and the forward's P in one launch, against the five launches it
+    stands for (four strided-batched products and the scaled softmax's backward) and against numpy in double; the
+    gradient buffer starts out full of NaN, so a cell the launch leaves unwritten shows."""
+    import ctypes
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.exceptions import ArgumentException, check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    lib = _lib.load()
+    nw, heads, wt = cfg
+    hd, dtype = 32, np.float32
+    C = heads * hd
+    QKV = seeded.normal(78, 1, (nw * wt, 3 * C), 1.0, dtype)
+    dO = seeded.normal(78, 2, (nw * wt, C), 1.0, dtype)
+    scale = 1.0 / np.sqrt(hd)
+    alloc = lambda r, c: DeviceBuffer.alloc(dtype, r, c)
+    bQKV, bdO = alloc(*QKV.shape), alloc(*dO.shape)
+    bQKV.upload(QKV); bdO.upload(dO)
+    P, O = alloc(heads * nw * wt, wt), alloc(nw * wt, C)
+    check(lib.prad_window_attention_fwd(bQKV.handle, P.handle, O.handle, nw, heads, wt, scale))
+    d1, d2 = alloc(nw * wt, 3 * C), alloc(nw * wt, 3 * C)
+    d1.upload(np.full((nw * wt, 3 * C), np.nan, dtype))
+    check(lib.prad_window_attention_bwd(bQKV.handle, P.handle, bdO.handle, d1.handle, nw, heads, wt, scale))
+    # the five launches
+    dP, dS = alloc(heads * nw * wt, wt), alloc(heads * nw * wt, wt)
+    ptr = lambda b, off: ctypes.c_void_p(b.ptr + off * 4)
+    q3, hs = 3 * C, nw * wt * wt
+    bat = lib.prad_gemm_strided_batched_2d_f32
+    check(bat(0, 1, wt, wt, hd, ptr(bdO, 0), C, wt * C, hd, ptr(bQKV, 2 * C), q3, wt * q3, hd, ptr(dP, 0), wt, wt * wt, hs, nw, heads, 0))
+    check(bat(1, 0, wt, hd, wt, ptr(P, 0), wt, wt * wt, hs, ptr(bdO, 0), C, wt * C, hd, ptr(d2, 2 * C), q3, wt * q3, hd, nw, heads, 0))
+    check(lib.prad_softmax_scaled_bwd(P.handle, dP.handle, scale, dS.handle))
+    check(bat(0, 0, wt, hd, wt, ptr(dS, 0), wt, wt * wt, hs, ptr(bQKV, C), q3, wt * q3, hd, ptr(d2, 0), q3, wt * q3, hd, nw, heads, 0))
+    check(bat(1, 0, wt, hd, wt, ptr(dS, 0), wt, wt * wt, hs, ptr(bQKV, 0), q3, wt * q3, hd, ptr(d2, C), q3, wt * q3, hd, nw, heads, 0))
+    g1 = d1.download()
+    assert np.isfinite(g1).all(), "cells left unwritten"
+    assert_parity(g1, d2.download(), dtype, "dQKV against the separate launches")
+    # numpy in double, from the same P
+    X = QKV.astype(np.float64).reshape(nw, wt, 3, heads, hd)
+    G = dO.astype(np.float64).reshape(nw, wt, heads, hd)
+    Pd = P.download().astype(np.float64).reshape(heads, nw, wt, wt)
+    dPd = np.einsum("wihd,wjhd->hwij", G, X[:, :, 2])
+    dSd = Pd * (dPd - (dPd * Pd).sum(axis=-1, keepdims=True)) * scale
+    ref = np.empty((nw, wt, 3, heads, hd))
+    ref[:, :, 0] = np.einsum("hwij,wjhd->wihd", dSd, X[:, :, 1])
+    ref[:, :, 1] = np.einsum("hwij,wihd->wjhd", dSd, X[:, :, 0])
+    ref[:, :, 2] = np.einsum("hwij,wihd->wjhd", Pd, G)
+    assert_parity(g1, ref.reshape(nw * wt, 3 * C).astype(dtype), dtype, "dQKV against numpy")
+    with pytest.raises(ArgumentException):
+        check(lib.prad_window_attention_bwd(bQKV.handle, P.handle, bdO.handle, bQKV.handle, nw, heads, wt, scale))   # output over an input
+    with pytest.raises(ArgumentException):
+        check(lib.prad_window_attention_bwd(bQKV.handle, P.handle, O.handle, d1.handle, nw, heads, wt + 1, scale))  # rows do not match
