@@ -324,6 +324,40 @@ __global__ void __launch_bounds__(256) mse_partial_kernel(const T* __restrict__ 
     __syncthreads();
     if (threadIdx.x == 0) part[blockIdx.x] = (w[0] + w[1]) + (w[2] + w[3]);
 }
+// The same pass in 16-byte accesses, four vectors of each operand in flight per thread (n a multiple of the vector
+// length, 16-byte aligned operands): 4-byte loads, one behind the other, left the pass at 40 % of a copy's rate.
+template <typename T, bool WITH_DY>
+__global__ void __launch_bounds__(256) mse_partial_vec_kernel(const T* __restrict__ y, const T* __restrict__ t, double* __restrict__ part,
+                                                              T* __restrict__ dy, int64_t n) {
+    constexpr int VEC = 16 / sizeof(T), FLY = 4;
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    const T scale = (T)2 / (T)n;
+    const int64_t nv = n / VEC, stride = (int64_t)gridDim.x * 256;
+    double s = 0.0;
+    for (int64_t v0 = (int64_t)blockIdx.x * 256 + threadIdx.x; v0 < nv; v0 += FLY * stride) {
+        Vec a[FLY], b[FLY];
+#pragma unroll
+        for (int u = 0; u < FLY; ++u) {
+            const int64_t v = min(v0 + u * stride, nv - 1);
+            a[u] = reinterpret_cast<const Vec*>(y)[v];
+            b[u] = reinterpret_cast<const Vec*>(t)[v];
+        }
+#pragma unroll
+        for (int u = 0; u < FLY; ++u) {
+            if (v0 + u * stride < nv) {
+                Vec d = a[u] - b[u];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) s += (double)(d[i] * d[i]);
+                if (WITH_DY) reinterpret_cast<Vec*>(dy)[v0 + u * stride] = d * scale;
+            }
+        }
+    }
+    s = wave_sum(s);
+    __shared__ double w[4];
+    if ((threadIdx.x & 63) == 0) w[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) part[blockIdx.x] = (w[0] + w[1]) + (w[2] + w[3]);
+}
 template <typename T>
 __global__ void __launch_bounds__(64) mse_final_kernel(const double* __restrict__ part, int nparts, T* __restrict__ loss, int64_t n) {
     double s = 0.0;
@@ -344,7 +378,11 @@ hipError_t launch_mse_fwd(const T* y, const T* t, T* loss, double* workspace, in
     int64_t blocks = (n + 255) / 256;
     if (blocks > MSE_PARTS) blocks = MSE_PARTS;
     if (blocks < 1) blocks = 1;
-    if (dy != nullptr) hipLaunchKernelGGL((mse_partial_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, dy, n);
+    const bool vec = n % (16 / sizeof(T)) == 0 && n >= 65536 && reinterpret_cast<uintptr_t>(y) % 16 == 0 && reinterpret_cast<uintptr_t>(t) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(dy) % 16 == 0;
+    if (vec && dy != nullptr) hipLaunchKernelGGL((mse_partial_vec_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, dy, n);
+    else if (vec) hipLaunchKernelGGL((mse_partial_vec_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, dy, n);
+    else if (dy != nullptr) hipLaunchKernelGGL((mse_partial_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, dy, n);
     else hipLaunchKernelGGL((mse_partial_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, s, y, t, workspace, dy, n);
     hipLaunchKernelGGL((mse_final_kernel<T>), dim3(1), dim3(64), 0, s, workspace, (int)blocks, loss, n);
     return hipGetLastError();

@@ -137,7 +137,7 @@ def test_scaled_softmax_forward_and_backward(gpu, oracle, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", [(1, 1), (7, 13), (128, 512), (3000, 97)])
+@pytest.mark.parametrize("shape", [(1, 1), (7, 13), (128, 512), (3000, 97), (2500, 1000)])
 def test_mean_squared_error_loss_and_gradient(gpu, oracle, dtype, shape):
     """MeanSquaredErrorLossOperation Forward and Backward against the oracle, separately and in one pass
     (prad_mse: the same values as the two launches, bit for bit)."""
