@@ -81,7 +81,7 @@ def test_strided_batched_products_on_column_blocks(gpu, oracle, dtype):
         == _lib.PRAD_ERR_ARG  # overlapping outputs
 
 
-@pytest.mark.parametrize("cfg", [(64, 3, 49), (5, 2, 64), (7, 4, 16), (33, 1, 33), (3, 3, 1)])
+@pytest.mark.parametrize("cfg", [(64, 3, 49), (5, 2, 64), (7, 4, 16), (33, 1, 33), (3, 3, 1), (9, 2, 52), (4, 2, 50)])
 def test_attention_of_all_windows_and_heads_in_one_launch(gpu, oracle, cfg):
     """Scores, scaling, softmax and P . V per window and head in one launch (float, head dimension 32): P and O against
     the three launches they stand for (strided-batched products and the scaled softmax) and against numpy in double;
