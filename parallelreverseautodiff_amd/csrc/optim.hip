@@ -25,6 +25,11 @@ constexpr int OPT_THREADS = 256;
 constexpr int OPT_CHUNK_SMALL = 4096;
 template <typename T> constexpr int OPT_CHUNK_LARGE = 32768 / (int)sizeof(T);
 constexpr int64_t LARGE_CHUNK_FROM = (int64_t)4 << 20;  // total elements of a launch
+// A model of less than a million parameters is not even one 4096-element chunk per compute unit (the 235 000 of the
+// 784-256-128-10 network: 58 workgroups, each moving its 229 KB at one compute unit's share of the bandwidth -
+// 11 us for 13 MB); chunks of 1024 spread it over four times as many.
+constexpr int OPT_CHUNK_TINY = 1024;
+constexpr int64_t TINY_CHUNK_BELOW = (int64_t)1 << 20;  // total elements of a launch
 
 template <typename T>
 struct DevTensor {
@@ -107,7 +112,7 @@ __global__ void __launch_bounds__(OPT_THREADS) clip_stats_kernel(const TensorTab
     const DevTensor<T> t = tab.t[ti];
     const int64_t begin = (chunk - t.first_chunk) * CHUNK;
     const int64_t end = min(begin + (int64_t)CHUNK, t.n);
-    constexpr int PER = CHUNK / OPT_THREADS;  // 16 (double) or 32 (float) elements per thread
+    constexpr int PER = CHUNK / OPT_THREADS;  // 4, 16 or 32 elements per thread
     double x[PER];
     int cnt = 0;
     double sum = 0.0;
@@ -392,8 +397,10 @@ size_t clip_workspace_bytes(const int64_t* n, int nt) {
     // Groups of MAX_TABLE tensors run one after another on the stream and reuse the space.
     size_t worst = 0;
     for (int g0 = 0; g0 < nt; g0 += MAX_TABLE) {
-        int64_t chunks = 0;
-        for (int i = g0; i < nt && i < g0 + MAX_TABLE; ++i) chunks += (n[i] + OPT_CHUNK_SMALL - 1) / OPT_CHUNK_SMALL;  // the smaller chunk: an upper bound
+        int64_t chunks = 0, total = 0;
+        for (int i = g0; i < nt && i < g0 + MAX_TABLE; ++i) total += n[i];
+        const int64_t chunk = total < TINY_CHUNK_BELOW ? OPT_CHUNK_TINY : OPT_CHUNK_SMALL;  // (of the two larger ones the smaller: an upper bound)
+        for (int i = g0; i < nt && i < g0 + MAX_TABLE; ++i) chunks += (n[i] + chunk - 1) / chunk;
         const size_t need = (size_t)chunks * sizeof(Moments) + (size_t)MAX_TABLE * 16;
         if (need > worst) worst = need;
     }
@@ -440,7 +447,9 @@ static hipError_t launch_groups(const TensorDesc<T>* host, int nt, void* workspa
         const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
         int64_t total = 0;
         for (int i = 0; i < gn; ++i) total += host[g0 + i].n;
-        const hipError_t e = (OPT_CHUNK_LARGE<T> != OPT_CHUNK_SMALL && total >= LARGE_CHUNK_FROM)
+        const hipError_t e = total < TINY_CHUNK_BELOW
+                                 ? launch_group<T, OPT_CHUNK_TINY, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs)
+                             : (OPT_CHUNK_LARGE<T> != OPT_CHUNK_SMALL && total >= LARGE_CHUNK_FROM)
                                  ? launch_group<T, OPT_CHUNK_LARGE<T>, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs)
                                  : launch_group<T, OPT_CHUNK_SMALL, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs);
         if (e != hipSuccess) return e;
