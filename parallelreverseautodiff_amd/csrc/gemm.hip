@@ -1137,11 +1137,35 @@ bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
     return t != TILE_128x128 && wgs >= 128 && wgs <= GEMM_SPLIT_MAX_TILES && K >= 32 * slab_depth(t, elem_size);
 }
 
+// A product of few 128 x 128 tiles and a long K (a weight gradient over thousands of rows: 256 x 2048 with K = 8192
+// is 32 such tiles) would run on 64 x 64 or 32 x 32 tiles to fill the chip, at their lower ratio of MFMAs to LDS
+// traffic.  With K long enough every 128 x 128 tile is shared by `ways` workgroups instead (the mechanism of
+// gemm_shared_tiles_plan with all tiles shared): four ways or more, at least 192 workgroups, at least 32 slabs of K
+// each, little padding.
+// Returns the ways (0: not such a product) and the number of tiles.
+static int few_tiles_long_k_plan(int64_t M, int64_t N, int64_t K, int elem_size, int* tiles_out) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_FEW_TILES"); return !(e && e[0] == '0'); }();  // tuning aid
+    if (!enabled || choose_tile(M, N, 1, false) == TILE_128x128) return 0;
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles * 128 * 128 * 4 > M * N * 5) return 0;  // more than a quarter of padding: the smaller tiles multiply less
+    const int64_t bk = slab_depth(TILE_128x128, elem_size);
+    int64_t ways = 256 / tiles;
+    if (ways > 16) ways = 16;
+    if (ways > K / (32 * bk)) ways = K / (32 * bk);
+    // (two ways were measured level with the smaller tiles once the launch that adds the partial tiles is counted:
+    // 8192 x 256 with K = 2048, 70.9 + 7.4 us against 69.5)
+    if (ways < 4 || tiles * ways < 192) return 0;
+    *tiles_out = (int)tiles;
+    return (int)ways;
+}
+
 int gemm_shared_tiles_plan(int64_t M, int64_t N, int64_t K, int batch, int elem_size, int* shared_tiles) {
     static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_SHARED"); return !(e && e[0] == '0'); }();  // tuning aid
     *shared_tiles = 0;
-    if (!enabled || batch != 1 || choose_tile(M, N, batch, false) != TILE_128x128) return 0;
+    if (!enabled || batch != 1) return 0;
     if (gemm_split_factor(M, N, K, batch, elem_size) > 1) return 0;
+    if (const int ways = few_tiles_long_k_plan(M, N, K, elem_size, shared_tiles)) return ways;
+    if (choose_tile(M, N, batch, false) != TILE_128x128) return 0;
     constexpr int64_t SLOTS = 512;  // two workgroups of the 128 x 128 kernels per compute unit
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     // (fewer tiles than slots - 256 tiles, one per compute unit - were measured with every tile shared two ways: +2 %,
@@ -1280,13 +1304,14 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         hipLaunchKernelGGL((split_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, a, a.split_ws, splits);
         return hipGetLastError();
     }
-    const TileShape tile = choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr);
+    TileShape tile = choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr);
     a.shared_tiles = 0; a.shared_splits = 0;
     int shared_tiles = 0;
-    const int shared_ways = (tile == TILE_128x128 && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
+    const int shared_ways = (a.tile_sums == nullptr && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
                              a.batch_inner <= 1 && a.colsum_dst == nullptr)
                                 ? gemm_shared_tiles_plan(a.M, a.N, a.K, a.batch, (int)sizeof(T), &shared_tiles) : 0;
     if (shared_ways > 1) {
+        tile = TILE_128x128;  // (few tiles and a long K: the plan puts a product of smaller tiles on shared 128 x 128 ones)
         const int64_t bk = slab_depth(tile, (int)sizeof(T));
         a.ksplit = ((a.K + shared_ways - 1) / shared_ways + bk - 1) / bk * bk;
         a.shared_splits = (int)((a.K + a.ksplit - 1) / a.ksplit);

@@ -496,10 +496,11 @@ def test_both_gradients_in_one_launch(gpu, dtype, accumulate, shape):
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
-@pytest.mark.parametrize("shape", [(512, 2048, 512), (1024, 1024, 1024), (384, 2100, 500), (512, 4096, 512)])
+@pytest.mark.parametrize("shape", [(512, 2048, 512), (1024, 1024, 1024), (384, 2100, 500), (512, 4096, 512), (256, 8192, 2048), (500, 6000, 1000)])
 def test_products_of_few_tiles_and_long_k(gpu, oracle, dtype, shape):
     """Shapes whose 64 x 64 or 32 x 32 tiles fill between half and one and a half of the chip's workgroup slots and
-    whose K holds at least 32 slabs (which of these shapes do depends on the element type): parity with the oracle
+    whose K holds at least 32 slabs (which of these shapes do depends on the element type), and shapes of few 128 x 128
+    tiles and a K of thousands, whose tiles are each shared by several workgroups: parity with the oracle
     for the forward and both backward layouts, fused epilogue included, and the same bits on every run.  With
     PRAD_GEMM_PAIRS=1 in the environment (test_workgroup_pairs_when_switched_on runs this test that way) they run
     with two workgroups per tile, half of K each, the later one adding the other's partial tile: the same bits then
@@ -532,7 +533,10 @@ def test_products_of_few_tiles_and_long_k(gpu, oracle, dtype, shape):
         # blocked sums are; both are therefore held against the product taken in double and rounded once.
         wide = lambda x: x.astype(np.float64)
         rC = oracle.matmul_fwd(wide(A), wide(B), threads=8).astype(dtype)
-        assert_parity(oracle.matmul_fwd(A, B, threads=8), rC, dtype, "oracle C against the double product")
+        # (the oracle's own sum: every entry within its rounding bound of the double product - at K = 8192 its normwise
+        # error is already 1.3e-5)
+        off = np.abs(oracle.matmul_fwd(A, B, threads=8).astype(np.float64) - rC.astype(np.float64))
+        assert np.all(off <= dot_bound(A, B, dtype)), "oracle C against the double product"
     else:
         rC = oracle.matmul_fwd(A, B, threads=8)
     rdA, rdB = oracle.matmul_bwd(dC, A, B, threads=8)
@@ -676,7 +680,7 @@ def test_workgroup_pairs_when_switched_on(gpu):
                         "-k", "test_products_of_few_tiles_and_long_k", "-p", "no:cacheprovider"],
                        cwd=root, env=env, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
-    assert "8 passed" in r.stdout, r.stdout[-2000:]
+    assert "12 passed" in r.stdout, r.stdout[-2000:]
 
 
 @pytest.mark.parametrize("shape", [(50176, 96, 288), (8192, 96, 96), (16384, 384, 96), (12288, 96, 384), (4096, 64, 320), (20000, 32, 48)])
