@@ -85,6 +85,15 @@ __device__ __forceinline__ bool wait_for_group(const unsigned* flags, int blocks
     return *verdict != 0;
 }
 
+// The cell's sigmoid and tanh for the sequence kernel: float arithmetic on the hardware exponential and reciprocal
+// (within 3e-7 of the double-precision evaluation the per-step kernels round to float) - five transcendental functions
+// per element sit on every time step's critical path, and in double they cost half a microsecond of it.
+__device__ __forceinline__ float seq_sigmoid(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+__device__ __forceinline__ float seq_tanh(float x) {
+    const float t = __expf(-2.0f * fabsf(x));
+    return copysignf((1.0f - t) * __builtin_amdgcn_rcpf(1.0f + t), x);
+}
+
 // ---- forward ----------------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_fwd_kernel(const LstmSeqArgs p) {
     const int H = p.hidden, B = p.batch, NJ = H / 16, groups = B / 16, blocks = H / 16;
@@ -160,13 +169,13 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_fwd_kernel(const Lstm
         for (int rr = 0; rr < 4; ++rr) exch[(q * 16 + 4 * g + rr) * 16 + n] = acc0[rr] + acc1[rr];
         __syncthreads();
         // the cell, as lstm_cell_fwd_kernel writes it
-        const float i_ = act_forward<float>(ACT_SIGMOID, pre[0] + exch[(0 * 16 + row) * 16 + u], 0.f);
-        const float f_ = act_forward<float>(ACT_SIGMOID, pre[1] + exch[(1 * 16 + row) * 16 + u], 0.f);
-        const float g_ = act_forward<float>(ACT_TANH, pre[2] + exch[(2 * 16 + row) * 16 + u], 0.f);
-        const float o_ = act_forward<float>(ACT_SIGMOID, pre[3] + exch[(3 * 16 + row) * 16 + u], 0.f);
+        const float i_ = seq_sigmoid(pre[0] + exch[(0 * 16 + row) * 16 + u]);
+        const float f_ = seq_sigmoid(pre[1] + exch[(1 * 16 + row) * 16 + u]);
+        const float g_ = seq_tanh(pre[2] + exch[(2 * 16 + row) * 16 + u]);
+        const float o_ = seq_sigmoid(pre[3] + exch[(3 * 16 + row) * 16 + u]);
         grow[0] = i_; grow[H] = f_; grow[2 * H] = g_; grow[3 * H] = o_;
         const float cn = (f_ * c_prev) + (i_ * g_);
-        const float tc = act_forward<float>(ACT_TANH, cn, 0.f);
+        const float tc = seq_tanh(cn);
         const int64_t blk = (int64_t)B * H;
         p.C[(t + 1) * blk + own] = cn;
         p.TC[t * blk + own] = tc;
