@@ -25,11 +25,11 @@ constexpr int OPT_THREADS = 256;
 constexpr int OPT_CHUNK_SMALL = 4096;
 template <typename T> constexpr int OPT_CHUNK_LARGE = 32768 / (int)sizeof(T);
 constexpr int64_t LARGE_CHUNK_FROM = (int64_t)4 << 20;  // total elements of a launch
-// A model of less than a million parameters is not even one 4096-element chunk per compute unit (the 235 000 of the
-// 784-256-128-10 network: 58 workgroups, each moving its 229 KB at one compute unit's share of the bandwidth -
-// 11 us for 13 MB); chunks of 1024 spread it over four times as many.
+// A model of a few million parameters or less is only a few 4096-element chunks per compute unit, a small one not even
+// one (the 235 000 of the 784-256-128-10 network: 58 workgroups, each moving its 229 KB at one compute unit's share of
+// the bandwidth - 11 us for 13 MB); chunks of 1024 spread it over four times as many.
 constexpr int OPT_CHUNK_TINY = 1024;
-constexpr int64_t TINY_CHUNK_BELOW = (int64_t)1 << 20;  // total elements of a launch
+constexpr int64_t TINY_CHUNK_BELOW = (int64_t)4 << 20;  // total elements of a launch
 
 template <typename T>
 struct DevTensor {
