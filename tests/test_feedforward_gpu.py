@@ -231,8 +231,8 @@ def test_workspace_growth_while_a_recorded_sequence_is_alive(gpu, oracle):
         assert np.array_equal(c.download(), eager)
     check(lib.prad_graph_destroy(g))
     # growth during a recording is refused with a message that says what to do: a sum of 16 products whose partial
-    # results (16 x 512 x 512 doubles = 32 MiB) outgrow everything above
-    P, m, k, n = 16, 512, 64, 512
+    # results (16 x 1536 x 1536 doubles = 288 MiB) outgrow everything above and whatever tests run before this one left
+    P, m, k, n = 16, 1536, 64, 1536
     da, db, dc = DeviceBuffer.alloc(dtype, m, k, depth=P), DeviceBuffer.alloc(dtype, k, n, depth=P), DeviceBuffer.alloc(dtype, m, n)
     check(lib.prad_graph_begin())
     try:
