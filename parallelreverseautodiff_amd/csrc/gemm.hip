@@ -991,7 +991,13 @@ template <typename T>
 static bool gemm_thin_eligible(const GemmArgs<T>& a, bool edge, int epi, int64_t tiles) {
     static const int64_t max_k = [] { const char* e = getenv("PRAD_GEMM_THIN_MAX_K"); return e ? (int64_t)atoll(e) : (int64_t)128; }();
     static const int64_t min_tiles = [] { const char* e = getenv("PRAD_GEMM_THIN_MIN_TILES"); return e ? (int64_t)atoll(e) : (int64_t)384; }();
-    if (edge || a.ksplit != 0 || a.shared_splits > 1 || a.colsum_dst != nullptr || a.K > max_k || (PRAD_GEMM_FOLD_K > 0 && a.K > PRAD_GEMM_FOLD_K) || tiles * a.batch < min_tiles) return false;  // (no fold on it)
+    // A K of up to 384 goes there too while the tiles are no more than the full-depth kernel's 512 slots (two
+    // workgroups per compute unit): all tiles are resident at once either way, and three half-depth workgroups per
+    // compute unit start the later ones' loads sooner (the attention block's 288- and 384-deep layers on 392 tiles: +1 %
+    // on the step); on a thousand tiles, two full rounds of the full-depth kernel, K = 256 was measured 5 % slower.
+    static const int64_t one_round_max_k = [] { const char* e = getenv("PRAD_GEMM_THIN_ONE_ROUND_MAX_K"); return e ? (int64_t)atoll(e) : (int64_t)384; }();
+    const int64_t k_limit = (max_k > 0 && tiles * a.batch <= 512 && one_round_max_k > max_k) ? one_round_max_k : max_k;
+    if (edge || a.ksplit != 0 || a.shared_splits > 1 || a.colsum_dst != nullptr || a.K > k_limit || (PRAD_GEMM_FOLD_K > 0 && a.K > PRAD_GEMM_FOLD_K) || tiles * a.batch < min_tiles) return false;  // (no fold on it)
     return epi == EPI_PLAIN || epi == EPI_ELEMENTWISE;
 }
 
