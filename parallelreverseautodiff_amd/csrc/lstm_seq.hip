@@ -62,7 +62,7 @@ __device__ __forceinline__ void wait_for_stores() {
 // Waits until the `blocks` flags at `flags` have all reached `want` (called by every thread of the workgroup; the
 // first wavefront polls, one lane per flag).  Returns false - for the whole workgroup - when it gave up.
 __device__ __forceinline__ bool wait_for_group(const unsigned* flags, int blocks, unsigned want, unsigned* abort_word, int spin_limit,
-                                               int* verdict /* LDS */) {
+                                               int* all_arrived /* LDS */) {
     if (threadIdx.x < 64) {
         bool done = (int)threadIdx.x >= blocks;
         int spins = 0;
@@ -78,11 +78,11 @@ __device__ __forceinline__ bool wait_for_group(const unsigned* flags, int blocks
         }
         if (threadIdx.x == 0) {
             if (!ok) __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            *verdict = ok ? 1 : 0;
+            *all_arrived = ok ? 1 : 0;
         }
     }
     __syncthreads();
-    return *verdict != 0;
+    return *all_arrived != 0;
 }
 
 // The cell's sigmoid and tanh for the sequence kernel: float arithmetic on the hardware exponential and reciprocal
@@ -103,7 +103,7 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_fwd_kernel(const Lstm
     const int row = tid >> 4, u = tid & 15;                      // the element this thread finishes: (row, unit u)
     __shared__ __attribute__((aligned(16))) float hblock[SEQ_LDS_FLOATS];  // h_{t-1} rows of the group, as MFMA fragments (16 x hidden used)
     __shared__ float exch[4 * 16 * 16];                              // the four gates' products, [gate][row][unit]
-    __shared__ int verdict;
+    __shared__ int all_arrived;
     keep_allocated(hblock);
 
     // W_h slice of this wavefront in registers: vector j of lane (n, g) = W_h[16 j + 4 g + i][q H + 16 c + n], i = 0..3
@@ -142,7 +142,7 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_fwd_kernel(const Lstm
         float pre[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) pre[k] = grow[k * H];
-        if (t > 0 && !wait_for_group(group_flags, blocks, (unsigned)t, p.abort_word, p.spin_limit, &verdict)) return;
+        if (t > 0 && !wait_for_group(group_flags, blocks, (unsigned)t, p.abort_word, p.spin_limit, &all_arrived)) return;
         // h_{t-1} rows of the group -> LDS in fragment order: vector (j, g') of row m = h[m][16 j + 4 g' .. + 3] at slot (4 j + g') * 17 + m
         const float* hsrc = p.Hs + (int64_t)(t * B + 16 * r) * H;
         f4v hv[SEQ_STAGE];
@@ -196,7 +196,7 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_bwd_kernel(const Lstm
     const int row = tid >> 4, u = tid & 15;
     __shared__ __attribute__((aligned(16))) float dgblock[SEQ_LDS_FLOATS];  // this workgroup's dG block as fragments: vector (q, g', m) (16 x 64 used)
     keep_allocated(dgblock);
-    __shared__ int verdict;
+    __shared__ int all_arrived;
 
     // Rows of W_h^T for this workgroup's 64 gate columns, spread over the wavefronts by output unit: wavefront wv
     // produces partial dh for units [tile * 16, tile * 16 + 16), tile = wv + 4 y (y < blocks / 4); vector (y, q) of lane
@@ -272,7 +272,7 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_bwd_kernel(const Lstm
         __syncthreads();  // (also: dgblock is free again)
         if (tid == 0) __hip_atomic_store(my_flag, (unsigned)(s + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         in = load_step(t - 1);
-        if (!wait_for_group(group_flags, blocks, (unsigned)(s + 1), p.abort_word, p.spin_limit, &verdict)) return;
+        if (!wait_for_group(group_flags, blocks, (unsigned)(s + 1), p.abort_word, p.spin_limit, &all_arrived)) return;
         // the blocks meant for this workgroup, added in producer order
         const float* src = pbase + ((int64_t)(r * blocks + c) * blocks * 16) * 16 + row * 16 + u;
         float part[SEQ_MAX_J];
