@@ -29,6 +29,24 @@ def test_swin_block_matches_node_by_node_oracle(gpu, oracle, dtype, cfg):
     assert_parity(blk.dX.download(), dX, dtype, "dX")
 
 
+def test_swin_block_with_separate_attention_launches(gpu, oracle):
+    """The float block with the attention nodes as separate launches (strided-batched products, scaled softmax and its
+    backward) instead of one launch each way: against the oracle, and against the block as it runs by default."""
+    cfg = dict(images=2, side=28, embed=96, heads=3, dtype=np.float32)
+    apart, fused = SwinBlock(fused_attention=False, **cfg), SwinBlock(**cfg)
+    assert not apart.fused_attention and fused.fused_attention
+    apart.step(update=False); fused.step(update=False)
+    params = {k: apart.host[k] for k in apart.names}
+    loss, Y2, g, dX = compose.swin_block_forward_backward(params, apart.host["X"], apart.host["T"], apart.nw, apart.wt, 3)
+    assert abs(float(apart.loss.download()[0, 0]) - loss) <= 1e-5 * abs(loss)
+    assert_parity(apart.Y2.download(), Y2, np.float32, "block output")
+    assert_parity(apart.dX.download(), dX, np.float32, "dX")
+    for k in apart.names:
+        assert_parity(apart.g[k].download(), g[k], np.float32, "gradient of " + k)
+        assert_parity(fused.g[k].download(), apart.g[k].download(), np.float32, "gradient of %s, one launch against separate ones" % k)
+    assert_parity(fused.dQKV.download(), apart.dQKV.download(), np.float32, "dQKV, one launch against separate ones")
+
+
 def test_swin_benchmark_configuration_full_size(gpu, oracle):
     """The configuration the benchmark times, at its full size: 16 images of 56 x 56 tokens in 7 x 7 windows, embed 96,
     3 heads, float (50 176 token rows, 1024 windows).  The four weight gradients are sums over all 50 176 rows: see
