@@ -1,6 +1,7 @@
-// Windowed self-attention of one block, forward, per window and head in one launch (float, head dimension 32, up to 64
-// tokens per window): S = Q . K^T (MatrixMultiplyOperation, src/RMAD/MatrixMultiplyOperation.cs:50-86), scaled
-// (MatrixMultiplyScalarOperation), P = softmax rows (src/RMAD/SoftmaxOperation.cs:45-110), O = P . V - the node sequence
+// Windowed self-attention of one block per window and head, one launch forward and one backward (float, head dimension
+// 32, up to 64 tokens per window; the backward kernel is described where it stands).  Forward: S = Q . K^T
+// (MatrixMultiplyOperation, src/RMAD/MatrixMultiplyOperation.cs:50-86), scaled (MatrixMultiplyScalarOperation),
+// P = softmax rows (src/RMAD/SoftmaxOperation.cs:45-110), O = P . V - the node sequence
 // of examples/swin/SwinExample/SwinTransformerTools.cs:348-399.  As separate launches the 49 x 49 scores of 9216
 // windows x heads go to memory and back twice (two products of K = 32 and 49 at 26 us each and a softmax pass at 25 us,
 // all bound by that traffic).  Here one wavefront takes one (window, head): the scores stay in its accumulators and its
