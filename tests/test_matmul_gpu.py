@@ -528,6 +528,9 @@ def test_products_of_few_tiles_and_long_k(gpu, oracle, dtype, shape):
         else:
             for a, b2 in zip(first, got):
                 assert np.array_equal(a, b2), "run %d differs from run 0" % run
+    # accumulation into the output: the same product added to itself is exactly twice its bits
+    check(lib.prad_gemm(0, 0, bA.handle, bB.handle, C.handle, 1))
+    assert np.array_equal(C.download(), first[0] + first[0]), "C += A . B"
     if dtype == np.float32 and K >= 4096:
         # The float oracle adds 4096 terms one by one and is itself about 1e-5 off the exact sum, more than the GPU's
         # blocked sums are; both are therefore held against the product taken in double and rounded once.
