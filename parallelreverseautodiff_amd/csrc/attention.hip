@@ -2,7 +2,7 @@
 // 32, up to 64 tokens per window; the backward kernel is described where it stands).  Forward: S = Q . K^T
 // (MatrixMultiplyOperation, src/RMAD/MatrixMultiplyOperation.cs:50-86), scaled (MatrixMultiplyScalarOperation),
 // P = softmax rows (src/RMAD/SoftmaxOperation.cs:45-110), O = P . V - the node sequence
-// of examples/swin/SwinExample/SwinTransformerTools.cs:348-399.  As separate launches the 49 x 49 scores of 9216
+// of examples/swin/SwinExample/SwinTransformerTools.cs:348-399.  As separate launches the 49 x 49 scores of 3072
 // windows x heads go to memory and back twice (two products of K = 32 and 49 at 26 us each and a softmax pass at 25 us,
 // all bound by that traffic).  Here one wavefront takes one (window, head): the scores stay in its accumulators and its
 // LDS tile, only P - which the backward pass needs - is written, and Q, K, V are read once.
@@ -58,13 +58,19 @@ __device__ __forceinline__ float dot8(const f4a (&a)[2], const f4a (&b)[2]) {
 // exactly 49 tokens - three 16 x 16 tiles each way on the matrix cores and the 49th row and column (a fringe that would
 // cost seven more tiles of sixteen, all but one row or column of each padding) as dot products on the vector unit.
 template <int KS, bool FR>
-__global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel(const AttArgs p) {
+__global__ void __launch_bounds__(64 * ATT_WAVES, FR ? 3 : 2) window_attention_fwd_kernel(const AttArgs p) {
     constexpr int TX = FR ? 3 : 4;    // 16 x 16 tiles each way on the matrix cores
     constexpr int NC = FR ? 49 : 64;  // columns the softmax walks
+    // FR: nothing reaches past row 48 or column 51, and a tile of 49 x 53 lets three workgroups share a compute unit
+    // instead of two: the 3072 (window, head) pairs of the 16 x 56 x 56 block are then resident at once, three to a SIMD,
+    // instead of a round and a half of two (31 -> 27 us).  The backward kernel needs 220 registers, more than three
+    // wavefronts to a SIMD leave each (168): tried with the loads of its last operands moved down, it spilled and ran at
+    // 49 us against 46.
+    constexpr int ROWS = FR ? 49 : 64, PITCH = FR ? 53 : ATT_PITCH;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int li = lane & 15, g = lane >> 4;
     const int64_t pair = (int64_t)blockIdx.x * ATT_WAVES + wave;  // (window, head), heads innermost
-    __shared__ float tiles[ATT_WAVES][64 * ATT_PITCH];
+    __shared__ float tiles[ATT_WAVES][ROWS * PITCH];
     if (pair >= (int64_t)p.windows * p.heads) return;
     const int w = (int)(pair / p.heads), h = (int)(pair % p.heads);
     const int wt = FR ? 49 : p.tokens, C = p.heads * ATT_HD, ld = 3 * C;
@@ -117,10 +123,10 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel
         if (g == 0) {
 #pragma unroll
             for (int y = 0; y < 3; ++y) {
-                tile[48 * ATT_PITCH + 16 * y + li] = fr[y];
-                tile[(16 * y + li) * ATT_PITCH + 48] = fc[y];
+                tile[48 * PITCH + 16 * y + li] = fr[y];
+                tile[(16 * y + li) * PITCH + 48] = fc[y];
             }
-            if (li == 0) tile[48 * ATT_PITCH + 48] = corner;
+            if (li == 0) tile[48 * PITCH + 48] = corner;
         }
     }
 #pragma unroll
@@ -128,15 +134,15 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel
 #pragma unroll
         for (int y = 0; y < TX; ++y)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) tile[(16 * x + 4 * g + r) * ATT_PITCH + 16 * y + li] = acc[x][y][r];
+            for (int r = 0; r < 4; ++r) tile[(16 * x + 4 * g + r) * PITCH + 16 * y + li] = acc[x][y][r];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     // softmax of row `lane` (the arithmetic of softmax_fwd_rows_kernel); the columns past the window become zeros
     // (with FR the rows past the window hold whatever the tile held: nothing reads them)
-    {
-        float* __restrict__ row = tile + lane * ATT_PITCH;
+    if (!FR || lane < ROWS) {
+        float* __restrict__ row = tile + lane * PITCH;
         float v[NC];
 #pragma unroll
         for (int j = 0; j < NC; ++j) v[j] = j < wt ? row[j] * p.scale : -INFINITY;
@@ -164,7 +170,7 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel
         int r = lane / wt, c = lane % wt;  // element lane + 64 i
         const int dr = 64 / wt, dc = 64 % wt;
         for (int e = lane; e < wt * wt; e += 64) {
-            dst[e] = tile[r * ATT_PITCH + c];
+            dst[e] = tile[r * PITCH + c];
             r += dr; c += dc;
             if (c >= wt) { c -= wt; ++r; }
         }
@@ -181,7 +187,7 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel
     for (int s = 0; s < KS; ++s) {
         float a[TX];
 #pragma unroll
-        for (int x = 0; x < TX; ++x) a[x] = tile[(16 * x + li) * ATT_PITCH + 4 * s + g];
+        for (int x = 0; x < TX; ++x) a[x] = tile[(16 * x + li) * PITCH + 4 * s + g];
 #pragma unroll
         for (int x = 0; x < TX; ++x)
 #pragma unroll
@@ -192,7 +198,7 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, 2) window_attention_fwd_kernel
         float o2[2] = {0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-            const float pv = tile[48 * ATT_PITCH + 4 * s + g];
+            const float pv = tile[48 * PITCH + 4 * s + g];
 #pragma unroll
             for (int y = 0; y < 2; ++y) o2[y] += pv * vf[s][y];
         }
