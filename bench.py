@@ -2,7 +2,9 @@
 
 One step = MatrixMultiplyOperation forward (C = A.B) plus backward (dA = dC.B^T, dB = A^T.dC) on
 device-resident square double matrices, N = 4096 by default: three launches of the MFMA product
-kernel, 6 N^3 floating-point operations.  Prints ONE JSON line.
+kernel, 6 N^3 floating-point operations.  The LAST line printed is one compact JSON object (the
+figures of the headline leg with its roofline and CPU baseline, under 1800 characters); the line
+before it, also written to gpurun_out/bench_detail.json, carries every other leg and the table.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--n N] [--dtype f64|f32] [--no-cpu]
 """
@@ -104,6 +106,23 @@ def gpu_leg(n, dtype_name, steps, warmup, with_errors=True):
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms = ctypes.c_float()
     check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    # each of the three launches alone between two events, the stream idle before it: the duration a kernel trace shows
+    # for a launch, where back-to-back launches above overlap one launch's drain with the next one's ramp
+    isolated = {}
+    for name, call in (("NN C=A.B", lambda: lib.prad_gemm(0, 0, h["A"], h["B"], h["C"], 0)),
+                       ("NT dA=dC.B^T", lambda: lib.prad_gemm(0, 1, h["dC"], h["B"], h["dA"], 0)),
+                       ("TN dB=A^T.dC", lambda: lib.prad_gemm(1, 0, h["A"], h["dC"], h["dB"], 0))):
+        total = 0.0
+        reps = max(3, min(steps, 10))
+        for _ in range(reps):
+            check(lib.prad_stream_sync())
+            check(lib.prad_event_record(e0))
+            check(call())
+            check(lib.prad_event_record(e1))
+            one = ctypes.c_float()
+            check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(one)))
+            total += one.value
+        isolated[name] = total / reps
     # spot check of the timed buffers: a few entries against exactly rounded dot products
     import math
     C = bufs["C"].download()
@@ -117,7 +136,7 @@ def gpu_leg(n, dtype_name, steps, warmup, with_errors=True):
     if not worst <= tol:
         raise SystemExit("benchmark output failed its spot check: %.3e" % worst)
     errors = gemm_sample_errors(A, B, dC, C, bufs["dA"].download(), bufs["dB"].download(), dtype) if with_errors else None
-    return {"ms": float(ms.value), "wall_ms": wall_ms, "spot": worst, "errors": errors}
+    return {"ms": float(ms.value), "wall_ms": wall_ms, "spot": worst, "errors": errors, "isolated_launch_ms": isolated}
 
 
 def bandwidth_leg(n_elems, dtype_name, steps, warmup, only=None):
@@ -456,6 +475,56 @@ def mlp_leg(dtype_name, steps, warmup, with_cpu):
     return out
 
 
+def mlp_ops_leg(dtype_name, steps, warmup):
+    """The configs[0] step driven operation by operation through the operation classes, in the reference's order
+    (MatrixMultiplyOperation.Forward -> MatrixAddBroadcastingOperation -> LeakyReLUOperation ... -> loss -> the
+    Backward chain with accumulate_gradient into the gradient destinations -> GradientClearer / GradientClipper.Clip /
+    AdamOptimizer.Optimize): no fused entry point, no recorded sequence, a fresh output Matrix per call.  This is the
+    rate an unchanged caller of the operation classes gets; the host side here is Python, so its figure is the wall
+    clock of the loop, and the time the device is busy is given beside it."""
+    from parallelreverseautodiff_amd import _lib, seeded
+    from parallelreverseautodiff_amd.cudablas import CudaBlas
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.feedforward import OperationWalkNetwork
+
+    lib = _lib.load()
+    CudaBlas.Instance.DeviceId = 0
+    CudaBlas.Instance.Initialize()
+    dtype = np.float64 if dtype_name == "f64" else np.float32
+    net = OperationWalkNetwork(dtype=dtype)
+    net.set_batch(seeded.uniform(seeded.DEFAULT_SEED, 1, (64, 784), 0.0, 1.0, dtype),
+                  seeded.one_hot_labels(seeded.DEFAULT_SEED, 2, 64, 10, dtype))
+
+    def stats():
+        vals = [ctypes.c_int64() for _ in range(5)]
+        check(lib.prad_alloc_stats(*[ctypes.byref(v) for v in vals]))
+        return [v.value for v in vals]
+
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.prad_event_create(ctypes.byref(e0)))
+    check(lib.prad_event_create(ctypes.byref(e1)))
+    for _ in range(max(warmup, 3)):
+        net.step()
+    check(lib.prad_stream_sync())
+    before = stats()
+    t0 = time.perf_counter()
+    check(lib.prad_event_record(e0))
+    for _ in range(steps):
+        net.step()
+    check(lib.prad_event_record(e1))
+    issue_ms = (time.perf_counter() - t0) * 1e3 / steps      # host time to issue a step (nothing waits for the device)
+    check(lib.prad_stream_sync())
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    after = stats()
+    ms = ctypes.c_float()
+    check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    return {"wall_ms_per_step": wall_ms, "host_issue_ms_per_step": issue_ms, "device_ms_per_step": ms.value / steps,
+            "steps_per_s": 1e3 / wall_ms, "loss_after": float(net.loss.to_numpy()[0, 0]), "flop_per_step": net.flops_per_step(),
+            "operations_per_step": 2 * len(net.nodes) + 2, "device_mallocs_in_timed_steps": after[0] - before[0],
+            "device_frees_in_timed_steps": after[1] - before[1], "stream_waits_in_timed_steps": after[2] - before[2],
+            "pool_hits_in_timed_steps": after[3] - before[3]}
+
+
 def mlp_cpu_leg(W0, X, T, params, dtype, budget_s=15.0):
     """The same step composed from the oracle's restatements of the reference operations, on the host."""
     from oracle import oracle
@@ -537,7 +606,7 @@ def main():
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="gemm mode: skip the other-precision and MLP legs")
-    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "matmul_sum", "lstm", "swin", "oneshot"], default="gemm",
+    ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "mlp_ops", "matmul_sum", "lstm", "swin", "oneshot"], default="gemm",
                     help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
                          "mlp: the feed-forward training step of configs[0]")
     ap.add_argument("--elems", type=int, default=64 * 1024 * 1024, help="elements per tensor in bandwidth mode")
@@ -588,6 +657,15 @@ def main():
                                                  "cross-entropy, clip(4), Adam(lr 1e-3): forward + backward + update"},
                           "detail": res}))
         return
+    if args.mode == "mlp_ops":
+        res = mlp_ops_leg(args.dtype, args.steps, args.warmup)
+        print(json.dumps({"metric": "MLP train steps/sec, operation by operation", "unit": "steps/s", "value": res["steps_per_s"],
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
+                          "higher_is_better": True, "ms_per_step": res["wall_ms_per_step"],
+                          "config": {"workload": "configs[0] driven through the operation classes one Forward / Backward at a time: "
+                                                 "fresh outputs per call, accumulate_gradient, GradientClipper.Clip, AdamOptimizer.Optimize"},
+                          "detail": res}))
+        return
     if args.mode == "bandwidth":
         res, n = bandwidth_leg(args.elems, args.dtype, args.steps, args.warmup, [x for x in args.only.split(",") if x])
         best = max(res.values(), key=lambda r: r["GB/s"])
@@ -598,42 +676,112 @@ def main():
         return
 
     head = gpu_leg(args.n, args.dtype, args.steps, args.warmup, with_errors=not args.no_cpu)
-    ms, wall_ms, spot = head["ms"], head["wall_ms"], head["spot"]
-    flops_per_step = 6.0 * args.n ** 3
-    ms_per_step = ms / args.steps
+    cpu = None if args.no_cpu else cpu_leg()
+    ms_per_step = head["ms"] / args.steps
+    table = [gemm_row(args.n, args.dtype, ms_per_step, head["errors"], cpu)]
+    also = None if args.no_also else also_legs(args, table)
+    line, detail = headline_lines(args, head, cpu, also, table)
+    text = json.dumps({"detail": detail})
+    print(text)
+    try:  # the same detail as a file, for runs whose captured output is cut short
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_detail.json"), "w") as f:
+            f.write(text + "\n")
+    except OSError:
+        pass
+    sys.stdout.flush()
+    print(json.dumps(line, separators=(",", ":")))
+
+
+MAX_LINE_CHARS = 1800  # the harness that runs this keeps the tail of stdout: the last line has to fit in it
+
+
+def headline_lines(args, head, cpu, also, table):
+    """(the compact last line, the detail object) of the headline run from its legs' results.  Everything bulky - the
+    error blocks, the other legs with their rooflines, the table - goes into the detail object; the last line holds
+    the contract's fields, the roofline and CPU baseline of the headline kernel, and a few scalars of the other legs."""
+    n, steps = args.n, args.steps
+    flops_per_step = 6.0 * n ** 3
+    ms_per_step = head["ms"] / steps
     tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
     peak = PEAK_TFLOPS[args.dtype]
     # dominant kernel: the MFMA product kernel, three launches per step of 2 N^3 flop each
-    launch_ms = ms / (3 * args.steps)
-    achieved = 2.0 * args.n ** 3 / (launch_ms * 1e-3) / 1e12
+    launch_ms = head["ms"] / (3 * steps)
+    achieved = 2.0 * n ** 3 / (launch_ms * 1e-3) / 1e12
+    iso = head.get("isolated_launch_ms") or {}
+    iso_mean = sum(iso.values()) / len(iso) if iso else None
+    sig = lambda x, d=5: None if x is None else float("%.*g" % (d, x))
     line = {
-        "metric": METRIC, "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "metric": METRIC, "value": sig(tflops), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": sig(ms_per_step), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": "configs[1]: single MatrixMultiplyOperation forward+backward, %s, square M=N=K=%d, "
-                               "A,B~U[-1,1], dC~N(0,1), seed %d, device-resident" % (args.dtype, args.n, 20240611),
-                   "flop_per_step": flops_per_step, "launches_per_step": 3},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
-                     "traffic": load_traffic(args.n, args.dtype), "kernel": "prad::gemm_kernel<%s> (NN, NT, TN instantiations)" %
-                     ("double" if args.dtype == "f64" else "float"), "launch_ms": launch_ms},
-        "wall_ms_per_step": wall_ms / args.steps, "spot_check_error": spot,
+        "config": {"workload": "configs[1]: MatrixMultiplyOperation forward+backward, %s, M=N=K=%d, A,B~U[-1,1], dC~N(0,1), seed %d, "
+                               "device-resident, 3 launches, 6N^3 flop/step" % (args.dtype, n, 20240611)},
+        "roofline": {"bound": "mfma", "achieved": sig(achieved), "peak": peak, "unit": "TFLOP/s", "frac": sig(achieved / peak, 4),
+                     "traffic": load_traffic(n, args.dtype), "kernel": "prad::gemm_kernel<%s> NN/NT/TN" % ("double" if args.dtype == "f64" else "float"),
+                     "launch_ms": sig(launch_ms), "launch_ms_isolated": sig(iso_mean),
+                     "frac_isolated": None if not iso_mean else sig(2.0 * n ** 3 / (iso_mean * 1e-3) / 1e12 / peak, 4)},
     }
-    if head["errors"] is not None:
-        line["errors"] = head["errors"]
-    cpu = None if args.no_cpu else cpu_leg()
-    table = [gemm_row(args.n, args.dtype, ms_per_step, head["errors"], cpu)]
-    if not args.no_also:
-        line["also"] = also_legs(args, table)
     if cpu is not None:
-        line["cpu_baseline"] = cpu
-    line["table"] = table
-    print(json.dumps(line))
+        line["cpu_baseline"] = {"value": sig(cpu["value"]), "unit": cpu["unit"], "cores": cpu["cores"], "kind": cpu["kind"],
+                                "sample": "fp64 fwd+bwd at N=%d, 1 pass, %.1f s" % (cpu["n"], cpu["secs"])}
+    detail = {"headline": {"wall_ms_per_step": head["wall_ms"] / steps, "spot_check_error": head["spot"], "errors": head["errors"],
+                           "isolated_launch_ms": iso, "flop_per_step": flops_per_step, "launches_per_step": 3},
+              "cpu_baseline": cpu, "also": also, "table": table}
+    if head["errors"] is not None:
+        line["err_vs_reference_arithmetic"] = sig(head["errors"]["against_reference_arithmetic"]["elementwise_floor_rms"], 3)
+    extras = summary_scalars(also) if also else {}
+    for key, value in extras.items():  # scalars of the other legs, as many as fit
+        line.setdefault("also", {})[key] = value
+        if len(json.dumps(line, separators=(",", ":"))) > MAX_LINE_CHARS:
+            del line["also"][key]
+            break
+    return line, detail
 
 
-def mfma_roofline(flops, ms, dtype_name, kernel):
+def summary_scalars(also):
+    """A few scalars of the other legs for the last line (their full results are in the detail object)."""
+    out = {}
+    sig = lambda x: float("%.4g" % x)
+
+    def put(key, leg, *path):
+        try:
+            v = also[leg]
+            for k in path:
+                v = v[k]
+            out[key] = sig(v)
+        except (KeyError, TypeError):
+            pass
+    for leg in also:
+        if leg.startswith("matmul_fwd_bwd_"):
+            put(leg.replace("matmul_fwd_bwd_", "") + "_frac", leg, "roofline", "frac")
+    put("mlp_f64_steps_s", "mlp_train_steps_per_s_f64", "value")
+    put("mlp_f64_cpu_steps_s", "mlp_train_steps_per_s_f64", "cpu_baseline", "steps_per_s")
+    put("mlp_ops_f64_steps_s", "mlp_operation_walk_f64", "value")
+    put("mlp_f32_steps_s", "mlp_train_steps_per_s_f32", "value")
+    put("mlp_ops_f32_steps_s", "mlp_operation_walk_f32", "value")
+    put("lstm_f32_steps_s", "lstm_train_steps_per_s_f32", "value")
+    put("lstm_f32_frac", "lstm_train_steps_per_s_f32", "roofline", "frac")
+    put("swin_f32_steps_s", "swin_block_train_steps_per_s_f32", "value")
+    put("swin_f32_frac", "swin_block_train_steps_per_s_f32", "roofline", "frac")
+    put("matmulsum_fwd_frac", "matmul_and_sum_f32", "forward", "roofline", "frac")
+    put("matmulsum_bwd_hbm_frac", "matmul_and_sum_f32", "backward", "roofline", "frac")
+    for d in ("f64", "f32"):
+        leg = also.get("gradient_kernels_64Mi_" + d)
+        if isinstance(leg, dict) and "error" not in leg:
+            fr = {k: v["roofline"]["frac"] for k, v in leg.items()}
+            out["adam_%s_hbm_frac" % d] = sig(fr.get("adam", 0.0))
+            out["min_act_bwd_%s_hbm_frac" % d] = sig(min(v for k, v in fr.items() if k.endswith("_bwd")))
+    failed = [k for k, v in also.items() if isinstance(v, dict) and "error" in v]
+    if failed:
+        out["failed_legs"] = len(failed)
+    return out
+
+
+def mfma_roofline(flops, ms, dtype_name, kernel, traffic=None):
     achieved = flops / (ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS[dtype_name], "unit": "TFLOP/s",
-            "frac": achieved / PEAK_TFLOPS[dtype_name], "traffic": None, "kernel": kernel}
+            "frac": achieved / PEAK_TFLOPS[dtype_name], "traffic": traffic, "kernel": kernel}
 
 
 def hbm_roofline(nbytes, ms, kernel):
@@ -689,8 +837,9 @@ def also_legs(args, table):
             r = gpu_leg(n, d, steps, args.warmup, with_errors=with_cpu)
             per = r["ms"] / steps
             out[key] = {"TFLOPs": 6.0 * n ** 3 / (per * 1e-3) / 1e12, "n": n, "ms_per_step": per, "spot_check_error": r["spot"],
-                        "roofline": mfma_roofline(2.0 * n ** 3, per / 3, d, "prad::gemm_kernel<%s>" % ("double" if d == "f64" else "float")),
-                        "errors": r["errors"]}
+                        "roofline": mfma_roofline(2.0 * n ** 3, per / 3, d, "prad::gemm_kernel<%s>" % ("double" if d == "f64" else "float"),
+                                                  traffic=load_traffic(n, d)),
+                        "isolated_launch_ms": r["isolated_launch_ms"], "errors": r["errors"]}
             table.append(gemm_row(n, d, per, r["errors"], None))
         except Exception as e:  # noqa: BLE001 - reported, not hidden
             out[key] = {"error": repr(e)}
@@ -707,6 +856,18 @@ def also_legs(args, table):
             table.append(step_row("configs[0] MLP 784-256-128-10 batch 64 step", d, r))
         except Exception as e:  # noqa: BLE001
             out["mlp_train_steps_per_s_" + d] = {"error": repr(e)}
+    for d in ("f64", "f32"):
+        try:
+            r = mlp_ops_leg(d, 300, 20)
+            out["mlp_operation_walk_" + d] = {"value": r["steps_per_s"], "unit": "steps/s", "ms_per_step": r["wall_ms_per_step"], "detail": r,
+                                               "roofline": mfma_roofline(r["flop_per_step"], r["wall_ms_per_step"], d,
+                                                                         "whole step, one launch per operation (%d operations)" % r["operations_per_step"])}
+            table.append({"config": "configs[0] MLP step, operation by operation through the operation classes", "precision": d,
+                          "gpu_ms": r["wall_ms_per_step"], "rate": r["steps_per_s"], "unit": "steps/s", "bound": "mfma",
+                          "frac_of_peak": r["flop_per_step"] / (r["wall_ms_per_step"] * 1e-3) / 1e12 / PEAK_TFLOPS[d],
+                          "cpu_ms": None, "cpu_cores": None, "speedup": None, "err_normwise": None, "err_elementwise_floor_1e-3_rms": None})
+        except Exception as e:  # noqa: BLE001
+            out["mlp_operation_walk_" + d] = {"error": repr(e)}
     for name, fn, config, kernel in (
             ("lstm_train_steps_per_s_f32", lstm_leg, "configs[3] LSTM 256->512 batch 128 T=64 step",
              "whole step: 2 x 64 recurrent launches + 5 large products"),
@@ -732,7 +893,7 @@ def also_legs(args, table):
                       "cpu_ms": None, "cpu_cores": None, "speedup": None, "err_normwise": None, "err_elementwise_floor_1e-3_rms": None})
         table.append({"config": "configs[2] MatrixMultiplyAndSum backward (as the reference writes it)", "precision": "f32", "gpu_ms": r["bwd_ms"],
                       "rate": r["bwd_GBps"], "unit": "GB/s", "bound": "hbm", "frac_of_peak": r["bwd_frac_of_8TBps"],
-                      "cpu_ms": None, "cpu_cores": None, "speedup": None, "err_normwise": 0.0, "err_elementwise_floor_1e-3_rms": 0.0})
+                      "cpu_ms": None, "cpu_cores": None, "speedup": None, "err_normwise": None, "err_elementwise_floor_1e-3_rms": None})
     except Exception as e:  # noqa: BLE001
         out["matmul_and_sum_f32"] = {"error": repr(e)}
     for d in ("f64", "f32"):

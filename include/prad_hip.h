@@ -77,9 +77,27 @@ void* prad_stream(void);           /* getter: the library's hipStream_t, for cal
  *      GetAsArray2D / ToJagged of src/RMAD/GpuMatrixMultiplyOperation.cs:170-271 ----------- */
 int32_t prad_buf_alloc(int32_t dtype, int64_t rows, int64_t cols, prad_buf_t* out); /* zero-filled, like new Matrix(rows, cols) */
 int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out); /* DeepMatrix: depth contiguous slices; src/RMAD/DeepMatrix.cs:22 */
+/* The same without the zero fill, for an output that the next call overwrites whole (a product with accumulate == 0, an
+ * activation, a transpose): the fresh output Matrix every Forward / Backward of the reference allocates
+ * (e.g. src/RMAD/MatrixMultiplyOperation.cs:64, :91, :107) without a launch spent on zeros that are never read.
+ * Contents are undefined until written. */
+int32_t prad_buf_alloc_output(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out);
 int32_t prad_buf_wrap(int32_t dtype, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out); /* borrow caller-owned device memory */
 int32_t prad_buf_wrap_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out); /* the same for depth contiguous slices (a tensor of more than two dimensions: Tensor.Shape, src/PRAD/Tensor.cs) */
+/* Owned device memory goes back to a pool inside the library, by size class, without waiting for the device and
+ * without hipFree: the reference's pattern is a fresh output Matrix per operation per step, released by the garbage
+ * collector (src/RMAD/GpuMatrixMultiplyOperation.cs:190-201 allocates and drops three device arrays per call), and the
+ * next allocation of the class takes the block back.  One in-order stream makes the reuse safe.  A buffer that a
+ * recorded launch sequence addresses must outlive the sequence. */
 int32_t prad_buf_free(prad_buf_t b);
+/* Gives the pooled blocks back to the device (waits for the stream).  The pool also releases them by itself when an
+ * allocation would otherwise fail, and never holds more than half of the device memory (PRAD_POOL_MAX_BYTES overrides). */
+int32_t prad_pool_trim(void);
+/* Counters since the library was loaded, any of which may be NULL: hipMalloc calls and hipFree calls for matrices,
+ * waits for the stream, allocations served from the pool, bytes the pool holds now.  For tests and tuning: a training
+ * step in its steady state adds nothing to the first three. */
+int32_t prad_alloc_stats(int64_t* device_mallocs, int64_t* device_frees, int64_t* stream_syncs, int64_t* pool_hits,
+                         int64_t* pooled_bytes);
 int32_t prad_buf_shape(prad_buf_t b, int64_t* depth, int64_t* rows, int64_t* cols, int32_t* dtype);
 void* prad_buf_device_ptr(prad_buf_t b); /* getter: NULL for a bad handle */
 int32_t prad_buf_zero(prad_buf_t b);

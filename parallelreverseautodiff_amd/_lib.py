@@ -44,6 +44,9 @@ SIGNATURES = {
     "prad_stream": (_vp, []),
     "prad_buf_alloc": (_i32, [_i32, _i64, _i64, _vpp]),
     "prad_buf_alloc_deep": (_i32, [_i32, _i64, _i64, _i64, _vpp]),
+    "prad_buf_alloc_output": (_i32, [_i32, _i64, _i64, _i64, _vpp]),
+    "prad_pool_trim": (_i32, []),
+    "prad_alloc_stats": (_i32, [_i64p, _i64p, _i64p, _i64p, _i64p]),
     "prad_buf_wrap": (_i32, [_i32, _i64, _i64, _vp, _vpp]),
     "prad_buf_wrap_deep": (_i32, [_i32, _i64, _i64, _i64, _vp, _vpp]),
     "prad_buf_free": (_i32, [_vp]),

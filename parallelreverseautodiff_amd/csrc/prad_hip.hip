@@ -15,6 +15,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <map>
 #include <string>
 #include <thread>
 #include <vector>
@@ -27,6 +28,7 @@ struct prad_buf {
     int64_t depth, rows, cols;
     void* ptr;
     bool owned;
+    size_t block_bytes;  // size class of the device block behind an owned buffer (0 for borrowed memory)
 };
 
 // Scratch of the allocation-free entry point (prad_clip_adam_multi_noalloc): device memory that exists from the
@@ -68,6 +70,14 @@ struct Context {
     unsigned* seq_flags = nullptr;
     unsigned* seq_abort = nullptr;          // hipHostMalloc'ed, also the address the kernels use
     int compute_units = 0;
+    // Device blocks that prad_buf_free handed back, by size class.  Everything the library enqueues runs on the one
+    // stream in lock order, so a block may be handed out again at once: whatever still reads or writes it is ahead
+    // in the stream of whatever the next owner enqueues.
+    std::map<size_t, std::vector<void*>> pool;
+    size_t pool_bytes = 0;
+    size_t pool_limit = 0;                  // half of the device memory, or PRAD_POOL_MAX_BYTES
+    bool poison_outputs = false;            // PRAD_POISON_OUTPUTS=1: unfilled outputs start as NaN bit patterns (a testing aid)
+    int64_t stat_device_mallocs = 0, stat_device_frees = 0, stat_stream_syncs = 0, stat_pool_hits = 0;
 };
 Context g_ctx;
 #define CUR_STREAM (g_ctx.stream)
@@ -122,6 +132,7 @@ inline int64_t count(prad_buf_t b) { return b->depth * b->rows * b->cols; }
 
 // Lock must be held.  Waits for everything enqueued on the library stream.
 int32_t sync_all() {
+    ++g_ctx.stat_stream_syncs;
     if (g_ctx.stream) HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
     if (g_ctx.seq_abort != nullptr && *static_cast<volatile unsigned*>(g_ctx.seq_abort) != 0u) {
         *static_cast<volatile unsigned*>(g_ctx.seq_abort) = 0u;
@@ -166,6 +177,60 @@ int32_t ensure_workspace(size_t bytes) {
     }
     g_ctx.workspace = fresh;
     g_ctx.workspace_bytes = bytes;
+    return PRAD_OK;
+}
+
+// ---- device blocks of the matrices -----------------------------------------------------------------------
+// Size class of a block: quarter-octave steps (at most a quarter more than asked for), 256 bytes at least.
+inline size_t size_class(size_t bytes) {
+    if (bytes <= 256) return 256;
+    const int top = 63 - __builtin_clzll((unsigned long long)(bytes - 1));  // bytes - 1 lies in [2^top, 2^(top+1))
+    const size_t step = (size_t)1 << (top - 2);
+    return (bytes + step - 1) & ~(step - 1);
+}
+// Lock held.  Gives every pooled block back to the device (after waiting for the stream: queued work may still use them).
+int32_t pool_release_all() {
+    if (g_ctx.pool_bytes == 0) return PRAD_OK;
+    if (int32_t st = sync_all()) return st;
+    for (auto& kv : g_ctx.pool)
+        for (void* p : kv.second) { (void)hipFree(p); ++g_ctx.stat_device_frees; }
+    g_ctx.pool.clear();
+    g_ctx.pool_bytes = 0;
+    return PRAD_OK;
+}
+// Lock held.  A block of at least `bytes`: one that prad_buf_free handed back if there is one of that class, else a
+// fresh one (when the device is out of memory the pooled blocks are released and the allocation is tried again).
+int32_t pool_take(size_t bytes, void** out, size_t* klass) {
+    *klass = size_class(bytes);
+    auto it = g_ctx.pool.find(*klass);
+    if (it != g_ctx.pool.end() && !it->second.empty()) {
+        *out = it->second.back();
+        it->second.pop_back();
+        g_ctx.pool_bytes -= *klass;
+        ++g_ctx.stat_pool_hits;
+        return PRAD_OK;
+    }
+    hipError_t e = hipMalloc(out, *klass);
+    if (e == hipErrorOutOfMemory && g_ctx.pool_bytes > 0) {
+        (void)hipGetLastError();
+        if (int32_t st = pool_release_all()) return st;
+        e = hipMalloc(out, *klass);
+    }
+    if (e != hipSuccess) return fail(PRAD_ERR_ALLOC, "hipMalloc of %zu bytes failed: %s", *klass, hipGetErrorString(e));
+    ++g_ctx.stat_device_mallocs;
+    return PRAD_OK;
+}
+// Lock held.  No wait and no hipFree: the block is kept for the next allocation of its class, unless the pool
+// already holds its share of the device memory.
+int32_t pool_give(void* p, size_t klass) {
+    if (g_ctx.pool_bytes + klass > g_ctx.pool_limit) {
+        if (int32_t st = sync_all()) return st;
+        HIP_TRY(hipFree(p), PRAD_ERR_ALLOC);
+        ++g_ctx.stat_device_frees;
+        return PRAD_OK;
+    }
+    g_ctx.pool[klass].push_back(p);
+    g_ctx.pool_bytes += klass;
     return PRAD_OK;
 }
 
@@ -480,6 +545,9 @@ int32_t prad_init(int32_t device_id) {
     HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&g_ctx.seq_abort), 64, hipHostMallocDefault), PRAD_ERR_ALLOC);
     *g_ctx.seq_abort = 0u;
     g_ctx.compute_units = std::min<int>(prop.multiProcessorCount, (int)(SEQ_FLAG_BYTES / sizeof(unsigned)));
+    g_ctx.pool_limit = prop.totalGlobalMem / 2;
+    if (const char* cap = getenv("PRAD_POOL_MAX_BYTES")) g_ctx.pool_limit = (size_t)strtoull(cap, nullptr, 10);
+    if (const char* poison = getenv("PRAD_POISON_OUTPUTS")) g_ctx.poison_outputs = poison[0] == '1';
     g_ctx.recording = false;
     g_ctx.live_graphs = 0;
     g_ctx.device = device_id;
@@ -492,6 +560,7 @@ int32_t prad_shutdown(void) {
     if (!g_ctx.initialized.load()) return PRAD_OK;
     (void)hipSetDevice(g_ctx.device);
     (void)sync_all();
+    (void)pool_release_all();
     if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
     if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
     free_retired_workspaces();
@@ -524,7 +593,9 @@ int32_t prad_stream_sync(void) {
 }
 
 // ---------------------------------------------------------------------------------------------
-int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out) {
+// Lock taken here.  zero_fill: new Matrix(rows, cols) starts at zero (src/RMAD/Matrix.cs:43-55); an output that the
+// next kernel overwrites whole needs no fill launch.
+static int32_t buf_alloc(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, bool zero_fill, prad_buf_t* out) {
     REQUIRE_INIT();
     if (out == nullptr) return fail(PRAD_ERR_ARG, "out is NULL");
     *out = nullptr;
@@ -532,21 +603,50 @@ int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t 
     if (depth <= 0 || rows <= 0 || cols <= 0) return fail(PRAD_ERR_ARG, "matrix dimensions must be positive");
     const size_t bytes = (size_t)depth * rows * cols * elem_size(dtype);
     void* p = nullptr;
+    size_t klass = 0;
     ENQUEUE_LOCK();
     NOT_WHILE_RECORDING("an allocation");
-    HIP_TRY(hipMalloc(&p, bytes), PRAD_ERR_ALLOC);
-    {
+    if (int32_t st = pool_take(bytes, &p, &klass)) return st;
+    if (zero_fill) {
         hipError_t e = dtype == PRAD_F64 ? launch_fill_zero<double>(static_cast<double*>(p), depth * rows * cols, CUR_STREAM)
                                          : launch_fill_zero<float>(static_cast<float*>(p), depth * rows * cols, CUR_STREAM);
-        if (e != hipSuccess) { (void)hipFree(p); return fail(PRAD_ERR_LAUNCH, "zero fill failed: %s", hipGetErrorString(e)); }
+        if (e != hipSuccess) { (void)pool_give(p, klass); return fail(PRAD_ERR_LAUNCH, "zero fill failed: %s", hipGetErrorString(e)); }
+    } else if (g_ctx.poison_outputs) {
+        // every byte 0xFF is a NaN in both element types: an output that its kernel does not write whole shows up in any comparison
+        if (hipMemsetAsync(p, 0xFF, bytes, CUR_STREAM) != hipSuccess) { (void)pool_give(p, klass); return fail(PRAD_ERR_LAUNCH, "poison fill failed"); }
     }
-    prad_buf* b = new prad_buf{BUF_MAGIC, dtype, depth, rows, cols, p, true};
-    *out = b;
+    *out = new prad_buf{BUF_MAGIC, dtype, depth, rows, cols, p, true, klass};
     return PRAD_OK;
 }
 
+int32_t prad_buf_alloc_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out) {
+    return buf_alloc(dtype, depth, rows, cols, true, out);
+}
+
 int32_t prad_buf_alloc(int32_t dtype, int64_t rows, int64_t cols, prad_buf_t* out) {
-    return prad_buf_alloc_deep(dtype, 1, rows, cols, out);
+    return buf_alloc(dtype, 1, rows, cols, true, out);
+}
+
+int32_t prad_buf_alloc_output(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, prad_buf_t* out) {
+    return buf_alloc(dtype, depth, rows, cols, false, out);
+}
+
+int32_t prad_pool_trim(void) {
+    REQUIRE_INIT();
+    ENQUEUE_LOCK();
+    NOT_WHILE_RECORDING("releasing pooled device memory");
+    return pool_release_all();
+}
+
+int32_t prad_alloc_stats(int64_t* device_mallocs, int64_t* device_frees, int64_t* stream_syncs, int64_t* pool_hits,
+                         int64_t* pooled_bytes) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (device_mallocs) *device_mallocs = g_ctx.stat_device_mallocs;
+    if (device_frees) *device_frees = g_ctx.stat_device_frees;
+    if (stream_syncs) *stream_syncs = g_ctx.stat_stream_syncs;
+    if (pool_hits) *pool_hits = g_ctx.stat_pool_hits;
+    if (pooled_bytes) *pooled_bytes = (int64_t)g_ctx.pool_bytes;
+    return PRAD_OK;
 }
 
 int32_t prad_buf_wrap_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t cols, void* device_ptr, prad_buf_t* out) {
@@ -554,7 +654,7 @@ int32_t prad_buf_wrap_deep(int32_t dtype, int64_t depth, int64_t rows, int64_t c
     if (out == nullptr || device_ptr == nullptr) return fail(PRAD_ERR_ARG, "NULL argument");
     if (dtype != PRAD_F64 && dtype != PRAD_F32) return fail(PRAD_ERR_DTYPE, "unknown dtype %d", dtype);
     if (depth <= 0 || rows <= 0 || cols <= 0) return fail(PRAD_ERR_ARG, "matrix dimensions must be positive");
-    *out = new prad_buf{BUF_MAGIC, dtype, depth, rows, cols, device_ptr, false};
+    *out = new prad_buf{BUF_MAGIC, dtype, depth, rows, cols, device_ptr, false, 0};
     return PRAD_OK;
 }
 
@@ -569,9 +669,9 @@ int32_t prad_buf_free(prad_buf_t b) {
         REQUIRE_INIT();
         ENQUEUE_LOCK();
         NOT_WHILE_RECORDING("freeing a buffer");
-        // Work that still uses the buffer may be queued.
-        if (int32_t st = sync_all()) return st;
-        HIP_TRY(hipFree(b->ptr), PRAD_ERR_ALLOC);
+        // Work that still uses the buffer may be queued: the block goes back to the pool, and whoever gets it next
+        // enqueues behind that work.
+        if (int32_t st = pool_give(b->ptr, b->block_bytes)) return st;
     }
     b->magic = 0;
     delete b;
@@ -621,6 +721,7 @@ int32_t prad_buf_upload_rows(prad_buf_t b, const void* const* row_ptrs, const in
         for (int64_t i = 0; i < nr; ++i) memcpy(stage + (size_t)i * row_bytes, row_ptrs[r0 + i], row_bytes);
         HIP_TRY(hipMemcpyAsync(static_cast<char*>(b->ptr) + (size_t)r0 * row_bytes, stage, (size_t)nr * row_bytes,
                                hipMemcpyHostToDevice, g_ctx.stream), PRAD_ERR_LAUNCH);
+        ++g_ctx.stat_stream_syncs;
         HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
     }
     return PRAD_OK;
@@ -645,6 +746,7 @@ int32_t prad_buf_download_rows(prad_buf_t b, void* const* row_ptrs) {
         char* stage = static_cast<char*>(g_ctx.pinned);
         HIP_TRY(hipMemcpyAsync(stage, static_cast<char*>(b->ptr) + (size_t)r0 * row_bytes, (size_t)nr * row_bytes,
                                hipMemcpyDeviceToHost, g_ctx.stream), PRAD_ERR_LAUNCH);
+        ++g_ctx.stat_stream_syncs;
         HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
         for (int64_t i = 0; i < nr; ++i) memcpy(row_ptrs[r0 + i], stage + (size_t)i * row_bytes, row_bytes);
     }
@@ -660,6 +762,7 @@ int32_t prad_buf_upload(prad_buf_t b, const void* src, int64_t ld) {
     NOT_WHILE_RECORDING("a copy to or from the host");
     HIP_TRY(hipMemcpy2DAsync(b->ptr, (size_t)b->cols * es, src, (size_t)ld * es, (size_t)b->cols * es,
                              (size_t)(b->depth * b->rows), hipMemcpyHostToDevice, g_ctx.stream), PRAD_ERR_LAUNCH);
+    ++g_ctx.stat_stream_syncs;
     HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -673,6 +776,7 @@ int32_t prad_buf_download(prad_buf_t b, void* dst, int64_t ld) {
     NOT_WHILE_RECORDING("a copy to or from the host");
     HIP_TRY(hipMemcpy2DAsync(dst, (size_t)ld * es, b->ptr, (size_t)b->cols * es, (size_t)b->cols * es,
                              (size_t)(b->depth * b->rows), hipMemcpyDeviceToHost, g_ctx.stream), PRAD_ERR_LAUNCH);
+    ++g_ctx.stat_stream_syncs;
     HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -1529,7 +1633,7 @@ int32_t prad_buf_view_rows(prad_buf_t parent, int64_t row0, int64_t rows, prad_b
     if (out == nullptr) return fail(PRAD_ERR_ARG, "out is NULL");
     if (parent->depth != 1 || row0 < 0 || rows <= 0 || row0 + rows > parent->rows) return fail(PRAD_ERR_ARG, "row range outside the buffer");
     char* base = static_cast<char*>(parent->ptr) + (size_t)row0 * parent->cols * elem_size(parent->dtype);
-    *out = new prad_buf{BUF_MAGIC, parent->dtype, 1, rows, parent->cols, base, false};
+    *out = new prad_buf{BUF_MAGIC, parent->dtype, 1, rows, parent->cols, base, false, 0};
     return PRAD_OK;
 }
 

@@ -158,3 +158,77 @@ class FeedForwardNetwork:
 
     def parameter_count(self):
         return sum(self.sizes[l] * self.sizes[l + 1] + self.sizes[l + 1] for l in range(len(self.W)))
+
+
+class OperationWalkNetwork:
+    """The same network and step, driven the way the reference's own loop drives it and with nothing fused: one
+    operation object per graph node, Forward called node by node in graph order, the loss, Backward called node by node
+    in reverse with each node's results added into its gradient destinations (OperationBase.AccumulateGradient,
+    src/RMAD/OperationBase.cs:273-304), then GradientClearer / GradientClipper / AdamOptimizer over the layers
+    (examples/feedforward/ParallelReverseAutoDiff.FeedForwardExample/FeedForwardNeuralNetwork.cs:212-303,
+    src/RMAD/OperationNeuralNetworkVisitor.cs:198-215, :287-329).  Every Forward / Backward returns a fresh output
+    Matrix, as in the reference; those come from the library's block pool, so a step in its steady state allocates
+    nothing on the device and never waits for it.  This is what an unchanged caller of the operation classes gets."""
+
+    def __init__(self, sizes=(784, 256, 128, 10), batch=64, dtype=np.float64, seed=seeded.DEFAULT_SEED, parameters=None,
+                 multiply="MatrixMultiplyOperation"):
+        from . import operations as ops
+        from .matrix import Matrix
+        from .optim import AdamOptimizer, GradientClearer, GradientClipper, ModelLayer
+        _ensure_initialized()
+        self.dtype = np.dtype(dtype)
+        self.sizes, self.batch = tuple(sizes), batch
+        self.Parameters = parameters or NeuralNetworkParameters(lite=self.dtype == np.float32)
+        L = len(sizes) - 1
+        self.host_W = [seeded.xavier(seed, 10 + l, sizes[l], sizes[l + 1], self.dtype) for l in range(L)]
+        self.W = [Matrix.from_numpy(w) for w in self.host_W]
+        self.b = [Matrix(1, sizes[l + 1], self.dtype) for l in range(L)]
+        self.layers = []
+        for l in range(L):
+            layer = ModelLayer().AddModelElementGroup("W", self.W[l]).AddModelElementGroup("B", self.b[l])
+            self.layers.append(layer)
+        self.dW = [layer["W", "Gradient"] for layer in self.layers]
+        self.db = [layer["B", "Gradient"] for layer in self.layers]
+        for m in self.dW + self.db + [layer[i, e] for layer in self.layers for i in ("W", "B") for e in ("FirstMoment", "SecondMoment")]:
+            m.device()
+        # the graph: [multiply -> add bias -> LeakyReLU] x (L - 1) -> multiply -> add bias -> softmax; loss = cross-entropy
+        multiply_type = getattr(ops, multiply)
+        self.nodes = []   # (operation, names of its inputs, gradient destinations per result)
+        for l in range(L):
+            self.nodes.append((multiply_type.Instantiate(self), ("prev", ("W", l)), (None, self.dW[l])))
+            self.nodes.append((ops.MatrixAddBroadcastingOperation.Instantiate(self), ("prev", ("b", l)), (None, self.db[l])))
+            self.nodes.append((ops.LeakyReLUOperation.Instantiate(self) if l < L - 1 else ops.SoftmaxOperation.Instantiate(self),
+                               ("prev",), (None,)))
+        self.loss_op = ops.CategoricalCrossEntropyLossOperation.Instantiate(self)
+        self._accumulate = ops.accumulate_gradient
+        self.clearer, self.clipper, self.adam = GradientClearer(), GradientClipper(self), AdamOptimizer(self)
+        self.iteration = 0
+        self.Input = self.Target = self.Output = self.loss = None
+
+    def set_batch(self, X, T):
+        from .matrix import Matrix
+        self.Input, self.Target = Matrix.from_numpy(np.asarray(X, self.dtype)), Matrix.from_numpy(np.asarray(T, self.dtype))
+        self.Input.device(); self.Target.device()
+
+    def step(self):
+        self.iteration += 1
+        self.Parameters.AdamIteration = float(self.iteration)
+        self.clearer.Clear(self.layers)
+        value = self.Input
+        for op, inputs, _ in self.nodes:                                   # forward walk, graph order
+            args = [value if name == "prev" else (self.W if name[0] == "W" else self.b)[name[1]] for name in inputs]
+            value = op.Forward(*args)
+        self.Output = value
+        self.loss = self.loss_op.Forward(self.Output, self.Target)
+        grad = self.loss_op.Backward(self.Output).Item1
+        for op, _, destinations in reversed(self.nodes):                   # backward walk
+            results = op.Backward(grad).Results
+            for dest, result in zip(destinations, results):
+                if dest is not None:
+                    self._accumulate(dest, result)
+            grad = results[0]
+        self.clipper.Clip(self.layers)
+        self.adam.Optimize(self.layers)
+
+    def flops_per_step(self):
+        return 3.0 * sum(2.0 * self.batch * self.sizes[l] * self.sizes[l + 1] for l in range(len(self.W)))

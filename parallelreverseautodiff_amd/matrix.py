@@ -54,9 +54,18 @@ class DeviceBuffer:
 
     @classmethod
     def alloc(cls, dtype, rows, cols, depth=1):
+        """A zero-filled buffer, like new Matrix(rows, cols)."""
         lib = _lib.load()
         h = ctypes.c_void_p()
         check(lib.prad_buf_alloc_deep(_dtype_code(dtype), depth, rows, cols, ctypes.byref(h)))
+        return cls(h, dtype, depth, rows, cols)
+
+    @classmethod
+    def alloc_output(cls, dtype, rows, cols, depth=1):
+        """A buffer whose contents are undefined until the next kernel overwrites all of it (no fill launch)."""
+        lib = _lib.load()
+        h = ctypes.c_void_p()
+        check(lib.prad_buf_alloc_output(_dtype_code(dtype), depth, rows, cols, ctypes.byref(h)))
         return cls(h, dtype, depth, rows, cols)
 
     def slice(self, d):

@@ -141,7 +141,7 @@ class MatrixMultiplyOperation(Operation):
             raise InvalidOperationException("Input 1 columns do not match Input 2 rows")
         if input1.dtype != input2.dtype:
             raise ArgumentException("buffers of different element types in one call")
-        out = DeviceBuffer.alloc(input1.dtype, input1.Rows, input2.Cols)
+        out = DeviceBuffer.alloc_output(input1.dtype, input1.Rows, input2.Cols)
         check(_lib.load().prad_matmul_fwd(input1.device().handle, input2.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
@@ -149,8 +149,8 @@ class MatrixMultiplyOperation(Operation):
     def Backward(self, dOutput):
         self._check_device()
         a, b = self.input1, self.input2
-        d_in1 = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols)
-        d_in2 = DeviceBuffer.alloc(b.dtype, b.Rows, b.Cols)
+        d_in1 = DeviceBuffer.alloc_output(a.dtype, a.Rows, a.Cols)
+        d_in2 = DeviceBuffer.alloc_output(b.dtype, b.Rows, b.Cols)
         check(_lib.load().prad_matmul_bwd(dOutput.device().handle, a.device().handle, b.device().handle,
                                          d_in1.handle, d_in2.handle, 0, 0))
         return (BackwardResultBuilder()
@@ -208,7 +208,7 @@ class _BatchMatrixMultiplyBase(Operation):
         if input1.Cols != input2.Rows:
             raise InvalidOperationException("Input 1 columns do not match Input 2 rows")
         self._in1, self._in2 = input1, input2
-        out = DeviceBuffer.alloc(input1.dtype, input1.Rows, input2.Cols, depth=depth)
+        out = DeviceBuffer.alloc_output(input1.dtype, input1.Rows, input2.Cols, depth=depth)
         check(_lib.load().prad_gemm_batched(0, 0, input1.device().handle, input2.device().handle, out.handle, 0))
         self.DeepOutput = DeepMatrix._from_device(out)
         return self.DeepOutput
@@ -219,8 +219,8 @@ class _BatchMatrixMultiplyBase(Operation):
         lib = _lib.load()
         depth = dOutput.Depth
         a, b = self._in1, self._in2
-        d1 = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols, depth=depth)
-        d2 = DeviceBuffer.alloc(b.dtype, b.Rows, b.Cols, depth=depth)
+        d1 = DeviceBuffer.alloc_output(a.dtype, a.Rows, a.Cols, depth=depth)
+        d2 = DeviceBuffer.alloc_output(b.dtype, b.Rows, b.Cols, depth=depth)
         g = dOutput.device()
         check(lib.prad_gemm_batched(0, 1, g.handle, b.device().handle, d1.handle, 0))  # dA_i = dC_i . B_i^T
         check(lib.prad_gemm_batched(1, 0, a.device().handle, g.handle, d2.handle, 0))  # dB_i = A_i^T . dC_i
@@ -277,7 +277,7 @@ class MatrixMultiplyAndSumOperation(Operation):
         self.a, self.b = a, b
         if a.Cols != b.Rows:
             raise InvalidOperationException("Matrix dimensions must be compatible for multiplication.")
-        out = DeviceBuffer.alloc(a.dtype, 1, b.Depth)
+        out = DeviceBuffer.alloc_output(a.dtype, 1, b.Depth)
         check(_lib.load().prad_matmul_sum_fwd(a.device().handle, b.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
@@ -286,8 +286,8 @@ class MatrixMultiplyAndSumOperation(Operation):
         if self._needs_init:
             _require_initialized()
         a, b = self.a, self.b
-        d_a = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols)
-        d_b = DeviceBuffer.alloc(a.dtype, a.Cols, a.Rows, depth=b.Depth)
+        d_a = DeviceBuffer.alloc_output(a.dtype, a.Rows, a.Cols)
+        d_b = DeviceBuffer.alloc_output(a.dtype, a.Cols, a.Rows, depth=b.Depth)
         check(_lib.load().prad_matmul_sum_bwd(a.device().handle, b.device().handle, dOutput.device().handle,
                                              d_a.handle, d_b.handle))
         return (BackwardResultBuilder()
@@ -341,7 +341,7 @@ class _BatchMatrixMultiplyAndSumBase(Operation):
         if input1.Cols != input2.Rows:
             raise InvalidOperationException("Matrix dimensions must be compatible for multiplication.")
         self._in1, self._in2 = input1, input2
-        out = DeviceBuffer.alloc(input1.dtype, 1, input2.Depth, depth=input1.Depth)
+        out = DeviceBuffer.alloc_output(input1.dtype, 1, input2.Depth, depth=input1.Depth)
         check(_lib.load().prad_matmul_sum_fwd(input1.device().handle, input2.device().handle, out.handle))
         self.DeepOutput = DeepMatrix._from_device(out)
         return self.DeepOutput
@@ -353,8 +353,8 @@ class _BatchMatrixMultiplyAndSumBase(Operation):
         S, P = a.Depth, b.Depth
         if dOutput.Depth != S:
             raise ArgumentException("upstream gradient must hold one matrix per sample")
-        d_a = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols, depth=S)
-        d_b = DeviceBuffer.alloc(a.dtype, a.Cols, a.Rows, depth=S * P)
+        d_a = DeviceBuffer.alloc_output(a.dtype, a.Rows, a.Cols, depth=S)
+        d_b = DeviceBuffer.alloc_output(a.dtype, a.Cols, a.Rows, depth=S * P)
         check(_lib.load().prad_matmul_sum_bwd(a.device().handle, b.device().handle, dOutput.device().handle, d_a.handle, d_b.handle))
         m_a, m_b = DeepMatrix._from_device(d_a), DeepMatrix._from_device(d_b)
         return [BackwardResultBuilder().AddInputGradient(m_a[i]).AddInputGradientArray([m_b[i * P + q] for q in range(P)]).Build()
@@ -401,7 +401,7 @@ class BatchMatrixMultiplySumOperation(Operation):
         self.a, self.b, self.bias = a, b, bias
         if a.Cols != b.Rows:
             raise InvalidOperationException("Input 1 columns do not match Input 2 rows")
-        out = DeviceBuffer.alloc(a.dtype, a.Rows, b.Cols)
+        out = DeviceBuffer.alloc_output(a.dtype, a.Rows, b.Cols)
         check(_lib.load().prad_matmul_batch_sum_fwd(a.device().handle, b.device().handle,
                                                    None if bias is None else bias.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
@@ -409,9 +409,9 @@ class BatchMatrixMultiplySumOperation(Operation):
 
     def Backward(self, dOutput):
         a, b = self.a, self.b
-        d_a = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols, depth=a.Depth)
-        d_b = DeviceBuffer.alloc(a.dtype, b.Rows, b.Cols, depth=b.Depth)
-        d_bias = None if self.bias is None else DeviceBuffer.alloc(a.dtype, 1, b.Cols)
+        d_a = DeviceBuffer.alloc_output(a.dtype, a.Rows, a.Cols, depth=a.Depth)
+        d_b = DeviceBuffer.alloc_output(a.dtype, b.Rows, b.Cols, depth=b.Depth)
+        d_bias = None if self.bias is None else DeviceBuffer.alloc_output(a.dtype, 1, b.Cols)
         check(_lib.load().prad_matmul_batch_sum_bwd(dOutput.device().handle, a.device().handle, b.device().handle, d_a.handle,
                                                    d_b.handle, None if d_bias is None else d_bias.handle))
         builder = BackwardResultBuilder().AddInputGradient(DeepMatrix._from_device(d_a)).AddInputGradient(DeepMatrix._from_device(d_b))
@@ -440,7 +440,7 @@ class _ActivationOperation(Operation):
     def Forward(self, input):
         _ensure_initialized()
         self.input = input
-        out = DeviceBuffer.alloc(input.dtype, input.Rows, input.Cols)
+        out = DeviceBuffer.alloc_output(input.dtype, input.Rows, input.Cols)
         check(_lib.load().prad_act_fwd(self._act, input.device().handle, out.handle, float(self.alpha)))
         self.Output = Matrix._from_device(out)
         return self.Output
@@ -448,7 +448,7 @@ class _ActivationOperation(Operation):
     def Backward(self, dOutput):
         _ensure_initialized()
         src = self.input if self._caches == "input" else self.Output
-        dx = DeviceBuffer.alloc(src.dtype, src.Rows, src.Cols)
+        dx = DeviceBuffer.alloc_output(src.dtype, src.Rows, src.Cols)
         check(_lib.load().prad_act_bwd(self._act, src.device().handle, dOutput.device().handle, dx.handle, float(self.alpha)))
         return BackwardResultBuilder().AddInputGradient(Matrix._from_device(dx)).Build()
 
@@ -522,7 +522,7 @@ class HadamardProductOperation(Operation):
         self.input1, self.input2 = input1, input2
         if input1.Rows != input2.Rows or input1.Cols != input2.Cols:
             raise ArgumentException("Matrices must have the same dimensions.")
-        out = DeviceBuffer.alloc(input1.dtype, input1.Rows, input1.Cols)
+        out = DeviceBuffer.alloc_output(input1.dtype, input1.Rows, input1.Cols)
         check(_lib.load().prad_hadamard_fwd(input1.device().handle, input2.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
@@ -530,8 +530,8 @@ class HadamardProductOperation(Operation):
     def Backward(self, dOutput):
         _ensure_initialized()
         a, b = self.input1, self.input2
-        da = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols)
-        db = DeviceBuffer.alloc(a.dtype, a.Rows, a.Cols)
+        da = DeviceBuffer.alloc_output(a.dtype, a.Rows, a.Cols)
+        db = DeviceBuffer.alloc_output(a.dtype, a.Rows, a.Cols)
         check(_lib.load().prad_hadamard_bwd(a.device().handle, b.device().handle, dOutput.device().handle, da.handle, db.handle))
         return (BackwardResultBuilder()
                 .AddInputGradient(Matrix._from_device(da))
@@ -559,7 +559,7 @@ class MatrixAddOperation(Operation):
 
     def Forward(self, inputA, inputB):
         _ensure_initialized()
-        out = DeviceBuffer.alloc(inputA.dtype, inputA.Rows, inputA.Cols)
+        out = DeviceBuffer.alloc_output(inputA.dtype, inputA.Rows, inputA.Cols)
         check(_lib.load().prad_add(inputA.device().handle, inputB.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
@@ -578,7 +578,7 @@ class MatrixAddThreeOperation(Operation):
 
     def Forward(self, inputA, inputB, bias):
         _ensure_initialized()
-        out = DeviceBuffer.alloc(inputA.dtype, inputA.Rows, inputA.Cols)
+        out = DeviceBuffer.alloc_output(inputA.dtype, inputA.Rows, inputA.Cols)
         check(_lib.load().prad_add_three(inputA.device().handle, inputB.device().handle, bias.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
@@ -597,7 +597,7 @@ class MatrixTransposeOperation(Operation):
     @staticmethod
     def _transpose(m):
         _ensure_initialized()
-        out = DeviceBuffer.alloc(m.dtype, m.Cols, m.Rows)
+        out = DeviceBuffer.alloc_output(m.dtype, m.Cols, m.Rows)
         check(_lib.load().prad_transpose(m.device().handle, out.handle))
         return Matrix._from_device(out)
 
@@ -630,16 +630,16 @@ class LayerNormalizationOperation(Operation):
     def Forward(self, input):
         _ensure_initialized()
         self.input = input
-        out = DeviceBuffer.alloc(input.dtype, input.Rows, input.Cols)
-        self.mean = DeviceBuffer.alloc(input.dtype, 1, input.Rows)
-        self.stdDev = DeviceBuffer.alloc(input.dtype, 1, input.Rows)
+        out = DeviceBuffer.alloc_output(input.dtype, input.Rows, input.Cols)
+        self.mean = DeviceBuffer.alloc_output(input.dtype, 1, input.Rows)
+        self.stdDev = DeviceBuffer.alloc_output(input.dtype, 1, input.Rows)
         check(_lib.load().prad_layernorm_fwd(input.device().handle, out.handle, self.mean.handle, self.stdDev.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
 
     def Backward(self, gradOutput):
         _ensure_initialized()
-        dx = DeviceBuffer.alloc(self.input.dtype, self.input.Rows, self.input.Cols)
+        dx = DeviceBuffer.alloc_output(self.input.dtype, self.input.Rows, self.input.Cols)
         check(_lib.load().prad_layernorm_bwd(self.input.device().handle, self.mean.handle, self.stdDev.handle,
                                              gradOutput.device().handle, dx.handle))
         return BackwardResultBuilder().AddInputGradient(Matrix._from_device(dx)).Build()
@@ -658,14 +658,14 @@ class MatrixAddBroadcastingOperation(Operation):
         if input.Cols != bias.Cols:
             raise ArgumentException(
                 "The length of the bias vector must be the same as the number of columns in the input matrix.")
-        out = DeviceBuffer.alloc(input.dtype, input.Rows, input.Cols)
+        out = DeviceBuffer.alloc_output(input.dtype, input.Rows, input.Cols)
         check(_lib.load().prad_add_broadcast_fwd(input.device().handle, bias.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
 
     def Backward(self, dOutput):
         _ensure_initialized()
-        db = DeviceBuffer.alloc(dOutput.dtype, 1, dOutput.Cols)
+        db = DeviceBuffer.alloc_output(dOutput.dtype, 1, dOutput.Cols)
         check(_lib.load().prad_add_broadcast_bwd_bias(dOutput.device().handle, db.handle))
         return BackwardResultBuilder().AddInputGradient(dOutput).AddBiasGradient(Matrix._from_device(db)).Build()
 
@@ -693,7 +693,7 @@ class SoftmaxOperation(Operation):
 
     def Forward(self, input):
         _ensure_initialized()
-        out = DeviceBuffer.alloc(input.dtype, input.Rows, input.Cols)
+        out = DeviceBuffer.alloc_output(input.dtype, input.Rows, input.Cols)
         check(_lib.load().prad_softmax_fwd(input.device().handle, out.handle))
         self.Output = Matrix._from_device(out)
         return self.Output
@@ -701,7 +701,7 @@ class SoftmaxOperation(Operation):
     def Backward(self, dLdOutput):
         _ensure_initialized()
         y = self.Output
-        dx = DeviceBuffer.alloc(y.dtype, y.Rows, y.Cols)
+        dx = DeviceBuffer.alloc_output(y.dtype, y.Rows, y.Cols)
         check(_lib.load().prad_softmax_bwd(y.device().handle, dLdOutput.device().handle, dx.handle))
         return BackwardResultBuilder().AddInputGradient(Matrix._from_device(dx)).Build()
 
@@ -724,13 +724,13 @@ class CategoricalCrossEntropyLossOperation(Operation):
         if output.Rows != target.Rows or output.Cols != target.Cols:
             raise ArgumentException("Output and target matrices must have the same dimensions.")
         self.target = target
-        loss = DeviceBuffer.alloc(output.dtype, 1, 1)
+        loss = DeviceBuffer.alloc_output(output.dtype, 1, 1)
         check(_lib.load().prad_cce_fwd(output.device().handle, target.device().handle, loss.handle))
         self.Output = Matrix._from_device(loss)
         return self.Output
 
     def Backward(self, output):
         _ensure_initialized()
-        dp = DeviceBuffer.alloc(output.dtype, output.Rows, output.Cols)
+        dp = DeviceBuffer.alloc_output(output.dtype, output.Rows, output.Cols)
         check(_lib.load().prad_cce_bwd(output.device().handle, self.target.device().handle, dp.handle))
         return BackwardResultBuilder().AddInputGradient(Matrix._from_device(dp)).Build()

@@ -8,6 +8,8 @@ lite/src/ParallelReverseAutoDiffLite/Lite/NeuralNetworkParameters.cs).
 """
 import json
 
+import numpy as np
+
 from . import _lib
 from .exceptions import InvalidOperationException, check
 from .matrix import DeepMatrix, Matrix
@@ -136,6 +138,22 @@ def _collect(layers, element):
                 raise InvalidOperationException("%s cannot be null." % element)
             out.append(m)
     return out
+
+
+class GradientClearer:
+    """src/RMAD/GradientClearer.cs:21-86: every gradient of every layer back to zero.  The reference replaces each
+    row by a new zero array; a gradient that lives on the device is zero-filled there instead (one launch, no copy),
+    a host-only one gets new zero rows as in the reference."""
+
+    def Clear(self, layers):
+        for g in _collect(layers, "Gradient"):
+            for m in (g if isinstance(g, DeepMatrix) else [g]):
+                if m._dev is not None:
+                    m._dev.zero()
+                    m._device_written()
+                else:
+                    for i in range(m.Rows):
+                        m[i] = np.zeros(m.Cols, dtype=m.dtype)
 
 
 class GradientClipper:

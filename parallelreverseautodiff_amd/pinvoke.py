@@ -25,12 +25,13 @@ _TYPES = [
     (r"int64_t\s*\*", "out long"),
     (r"int32_t\s*\*", "out int"),
     (r"const (double|float)\s*\*", "IntPtr"),
-    (r"float\s*\*", "out float"),     # prad_event_elapsed_ms
-    (r"double\s*\*", "IntPtr"),
+    (r"(double|float)\s*\*", "IntPtr"),   # device memory; the host out-parameters are listed in _HOST_OUT
     (r"int64_t", "long"),
     (r"int32_t", "int"),
     (r"double", "double"),
 ]
+# (function, parameter) pairs whose float* / double* points at a host variable that the call fills in.
+_HOST_OUT = {("prad_event_elapsed_ms", "ms"): "out float"}
 _RESERVED = {"out", "in", "ref", "params", "base", "lock", "event", "object", "string"}
 
 
@@ -52,7 +53,9 @@ def prototypes(header_text=None):
     return out
 
 
-def csharp_type(ctype):
+def csharp_type(ctype, function=None, parameter=None):
+    if (function, parameter) in _HOST_OUT:
+        return _HOST_OUT[(function, parameter)]
     for pattern, cs in _TYPES:
         if re.fullmatch(pattern, ctype):
             return cs
@@ -63,9 +66,10 @@ def declaration(ret, name, params):
     cs_ret = "int" if ret == "int32_t" else "IntPtr"
     args = []
     for ctype, pname in params:
+        cs = csharp_type(ctype, name, pname)
         if pname in _RESERVED:
             pname = "@" + pname
-        args.append("%s %s" % (csharp_type(ctype), pname))
+        args.append("%s %s" % (cs, pname))
     return "[DllImport(Lib)] public static extern %s %s(%s);" % (cs_ret, name, ", ".join(args))
 
 

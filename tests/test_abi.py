@@ -80,3 +80,23 @@ def test_integration_notes_declare_every_function_for_pinvoke():
     header_names = {p[1] for p in protos}
     from parallelreverseautodiff_amd import _lib
     assert header_names == set(_lib.SIGNATURES)
+
+
+def test_pinvoke_device_pointers_are_not_out_parameters():
+    """Device memory travels as IntPtr in the generated C# declarations, for float as for double: `out` is only for
+    host variables that a call fills in (handles, shapes, counters, an event's elapsed time)."""
+    import re
+    from parallelreverseautodiff_amd import pinvoke
+    protos = {p[1]: p for p in pinvoke.prototypes()}
+    for name, (_, _, params) in protos.items():
+        decl = pinvoke.declaration(*protos[name])
+        for ctype, pname in params:
+            cs = pinvoke.csharp_type(ctype, name, pname)
+            if name.startswith("prad_gemm") and pname in ("A", "B", "C"):
+                assert cs == "IntPtr", (name, pname, cs)
+            if re.fullmatch(r"(const )?(double|float)\s*\*", ctype) and (name, pname) not in pinvoke._HOST_OUT:
+                assert cs == "IntPtr", (name, pname, cs)
+        if name.endswith("_f32") and name[:-4] + "_f64" in protos:   # the two precisions differ in nothing but the name
+            twin = pinvoke.declaration(*protos[name[:-4] + "_f64"])
+            assert decl.replace("_f32(", "_f64(") == twin
+    assert "out float ms" in pinvoke.declaration(*protos["prad_event_elapsed_ms"])

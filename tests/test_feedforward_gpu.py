@@ -269,3 +269,60 @@ def test_fused_softmax_cross_entropy_equals_separate_launches(gpu, dtype, shape)
         assert np.array_equal(a.download(), b2.download())
     check(lib.prad_softmax_cce(bx.handle, bt.handle, p2.handle, None, dp2.handle, dx2.handle))   # loss is optional
     assert np.array_equal(dx1.download(), dx2.download())
+
+
+def _alloc_stats():
+    import ctypes
+    from parallelreverseautodiff_amd import _lib
+    vals = [ctypes.c_int64() for _ in range(5)]
+    assert _lib.load().prad_alloc_stats(*[ctypes.byref(v) for v in vals]) == 0
+    return dict(zip(("mallocs", "frees", "syncs", "pool_hits", "pooled_bytes"), (v.value for v in vals)))
+
+
+@pytest.mark.parametrize("multiply", ["MatrixMultiplyOperation", "GpuMatrixMultiplyOperation", "CudaMatrixMultiplyOperation"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_operation_by_operation_walk(gpu, oracle, dtype, multiply):
+    """The step driven through the operation classes one Forward / Backward at a time (fresh output Matrix per call,
+    results added into the gradient destinations, then GradientClipper and AdamOptimizer over the layers) against the
+    oracle's composition, and against the fused launch sequence: same arithmetic per operation, so the same bits."""
+    from parallelreverseautodiff_amd.feedforward import OperationWalkNetwork
+    X = seeded.uniform(seeded.DEFAULT_SEED, 1, (64, 784), 0.0, 1.0, dtype)
+    T = seeded.one_hot_labels(seeded.DEFAULT_SEED, 2, 64, 10, dtype)
+    walk, fused = OperationWalkNetwork(dtype=dtype, multiply=multiply), FeedForwardNetwork(dtype=dtype)
+    walk.set_batch(X, T); fused.set_batch(X, T)
+    W = [w.copy() for w in walk.host_W]
+    b = [np.zeros((1, s), dtype) for s in walk.sizes[1:]]
+    m = [np.zeros_like(x) for x in W + b]
+    v = [np.zeros_like(x) for x in W + b]
+    for t in (1, 2, 3):
+        walk.step(); fused.step()
+        dev_grads = [g.to_numpy() for g in walk.dW + walk.db]
+        loss, raw, clipped, new = oracle_step(oracle, W, b, m, v, X, T, walk.Parameters, t, dtype,
+                                              adam_grads=dev_grads if dtype == np.float32 else None)
+        assert abs(float(walk.loss.to_numpy()[0, 0]) - loss) <= (1e-12 if dtype == np.float64 else 1e-5) * abs(loss)
+        for i, (g_dev, g_ref) in enumerate(zip(dev_grads, clipped)):
+            assert_parity(g_dev, g_ref, dtype, "clipped gradient %d step %d" % (i, t))
+        L = len(W)
+        W = [n[0] for n in new[:L]]; b = [n[0] for n in new[L:]]
+        m = [n[1] for n in new]; v = [n[2] for n in new]
+        for i, (w_dev, w_ref) in enumerate(zip(walk.W + walk.b, W + b)):
+            assert_parity(w_dev.to_numpy(), w_ref, dtype, "weight %d step %d" % (i, t))
+        for i, (w_walk, w_fused) in enumerate(zip(walk.W + walk.b, fused._weights)):
+            assert np.array_equal(w_walk.to_numpy(), w_fused.download()), "weight %d step %d: walk and fused sequence differ" % (i, t)
+
+
+def test_operation_walk_steady_state_allocates_nothing(gpu):
+    """After the first steps the walk takes every output block from the library's pool: no hipMalloc, no hipFree and
+    no wait for the stream per step, although every operation returns a fresh Matrix."""
+    from parallelreverseautodiff_amd.feedforward import OperationWalkNetwork
+    net = OperationWalkNetwork()
+    net.set_batch(seeded.uniform(5, 1, (64, 784), 0.0, 1.0), seeded.one_hot_labels(5, 2, 64, 10))
+    for _ in range(3):
+        net.step()
+    before = _alloc_stats()
+    for _ in range(5):
+        net.step()
+    after = _alloc_stats()
+    assert after["mallocs"] == before["mallocs"] and after["frees"] == before["frees"] and after["syncs"] == before["syncs"], (before, after)
+    assert after["pool_hits"] - before["pool_hits"] >= 5 * 20
+    assert np.isfinite(net.loss.to_numpy()[0, 0])
