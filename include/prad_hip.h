@@ -294,12 +294,23 @@ int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, 
  *             the following blocks; tanh_c (steps*batch x hidden) receives tanh(c_t).
  *   backward: dh_loss (steps*batch x hidden) is the loss gradient with respect to every h_t; dG receives the gradient of
  *             the pre-activations of every step.  (dh_{-1} and dc_{-1}, which nothing consumes, are not formed.)
- * Shapes: float only, batch a multiple of 16, hidden a multiple of 64 up to 512, and (batch/16)*(hidden/16) workgroups
- * must fit the device at once (one per compute unit): prad_lstm_sequence_supported says 1 or 0 for a shape, and the
- * two calls return PRAD_ERR_ARG for others.  Every wait inside the kernels is bounded (PRAD_LSTM_SPIN_LIMIT polls,
- * default 2^22): if the device did not run the whole grid at once - other work held compute units for seconds -
- * the kernels end early and the next call that waits for the stream returns PRAD_ERR_LAUNCH. */
+ * The one-launch kernels take float, batch a multiple of 16, hidden a multiple of 64 up to 512, and need
+ * (batch/16)*(hidden/16) workgroups on the device at once, one per compute unit: prad_lstm_sequence_supported says 1 or 0
+ * for a shape (0 for every shape once the kernels are off, see below).  Every other shape and element type, and every
+ * call while the kernels are off, runs the same sequence as one launch per time step inside these two calls
+ * (prad_lstm_step_fwd / prad_lstm_step_bwd on windows of the same buffers), so the calls are always valid.
+ * Whether the device holds the whole grid is asked, not assumed: the first call for a grid larger than any before runs a
+ * probe kernel of the same grid and footprint that only takes a roll call, and waits for it (once per process and grid
+ * size; inside a recording an unproven grid takes the per-step path).  A probe that fails - another process or a
+ * compute-unit mask holds compute units - turns the kernels off, leaves a note in prad_last_error and the call goes on
+ * per time step and returns PRAD_OK.  Every wait inside the kernels is bounded as well (PRAD_LSTM_SPIN_LIMIT polls,
+ * default 2^22): if compute units are taken away later, the kernels end early, the next call that waits for the stream
+ * returns PRAD_ERR_LAUNCH (what was computed since the last successful wait is invalid), and the kernels stay off from
+ * then on.  prad_lstm_sequence_enable(1) turns them back on (the next call probes again), (0) turns them off;
+ * PRAD_LSTM_SEQUENCE=0 in the environment starts with them off.  A recorded launch sequence keeps the path it was
+ * recorded with. */
 int32_t prad_lstm_sequence_supported(int32_t dtype, int64_t batch, int64_t hidden, int64_t steps);
+int32_t prad_lstm_sequence_enable(int32_t on);
 int32_t prad_lstm_sequence_fwd(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_buf_t Hs, prad_buf_t tanh_c, int64_t steps);
 int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, prad_buf_t tanh_c, prad_buf_t dh_loss, prad_buf_t dG,
                                int64_t steps);

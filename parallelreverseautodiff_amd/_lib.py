@@ -109,6 +109,7 @@ SIGNATURES = {
     "prad_window_attention_fwd": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_double]),
     "prad_window_attention_bwd": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_double]),
     "prad_lstm_sequence_supported": (_i32, [_i32, _i64, _i64, _i64]),
+    "prad_lstm_sequence_enable": (_i32, [_i32]),
     "prad_lstm_sequence_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64]),
     "prad_lstm_sequence_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64]),
     "prad_buf_view_rows": (_i32, [_vp, _i64, _i64, _vpp]),

@@ -335,6 +335,7 @@ struct LstmSeqArgs {
 bool lstm_seq_eligible(int64_t batch, int64_t hidden, int64_t steps, int compute_units);
 size_t lstm_seq_partial_bytes(int64_t batch, int64_t hidden);
 hipError_t launch_lstm_seq(const LstmSeqArgs& a, bool backward, hipStream_t s);
+hipError_t launch_lstm_seq_probe(int64_t batch, int64_t hidden, unsigned* flags, unsigned* abort_word, int spin_limit, hipStream_t s);
 
 // Windowed self-attention, forward, one launch (csrc/attention.hip; float, head dimension 32, <= 64 tokens per window)
 bool window_attention_supported(int64_t tokens, int64_t head_dim);

@@ -286,11 +286,38 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_bwd_kernel(const Lstm
     }
 }
 
+// ---- co-residency probe -------------------------------------------------------------------------------------------
+// The sequence kernels need every workgroup of a row group on the device at the same time.  Whether the device can
+// hold the grid right now (it cannot when another process or a compute-unit mask takes compute units away) is asked
+// once, with a kernel of the same grid, workgroup size and LDS footprint that does nothing but the roll call: every
+// workgroup raises its flag and waits, bounded, for the flags of its row group.  Nothing is written but the flags.
+__global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_probe_kernel(unsigned* flags, unsigned* abort_word, int spin_limit, int groups,
+                                                                       int blocks) {
+    __shared__ __attribute__((aligned(16))) float footprint[SEQ_LDS_FLOATS];
+    __shared__ int all_arrived;
+    keep_allocated(footprint);
+    const int r = blockIdx.x % groups, c = blockIdx.x / groups;
+    if (spin_limit < 0) {  // forced from the host (tests of the fallback): report failure, wait for nobody
+        if (threadIdx.x == 0) __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        return;
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(flags + r * blocks + c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    (void)wait_for_group(flags + r * blocks, blocks, 1u, abort_word, spin_limit, &all_arrived);
+}
+
+hipError_t launch_lstm_seq_probe(int64_t batch, int64_t hidden, unsigned* flags, unsigned* abort_word, int spin_limit, hipStream_t s) {
+    const int groups = (int)(batch / 16), blocks = (int)(hidden / 16);
+    const unsigned grid = (unsigned)(groups * blocks);
+    hipError_t e = launch_fill_zero<float>(reinterpret_cast<float*>(flags), grid, s);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(lstm_seq_probe_kernel, dim3(grid), dim3(SEQ_THREADS), 0, s, flags, abort_word, spin_limit, groups, blocks);
+    return hipGetLastError();
+}
+
 // Shapes the sequence kernels take: float, hidden a multiple of 64 up to 512 (the slice of W_h in registers, the
 // backward tiles four wavefronts wide), batch a multiple of 16, one workgroup per compute unit for the whole grid.
 bool lstm_seq_eligible(int64_t batch, int64_t hidden, int64_t steps, int compute_units) {
-    static const bool enabled = [] { const char* e = getenv("PRAD_LSTM_SEQUENCE"); return !(e && e[0] == '0'); }();  // tuning aid
-    if (!enabled || steps < 1 || batch < 16 || batch % 16 != 0 || hidden < 64 || hidden % 64 != 0 || hidden > 16 * SEQ_MAX_J) return false;
+    if (steps < 1 || batch < 16 || batch % 16 != 0 || hidden < 64 || hidden % 64 != 0 || hidden > 16 * SEQ_MAX_J) return false;
     return (batch / 16) * (hidden / 16) <= compute_units;
 }
 size_t lstm_seq_partial_bytes(int64_t batch, int64_t hidden) {

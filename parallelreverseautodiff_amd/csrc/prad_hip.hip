@@ -70,6 +70,13 @@ struct Context {
     unsigned* seq_flags = nullptr;
     unsigned* seq_abort = nullptr;          // hipHostMalloc'ed, also the address the kernels use
     int compute_units = 0;
+    // Sequence kernels: off when PRAD_LSTM_SEQUENCE=0, when prad_lstm_sequence_enable(0) said so, when the co-residency
+    // probe of a grid failed, or - sticky - once a sequence kernel gave up; seq_proven_grid is the largest grid
+    // (workgroups) that a probe has shown the device to hold at once.
+    bool seq_enabled = true;
+    int seq_proven_grid = 0;
+    void* seq_step_scratch = nullptr;       // dh and dc ping-pong blocks of the per-time-step backward (kept: recordings address it)
+    size_t seq_step_scratch_bytes = 0, seq_step_scratch_class = 0;
     // Device blocks that prad_buf_free handed back, by size class.  Everything the library enqueues runs on the one
     // stream in lock order, so a block may be handed out again at once: whatever still reads or writes it is ahead
     // in the stream of whatever the next owner enqueues.
@@ -136,8 +143,12 @@ int32_t sync_all() {
     if (g_ctx.stream) HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
     if (g_ctx.seq_abort != nullptr && *static_cast<volatile unsigned*>(g_ctx.seq_abort) != 0u) {
         *static_cast<volatile unsigned*>(g_ctx.seq_abort) = 0u;
+        g_ctx.seq_enabled = false;
+        g_ctx.seq_proven_grid = 0;
         return fail(PRAD_ERR_LAUNCH, "an LSTM sequence kernel gave up waiting for its peer workgroups (the device did not run its whole "
-                                     "grid at once); the buffers it was writing hold partial results");
+                                     "grid at once); the buffers written since the last successful wait hold partial results.  The "
+                                     "sequence kernels are now off: prad_lstm_sequence_fwd / _bwd run one launch per time step from here "
+                                     "on (prad_lstm_sequence_enable(1) turns them back on)");
     }
     return PRAD_OK;
 }
@@ -545,6 +556,11 @@ int32_t prad_init(int32_t device_id) {
     HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&g_ctx.seq_abort), 64, hipHostMallocDefault), PRAD_ERR_ALLOC);
     *g_ctx.seq_abort = 0u;
     g_ctx.compute_units = std::min<int>(prop.multiProcessorCount, (int)(SEQ_FLAG_BYTES / sizeof(unsigned)));
+    {
+        const char* e = getenv("PRAD_LSTM_SEQUENCE");
+        g_ctx.seq_enabled = !(e && e[0] == '0');
+        g_ctx.seq_proven_grid = 0;
+    }
     g_ctx.pool_limit = prop.totalGlobalMem / 2;
     if (const char* cap = getenv("PRAD_POOL_MAX_BYTES")) g_ctx.pool_limit = (size_t)strtoull(cap, nullptr, 10);
     if (const char* poison = getenv("PRAD_POISON_OUTPUTS")) g_ctx.poison_outputs = poison[0] == '1';
@@ -560,6 +576,8 @@ int32_t prad_shutdown(void) {
     if (!g_ctx.initialized.load()) return PRAD_OK;
     (void)hipSetDevice(g_ctx.device);
     (void)sync_all();
+    if (g_ctx.seq_step_scratch) (void)pool_give(g_ctx.seq_step_scratch, g_ctx.seq_step_scratch_class);
+    g_ctx.seq_step_scratch = nullptr; g_ctx.seq_step_scratch_bytes = 0;
     (void)pool_release_all();
     if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
     if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
@@ -1519,21 +1537,19 @@ int32_t prad_lstm_step_bwd(prad_buf_t dG_next, prad_buf_t Wh, prad_buf_t gates, 
                : lstm_step_bwd_t<float>(dG_next, Wh, gates, c_prev, tanh_c, dh_loss, dc_in, dG, dc_prev, dh_scratch);
 }
 
-// Whole-sequence kernels: shape checks shared by both directions.  `gates` is steps*batch x 4*hidden.
+// Whole sequences: shape checks shared by both directions.  `gates` is steps*batch x 4*hidden.
 static int32_t lstm_sequence_check(prad_buf_t Wh, prad_buf_t gates, int64_t steps, int64_t* batch, int64_t* hidden) {
     if (steps < 1 || gates->depth != 1 || gates->rows % steps != 0 || gates->cols % 4 != 0)
         return fail(PRAD_ERR_ARG, "gates must be steps*batch x 4*hidden");
     *batch = gates->rows / steps;
     *hidden = gates->cols / 4;
     if (Wh->depth != 1 || Wh->rows != *hidden || Wh->cols != 4 * *hidden) return fail(PRAD_ERR_SHAPE, "recurrent weight must be hidden x 4*hidden");
-    if (gates->dtype != PRAD_F32 || !lstm_seq_eligible(*batch, *hidden, steps, g_ctx.compute_units))
-        return fail(PRAD_ERR_ARG, "the sequence kernels take float, batch a multiple of 16, hidden a multiple of 64 up to 512 and "
-                                  "(batch/16)*(hidden/16) <= %d workgroups; ask prad_lstm_sequence_supported first", g_ctx.compute_units);
     return PRAD_OK;
 }
 static int lstm_spin_limit() {
     const char* e = getenv("PRAD_LSTM_SPIN_LIMIT");  // polls of a peer's flag before a workgroup gives up
     const long v = e ? atol(e) : 0;
+    if (v < 0) return -1;  // a testing aid: the co-residency probe reports failure without polling
     return v > 0 ? (int)std::min<long>(v, 1L << 30) : (1 << 22);
 }
 static int32_t expect_rows(prad_buf_t b, int64_t rows, int64_t cols, const char* what) {
@@ -1543,8 +1559,98 @@ static int32_t expect_rows(prad_buf_t b, int64_t rows, int64_t cols, const char*
 
 int32_t prad_lstm_sequence_supported(int32_t dtype, int64_t batch, int64_t hidden, int64_t steps) {
     if (!g_ctx.initialized.load()) return 0;
-    return dtype == PRAD_F32 && lstm_seq_eligible(batch, hidden, steps, g_ctx.compute_units) ? 1 : 0;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return g_ctx.seq_enabled && dtype == PRAD_F32 && lstm_seq_eligible(batch, hidden, steps, g_ctx.compute_units) ? 1 : 0;
 }
+
+int32_t prad_lstm_sequence_enable(int32_t on) {
+    REQUIRE_INIT();
+    ENQUEUE_LOCK();
+    g_ctx.seq_enabled = on != 0;
+    g_ctx.seq_proven_grid = 0;  // the next sequence call asks the device again
+    return PRAD_OK;
+}
+
+// A 2-D window of `rows` rows of a buffer, starting at row0 (lives on the caller's stack).
+static prad_buf row_window(prad_buf_t b, int64_t row0, int64_t rows) {
+    return prad_buf{BUF_MAGIC, b->dtype, 1, rows, b->cols, static_cast<char*>(b->ptr) + (size_t)row0 * b->cols * elem_size(b->dtype), false, 0};
+}
+
+// Lock held.  Whether this call may use the sequence kernels: the shape fits, they are on, and the device has been
+// seen to hold a grid of this size at once.  The first call for a larger grid than any before asks the device with
+// the probe kernel and waits for its answer (once; not inside a recording, where an unproven grid takes the per-step
+// path); a probe that gives up turns the sequence kernels off.
+static int32_t sequence_kernels_usable(int32_t dtype, int64_t batch, int64_t hidden, int64_t steps, bool* usable) {
+    *usable = false;
+    if (!g_ctx.seq_enabled || dtype != PRAD_F32 || !lstm_seq_eligible(batch, hidden, steps, g_ctx.compute_units)) return PRAD_OK;
+    const int grid = (int)((batch / 16) * (hidden / 16));
+    if (grid <= g_ctx.seq_proven_grid) { *usable = true; return PRAD_OK; }
+    if (g_ctx.recording) return PRAD_OK;
+    if (int32_t st = sync_all()) return st;
+    HIP_TRY(launch_lstm_seq_probe(batch, hidden, g_ctx.seq_flags, g_ctx.seq_abort, lstm_spin_limit(), CUR_STREAM), PRAD_ERR_LAUNCH);
+    ++g_ctx.stat_stream_syncs;
+    HIP_TRY(hipStreamSynchronize(g_ctx.stream), PRAD_ERR_LAUNCH);
+    if (*static_cast<volatile unsigned*>(g_ctx.seq_abort) != 0u) {
+        *static_cast<volatile unsigned*>(g_ctx.seq_abort) = 0u;
+        g_ctx.seq_enabled = false;
+        tl_error = "the device does not hold the LSTM sequence kernels' whole grid at once (other work holds compute units): "
+                   "prad_lstm_sequence_fwd / _bwd run one launch per time step";
+        return PRAD_OK;
+    }
+    g_ctx.seq_proven_grid = grid;
+    *usable = true;
+    return PRAD_OK;
+}
+
+extern "C++" {
+// The same sequence as `steps` launches each way (lock held): the path of every shape and element type the sequence
+// kernels do not take, and of every call once they are off.
+template <typename T>
+static int32_t lstm_sequence_fwd_steps(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_buf_t Hs, prad_buf_t TC, int64_t steps, int64_t B) {
+    for (int64_t t = 0; t < steps; ++t) {
+        prad_buf h_prev = row_window(Hs, t * B, B), g = row_window(G, t * B, B), c_prev = row_window(C, t * B, B);
+        prad_buf c = row_window(C, (t + 1) * B, B), tc = row_window(TC, t * B, B), h = row_window(Hs, (t + 1) * B, B);
+        if (int32_t st = lstm_step_fwd_t<T>(&h_prev, Wh, &g, &c_prev, &c, &tc, &h)) return st;
+    }
+    return PRAD_OK;
+}
+
+template <typename T>
+static int32_t lstm_sequence_bwd_steps(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, prad_buf_t TC, prad_buf_t dHl, prad_buf_t dG,
+                                       int64_t steps, int64_t B, int64_t H) {
+    const size_t block = (((size_t)B * H * sizeof(T)) + 255) & ~(size_t)255;
+    if (g_ctx.seq_step_scratch_bytes < 4 * block) {
+        if (g_ctx.recording)
+            return fail(PRAD_ERR_RECORDING, "the per-time-step scratch would have to grow during a recording: run the sequence once before recording it");
+        void* fresh = nullptr;
+        size_t klass = 0;
+        if (int32_t st = pool_take(4 * block, &fresh, &klass)) return st;
+        if (g_ctx.seq_step_scratch) (void)pool_give(g_ctx.seq_step_scratch, g_ctx.seq_step_scratch_class);
+        g_ctx.seq_step_scratch = fresh; g_ctx.seq_step_scratch_bytes = 4 * block; g_ctx.seq_step_scratch_class = klass;
+    }
+    char* base = static_cast<char*>(g_ctx.seq_step_scratch);
+    prad_buf rec[2], dc[2];
+    for (int i = 0; i < 2; ++i) {
+        rec[i] = prad_buf{BUF_MAGIC, gates->dtype, 1, B, H, base + (size_t)i * block, false, 0};
+        dc[i] = prad_buf{BUF_MAGIC, gates->dtype, 1, B, H, base + (size_t)(2 + i) * block, false, 0};
+    }
+    for (int64_t t = steps - 1; t >= 0; --t) {
+        prad_buf g = row_window(gates, t * B, B), c_prev = row_window(C, t * B, B), tc = row_window(TC, t * B, B);
+        prad_buf dhl = row_window(dHl, t * B, B), dg = row_window(dG, t * B, B);
+        prad_buf* dc_in = &dc[t % 2];
+        prad_buf* dc_out = &dc[(t + 1) % 2];
+        if (t == steps - 1) {  // the last time step has no recurrent part and no dc arriving
+            HIP_TRY(launch_lstm_cell_bwd<T>(static_cast<const T*>(g.ptr), static_cast<const T*>(c_prev.ptr), static_cast<const T*>(tc.ptr),
+                                            static_cast<const T*>(dhl.ptr), nullptr, nullptr, static_cast<T*>(dg.ptr),
+                                            static_cast<T*>(dc_out->ptr), B, H, CUR_STREAM), PRAD_ERR_LAUNCH);
+            continue;
+        }
+        prad_buf dg_next = row_window(dG, (t + 1) * B, B);
+        if (int32_t st = lstm_step_bwd_t<T>(&dg_next, Wh, &g, &c_prev, &tc, &dhl, dc_in, &dg, dc_out, &rec[t % 2])) return st;
+    }
+    return PRAD_OK;
+}
+}  // extern "C++"
 
 int32_t prad_lstm_sequence_fwd(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_buf_t Hs, prad_buf_t tanh_c, int64_t steps) {
     REQUIRE_INIT();
@@ -1556,6 +1662,11 @@ int32_t prad_lstm_sequence_fwd(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_b
     if (int32_t st = expect_rows(Hs, (steps + 1) * batch, hidden, "Hs")) return st;
     if (int32_t st = expect_rows(tanh_c, steps * batch, hidden, "tanh_c")) return st;
     ENQUEUE_LOCK();
+    bool usable = false;
+    if (int32_t st = sequence_kernels_usable(G->dtype, batch, hidden, steps, &usable)) return st;
+    if (!usable)
+        return G->dtype == PRAD_F64 ? lstm_sequence_fwd_steps<double>(Wh, G, C, Hs, tanh_c, steps, batch)
+                                    : lstm_sequence_fwd_steps<float>(Wh, G, C, Hs, tanh_c, steps, batch);
     LstmSeqArgs a{};
     a.Wh = F(Wh); a.G = F(G); a.C = F(C); a.Hs = F(Hs); a.TC = F(tanh_c);
     a.flags = g_ctx.seq_flags; a.abort_word = g_ctx.seq_abort;
@@ -1576,6 +1687,11 @@ int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, pr
     if (int32_t st = expect_rows(dh_loss, steps * batch, hidden, "dh_loss")) return st;
     if (int32_t st = expect_rows(dG, steps * batch, 4 * hidden, "dG")) return st;
     ENQUEUE_LOCK();
+    bool usable = false;
+    if (int32_t st = sequence_kernels_usable(gates->dtype, batch, hidden, steps, &usable)) return st;
+    if (!usable)
+        return gates->dtype == PRAD_F64 ? lstm_sequence_bwd_steps<double>(Wh, gates, C, tanh_c, dh_loss, dG, steps, batch, hidden)
+                                        : lstm_sequence_bwd_steps<float>(Wh, gates, C, tanh_c, dh_loss, dG, steps, batch, hidden);
     if (int32_t st = ensure_workspace(lstm_seq_partial_bytes(batch, hidden))) return st;
     LstmSeqArgs a{};
     a.Wh = F(Wh); a.G = F(gates); a.C = F(C); a.TC = F(tanh_c); a.dHl = F(dh_loss); a.dG = F(dG);

@@ -8,6 +8,7 @@ import pytest
 
 from conftest import assert_long_sum_parity, assert_parity, norm_err, strict_err
 from oracle import compose
+from parallelreverseautodiff_amd import _lib
 from parallelreverseautodiff_amd.exceptions import ArgumentException, InvalidOperationException
 from parallelreverseautodiff_amd.lstm import LSTMLayer
 
@@ -119,11 +120,50 @@ def test_whole_sequence_shapes_it_does_not_take(gpu):
     assert layer.lib.prad_lstm_sequence_fwd(layer.Wh.handle, layer.G.handle, layer.C.handle, layer.Hs.handle, layer.TC.handle, 3) != 0   # rows % steps
 
 
+def _error_text(lib):
+    return lib.prad_last_error().decode()
+
+
+def test_whole_sequence_falls_back_when_the_device_does_not_hold_the_grid(gpu):
+    """The first sequence call asks the device, with a roll-call kernel of the same grid and footprint, whether it holds
+    the whole grid at once.  Forced to fail from the host (a negative poll limit makes the probe report failure without
+    waiting for anybody; every kernel ends normally), the sequence kernels go off, the calls run one launch per time step instead and
+    succeed, and the results are those of the per-step layer bit for bit."""
+    shape = (64, 512, 128, 16)
+    code = _lib.PRAD_F32
+    lib = _lib.load()
+    assert lib.prad_lstm_sequence_enable(1) == 0
+    os.environ["PRAD_LSTM_SPIN_LIMIT"] = "-1"
+    try:
+        layer, ref = LSTMLayer(*shape, dtype=np.float32), LSTMLayer(*shape, dtype=np.float32, sequence=False)
+        assert layer.sequence and not ref.sequence
+        layer.step(); ref.step()
+        gpu.Synchronize()                                               # no error: nothing partial was written
+        assert "one launch per time step" in _error_text(lib)
+        assert lib.prad_lstm_sequence_supported(code, shape[2], shape[1], shape[3]) == 0
+    finally:
+        del os.environ["PRAD_LSTM_SPIN_LIMIT"]
+    for _ in range(2):
+        layer.step(); ref.step()
+    gpu.Synchronize()
+    for x, y in ((layer.W, ref.W), (layer.dW, ref.dW), (layer.dG, ref.dG), (layer.Hs, ref.Hs), (layer.dX, ref.dX), (layer.loss, ref.loss)):
+        assert np.array_equal(x.download(), y.download())
+    assert lib.prad_lstm_sequence_enable(1) == 0
+    assert lib.prad_lstm_sequence_supported(code, shape[2], shape[1], shape[3]) == 1
+
+
 def test_whole_sequence_kernel_gives_up_instead_of_waiting_forever(gpu):
-    """Every wait on a peer workgroup is bounded.  With a limit of one poll some workgroup gives up at once; all the
-    others then leave at their next wait, the kernels end normally, and the next wait for the stream reports it.  The
-    step after, with the default limit, is unaffected."""
-    layer, ref = LSTMLayer(64, 512, 128, 16, dtype=np.float32, sequence=True), LSTMLayer(64, 512, 128, 16, dtype=np.float32, sequence=True)
+    """Every wait on a peer workgroup is bounded.  After a grid has been proven, a limit of one poll makes some workgroup
+    give up at once inside the sequence kernels; all the others then leave at their next wait, the kernels end
+    normally, the next wait for the stream reports it, and the sequence kernels stay off: the steps after that run
+    per time step and are right.  Turning the kernels on again restores the one-launch path."""
+    shape = (64, 512, 128, 16)
+    lib = _lib.load()
+    assert lib.prad_lstm_sequence_enable(1) == 0
+    layer, ref = LSTMLayer(*shape, dtype=np.float32), LSTMLayer(*shape, dtype=np.float32, sequence=False)
+    seq = LSTMLayer(*shape, dtype=np.float32)
+    layer.step(update=False); seq.step(update=False)                   # proves the grid with the default limit
+    gpu.Synchronize()
     os.environ["PRAD_LSTM_SPIN_LIMIT"] = "1"
     try:
         layer.step(update=False)
@@ -131,6 +171,24 @@ def test_whole_sequence_kernel_gives_up_instead_of_waiting_forever(gpu):
             gpu.Synchronize()
     finally:
         del os.environ["PRAD_LSTM_SPIN_LIMIT"]
-    layer.step(update=False); ref.step(update=False)
+    assert lib.prad_lstm_sequence_supported(_lib.PRAD_F32, shape[2], shape[1], shape[3]) == 0
+    layer.step(update=False); ref.step(update=False)                   # per time step inside the sequence calls
     gpu.Synchronize()
     assert np.array_equal(layer.dW.download(), ref.dW.download())
+    assert np.array_equal(layer.Hs.download(), ref.Hs.download())
+    assert lib.prad_lstm_sequence_enable(1) == 0
+    layer.step(update=False); seq.step(update=False)                   # the one-launch path again, after a fresh probe
+    gpu.Synchronize()
+    assert np.array_equal(layer.dW.download(), seq.dW.download())
+
+
+def test_sequence_calls_take_every_shape_and_element_type(gpu, oracle):
+    """Shapes and element types the one-launch kernels do not take run per time step inside the same two calls."""
+    for dtype, shape in ((np.float64, (16, 64, 16, 4)), (np.float32, (16, 32, 8, 5))):
+        a = LSTMLayer(*shape, dtype=dtype, sequence=False)
+        b = LSTMLayer(*shape, dtype=dtype, sequence=False)
+        b.sequence = True                                              # drive the sequence entry points anyway
+        a.step(); b.step()
+        gpu.Synchronize()
+        for x, y in ((a.W, b.W), (a.dW, b.dW), (a.Hs, b.Hs), (a.dX, b.dX)):
+            assert np.array_equal(x.download(), y.download())
