@@ -226,6 +226,10 @@ bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size);
 bool gemm_skinny_eligible(const GemmArgs<float>& a);
 size_t gemm_skinny_workspace_bytes(const GemmArgs<float>& a);
 hipError_t launch_gemm_skinny(const GemmArgs<float>& a, hipStream_t stream);
+// A . op(B) in float with tens of thousands of rows and a right operand small enough to stay in LDS (csrc/gemm_tall.hip),
+// any elementwise epilogue; returns hipErrorNotSupported for other products.
+bool gemm_tall_eligible(const GemmArgs<float>& a);
+hipError_t launch_gemm_tall(const GemmArgs<float>& a, hipStream_t stream);
 // A product on 128 x 128 tiles whose tile count leaves a poorly filled last round of workgroups (576 tiles over 512
 // workgroup slots: 64 tiles would run alone on 64 compute units while 192 sit idle) splits that many tiles along K
 // so that they fill the chip too.  Returns how many ways (0: none) and, through shared_tiles, how many tiles;

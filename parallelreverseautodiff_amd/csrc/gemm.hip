@@ -1257,6 +1257,10 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
             const hipError_t e = launch_gemm_skinny(a, stream);
             if (e != hipErrorNotSupported) return e;
         }
+        if (epi != EPI_TILE_SUM) {
+            const hipError_t e = launch_gemm_tall(a, stream);
+            if (e != hipErrorNotSupported) return e;
+        }
     }
     if (a.nseg > 1) {
         // Sum of nseg products: one operand pair per split, partial results added in pair order.

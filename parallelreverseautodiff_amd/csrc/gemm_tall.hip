@@ -1,0 +1,383 @@
+// Tall products in float: C[M x N] = A[M x K] . op(B) with tens of thousands of rows and a small right operand
+// (K x N floats fit one compute unit's LDS) - a layer of 96 to 384 units applied to every token of a batch, forward
+// (MatrixMultiplyOperation.Forward, src/RMAD/MatrixMultiplyOperation.cs:50-80, with the bias add and activation that
+// follow it in the graph) and the input gradient of the same layer (dA = dC . B^T, :94-104, with the upstream
+// activation's Backward).  On 128 x 128 output tiles such a product is a single round of workgroups that all load, then
+// all multiply, then all store: nothing overlaps, and it runs at a quarter of what either the matrix cores or the
+// memory could do.  Here the right operand is resident and the rows stream:
+//
+//   * every workgroup (one per compute unit, sixteen wavefronts) first copies the whole of B into LDS, already cut into
+//     MFMA fragments: element (y, j, i, g, n) is B[16 j + 4 g + i][16 y + n], so that a wavefront's 64 lanes (g, n) read 64
+//     consecutive floats for one MFMA step (no bank conflicts; 16-byte reads per lane were measured with 60 % of the LDS
+//     cycles lost to conflicts);
+//   * the work is cut into units of 16 rows by NYW 16-column tiles (NYW = 4, 3 or 2: many small units, so that a compute
+//     unit's four matrix cores get shares that differ by little); a workgroup owns a contiguous range of units
+//     and each of its wavefronts walks its share of them alone (no barrier after the fill).  A lane (m, g) of the
+//     wavefront loads 16 bytes A[row0 + m][16 j + 4 g .. + 3] straight into registers - the four k of a lane's vector are
+//     four MFMA steps, paired with the B values of the same (j, g) - 96 columns of a unit at a time, each half of them
+//     fetched again (for the next 96 columns, or the next unit) as soon as its MFMAs are issued, so a load has the other
+//     half's multiplications to arrive;
+//   * the MFMA takes the B fragment as its first operand and the A fragment as its second: the 16 x 16 result is then
+//     C^T, and a lane holds C[row0 + m][16 y + 4 g .. + 3] - four neighbours of one row - so bias, pre-activation copy,
+//     activation, the upstream activation's derivative and the store are all 16-byte accesses with no trip through LDS.
+//
+// Per element the arithmetic is that of the tiled kernels' elementwise epilogue, in the same order; only the order of the
+// sum along K differs (one chain of K / 4 MFMA steps; K <= 384 here).
+#include "common.h"
+
+#include <cstdlib>
+
+#ifdef PRAD_TALL_TRACE
+__device__ long long prad_tall_trace[256 * 16 * 4];  // (a tuning aid: per-wavefront clock readings)
+#endif
+
+namespace prad {
+
+namespace {
+
+typedef float f4t __attribute__((ext_vector_type(4)));
+
+constexpr int TALL_THREADS = 1024;
+constexpr int TALL_WAVES = TALL_THREADS / 64;
+constexpr int TALL_CH = 6;                       // 16-wide k groups per chunk: 96 columns of A per load round
+constexpr int HALF = TALL_CH / 2;
+constexpr size_t TALL_MAX_B = 144 * 1024;        // K * N * 4 bytes at most (96 x 384, 384 x 96)
+constexpr size_t TALL_MAX_LDS = TALL_MAX_B + 2048;  // and the bias, N <= 384 floats
+constexpr int64_t TALL_MIN_ROWS = 8192;
+
+struct TallArgs {
+    const float* A; const float* B; float* C;
+    const float* bias; float* Z; const float* act_src;
+    long lda, ldb, ldc, ldz, ld_act;
+    int M, N, K;
+    int transB, accumulate, act_fwd, act_bwd;
+    float alpha;
+    int blocks;  // 16-row blocks in all
+    int parts;   // column parts per block: N / 16 / NYW
+};
+
+__device__ __forceinline__ f4t load16(const float* base, unsigned byte_offset) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, -1, 0x00020000);
+    return __builtin_bit_cast(f4t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0));
+}
+
+// What follows a unit's multiplications.  TALL_STORE: store (or add into) C, with the bias if there is one: straight-line
+// code, a few instructions per 16 bytes.  TALL_GENERAL: everything (pre-activation copy, activation, upstream activation's
+// derivative) in a runtime loop, see `finish_general`.
+constexpr int TALL_STORE = 0, TALL_GENERAL = 1;
+
+// NYW: 16-column tiles (accumulators per lane) of a unit.  ONE_CHUNK: K == 96, every pass of the main loop is a whole unit.
+template <int NYW, int EPI, bool ONE_CHUNK>
+__global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallArgs p) {
+    extern __shared__ __attribute__((aligned(16))) float bfrag[];  // [y][j][i][g][n], then the bias
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (said to be uniform: loop counts and load bases that depend on it stay scalar)
+    const int li = lane & 15, g = lane >> 4;
+    const int KJ = p.K / 16;
+#ifdef PRAD_TALL_TRACE
+    const long long t_begin = wall_clock64();
+    long long t_first = 0;
+#endif
+
+    // ---- this wavefront's units: the workgroup owns [first, first + count), its wavefronts take every sixteenth ----
+    const int units = p.blocks * p.parts;
+    const int first = (int)((long)blockIdx.x * units / gridDim.x);
+    const int count = (int)((long)(blockIdx.x + 1) * units / gridDim.x) - first;
+    const int nchunks = KJ / TALL_CH;
+    const int my_units = count > wave ? (count - wave + TALL_WAVES - 1) / TALL_WAVES : 0;
+    const int total = my_units * nchunks;  // (unit, chunk) pairs of this wavefront, walked in order
+
+    auto pair_unit = [&](int q) { return first + wave + TALL_WAVES * (q / nchunks); };
+    // lane part of the A address: row li of the unit's block, 16 bytes at k = 4 g of a 16-wide group
+    auto a_offset = [&](int unit) {
+        const int row = min(16 * (unit / p.parts) + li, p.M - 1);  // rows past the end repeat the last one; they are never stored
+        return (unsigned)(((long)row * p.lda + 4 * g) * 4);
+    };
+    f4t a[TALL_CH];
+    // half a chunk's loads: the registers are refilled as soon as the MFMAs that read them have been issued
+    auto load_half = [&](int q, int h) {
+        const int c = q % nchunks;
+        const unsigned off = a_offset(pair_unit(q));
+#pragma unroll
+        for (int j = 0; j < HALF; ++j) a[h * HALF + j] = load16(p.A + (c * TALL_CH + h * HALF + j) * 16, off);
+    };
+
+    // (the first unit's rows are on their way while B is copied)
+    if (my_units > 0) {
+        load_half(0, 0);
+        load_half(0, 1);
+    }
+
+    // ---- B -> LDS as fragments.  One 16-byte load per lane and step; a wavefront's 64 lanes take one (y, j) pair, the
+    // 256 consecutive floats of the fragment array, so that its LDS stores fall on distinct banks (walking B row by row
+    // instead had the 64 lanes of a store 16 deep on the same banks: 7 us of a 42 us launch).  Eight loads are in flight
+    // per thread: the copy is latency, not volume.
+    {
+        constexpr int FILL = 8;
+        const int nvec = (p.N / 16) * KJ * 64;  // = K * N / 4
+        for (int v0 = tid; v0 < nvec; v0 += FILL * TALL_THREADS) {
+            f4t x[FILL];
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int v = min(v0 + u * TALL_THREADS, nvec - 1);
+                const int pair = v >> 6, l = v & 63, y = pair / KJ, j = pair - y * KJ;
+                // transposed B is stored [n][k]: lane (gg, nn) reads the four i of (j, gg) for column 16 y + nn;
+                // plain B is stored [k][n]: lane (i, gg, n4) reads four neighbouring columns of row k = 16 j + 4 gg + i
+                const long at = p.transB ? (long)(16 * y + (l & 15)) * p.ldb + 16 * j + 4 * (l >> 4)
+                                         : (long)(16 * j + 4 * ((l >> 2) & 3) + (l >> 4)) * p.ldb + 16 * y + 4 * (l & 3);
+                x[u] = *reinterpret_cast<const f4t*>(p.B + at);
+            }
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int v = v0 + u * TALL_THREADS;
+                if (v >= nvec) continue;
+                const int pair = v >> 6, l = v & 63;
+                float* dst = bfrag + pair * 256;
+                if (p.transB) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) dst[i * 64 + l] = x[u][i];
+                } else {
+                    *reinterpret_cast<f4t*>(dst + (l >> 4) * 64 + ((l >> 2) & 3) * 16 + 4 * (l & 3)) = x[u];
+                }
+            }
+        }
+    }
+    if (p.bias != nullptr)
+        for (int n = tid; n < p.N; n += TALL_THREADS) bfrag[p.K * p.N + n] = p.bias[n];
+    __syncthreads();
+#ifdef PRAD_TALL_TRACE
+    const long long t_fill = wall_clock64();
+#endif
+
+    if (my_units == 0) return;
+    f4t acc[NYW];
+    // One k step (j, i) at a time across all NYW accumulators, so that consecutive MFMAs never depend on each other; the
+    // NYW values of B for a step are read from LDS one step ahead of the MFMAs that use them.
+    auto multiply_half = [&](int unit, int c, int h) {
+        int b_index = ((unit % p.parts) * NYW * KJ + c * TALL_CH + h * HALF) * 256 + lane;
+        // (opaque per pass: with K == 96 the addresses never change and every B value would be hoisted into registers;
+        // the index, not the pointer, so that the reads stay LDS reads)
+        asm volatile("" : "+v"(b_index));
+        const float* b0 = bfrag + b_index;
+        constexpr int STEPS = HALF * 4;
+        float b[2][NYW];
+        auto read_b = [&](int t) {  // t = 4 jj + i
+            const float* q = b0 + t * 64;
+#pragma unroll
+            for (int y = 0; y < NYW; ++y) b[t & 1][y] = q[(long)y * KJ * 256];
+        };
+        read_b(0);
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+            const int j = h * HALF + t / 4, i = t % 4;
+            if (t + 1 < STEPS) read_b(t + 1);
+#pragma unroll
+            for (int y = 0; y < NYW; ++y) acc[y] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[t & 1][y], a[j][i], acc[y], 0, 0, 0);
+        }
+    };
+    const float* bias_lds = bfrag + p.K * p.N;
+    // The finished unit, TALL_STORE: per 16-column tile one LDS read (bias), four additions, one 16-byte store.
+    auto finish_store = [&](int unit) {
+        const int row = 16 * (unit / p.parts) + li, col0 = 16 * NYW * (unit % p.parts) + 4 * g;
+        if (row >= p.M) return;
+        float* crow = p.C + (long)row * p.ldc + col0;
+#pragma unroll
+        for (int y = 0; y < NYW; ++y) {
+            f4t v = acc[y];
+            if (p.bias != nullptr) {
+                const f4t bv = *reinterpret_cast<const f4t*>(bias_lds + col0 + 16 * y);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] + bv[e];
+            }
+            f4t* out = reinterpret_cast<f4t*>(crow + 16 * y);
+            if (p.accumulate) {
+                const f4t old = *out;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = old[e] + v[e];
+            }
+            *out = v;
+        }
+    };
+    // The finished unit, TALL_GENERAL.  A runtime loop over its tiles (the activation code is there once, not once per
+    // accumulator); the accumulators, and the values the upstream activation's derivative is taken of, rotate through
+    // element 0 so that no register is indexed at run time.  Those values are fetched while the unit's last 96 columns are
+    // multiplied.
+    f4t src[NYW];
+    auto fetch_src = [&](int unit) {
+        const int row = min(16 * (unit / p.parts) + li, p.M - 1);
+        const float* s0 = p.act_src + (long)row * p.ld_act + 16 * NYW * (unit % p.parts) + 4 * g;
+#pragma unroll
+        for (int y = 0; y < NYW; ++y) src[y] = *reinterpret_cast<const f4t*>(s0 + 16 * y);
+    };
+    auto finish_general = [&](int unit) {
+        const int row = 16 * (unit / p.parts) + li, col0 = 16 * NYW * (unit % p.parts) + 4 * g;
+        const bool live = row < p.M;
+        const long crow = (long)row * p.ldc, zrow = (long)row * p.ldz;
+#pragma unroll 1
+        for (int y = 0; y < NYW; ++y) {
+            const int col = col0 + 16 * y;
+            f4t v = acc[0];
+            const f4t sv = src[0];
+#pragma unroll
+            for (int k = 0; k + 1 < NYW; ++k) {
+                acc[k] = acc[k + 1];
+                src[k] = src[k + 1];
+            }
+            if (!live) continue;
+            if (p.bias != nullptr) {
+                const f4t bv = *reinterpret_cast<const f4t*>(bias_lds + col);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] + bv[e];
+            }
+            if (p.Z != nullptr) *reinterpret_cast<f4t*>(p.Z + zrow + col) = v;
+            if (p.act_fwd != ACT_NONE) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = act_forward<float>(p.act_fwd, v[e], p.alpha);
+            }
+            if (p.act_bwd != ACT_NONE) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * act_derivative<float>(p.act_bwd, sv[e], p.alpha);
+            }
+            f4t* out = reinterpret_cast<f4t*>(p.C + crow + col);
+            if (p.accumulate) {
+                const f4t old = *out;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = old[e] + v[e];
+            }
+            *out = v;
+        }
+    };
+    auto finish = [&](int unit) {
+        if (EPI == TALL_STORE) finish_store(unit);
+        else finish_general(unit);
+    };
+    auto zero = [&] {
+#pragma unroll
+        for (int y = 0; y < NYW; ++y) acc[y] = f4t{0.f, 0.f, 0.f, 0.f};
+    };
+    if (ONE_CHUNK) {
+        // A pass is a whole unit, in straight-line code (a wait placed after a branch around the stores would include them).
+        zero();
+#pragma unroll 1
+        for (int q = 0;; ++q) {
+            const int unit = pair_unit(q), next = min(q + 1, total - 1);  // (the last unit is fetched twice rather than branched around)
+            if (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE) fetch_src(unit);
+            multiply_half(unit, 0, 0);
+            load_half(next, 0);
+            multiply_half(unit, 0, 1);
+            load_half(next, 1);
+            finish(unit);
+#ifdef PRAD_TALL_TRACE
+            if (q == 0) t_first = wall_clock64();
+#endif
+            if (q + 1 >= total) break;
+            zero();
+        }
+    } else {
+#pragma unroll 1
+        for (int q = 0; q < total; ++q) {
+            const int unit = pair_unit(q), c = q % nchunks, next = min(q + 1, total - 1);
+            if (c == 0) zero();
+            if (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE && c == nchunks - 1) fetch_src(unit);
+            multiply_half(unit, c, 0);
+            load_half(next, 0);
+            multiply_half(unit, c, 1);
+            load_half(next, 1);
+            if (c == nchunks - 1) {
+                finish(unit);
+#ifdef PRAD_TALL_TRACE
+                if (q == nchunks - 1) t_first = wall_clock64();
+#endif
+            }
+        }
+    }
+#ifdef PRAD_TALL_TRACE
+    if (lane == 0 && blockIdx.x < 256) {
+        long long* o = prad_tall_trace + (blockIdx.x * TALL_WAVES + wave) * 4;
+        o[0] = t_begin; o[1] = t_fill; o[2] = t_first; o[3] = wall_clock64();
+    }
+#endif
+}
+
+int tall_compute_units() {
+    static const int v = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        return n;
+    }();
+    return v;
+}
+
+template <int NYW, int EPI, bool ONE_CHUNK>
+hipError_t launch_variant(const TallArgs& k, unsigned grid, size_t lds, hipStream_t stream) {
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tall_kernel<NYW, EPI, ONE_CHUNK>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)TALL_MAX_LDS);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL((gemm_tall_kernel<NYW, EPI, ONE_CHUNK>), dim3(grid), dim3(TALL_THREADS), lds, stream, k);
+    return hipGetLastError();
+}
+template <int NYW>
+hipError_t launch_nyw(const TallArgs& k, unsigned grid, size_t lds, hipStream_t stream) {
+    const bool general = k.Z != nullptr || k.act_fwd != ACT_NONE || k.act_bwd != ACT_NONE;
+    const bool one = k.K == 16 * TALL_CH;
+    if (general) return one ? launch_variant<NYW, TALL_GENERAL, true>(k, grid, lds, stream) : launch_variant<NYW, TALL_GENERAL, false>(k, grid, lds, stream);
+    return one ? launch_variant<NYW, TALL_STORE, true>(k, grid, lds, stream) : launch_variant<NYW, TALL_STORE, false>(k, grid, lds, stream);
+}
+
+// Tiles per unit for a product of `ny` 16-column tiles: four, three or two, whichever divides ny first.  Narrow units
+// keep the epilogue's registers few (the general one holds a second value per accumulator) and give every matrix core
+// many units, so that their shares differ by little; wider ones (six, eight, nine tiles) were measured no faster for
+// the plain store and up to 40 % slower for the general epilogue.
+int tall_unit_tiles(int64_t ny) {
+    static const int forced = [] { const char* e = getenv("PRAD_GEMM_TALL_UNIT_TILES"); return e ? atoi(e) : 0; }();  // tuning aid
+    for (int w : {4, 3, 2})
+        if (forced == w && ny % w == 0) return w;
+    for (int w : {4, 3, 2})
+        if (ny % w == 0) return w;
+    return 0;
+}
+
+bool aligned16(const void* q, int64_t ld) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) % 16 == 0 && ld % 4 == 0); }
+
+}  // namespace
+
+// Shapes that go to the kernel above: float, A not transposed, one product, at least TALL_MIN_ROWS rows, K a multiple of
+// 96 and N a multiple of 32 or 48 with K * N floats within 144 KB, every row 16-byte aligned.
+// PRAD_GEMM_TALL=0 switches it off (a tuning aid).
+bool gemm_tall_eligible(const GemmArgs<float>& a) {
+    static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_TALL"); return !(e && e[0] == '0'); }();
+    static const int64_t min_rows = [] { const char* e = getenv("PRAD_GEMM_TALL_MIN_ROWS"); return e ? (int64_t)atoll(e) : TALL_MIN_ROWS; }();
+    if (!enabled || a.transA || a.batch != 1 || a.batch_inner > 1 || a.nseg > 1 || a.tile_sums != nullptr || a.colsum_dst != nullptr ||
+        a.lstm_hidden != 0)
+        return false;
+    if (a.M < min_rows || a.M >= (1 << 27) || a.K < 16 * TALL_CH || a.K % (16 * TALL_CH) != 0 || a.N % 16 != 0) return false;
+    if (tall_unit_tiles(a.N / 16) == 0) return false;
+    if ((size_t)a.K * a.N * sizeof(float) > TALL_MAX_B) return false;
+    if (!aligned16(a.A, a.lda) || !aligned16(a.B, a.ldb) || !aligned16(a.C, a.ldc) || !aligned16(a.Z, a.ldz) ||
+        !aligned16(a.act_src, a.ld_act) || !aligned16(a.bias, 4))
+        return false;
+    if (a.lda >= (1 << 20)) return false;  // (a lane's byte offset into A is kept in 32 bits: rows * lda * 4 < 2^32 is checked at launch)
+    return true;
+}
+
+hipError_t launch_gemm_tall(const GemmArgs<float>& a, hipStream_t stream) {
+    if (!gemm_tall_eligible(a) || (uint64_t)a.M * (uint64_t)a.lda * 4u >= ((uint64_t)1 << 32)) return hipErrorNotSupported;
+    TallArgs k{};
+    k.A = a.A; k.B = a.B; k.C = a.C; k.bias = a.bias; k.Z = a.Z; k.act_src = a.act_src;
+    k.lda = a.lda; k.ldb = a.ldb; k.ldc = a.ldc; k.ldz = a.ldz; k.ld_act = a.ld_act;
+    k.M = (int)a.M; k.N = (int)a.N; k.K = (int)a.K;
+    k.transB = a.transB; k.accumulate = a.accumulate; k.act_fwd = a.act_fwd; k.act_bwd = a.act_bwd; k.alpha = a.alpha;
+    k.blocks = (int)((a.M + 15) / 16);
+    const int nyw = tall_unit_tiles(a.N / 16);
+    k.parts = (int)(a.N / 16) / nyw;
+    const unsigned grid = (unsigned)std::min<int64_t>(tall_compute_units(), (int64_t)k.blocks * k.parts);
+    const size_t lds = ((size_t)a.K * a.N + (size_t)a.N) * sizeof(float);  // B as fragments, then the bias
+    switch (nyw) {
+        case 2: return launch_nyw<2>(k, grid, lds, stream);
+        case 3: return launch_nyw<3>(k, grid, lds, stream);
+        case 4: return launch_nyw<4>(k, grid, lds, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace prad

@@ -25,6 +25,11 @@ constexpr int OPT_THREADS = 256;
 constexpr int OPT_CHUNK_SMALL = 4096;
 template <typename T> constexpr int OPT_CHUNK_LARGE = 32768 / (int)sizeof(T);
 constexpr int64_t LARGE_CHUNK_FROM = (int64_t)4 << 20;  // total elements of a launch
+// Adam alone moves seven streams (four read, three written) per workgroup: there 16 KB per stream and workgroup is the
+// better cut (64 Mi doubles: 0.69 to 0.705 of 8 TB/s with 32 KB, 0.72 to 0.74 with 16 KB or 8 KB; the arithmetic does
+// not show in the time at all, and neither workgroups that loop over several chunks nor addresses of the four tensors
+// skewed against each other gain anything).
+template <typename T> constexpr int ADAM_CHUNK_LARGE = 16384 / (int)sizeof(T);
 // A model of a few million parameters or less is only a few 4096-element chunks per compute unit, a small one not even
 // one (the 235 000 of the 784-256-128-10 network: 58 workgroups, each moving its 229 KB at one compute unit's share of
 // the bandwidth - 11 us for 13 MB); chunks of 1024 spread it over four times as many.
@@ -447,10 +452,11 @@ static hipError_t launch_groups(const TensorDesc<T>* host, int nt, void* workspa
         const int gn = nt - g0 < MAX_TABLE ? nt - g0 : MAX_TABLE;
         int64_t total = 0;
         for (int i = 0; i < gn; ++i) total += host[g0 + i].n;
+        constexpr int LARGE = (ADAM && !CLIP) ? ADAM_CHUNK_LARGE<T> : OPT_CHUNK_LARGE<T>;
         const hipError_t e = total < TINY_CHUNK_BELOW
                                  ? launch_group<T, OPT_CHUNK_TINY, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs)
-                             : (OPT_CHUNK_LARGE<T> != OPT_CHUNK_SMALL && total >= LARGE_CHUNK_FROM)
-                                 ? launch_group<T, OPT_CHUNK_LARGE<T>, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs)
+                             : (LARGE != OPT_CHUNK_SMALL && total >= LARGE_CHUNK_FROM)
+                                 ? launch_group<T, LARGE, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs)
                                  : launch_group<T, OPT_CHUNK_SMALL, CLIP, ADAM>(host + g0, gn, workspace, clip_value, min_value, update, s, obs);
         if (e != hipSuccess) return e;
     }
