@@ -12,7 +12,7 @@
 //     cycles lost to conflicts);
 //   * the work is cut into units of 16 rows by NYW 16-column tiles (NYW = 4, 3 or 2: many small units, so that a compute
 //     unit's four matrix cores get shares that differ by little); a workgroup owns a contiguous range of units
-//     and each of its wavefronts walks its share of them alone (no barrier after the fill).  A lane (m, g) of the
+//     and each of its wavefronts takes one unit after another from it, alone (no barrier after the fill).  A lane (m, g) of the
 //     wavefront loads 16 bytes A[row0 + m][16 j + 4 g .. + 3] straight into registers - the four k of a lane's vector are
 //     four MFMA steps, paired with the B values of the same (j, g) - 96 columns of a unit at a time, each half of them
 //     fetched again (for the next 96 columns, or the next unit) as soon as its MFMAs are issued, so a load has the other
@@ -69,7 +69,7 @@ constexpr int TALL_STORE = 0, TALL_GENERAL = 1;
 // NYW: 16-column tiles (accumulators per lane) of a unit.  ONE_CHUNK: K == 96, every pass of the main loop is a whole unit.
 template <int NYW, int EPI, bool ONE_CHUNK>
 __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallArgs p) {
-    extern __shared__ __attribute__((aligned(16))) float bfrag[];  // [y][j][i][g][n], then the bias
+    extern __shared__ __attribute__((aligned(16))) float bfrag[];  // [y][j][i][g][n], then the bias, then the unit counter
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (said to be uniform: loop counts and load bases that depend on it stay scalar)
     const int li = lane & 15, g = lane >> 4;
@@ -79,15 +79,16 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
     long long t_first = 0;
 #endif
 
-    // ---- this wavefront's units: the workgroup owns [first, first + count), its wavefronts take every sixteenth ----
+    // ---- units: the workgroup owns [first, first + count); wavefront w starts with unit w and then takes the next unit
+    // nobody has taken yet (a counter in LDS), so that all sixteen finish within a unit of each other ----
     const int units = p.blocks * p.parts;
     const int first = (int)((long)blockIdx.x * units / gridDim.x);
     const int count = (int)((long)(blockIdx.x + 1) * units / gridDim.x) - first;
     const int nchunks = KJ / TALL_CH;
-    const int my_units = count > wave ? (count - wave + TALL_WAVES - 1) / TALL_WAVES : 0;
-    const int total = my_units * nchunks;  // (unit, chunk) pairs of this wavefront, walked in order
+    const bool working = wave < count;
+    int* next_counter = reinterpret_cast<int*>(bfrag + p.K * p.N + p.N);
+    if (tid == 0) *next_counter = TALL_WAVES;  // (published by the barrier after the copy of B)
 
-    auto pair_unit = [&](int q) { return first + wave + TALL_WAVES * (q / nchunks); };
     // lane part of the A address: row li of the unit's block, 16 bytes at k = 4 g of a 16-wide group
     auto a_offset = [&](int unit) {
         const int row = min(16 * (unit / p.parts) + li, p.M - 1);  // rows past the end repeat the last one; they are never stored
@@ -95,25 +96,25 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
     };
     f4t a[TALL_CH];
     // half a chunk's loads: the registers are refilled as soon as the MFMAs that read them have been issued
-    auto load_half = [&](int q, int h) {
-        const int c = q % nchunks;
-        const unsigned off = a_offset(pair_unit(q));
+    auto load_half = [&](int unit, int c, int h) {
+        const unsigned off = a_offset(unit);
 #pragma unroll
         for (int j = 0; j < HALF; ++j) a[h * HALF + j] = load16(p.A + (c * TALL_CH + h * HALF + j) * 16, off);
     };
 
     // (the first unit's rows are on their way while B is copied)
-    if (my_units > 0) {
-        load_half(0, 0);
-        load_half(0, 1);
+    if (working) {
+        load_half(first + wave, 0, 0);
+        load_half(first + wave, 0, 1);
     }
 
     // ---- B -> LDS as fragments.  One 16-byte load per lane and step; a wavefront's 64 lanes take one (y, j) pair, the
     // 256 consecutive floats of the fragment array, so that its LDS stores fall on distinct banks (walking B row by row
-    // instead had the 64 lanes of a store 16 deep on the same banks: 7 us of a 42 us launch).  Eight loads are in flight
-    // per thread: the copy is latency, not volume.
+    // instead had the 64 lanes of a store 16 deep on the same banks).  Up to nine loads are in flight per thread, which is
+    // all of the largest B in one round: the copy is latency, not volume.
     {
-        constexpr int FILL = 8;
+        constexpr int FILL = 9;
+        static_assert(TALL_MAX_B / 16 <= (size_t)FILL * TALL_THREADS, "one round copies the largest B");
         const int nvec = (p.N / 16) * KJ * 64;  // = K * N / 4
         for (int v0 = tid; v0 < nvec; v0 += FILL * TALL_THREADS) {
             f4t x[FILL];
@@ -149,7 +150,7 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
     const long long t_fill = wall_clock64();
 #endif
 
-    if (my_units == 0) return;
+    if (!working) return;
     f4t acc[NYW];
     // One k step (j, i) at a time across all NYW accumulators, so that consecutive MFMAs never depend on each other; the
     // NYW values of B for a step are read from LDS one step ahead of the MFMAs that use them.
@@ -255,41 +256,48 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
 #pragma unroll
         for (int y = 0; y < NYW; ++y) acc[y] = f4t{0.f, 0.f, 0.f, 0.f};
     };
-    if (ONE_CHUNK) {
-        // A pass is a whole unit, in straight-line code (a wait placed after a branch around the stores would include them).
-        zero();
+    // One unit per pass.  The next unit's number is asked for at the top of the pass and read when the first loads for
+    // it are due (half a chunk of MFMAs later).  With ONE_CHUNK the pass is straight-line code: a wait placed after a
+    // branch around the stores would include them.
+    int unit = first + wave;
 #pragma unroll 1
-        for (int q = 0;; ++q) {
-            const int unit = pair_unit(q), next = min(q + 1, total - 1);  // (the last unit is fetched twice rather than branched around)
+    for (int pass = 0;; ++pass) {
+        int ticket = 0;
+        if (lane == 0) ticket = __hip_atomic_fetch_add(next_counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        int next_unit = unit;
+        bool has_next = false;
+        auto resolve = [&] {
+            const int t = __builtin_amdgcn_readfirstlane(ticket);
+            has_next = t < count;
+            next_unit = has_next ? first + t : unit;  // (the last unit is fetched twice rather than branched around)
+        };
+        zero();
+        if (ONE_CHUNK) {
             if (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE) fetch_src(unit);
             multiply_half(unit, 0, 0);
-            load_half(next, 0);
+            resolve();
+            load_half(next_unit, 0, 0);
             multiply_half(unit, 0, 1);
-            load_half(next, 1);
-            finish(unit);
-#ifdef PRAD_TALL_TRACE
-            if (q == 0) t_first = wall_clock64();
-#endif
-            if (q + 1 >= total) break;
-            zero();
-        }
-    } else {
+            load_half(next_unit, 0, 1);
+        } else {
 #pragma unroll 1
-        for (int q = 0; q < total; ++q) {
-            const int unit = pair_unit(q), c = q % nchunks, next = min(q + 1, total - 1);
-            if (c == 0) zero();
-            if (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE && c == nchunks - 1) fetch_src(unit);
-            multiply_half(unit, c, 0);
-            load_half(next, 0);
-            multiply_half(unit, c, 1);
-            load_half(next, 1);
-            if (c == nchunks - 1) {
-                finish(unit);
-#ifdef PRAD_TALL_TRACE
-                if (q == nchunks - 1) t_first = wall_clock64();
-#endif
+            for (int c = 0; c < nchunks; ++c) {
+                const bool last = c == nchunks - 1;
+                if (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE && last) fetch_src(unit);
+                multiply_half(unit, c, 0);
+                if (last) resolve();
+                const int nu = last ? next_unit : unit, nc = last ? 0 : c + 1;
+                load_half(nu, nc, 0);
+                multiply_half(unit, c, 1);
+                load_half(nu, nc, 1);
             }
         }
+        finish(unit);
+#ifdef PRAD_TALL_TRACE
+        if (pass == 0) t_first = wall_clock64();
+#endif
+        if (!has_next) break;
+        unit = next_unit;
     }
 #ifdef PRAD_TALL_TRACE
     if (lane == 0 && blockIdx.x < 256) {
@@ -371,7 +379,7 @@ hipError_t launch_gemm_tall(const GemmArgs<float>& a, hipStream_t stream) {
     const int nyw = tall_unit_tiles(a.N / 16);
     k.parts = (int)(a.N / 16) / nyw;
     const unsigned grid = (unsigned)std::min<int64_t>(tall_compute_units(), (int64_t)k.blocks * k.parts);
-    const size_t lds = ((size_t)a.K * a.N + (size_t)a.N) * sizeof(float);  // B as fragments, then the bias
+    const size_t lds = ((size_t)a.K * a.N + (size_t)a.N + 4) * sizeof(float);  // B as fragments, the bias, the unit counter
     switch (nyw) {
         case 2: return launch_nyw<2>(k, grid, lds, stream);
         case 3: return launch_nyw<3>(k, grid, lds, stream);
