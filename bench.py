@@ -518,8 +518,16 @@ def mlp_ops_leg(dtype_name, steps, warmup):
     after = stats()
     ms = ctypes.c_float()
     check(lib.prad_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    # the same walk driven by compiled code (libprad_hostwalk.so: C ABI calls only), where the host is no interpreter
+    compiled = None
+    try:
+        from parallelreverseautodiff_amd.feedforward import compiled_operation_walk
+        c_ms, c_loss, _ = compiled_operation_walk(dtype=dtype, steps=max(steps, 500), warmup=50)
+        compiled = {"wall_ms_per_step": c_ms, "steps_per_s": 1e3 / c_ms, "loss_after": c_loss}
+    except Exception as e:  # noqa: BLE001 - reported, not hidden
+        compiled = {"error": repr(e)}
     return {"wall_ms_per_step": wall_ms, "host_issue_ms_per_step": issue_ms, "device_ms_per_step": ms.value / steps,
-            "steps_per_s": 1e3 / wall_ms, "loss_after": float(net.loss.to_numpy()[0, 0]), "flop_per_step": net.flops_per_step(),
+            "steps_per_s": 1e3 / wall_ms, "compiled_caller": compiled, "loss_after": float(net.loss.to_numpy()[0, 0]), "flop_per_step": net.flops_per_step(),
             "operations_per_step": 2 * len(net.nodes) + 2, "device_mallocs_in_timed_steps": after[0] - before[0],
             "device_frees_in_timed_steps": after[1] - before[1], "stream_waits_in_timed_steps": after[2] - before[2],
             "pool_hits_in_timed_steps": after[3] - before[3]}
@@ -758,8 +766,10 @@ def summary_scalars(also):
     put("mlp_f64_steps_s", "mlp_train_steps_per_s_f64", "value")
     put("mlp_f64_cpu_steps_s", "mlp_train_steps_per_s_f64", "cpu_baseline", "steps_per_s")
     put("mlp_ops_f64_steps_s", "mlp_operation_walk_f64", "value")
+    put("mlp_ops_compiled_f64_steps_s", "mlp_operation_walk_f64", "detail", "compiled_caller", "steps_per_s")
     put("mlp_f32_steps_s", "mlp_train_steps_per_s_f32", "value")
     put("mlp_ops_f32_steps_s", "mlp_operation_walk_f32", "value")
+    put("mlp_ops_compiled_f32_steps_s", "mlp_operation_walk_f32", "detail", "compiled_caller", "steps_per_s")
     put("lstm_f32_steps_s", "lstm_train_steps_per_s_f32", "value")
     put("lstm_f32_frac", "lstm_train_steps_per_s_f32", "roofline", "frac")
     put("swin_f32_steps_s", "swin_block_train_steps_per_s_f32", "value")
@@ -862,6 +872,12 @@ def also_legs(args, table):
             out["mlp_operation_walk_" + d] = {"value": r["steps_per_s"], "unit": "steps/s", "ms_per_step": r["wall_ms_per_step"], "detail": r,
                                                "roofline": mfma_roofline(r["flop_per_step"], r["wall_ms_per_step"], d,
                                                                          "whole step, one launch per operation (%d operations)" % r["operations_per_step"])}
+            if "steps_per_s" in (r.get("compiled_caller") or {}):
+                c = r["compiled_caller"]
+                table.append({"config": "configs[0] MLP step, operation by operation, compiled caller of the C ABI", "precision": d,
+                              "gpu_ms": c["wall_ms_per_step"], "rate": c["steps_per_s"], "unit": "steps/s", "bound": "mfma",
+                              "frac_of_peak": r["flop_per_step"] / (c["wall_ms_per_step"] * 1e-3) / 1e12 / PEAK_TFLOPS[d],
+                              "cpu_ms": None, "cpu_cores": None, "speedup": None, "err_normwise": None, "err_elementwise_floor_1e-3_rms": None})
             table.append({"config": "configs[0] MLP step, operation by operation through the operation classes", "precision": d,
                           "gpu_ms": r["wall_ms_per_step"], "rate": r["steps_per_s"], "unit": "steps/s", "bound": "mfma",
                           "frac_of_peak": r["flop_per_step"] / (r["wall_ms_per_step"] * 1e-3) / 1e12 / PEAK_TFLOPS[d],

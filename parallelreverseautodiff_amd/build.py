@@ -52,7 +52,17 @@ def build_library(verbose=False):
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), 8)) as pool:
         objs = list(pool.map(compile_one, SOURCES))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs)
+    build_host_walk()
     return LIB_PATH
+
+
+def build_host_walk():
+    """libprad_hostwalk.so: a compiled caller of the C ABI (csrc/host_walk.cpp, host code only), used by the
+    benchmark and one test to drive a training step operation by operation without an interpreter in between."""
+    out = os.path.join(HERE, "libprad_hostwalk.so")
+    _run(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden", os.path.join(CSRC, "host_walk.cpp"), "-o", out,
+          "-L" + HERE, "-lprad_hip", "-Wl,-rpath,$ORIGIN"])
+    return out
 
 
 if __name__ == "__main__":

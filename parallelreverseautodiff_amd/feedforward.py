@@ -232,3 +232,34 @@ class OperationWalkNetwork:
 
     def flops_per_step(self):
         return 3.0 * sum(2.0 * self.batch * self.sizes[l] * self.sizes[l + 1] for l in range(len(self.W)))
+
+
+def compiled_operation_walk(sizes=(784, 256, 128, 10), batch=64, dtype=np.float64, seed=seeded.DEFAULT_SEED, parameters=None,
+                            steps=1, warmup=0, X=None, T=None):
+    """The same operation-by-operation step as OperationWalkNetwork, driven by compiled code instead of Python
+    (libprad_hostwalk.so, csrc/host_walk.cpp: nothing but C ABI calls, one per operation): what the boundary costs a
+    compiled caller such as the reference's C# classes.  Runs `warmup` + `steps` steps from the seeded initial weights
+    and returns (wall-clock ms per timed step, last loss, final weight matrices)."""
+    import os
+    _ensure_initialized()
+    _lib.load()
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libprad_hostwalk.so")
+    if not os.path.exists(path):
+        raise ImportError("libprad_hostwalk.so is not built (python -m parallelreverseautodiff_amd.build)")
+    walk = ctypes.CDLL(path).prad_hostwalk_mlp
+    walk.restype = ctypes.c_int32
+    dtype = np.dtype(dtype)
+    p = parameters or NeuralNetworkParameters(lite=dtype == np.float32)
+    L = len(sizes) - 1
+    W = [np.ascontiguousarray(seeded.xavier(seed, 10 + l, sizes[l], sizes[l + 1], dtype)) for l in range(L)]
+    X = np.ascontiguousarray(seeded.uniform(seed, 1, (batch, sizes[0]), 0.0, 1.0, dtype) if X is None else np.asarray(X, dtype))
+    T = np.ascontiguousarray(seeded.one_hot_labels(seed, 2, batch, sizes[-1], dtype) if T is None else np.asarray(T, dtype))
+    out = [np.empty_like(w) for w in W]
+    ptrs = lambda arrays: (ctypes.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+    ms, loss = ctypes.c_double(), ctypes.c_double()
+    d = ctypes.c_double
+    check(walk(ctypes.c_int32(_lib.PRAD_F64 if dtype == np.float64 else _lib.PRAD_F32), ctypes.c_int32(batch), ctypes.c_int32(L),
+               (ctypes.c_int64 * (L + 1))(*sizes), ptrs(W), ctypes.c_void_p(X.ctypes.data), ctypes.c_void_p(T.ctypes.data),
+               ctypes.c_int32(steps), ctypes.c_int32(warmup), d(p.LeakyReLUAlpha), d(p.ClipValue), d(p.MinimumClipValue),
+               d(p.LearningRate), d(p.AdamBeta1), d(p.AdamBeta2), d(p.AdamEpsilon), ctypes.byref(ms), ctypes.byref(loss), ptrs(out)))
+    return ms.value, loss.value, out

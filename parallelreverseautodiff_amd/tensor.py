@@ -84,8 +84,18 @@ class Tensor:
         return DeviceBuffer(h, self.dtype, 1, dev.depth * dev.rows, dev.cols, parent=dev)
 
     def MatrixMultiply(self, other, alpha=1.0, beta=0.0):
-        """alpha * this . other on the last two dimensions.  ``beta`` multiplies the freshly zeroed result array in
-        the reference and has no effect; it is accepted for signature compatibility."""
+        """alpha * this . other for two-dimensional tensors; anything else raises the reference's ArgumentException
+        (src/PRAD/Tensor.cs:574-577).  ``beta`` multiplies the freshly zeroed result array in the reference and has no
+        effect; it is accepted for signature compatibility."""
+        if len(self.Shape) != 2 or len(other.Shape) != 2:
+            raise ArgumentException("Matrix multiplication is only supported for 2D tensors.")
+        return self.BatchMatrixMultiply(other, alpha)
+
+    def BatchMatrixMultiply(self, other, alpha=1.0):
+        """alpha * this . other on the last two dimensions of tensors of two or more dimensions: one product per
+        leading index ([..., m, k] . [..., k, n]), or a shared two-dimensional right operand ([..., m, k] . [k, n]).
+        The reference has no such method (its MatrixMultiply rejects these shapes); it is what its windowed-attention
+        example needs (examples/swin/SwinExample/SwinTransformerTools.cs:348-389)."""
         kind = _product_kind(self.Shape, other.Shape, "Matrix multiplication is only supported for 2D tensors.")
         if self.dtype != other.dtype:
             raise ArgumentException("buffers of different element types in one call")
@@ -148,9 +158,18 @@ class TensorReverse:
         self.InitialTensors = list(tensors)
 
     def MatrixMultiplyReverse(self, upstreamGradient):
-        """[dA, dB] for C = A . B: dA = dC . B^T and dB = A^T . dC on the last two dimensions (per slice for a
-        batched product; for a shared right operand dB adds up over all leading indices, which is the single
-        product of the flattened operands)."""
+        """[dA, dB] for C = A . B of two-dimensional tensors: dA = dC . B^T and dB = A^T . dC
+        (src/PRAD/TensorReverse.cs:94-157, which rejects other shapes)."""
+        if len(self.InitialTensors) != 2:
+            raise InvalidOperationException("MatrixMultiplyReverse expects exactly two initial tensors.")
+        if any(len(t.Shape) != 2 for t in self.InitialTensors) or len(upstreamGradient.Shape) != 2:
+            raise ArgumentException("Matrix multiplication gradients are only supported for 2D tensors.")
+        return self.BatchMatrixMultiplyReverse(upstreamGradient)
+
+    def BatchMatrixMultiplyReverse(self, upstreamGradient):
+        """The gradients of BatchMatrixMultiply on the last two dimensions (per slice for a batched product; for a
+        shared right operand dB adds up over all leading indices, which is the single product of the flattened
+        operands)."""
         if len(self.InitialTensors) != 2:
             raise InvalidOperationException("MatrixMultiplyReverse expects exactly two initial tensors.")
         a, b = self.InitialTensors

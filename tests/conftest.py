@@ -78,8 +78,10 @@ def assert_long_sum_parity(dev, ref, lhs, rhs, dtype, what=""):
     (the reference's own k-ascending float loop is 3e-5 from the exact product at K = 50 000), so where the direct
     comparison exceeds the bar the result is held to what reordering can change and no more: every entry within the
     order-independent rounding bound 8 sqrt(K) eps (|lhs|^T.|rhs|)_ij of the product evaluated in double from the
-    same operands, and no further from that double value (in the relative measure of the other checks) than the
-    bar or twice the distance of the reference's own arithmetic, whichever is larger.  Returns the three errors
+    same operands, no further from that double value (in the relative measure of the other checks) than the bar or
+    the distance of the reference's own arithmetic, whichever is larger, and within four times the bar of the
+    reference (measured at K = 50 176: device 2e-6 and reference 2.9e-5 from the double product, 3.0e-5 apart).
+    Returns the three errors
     (device vs reference, device vs double, reference vs double)."""
     tol = TOL[np.dtype(dtype)]
     direct = rel_err(dev, ref)
@@ -90,8 +92,8 @@ def assert_long_sum_parity(dev, ref, lhs, rhs, dtype, what=""):
         bound = 8.0 * np.sqrt(lhs64.shape[0]) * float(np.finfo(dtype).eps) * (np.abs(lhs64).T @ np.abs(rhs64))
         worst = float(np.max(np.abs(np.asarray(dev, np.float64) - exact) / bound))
         assert worst <= 1.0, "%s: an entry is off by %.2f x its rounding bound" % (what, worst)
-        assert e_dev <= max(tol, 2.0 * e_ref), "%s: %.3e from the double product, the reference's arithmetic %.3e" % (what, e_dev, e_ref)
-        assert direct <= 10.0 * tol, "%s: relative error %.3e against the reference" % (what, direct)
+        assert e_dev <= max(tol, e_ref), "%s: %.3e from the double product, the reference's arithmetic %.3e" % (what, e_dev, e_ref)
+        assert direct <= 4.0 * tol, "%s: relative error %.3e against the reference" % (what, direct)
     return direct, e_dev, e_ref
 
 

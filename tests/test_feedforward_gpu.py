@@ -326,3 +326,21 @@ def test_operation_walk_steady_state_allocates_nothing(gpu):
     assert after["mallocs"] == before["mallocs"] and after["frees"] == before["frees"] and after["syncs"] == before["syncs"], (before, after)
     assert after["pool_hits"] - before["pool_hits"] >= 5 * 20
     assert np.isfinite(net.loss.to_numpy()[0, 0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_compiled_operation_walk_equals_the_python_walk(gpu, dtype):
+    """The step walked by compiled code through the C ABI (one call per operation) gives the bits of the Python walk
+    through the operation classes: same entry points in the same order."""
+    from parallelreverseautodiff_amd.feedforward import OperationWalkNetwork, compiled_operation_walk
+    X = seeded.uniform(seeded.DEFAULT_SEED, 1, (64, 784), 0.0, 1.0, dtype)
+    T = seeded.one_hot_labels(seeded.DEFAULT_SEED, 2, 64, 10, dtype)
+    walk = OperationWalkNetwork(dtype=dtype)
+    walk.set_batch(X, T)
+    for _ in range(4):
+        walk.step()
+    ms, loss, weights = compiled_operation_walk(dtype=dtype, steps=3, warmup=1)
+    assert ms > 0
+    assert loss == float(walk.loss.to_numpy()[0, 0])
+    for got, ref in zip(weights, walk.W):
+        assert np.array_equal(got, ref.to_numpy())

@@ -46,10 +46,15 @@ def test_tensor_errors(gpu):
         a.MatrixMultiply(b)
     with pytest.raises(ArgumentException, match="only supported for 2D"):
         Tensor([4]).MatrixMultiply(b)
+    # the reference's own methods take two-dimensional tensors only (src/PRAD/Tensor.cs:574-577, TensorReverse.cs:96-110)
+    with pytest.raises(ArgumentException, match="only supported for 2D"):
+        Tensor([2, 3, 4]).MatrixMultiply(Tensor([2, 4, 2]))
+    with pytest.raises(ArgumentException, match="only supported for 2D"):
+        TensorReverse([Tensor([2, 3, 4]), Tensor([2, 4, 2])]).MatrixMultiplyReverse(Tensor([2, 3, 2]))
     with pytest.raises(ArgumentException, match="Incompatible shapes"):
-        Tensor([2, 3, 4]).MatrixMultiply(Tensor([3, 4, 2]))      # leading dimensions differ
+        Tensor([2, 3, 4]).BatchMatrixMultiply(Tensor([3, 4, 2]))      # leading dimensions differ
     with pytest.raises(ArgumentException, match="Incompatible shapes"):
-        Tensor([2, 3, 4]).MatrixMultiply(Tensor([2, 5, 2]))      # inner dimensions differ
+        Tensor([2, 3, 4]).BatchMatrixMultiply(Tensor([2, 5, 2]))      # inner dimensions differ
     with pytest.raises(InvalidOperationException):
         TensorReverse([a]).MatrixMultiplyReverse(a)
     with pytest.raises(ArgumentException):
@@ -61,7 +66,7 @@ def test_tensor_errors(gpu):
 def test_batched_tensor_product_and_reverse(gpu, oracle, dtype, case):
     """Products of tensors of more than two dimensions, which the windowed-attention example of the reference needs
     (examples/swin/SwinExample/SwinTransformerTools.cs:372-389) and its Tensor.MatrixMultiply rejects
-    (src/PRAD/Tensor.cs:574-577): one product per leading index, checked slice by slice against the oracle's
+    (src/PRAD/Tensor.cs:574-577), under names of their own: one product per leading index, checked slice by slice against the oracle's
     MatrixMultiplyOperation.  "scores" and "context" are the shapes of that example at 1024 windows x 3 heads:
     [1024, 3, 49, 32] . [1024, 3, 32, 49] and [1024, 3, 49, 49] . [1024, 3, 49, 32]."""
     lead, m, k, n = {"scores": ([1024, 3], 49, 32, 49), "context": ([1024, 3], 49, 49, 32), "small": ([2, 1, 3], 5, 7, 4)}[case]
@@ -70,9 +75,9 @@ def test_batched_tensor_product_and_reverse(gpu, oracle, dtype, case):
     B = seeded.uniform(113, 2, (L, k, n), -1.0, 1.0, dtype)
     dC = seeded.normal(113, 3, (L, m, n), 1.0, dtype)
     ta, tb, tg = Tensor(lead + [m, k], A.reshape(-1)), Tensor(lead + [k, n], B.reshape(-1)), Tensor(lead + [m, n], dC.reshape(-1))
-    tc = ta.MatrixMultiply(tb)
+    tc = ta.BatchMatrixMultiply(tb)
     assert tc.Shape == lead + [m, n]
-    gA, gB = TensorReverse([ta, tb]).MatrixMultiplyReverse(tg)
+    gA, gB = TensorReverse([ta, tb]).BatchMatrixMultiplyReverse(tg)
     assert gA.Shape == lead + [m, k] and gB.Shape == lead + [k, n]
     C, dA, dB = tc.to_numpy().reshape(L, m, n), gA.to_numpy().reshape(L, m, k), gB.to_numpy().reshape(L, k, n)
     for s in range(L):
@@ -80,7 +85,7 @@ def test_batched_tensor_product_and_reverse(gpu, oracle, dtype, case):
         rA, rB = oracle.matmul_bwd(dC[s], A[s], B[s])
         assert_parity(dA[s], rA, dtype, "dA of slice %d" % s, bound=dot_bound(dC[s], B[s].T, dtype))
         assert_parity(dB[s], rB, dtype, "dB of slice %d" % s, bound=dot_bound(A[s].T, dC[s], dtype))
-    half = ta.MatrixMultiply(tb, alpha=0.5)
+    half = ta.BatchMatrixMultiply(tb, alpha=0.5)
     assert np.array_equal(half.to_numpy(), tc.to_numpy() * dtype(0.5))
 
 
@@ -95,18 +100,18 @@ def test_tensor_product_with_a_shared_right_operand(gpu, oracle, dtype):
     B = seeded.uniform(114, 2, (k, n), -1.0, 1.0, dtype)
     dC = seeded.normal(114, 3, (L * m, n), 1.0, dtype)
     ta, tb, tg = Tensor(lead + [m, k], A.reshape(-1)), Tensor([k, n], B.reshape(-1)), Tensor(lead + [m, n], dC.reshape(-1))
-    tc = ta.MatrixMultiply(tb)
+    tc = ta.BatchMatrixMultiply(tb)
     assert tc.Shape == lead + [m, n]
     assert_parity(tc.to_numpy().reshape(L * m, n), oracle.matmul_fwd(A, B), dtype, "shared product", bound=dot_bound(A, B, dtype))
-    gA, gB = TensorReverse([ta, tb]).MatrixMultiplyReverse(tg)
+    gA, gB = TensorReverse([ta, tb]).BatchMatrixMultiplyReverse(tg)
     assert gA.Shape == lead + [m, k] and gB.Shape == [k, n]
     rA, rB = oracle.matmul_bwd(dC, A, B)
     assert_parity(gA.to_numpy().reshape(L * m, k), rA, dtype, "dA", bound=dot_bound(dC, B.T, dtype))
     assert_parity(gB.to_numpy(), rB, dtype, "dB summed over the windows", bound=dot_bound(A.T, dC, dtype))
     # a right operand with leading dimensions of one is the same product; results feed the next product from the device
     tb1 = Tensor([1, 1, k, n], B.reshape(-1))
-    assert np.array_equal(ta.MatrixMultiply(tb1).to_numpy(), tc.to_numpy())
-    chained = tc.MatrixMultiply(Tensor([n, 8], np.ones(n * 8, dtype)))
+    assert np.array_equal(ta.BatchMatrixMultiply(tb1).to_numpy(), tc.to_numpy())
+    chained = tc.BatchMatrixMultiply(Tensor([n, 8], np.ones(n * 8, dtype)))
     assert chained.Shape == lead + [m, 8]
     assert_parity(chained.to_numpy().reshape(L * m, 8), oracle.matmul_fwd(tc.to_numpy().reshape(L * m, n), np.ones((n, 8), dtype)), dtype)
 
