@@ -44,7 +44,7 @@ constexpr uint32_t BUF_MAGIC = 0x50524144u;  // "PRAD"
 constexpr size_t STAGING_CHUNK = (size_t)256 << 20;
 
 constexpr size_t COUNTER_BYTES = 4096;  // arrival counters: one per tile of a split or paired product, and a few
-constexpr size_t SEQ_FLAG_BYTES = 4096;  // one progress word per workgroup of an LSTM sequence kernel
+constexpr size_t SEQ_FLAG_BYTES = 8192;  // two words per workgroup of an LSTM sequence kernel: progress, and where it runs
 static_assert(COUNTER_BYTES >= GEMM_SPLIT_MAX_TILES * sizeof(unsigned), "a split product needs a counter per tile");
 
 // One stream, one kernel workspace (partial results of split products, clip moments, loss partial sums, tall
@@ -555,7 +555,7 @@ int32_t prad_init(int32_t device_id) {
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.seq_flags), SEQ_FLAG_BYTES), PRAD_ERR_ALLOC);
     HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&g_ctx.seq_abort), 64, hipHostMallocDefault), PRAD_ERR_ALLOC);
     *g_ctx.seq_abort = 0u;
-    g_ctx.compute_units = std::min<int>(prop.multiProcessorCount, (int)(SEQ_FLAG_BYTES / sizeof(unsigned)));
+    g_ctx.compute_units = std::min<int>(prop.multiProcessorCount, (int)(SEQ_FLAG_BYTES / (2 * sizeof(unsigned))));
     {
         const char* e = getenv("PRAD_LSTM_SEQUENCE");
         g_ctx.seq_enabled = !(e && e[0] == '0');
@@ -578,6 +578,7 @@ int32_t prad_shutdown(void) {
     (void)sync_all();
     if (g_ctx.seq_step_scratch) (void)pool_give(g_ctx.seq_step_scratch, g_ctx.seq_step_scratch_class);
     g_ctx.seq_step_scratch = nullptr; g_ctx.seq_step_scratch_bytes = 0;
+
     (void)pool_release_all();
     if (g_ctx.pinned) (void)hipHostFree(g_ctx.pinned);
     if (g_ctx.workspace) (void)hipFree(g_ctx.workspace);
@@ -1692,9 +1693,9 @@ int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, pr
     if (!usable)
         return gates->dtype == PRAD_F64 ? lstm_sequence_bwd_steps<double>(Wh, gates, C, tanh_c, dh_loss, dG, steps, batch, hidden)
                                         : lstm_sequence_bwd_steps<float>(Wh, gates, C, tanh_c, dh_loss, dG, steps, batch, hidden);
-    if (int32_t st = ensure_workspace(lstm_seq_partial_bytes(batch, hidden))) return st;
     LstmSeqArgs a{};
     a.Wh = F(Wh); a.G = F(gates); a.C = F(C); a.TC = F(tanh_c); a.dHl = F(dh_loss); a.dG = F(dG);
+    if (int32_t st = ensure_workspace(lstm_seq_partial_bytes(batch, hidden))) return st;
     a.partial = static_cast<float*>(CUR_WORKSPACE);
     a.flags = g_ctx.seq_flags; a.abort_word = g_ctx.seq_abort;
     a.batch = (int)batch; a.hidden = (int)hidden; a.steps = (int)steps; a.spin_limit = lstm_spin_limit();
