@@ -335,10 +335,12 @@ struct LstmSeqArgs {
     unsigned* abort_word;  // host-visible; a workgroup that gives up waiting writes 1
     int batch, hidden, steps;
     int spin_limit;
+    int local;             // the probe found every row group on one XCD: the kernels may exchange through that XCD's L2
 };
 bool lstm_seq_eligible(int64_t batch, int64_t hidden, int64_t steps, int compute_units);
 size_t lstm_seq_partial_bytes(int64_t batch, int64_t hidden);
 hipError_t launch_lstm_seq(const LstmSeqArgs& a, bool backward, hipStream_t s);
+bool lstm_seq_local(int64_t batch);
 hipError_t launch_lstm_seq_probe(int64_t batch, int64_t hidden, unsigned* flags, unsigned* abort_word, int spin_limit, hipStream_t s);
 
 // Windowed self-attention, forward, one launch (csrc/attention.hip; float, head dimension 32, <= 64 tokens per window)

@@ -412,8 +412,16 @@ __global__ void __launch_bounds__(SEQ_THREADS, 1) lstm_seq_probe_kernel(unsigned
         if (threadIdx.x == 0) __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         return;
     }
-    if (threadIdx.x == 0) __hip_atomic_store(flags + r * blocks + c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    (void)wait_for_group(flags + r * blocks, blocks, 1u, abort_word, spin_limit, &all_arrived);
+    // the flag value says where the workgroup runs (XCD + 1): the roll call also tells whether each row group sits on
+    // one XCD, which decides how the sequence kernels exchange (abort_word[1] is raised if one does not)
+    const unsigned mine = xcd_of_this_wave() + 1u;
+    if (threadIdx.x == 0) __hip_atomic_store(flags + r * blocks + c, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!wait_for_group(flags + r * blocks, blocks, 1u, abort_word, spin_limit, &all_arrived)) return;
+    if (threadIdx.x < 64) {
+        const bool same = (int)threadIdx.x >= blocks ||
+                          __hip_atomic_load(flags + r * blocks + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == mine;
+        if (!__all(same) && threadIdx.x == 0) __hip_atomic_store(abort_word + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
 hipError_t launch_lstm_seq_probe(int64_t batch, int64_t hidden, unsigned* flags, unsigned* abort_word, int spin_limit, hipStream_t s) {
@@ -460,7 +468,7 @@ bool lstm_seq_local(int64_t batch) {
 
 hipError_t launch_lstm_seq(const LstmSeqArgs& a, bool backward, hipStream_t s) {
     const unsigned grid = (unsigned)((a.batch / 16) * (a.hidden / 16));
-    const bool local = lstm_seq_local(a.batch);
+    const bool local = a.local != 0 && lstm_seq_local(a.batch);
     if (!backward && local) {
         // every h_t block that the launch will write starts as "not written yet"
         hipError_t e = fill_sentinel(a.Hs + (int64_t)a.batch * a.hidden, (int64_t)a.steps * a.batch * a.hidden, a.flags, (int)grid, s);

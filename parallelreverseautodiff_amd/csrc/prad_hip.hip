@@ -75,6 +75,7 @@ struct Context {
     // (workgroups) that a probe has shown the device to hold at once.
     bool seq_enabled = true;
     int seq_proven_grid = 0;
+    bool seq_groups_local = false;          // the last probe found every row group on one XCD
     void* seq_step_scratch = nullptr;       // dh and dc ping-pong blocks of the per-time-step backward (kept: recordings address it)
     size_t seq_step_scratch_bytes = 0, seq_step_scratch_class = 0;
     // Device blocks that prad_buf_free handed back, by size class.  Everything the library enqueues runs on the one
@@ -554,7 +555,7 @@ int32_t prad_init(int32_t device_id) {
     if (int32_t st = init_static_scratch(device_id)) return st;
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&g_ctx.seq_flags), SEQ_FLAG_BYTES), PRAD_ERR_ALLOC);
     HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&g_ctx.seq_abort), 64, hipHostMallocDefault), PRAD_ERR_ALLOC);
-    *g_ctx.seq_abort = 0u;
+    g_ctx.seq_abort[0] = 0u; g_ctx.seq_abort[1] = 0u;
     g_ctx.compute_units = std::min<int>(prop.multiProcessorCount, (int)(SEQ_FLAG_BYTES / (2 * sizeof(unsigned))));
     {
         const char* e = getenv("PRAD_LSTM_SEQUENCE");
@@ -1599,6 +1600,8 @@ static int32_t sequence_kernels_usable(int32_t dtype, int64_t batch, int64_t hid
         return PRAD_OK;
     }
     g_ctx.seq_proven_grid = grid;
+    g_ctx.seq_groups_local = static_cast<volatile unsigned*>(g_ctx.seq_abort)[1] == 0u;
+    static_cast<volatile unsigned*>(g_ctx.seq_abort)[1] = 0u;
     *usable = true;
     return PRAD_OK;
 }
@@ -1671,7 +1674,7 @@ int32_t prad_lstm_sequence_fwd(prad_buf_t Wh, prad_buf_t G, prad_buf_t C, prad_b
     LstmSeqArgs a{};
     a.Wh = F(Wh); a.G = F(G); a.C = F(C); a.Hs = F(Hs); a.TC = F(tanh_c);
     a.flags = g_ctx.seq_flags; a.abort_word = g_ctx.seq_abort;
-    a.batch = (int)batch; a.hidden = (int)hidden; a.steps = (int)steps; a.spin_limit = lstm_spin_limit();
+    a.batch = (int)batch; a.hidden = (int)hidden; a.steps = (int)steps; a.spin_limit = lstm_spin_limit(); a.local = g_ctx.seq_groups_local ? 1 : 0;
     HIP_TRY(launch_lstm_seq(a, false, CUR_STREAM), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }
@@ -1698,7 +1701,7 @@ int32_t prad_lstm_sequence_bwd(prad_buf_t Wh, prad_buf_t gates, prad_buf_t C, pr
     if (int32_t st = ensure_workspace(lstm_seq_partial_bytes(batch, hidden))) return st;
     a.partial = static_cast<float*>(CUR_WORKSPACE);
     a.flags = g_ctx.seq_flags; a.abort_word = g_ctx.seq_abort;
-    a.batch = (int)batch; a.hidden = (int)hidden; a.steps = (int)steps; a.spin_limit = lstm_spin_limit();
+    a.batch = (int)batch; a.hidden = (int)hidden; a.steps = (int)steps; a.spin_limit = lstm_spin_limit(); a.local = g_ctx.seq_groups_local ? 1 : 0;
     HIP_TRY(launch_lstm_seq(a, true, CUR_STREAM), PRAD_ERR_LAUNCH);
     return PRAD_OK;
 }

@@ -12,7 +12,7 @@ import threading
 import numpy as np
 import pytest
 
-from conftest import assert_parity, dot_bound
+from conftest import assert_parity, dot_bound, rel_err
 from parallelreverseautodiff_amd import _lib, seeded
 from parallelreverseautodiff_amd.exceptions import ArgumentException, InvalidOperationException
 from parallelreverseautodiff_amd.matrix import DeepMatrix, DeviceBuffer, Matrix
@@ -625,16 +625,23 @@ def test_tall_products_of_few_slabs(gpu, oracle, dtype, shape):
 
 @pytest.mark.parametrize("shape", [(16384, 96, 288), (9000, 96, 96), (8200, 384, 96), (12001, 288, 96), (8192, 64, 384), (10000, 20, 48)])
 def test_rows_of_a_tall_product_do_not_depend_on_how_many_rows_there_are(gpu, oracle, shape):
-    """Row i of a product depends on row i of A only, and every kernel adds along K in the same order, whatever tile
-    the sizes select (a tall product runs on 128 x 128 tiles or the half-depth kernel, its first 4096 rows alone on
-    smaller ones): the first 4096 rows of the tall product equal the product of the first 4096 rows bit for bit - for
-    every epilogue (bias, pre-activation copy, activation, the upstream activation's derivative, accumulation), both
-    layouts of B, and a ragged last tile."""
+    """Row i of a product depends on row i of A only, and the tiled kernels all add along K in the same order, whatever
+    tile the sizes select (a tall product runs on 128 x 128 tiles, its first 4096 rows alone on smaller ones): the first
+    4096 rows of the tall product equal the product of the first 4096 rows bit for bit - for every epilogue (bias,
+    pre-activation copy, activation, the upstream activation's derivative, accumulation), both layouts of B, and a
+    ragged last tile.  From 8192 rows on, products with K a multiple of 96 run on the streaming kernel, whose MFMA steps
+    group K differently (k = 16 j + 4 g + i instead of 4 s + g): there the two agree to rounding, not to the bit."""
     lib = _lib.load()
     from parallelreverseautodiff_amd.exceptions import check
     dtype = np.float32
     M, K, N = shape
     head = 4096
+    streaming = M >= 8192 and K % 96 == 0          # the full product runs on the streaming kernel, the head on tiles
+
+    def same(x, y):
+        if not streaming:
+            return np.array_equal(x, y)
+        return rel_err(x, y) <= 1e-5
     A = seeded.uniform(43, 1, (M, K), -1, 1, dtype)
     B = seeded.uniform(43, 2, (K, N), -1, 1, dtype)
     Bt = np.ascontiguousarray(B.T)                                  # N x K: the operand of dC . W^T
@@ -657,20 +664,20 @@ def test_rows_of_a_tall_product_do_not_depend_on_how_many_rows_there_are(gpu, or
     # plain store, and accumulation into C
     f, q = both(lambda a, s, c0, c1: (check(lib.prad_gemm(0, 0, a.handle, bB.handle, c0.handle, 0)),
                                       check(lib.prad_gemm(0, 0, a.handle, bB.handle, c1.handle, 1))))
-    assert np.array_equal(f[0][:head], q[0]) and np.array_equal(f[1][:head], q[1])
+    assert same(f[0][:head], q[0]) and same(f[1][:head], q[1])
     assert_parity(f[0], A.astype(np.float64) @ B.astype(np.float64), dtype, "A.B", bound=dot_bound(A, B, dtype))
     assert_parity(f[1], old + A.astype(np.float64) @ B.astype(np.float64), dtype, "C += A.B")
     # B stored N x K (the layout of dA = dC . W^T)
     f, q = both(lambda a, s, c0, c1: check(lib.prad_gemm(0, 1, a.handle, bBt.handle, c0.handle, 0)))
-    assert np.array_equal(f[0][:head], q[0])
+    assert same(f[0][:head], q[0])
     assert_parity(f[0], A.astype(np.float64) @ B.astype(np.float64), dtype, "A.(B^T)^T", bound=dot_bound(A, B, dtype))
     # bias, pre-activation copy, activation
     f, q = both(lambda a, s, c0, c1: check(lib.prad_matmul_fwd_fused(a.handle, bB.handle, bbias.handle, c1.handle, c0.handle, _lib.ACT_TANH, 0.0)))
-    assert np.array_equal(f[0][:head], q[0]) and np.array_equal(f[1][:head], q[1])
+    assert same(f[0][:head], q[0]) and same(f[1][:head], q[1])
     assert_parity(f[0][-200:], oracle.tanh_fwd(np.ascontiguousarray(f[1][-200:])), dtype, "tanh(Z), last rows")
     # the upstream activation's derivative on the way out (dA = (dC . W^T) (.) act'(src)): here "dC" = A, "W" = B^T
     f, q = both(lambda a, s, c0, c1: check(lib.prad_matmul_bwd_fused(a.handle, s.handle, bBt.handle, c0.handle, None, 0, _lib.ACT_SIGMOID, s.handle, 0.0)))
-    assert np.array_equal(f[0][:head], q[0])
+    assert same(f[0][:head], q[0])
 
 
 def test_workgroup_pairs_when_switched_on(gpu):
