@@ -890,7 +890,7 @@ def also_legs(args, table):
             ("swin_block_train_steps_per_s_f32", swin_leg, "configs[4] windowed attention block 16x56x56 embed 96 step",
              "whole step: 12 dense products, 6 batched window products, softmax, column sums")):
         try:
-            r = fn("f32", 10, 2, with_cpu)
+            r = fn("f32", 50, 10, with_cpu)
             leg = {"value": 1e3 / r["recorded_ms_per_step"], "unit": "steps/s", "ms_per_step": r["recorded_ms_per_step"],
                    "errors": r.get("errors"), "roofline": mfma_roofline(r["flop_per_step"], r["recorded_ms_per_step"], "f32", kernel)}
             if "cpu" in r:
