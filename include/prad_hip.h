@@ -361,6 +361,18 @@ int32_t prad_graph_destroy(void* graph);
  * src/RMAD/Loss/CategoricalCrossEntropyLossOperation.cs:37-86), in one launch. */
 int32_t prad_softmax_cce(prad_buf_t x, prad_buf_t target, prad_buf_t p, prad_buf_t loss, prad_buf_t dp, prad_buf_t dx);
 
+/* The output layer of a classifier with its loss, forward and backward: MatrixMultiplyOperation.Forward
+ * (src/RMAD/MatrixMultiplyOperation.cs:50-80) and MatrixAddBroadcastingOperation.Forward into z, then everything
+ * prad_softmax_cce does (p, loss, dp, dz), then the layer's Backward as prad_matmul_bias_bwd does it
+ * (src/RMAD/MatrixMultiplyOperation.cs:94-126): dbias, dW (+)= A^T . dz, dA = dz . W^T times the derivative of the
+ * activation below (act, act_src: what that activation cached, alpha) - the values of prad_matmul_fwd_fused +
+ * prad_softmax_cce + prad_matmul_bias_bwd.  One launch of one workgroup when there are at most 64 classes, fewer than
+ * 2048 rows and A, W and the class rows fit the compute unit's LDS (144 KB); the three launches otherwise.  bias, loss,
+ * dbias and act_src (with act = PRAD_ACT_NONE) may be NULL. */
+int32_t prad_dense_softmax_cce(prad_buf_t A, prad_buf_t W, prad_buf_t bias, prad_buf_t target, prad_buf_t z, prad_buf_t p,
+                               prad_buf_t loss, prad_buf_t dp, prad_buf_t dz, prad_buf_t dA, prad_buf_t dW, prad_buf_t dbias,
+                               int32_t accumulate_dW, int32_t act, prad_buf_t act_src, double alpha);
+
 /* ---- GradientClipper.ClipGradients, src/RMAD/GradientClipper.cs:118-157 and :212-253 (in place) */
 int32_t prad_clip(prad_buf_t g, double clip_value, double min_value);
 /* ---- AdamOptimizer.UpdateWeightWithAdam, src/RMAD/AdamOptimizer.cs:195-239 (in place on w, m, v) */

@@ -114,6 +114,7 @@ SIGNATURES = {
     "prad_lstm_sequence_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64]),
     "prad_buf_view_rows": (_i32, [_vp, _i64, _i64, _vpp]),
     "prad_softmax_cce": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp]),
+    "prad_dense_softmax_cce": (_i32, [_vp] * 12 + [_i32, _i32, _vp, _f64]),
     "prad_graph_begin": (_i32, []),
     "prad_graph_end": (_i32, [_vpp]),
     "prad_graph_launch": (_i32, [_vp]),

@@ -12,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libprad_hip.so")
-SOURCES = ["gemm.hip", "gemm_skinny.hip", "gemm_tall.hip", "elementwise.hip", "optim.hip", "matmul_sum.hip", "loss.hip", "lstm.hip", "lstm_seq.hip", "attention.hip", "norm.hip", "prad_hip.hip"]
+SOURCES = ["gemm.hip", "gemm_skinny.hip", "gemm_tall.hip", "elementwise.hip", "optim.hip", "matmul_sum.hip", "loss.hip", "head.hip", "lstm.hip", "lstm_seq.hip", "attention.hip", "norm.hip", "prad_hip.hip"]
 
 # -packed-fp32-ops is switched off: the compiler must not form packed FP32 instructions.
 HIPCC_FLAGS = [

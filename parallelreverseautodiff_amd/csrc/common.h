@@ -187,7 +187,8 @@ struct GemmArgs {
 // wavefronts take every fourth row, four accumulators each); part is 4 x 64 doubles of LDS.
 template <typename T, typename OUT>
 __device__ __forceinline__ void colsum_block(const T* __restrict__ dy, OUT* __restrict__ out, int64_t cols, int64_t r0, int64_t r1,
-                                             int64_t bx, double* part) {
+                                             int64_t bx, double* part, int64_t pitch = 0) {
+    if (pitch == 0) pitch = cols;  // (rows of dy are `pitch` elements apart)
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int64_t j = bx * 64 + lane;
     double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
@@ -197,16 +198,16 @@ __device__ __forceinline__ void colsum_block(const T* __restrict__ dy, OUT* __re
         for (; i + 60 < r1; i += 64) {
             double v[16];
 #pragma unroll
-            for (int u = 0; u < 16; ++u) v[u] = (double)dy[(i + 4 * u) * cols + j];
+            for (int u = 0; u < 16; ++u) v[u] = (double)dy[(i + 4 * u) * pitch + j];
 #pragma unroll
             for (int u = 0; u < 16; u += 4) { acc0 += v[u]; acc1 += v[u + 1]; acc2 += v[u + 2]; acc3 += v[u + 3]; }
         }
         for (; i + 12 < r1; i += 16) {
-            const double a = (double)dy[i * cols + j], b = (double)dy[(i + 4) * cols + j];
-            const double c = (double)dy[(i + 8) * cols + j], d = (double)dy[(i + 12) * cols + j];
+            const double a = (double)dy[i * pitch + j], b = (double)dy[(i + 4) * pitch + j];
+            const double c = (double)dy[(i + 8) * pitch + j], d = (double)dy[(i + 12) * pitch + j];
             acc0 += a; acc1 += b; acc2 += c; acc3 += d;
         }
-        for (; i < r1; i += 4) acc0 += (double)dy[i * cols + j];
+        for (; i < r1; i += 4) acc0 += (double)dy[i * pitch + j];
     }
     part[w * 64 + lane] = (acc0 + acc1) + (acc2 + acc3);
     __syncthreads();
@@ -302,12 +303,60 @@ template <typename T> hipError_t launch_clip_adam(const TensorDesc<T>* host_desc
 // Replaces c1 and c2 in the launch arguments of a recorded Adam kernel node of an instantiated graph.
 template <typename T> hipError_t adam_node_set_bias_correction(hipGraphExec_t exec, hipGraphNode_t node, T c1, T c2);
 
+// Reductions across a wavefront (a butterfly over lane distances 32, 16, ... 1) and the exponential of the short-row
+// softmax kernels, shared by csrc/loss.hip and csrc/head.hip so that both give the same bits.
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_max(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmax(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Reductions and exponentials in the element type for the short-row kernels: in float they move one register per
+// shuffle step instead of two and use the hardware exponential (within 2e-7 of the double evaluation rounded to
+// float, far inside the 1e-5 parity bar), which is what those kernels' time goes into.
+__device__ __forceinline__ float wave_sum_t(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_sum_t(double v) { return wave_sum(v); }
+__device__ __forceinline__ float wave_max_t(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ double wave_max_t(double v) { return wave_max(v); }
+__device__ __forceinline__ float short_exp(float x) { return __expf(x); }
+__device__ __forceinline__ double short_exp(double x) { return exp(x); }
+
 // softmax / categorical cross-entropy (csrc/loss.hip)
 template <typename T> hipError_t launch_softmax_fwd(const T* x, T* y, int64_t rows, int64_t cols, T alpha, hipStream_t s);
 template <typename T> hipError_t launch_softmax_bwd(const T* y, const T* dy, T* dx, int64_t rows, int64_t cols, T alpha, hipStream_t s);
 template <typename T> hipError_t launch_softmax_cce(const T* x, const T* t, T* y, T* dy, T* dx, T* loss, unsigned* counter, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_cce_fwd(const T* p, const T* t, T* loss, int64_t rows, int64_t cols, hipStream_t s);
 template <typename T> hipError_t launch_cce_bwd(const T* p, const T* t, T* dp, int64_t rows, int64_t cols, hipStream_t s);
+
+// The output layer of a classifier with softmax and categorical cross-entropy, forward and backward, in one launch of one
+// workgroup (csrc/head.hip): Z = A . W + bias, P = softmax(Z), loss, dP, dZ, then dbias, dW (+)= A^T . dZ and
+// dA = dZ . W^T (.) act'(act_src).  All matrices dense row-major; Z, loss, dbias, dW, dA may be nullptr.
+template <typename T>
+struct HeadArgs {
+    const T* A; const T* W; const T* bias; const T* target; const T* act_src;
+    T* Z; T* P; T* loss; T* dP; T* dZ; T* dA; T* dW; T* dbias;
+    int B, H, C;  // rows of the batch, inputs of the layer, classes
+    int act;      // activation of the layer below (its Backward multiplies dA), ACT_NONE: none
+    T alpha;
+    int accumulate_dW;
+};
+template <typename T> bool classifier_head_eligible(int64_t B, int64_t H, int64_t C);
+template <typename T> size_t classifier_head_lds_bytes(int64_t B, int64_t H, int64_t C);
+// hipErrorNotSupported for shapes the kernel does not take (the caller then uses the separate launches).
+template <typename T> hipError_t launch_classifier_head(const HeadArgs<T>& a, hipStream_t s);
 
 size_t mse_workspace_bytes();
 // dy != nullptr: the gradient is written in the same pass (the values of launch_mse_bwd).

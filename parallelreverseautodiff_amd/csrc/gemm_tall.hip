@@ -27,9 +27,6 @@
 
 #include <cstdlib>
 
-#ifdef PRAD_TALL_TRACE
-__device__ long long prad_tall_trace[256 * 16 * 4];  // (a tuning aid: per-wavefront clock readings)
-#endif
 
 namespace prad {
 
@@ -64,7 +61,10 @@ __device__ __forceinline__ f4t load16(const float* base, unsigned byte_offset) {
 // What follows a unit's multiplications.  TALL_STORE: store (or add into) C, with the bias if there is one: straight-line
 // code, a few instructions per 16 bytes.  TALL_GENERAL: everything (pre-activation copy, activation, upstream activation's
 // derivative) in a runtime loop, see `finish_general`.
-constexpr int TALL_STORE = 0, TALL_GENERAL = 1;
+// TALL_GELU_FWD / TALL_GELU_BWD: the general epilogue with the activation known at compile time (GELU forward with or
+// without the pre-activation copy; GELU's derivative of a cached operand): no dispatch per element, and the four elements
+// of a lane's vector are independent instruction chains that the compiler interleaves.
+constexpr int TALL_STORE = 0, TALL_GENERAL = 1, TALL_GELU_FWD = 2, TALL_GELU_BWD = 3;
 
 // NYW: 16-column tiles (accumulators per lane) of a unit.  ONE_CHUNK: K == 96, every pass of the main loop is a whole unit.
 template <int NYW, int EPI, bool ONE_CHUNK>
@@ -74,10 +74,6 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (said to be uniform: loop counts and load bases that depend on it stay scalar)
     const int li = lane & 15, g = lane >> 4;
     const int KJ = p.K / 16;
-#ifdef PRAD_TALL_TRACE
-    const long long t_begin = wall_clock64();
-    long long t_first = 0;
-#endif
 
     // ---- units: the workgroup owns [first, first + count); wavefront w starts with unit w and then takes the next unit
     // nobody has taken yet (a counter in LDS), so that all sixteen finish within a unit of each other ----
@@ -146,9 +142,6 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
     if (p.bias != nullptr)
         for (int n = tid; n < p.N; n += TALL_THREADS) bfrag[p.K * p.N + n] = p.bias[n];
     __syncthreads();
-#ifdef PRAD_TALL_TRACE
-    const long long t_fill = wall_clock64();
-#endif
 
     if (!working) return;
     f4t acc[NYW];
@@ -225,19 +218,27 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
                 src[k] = src[k + 1];
             }
             if (!live) continue;
-            if (p.bias != nullptr) {
+            if (EPI != TALL_GELU_BWD && p.bias != nullptr) {
                 const f4t bv = *reinterpret_cast<const f4t*>(bias_lds + col);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = v[e] + bv[e];
             }
-            if (p.Z != nullptr) *reinterpret_cast<f4t*>(p.Z + zrow + col) = v;
-            if (p.act_fwd != ACT_NONE) {
+            if (EPI != TALL_GELU_BWD && p.Z != nullptr) *reinterpret_cast<f4t*>(p.Z + zrow + col) = v;
+            if (EPI == TALL_GELU_FWD) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = act_forward<float>(p.act_fwd, v[e], p.alpha);
-            }
-            if (p.act_bwd != ACT_NONE) {
+                for (int e = 0; e < 4; ++e) v[e] = act_forward<float>(ACT_GELU, v[e], 0.f);
+            } else if (EPI == TALL_GELU_BWD) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = v[e] * act_derivative<float>(p.act_bwd, sv[e], p.alpha);
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * act_derivative<float>(ACT_GELU, sv[e], 0.f);
+            } else {
+                if (p.act_fwd != ACT_NONE) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = act_forward<float>(p.act_fwd, v[e], p.alpha);
+                }
+                if (p.act_bwd != ACT_NONE) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = v[e] * act_derivative<float>(p.act_bwd, sv[e], p.alpha);
+                }
             }
             f4t* out = reinterpret_cast<f4t*>(p.C + crow + col);
             if (p.accumulate) {
@@ -273,7 +274,7 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
         };
         zero();
         if (ONE_CHUNK) {
-            if (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE) fetch_src(unit);
+            if (EPI == TALL_GELU_BWD || (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE)) fetch_src(unit);
             multiply_half(unit, 0, 0);
             resolve();
             load_half(next_unit, 0, 0);
@@ -283,7 +284,7 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
 #pragma unroll 1
             for (int c = 0; c < nchunks; ++c) {
                 const bool last = c == nchunks - 1;
-                if (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE && last) fetch_src(unit);
+                if ((EPI == TALL_GELU_BWD || (EPI == TALL_GENERAL && p.act_bwd != ACT_NONE)) && last) fetch_src(unit);
                 multiply_half(unit, c, 0);
                 if (last) resolve();
                 const int nu = last ? next_unit : unit, nc = last ? 0 : c + 1;
@@ -293,18 +294,9 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
             }
         }
         finish(unit);
-#ifdef PRAD_TALL_TRACE
-        if (pass == 0) t_first = wall_clock64();
-#endif
         if (!has_next) break;
         unit = next_unit;
     }
-#ifdef PRAD_TALL_TRACE
-    if (lane == 0 && blockIdx.x < 256) {
-        long long* o = prad_tall_trace + (blockIdx.x * TALL_WAVES + wave) * 4;
-        o[0] = t_begin; o[1] = t_fill; o[2] = t_first; o[3] = wall_clock64();
-    }
-#endif
 }
 
 int tall_compute_units() {
@@ -328,6 +320,10 @@ template <int NYW>
 hipError_t launch_nyw(const TallArgs& k, unsigned grid, size_t lds, hipStream_t stream) {
     const bool general = k.Z != nullptr || k.act_fwd != ACT_NONE || k.act_bwd != ACT_NONE;
     const bool one = k.K == 16 * TALL_CH;
+    if (k.act_fwd == ACT_GELU && k.act_bwd == ACT_NONE)
+        return one ? launch_variant<NYW, TALL_GELU_FWD, true>(k, grid, lds, stream) : launch_variant<NYW, TALL_GELU_FWD, false>(k, grid, lds, stream);
+    if (k.act_bwd == ACT_GELU && k.act_fwd == ACT_NONE && k.Z == nullptr && k.bias == nullptr)
+        return one ? launch_variant<NYW, TALL_GELU_BWD, true>(k, grid, lds, stream) : launch_variant<NYW, TALL_GELU_BWD, false>(k, grid, lds, stream);
     if (general) return one ? launch_variant<NYW, TALL_GENERAL, true>(k, grid, lds, stream) : launch_variant<NYW, TALL_GENERAL, false>(k, grid, lds, stream);
     return one ? launch_variant<NYW, TALL_STORE, true>(k, grid, lds, stream) : launch_variant<NYW, TALL_STORE, false>(k, grid, lds, stream);
 }

@@ -7,35 +7,6 @@
 
 namespace prad {
 
-__device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-__device__ __forceinline__ double wave_max(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmax(v, __shfl_xor(v, off, 64));
-    return v;
-}
-
-// Reductions and exponentials in the element type for the short-row kernels: in float they move one register per
-// shuffle step instead of two and use the hardware exponential (within 2e-7 of the double evaluation rounded to
-// float, far inside the 1e-5 parity bar), which is what those kernels' time goes into.
-__device__ __forceinline__ float wave_sum_t(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-__device__ __forceinline__ double wave_sum_t(double v) { return wave_sum(v); }
-__device__ __forceinline__ float wave_max_t(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
-}
-__device__ __forceinline__ double wave_max_t(double v) { return wave_max(v); }
-__device__ __forceinline__ float short_exp(float x) { return __expf(x); }
-__device__ __forceinline__ double short_exp(double x) { return exp(x); }
-
 // y[i][j] = exp(x[i][j] - max_i) / sum_j exp(x[i][j] - max_i)
 template <typename T>
 __global__ void __launch_bounds__(64) softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t cols,

@@ -1879,6 +1879,61 @@ int32_t prad_softmax_cce(prad_buf_t x, prad_buf_t target, prad_buf_t p, prad_buf
     return PRAD_OK;
 }
 
+// The classifier's output layer with its loss in one launch where the shape allows, otherwise as the three launches it
+// stands for (prad_matmul_fwd_fused, prad_softmax_cce, prad_matmul_bias_bwd): same values either way.
+int32_t prad_dense_softmax_cce(prad_buf_t A, prad_buf_t W, prad_buf_t bias, prad_buf_t target, prad_buf_t z, prad_buf_t p,
+                               prad_buf_t loss, prad_buf_t dp, prad_buf_t dz, prad_buf_t dA, prad_buf_t dW, prad_buf_t dbias,
+                               int32_t accumulate_dW, int32_t act, prad_buf_t act_src, double alpha) {
+    REQUIRE_INIT();
+    REQUIRE_BUF(A); REQUIRE_BUF(W); REQUIRE_BUF(target); REQUIRE_BUF(z); REQUIRE_BUF(p); REQUIRE_BUF(dp); REQUIRE_BUF(dz);
+    REQUIRE_BUF(dA); REQUIRE_BUF(dW);
+    if (bias != nullptr) REQUIRE_BUF(bias);
+    if (loss != nullptr) REQUIRE_BUF(loss);
+    if (dbias != nullptr) REQUIRE_BUF(dbias);
+    if (act_src != nullptr) REQUIRE_BUF(act_src);
+    if (act < PRAD_ACT_NONE || act > PRAD_ACT_AMPLIFIED_SIGMOID) return fail(PRAD_ERR_ARG, "unknown activation %d", act);
+    if (act != PRAD_ACT_NONE && act_src == nullptr) return fail(PRAD_ERR_ARG, "an activation's Backward needs the operand it cached");
+    if (int32_t st = same_dtype({A, W, bias, target, z, p, loss, dp, dz, dA, dW, dbias, act_src})) return st;
+    const bool flat = A->depth == 1 && W->depth == 1 && target->depth == 1 && z->depth == 1 && p->depth == 1 && dp->depth == 1 &&
+                      dz->depth == 1 && dA->depth == 1 && dW->depth == 1 && (bias == nullptr || bias->depth == 1) &&
+                      (dbias == nullptr || dbias->depth == 1) && (act_src == nullptr || act_src->depth == 1);
+    const int64_t B = A->rows, H = A->cols, C = W->cols;
+    const bool shapes = flat && W->rows == H && target->rows == B && target->cols == C && z->rows == B && z->cols == C && p->rows == B &&
+                        p->cols == C && dp->rows == B && dp->cols == C && dz->rows == B && dz->cols == C && dA->rows == B &&
+                        dA->cols == H && dW->rows == H && dW->cols == C && (bias == nullptr || (bias->rows == 1 && bias->cols == C)) &&
+                        (dbias == nullptr || (dbias->rows == 1 && dbias->cols == C)) &&
+                        (act_src == nullptr || (act_src->rows == B && act_src->cols == H)) &&
+                        (loss == nullptr || (loss->rows == 1 && loss->cols == 1));
+    ENQUEUE_LOCK();
+    const bool one_launch = shapes && (A->dtype == PRAD_F64 ? prad::classifier_head_eligible<double>(B, H, C)
+                                                            : prad::classifier_head_eligible<float>(B, H, C));
+    if (!one_launch) {  // the separate launches, which also word the complaint about a shape that fits none of them
+        Epilogue fwd;
+        fwd.bias = bias; fwd.alpha = alpha;
+        if (int32_t st = enqueue_gemm(0, 0, A, W, z, 0, fwd, false)) return st;
+        if (z->rows != target->rows || z->cols != target->cols || target->depth != 1)
+            return fail(PRAD_ERR_ARG, "Output and target matrices must have the same dimensions.");
+        if (loss != nullptr && (loss->depth != 1 || loss->rows != 1 || loss->cols != 1)) return fail(PRAD_ERR_ARG, "loss must be 1 x 1");
+        for (prad_buf_t o : {p, dp, dz})
+            if (int32_t st = same_shape(z, o, "softmax + cross-entropy")) return st;
+        DISPATCH(z, launch_softmax_cce<double>(D(z), D(target), D(p), D(dp), D(dz), loss ? D(loss) : nullptr, g_ctx.counter, z->rows, z->cols, CUR_STREAM),
+                 launch_softmax_cce<float>(F(z), F(target), F(p), F(dp), F(dz), loss ? F(loss) : nullptr, g_ctx.counter, z->rows, z->cols, CUR_STREAM));
+        Epilogue bwd;
+        bwd.act_bwd = act; bwd.act_src = act_src; bwd.alpha = alpha;
+        return matmul_bwd_locked(dz, A, W, dA, dW, 0, accumulate_dW, bwd, dbias);
+    }
+#define HEAD_ARGS(T, PTR)                                                                                                   \
+    prad::HeadArgs<T> h{};                                                                                                  \
+    h.A = PTR(A); h.W = PTR(W); h.bias = bias ? PTR(bias) : nullptr; h.target = PTR(target);                               \
+    h.act_src = act_src ? PTR(act_src) : nullptr; h.Z = PTR(z); h.P = PTR(p); h.loss = loss ? PTR(loss) : nullptr;         \
+    h.dP = PTR(dp); h.dZ = PTR(dz); h.dA = PTR(dA); h.dW = PTR(dW); h.dbias = dbias ? PTR(dbias) : nullptr;                \
+    h.B = (int)B; h.H = (int)H; h.C = (int)C; h.act = act; h.alpha = (T)alpha; h.accumulate_dW = accumulate_dW ? 1 : 0;     \
+    HIP_TRY(prad::launch_classifier_head<T>(h, CUR_STREAM), PRAD_ERR_LAUNCH);
+    if (A->dtype == PRAD_F64) { HEAD_ARGS(double, D) } else { HEAD_ARGS(float, F) }
+#undef HEAD_ARGS
+    return PRAD_OK;
+}
+
 // ---------------------------------------------------------------------------------------------
 int32_t prad_clip_multi(const prad_buf_t* g, int32_t n, double clip_value, double min_value) {
     REQUIRE_INIT();

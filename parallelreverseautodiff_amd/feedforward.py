@@ -66,10 +66,10 @@ class FeedForwardNetwork:
         self.T.upload(T)
 
     # ---- one step, launch by launch ------------------------------------------------------------
-    def _enqueue_forward(self):
+    def _enqueue_forward(self, layers=None):
         lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
         a = self.X
-        for l in range(L):
+        for l in range(L if layers is None else layers):
             last = l == L - 1
             out = self.Z[l] if last else self.H[l]
             z = None if last else self.Z[l].handle
@@ -79,8 +79,14 @@ class FeedForwardNetwork:
 
     def _enqueue_forward_backward(self):
         lib, L, alpha = self.lib, len(self.W), float(self.params.LeakyReLUAlpha)
-        self._enqueue_forward()
-        if self.fused:
+        head = self.fused and L >= 2  # output layer, loss and the layer's backward in one call
+        self._enqueue_forward(L - 1 if head else None)
+        if head:
+            check(lib.prad_dense_softmax_cce(self.H[L - 2].handle, self.W[-1].handle, self.b[-1].handle, self.T.handle,
+                                             self.Z[-1].handle, self.P.handle, self.loss.handle, self.dP.handle, self.dZ[-1].handle,
+                                             self.dZ[L - 2].handle, self.dW[-1].handle, self.db[-1].handle, 0,
+                                             _lib.ACT_LEAKYRELU, self.Z[L - 2].handle, alpha))
+        elif self.fused:
             check(lib.prad_softmax_cce(self.Z[-1].handle, self.T.handle, self.P.handle, self.loss.handle, self.dP.handle,
                                        self.dZ[-1].handle))
         else:
@@ -88,7 +94,7 @@ class FeedForwardNetwork:
             check(lib.prad_cce_fwd(self.P.handle, self.T.handle, self.loss.handle))
             check(lib.prad_cce_bwd(self.P.handle, self.T.handle, self.dP.handle))
             check(lib.prad_softmax_bwd(self.P.handle, self.dP.handle, self.dZ[-1].handle))
-        for l in range(L - 1, -1, -1):
+        for l in range(L - 2 if head else L - 1, -1, -1):
             inp = self.X if l == 0 else self.H[l - 1]
             # MatrixMultiplyOperation.Backward always forms both gradients, also for the network input (l == 0)
             dA = self.dX if l == 0 else self.dZ[l - 1]
