@@ -7,22 +7,24 @@
 // memory could do.  Here the right operand is resident and the rows stream:
 //
 //   * every workgroup (one per compute unit, sixteen wavefronts) first copies the whole of B into LDS, already cut into
-//     MFMA fragments: element (y, j, i, g, n) is B[16 j + 4 g + i][16 y + n], so that a wavefront's 64 lanes (g, n) read 64
+//     MFMA fragments: element (y, j, i, g, n) is B[16 j + 4 i + g][16 y + n], so that a wavefront's 64 lanes (g, n) read 64
 //     consecutive floats for one MFMA step (no bank conflicts; 16-byte reads per lane were measured with 60 % of the LDS
 //     cycles lost to conflicts);
 //   * the work is cut into units of 16 rows by NYW 16-column tiles (NYW = 4, 3 or 2: many small units, so that a compute
 //     unit's four matrix cores get shares that differ by little); a workgroup owns a contiguous range of units
 //     and each of its wavefronts takes one unit after another from it, alone (no barrier after the fill).  A lane (m, g) of the
-//     wavefront loads 16 bytes A[row0 + m][16 j + 4 g .. + 3] straight into registers - the four k of a lane's vector are
-//     four MFMA steps, paired with the B values of the same (j, g) - 96 columns of a unit at a time, each half of them
-//     fetched again (for the next 96 columns, or the next unit) as soon as its MFMAs are issued, so a load has the other
-//     half's multiplications to arrive;
+//     wavefront loads 16 bytes A[row0 + m][16 j + 4 g .. + 3] straight into registers, 96 columns of a unit at a time, each
+//     half of them fetched again (for the next 96 columns, or the next unit) as soon as its MFMAs are issued, so a load has
+//     the other half's multiplications to arrive.  Before its MFMAs a vector is transposed across the wavefront's four
+//     lane groups (four lane-swap instructions per sixteen k), after which element i of lane group g is
+//     A[row0 + m][16 j + 4 i + g]: MFMA step 4 j + i then sees k = 4 (4 j + i) + g, the assignment of the tiled kernels;
 //   * the MFMA takes the B fragment as its first operand and the A fragment as its second: the 16 x 16 result is then
 //     C^T, and a lane holds C[row0 + m][16 y + 4 g .. + 3] - four neighbours of one row - so bias, pre-activation copy,
 //     activation, the upstream activation's derivative and the store are all 16-byte accesses with no trip through LDS.
 //
-// Per element the arithmetic is that of the tiled kernels' elementwise epilogue, in the same order; only the order of the
-// sum along K differs (one chain of K / 4 MFMA steps; K <= 384 here).
+// Per element the arithmetic is that of the tiled kernels' elementwise epilogue, in the same order, and the sum along K is
+// the same chain of MFMA steps over the same k (K <= 384 here: the float kernels' folding every 512 does not come into
+// it): a product has the same bits whichever kernel its shape selects.
 #include "common.h"
 
 #include <cstdlib>
@@ -69,7 +71,7 @@ constexpr int TALL_STORE = 0, TALL_GENERAL = 1, TALL_GELU_FWD = 2, TALL_GELU_BWD
 // NYW: 16-column tiles (accumulators per lane) of a unit.  ONE_CHUNK: K == 96, every pass of the main loop is a whole unit.
 template <int NYW, int EPI, bool ONE_CHUNK>
 __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallArgs p) {
-    extern __shared__ __attribute__((aligned(16))) float bfrag[];  // [y][j][i][g][n], then the bias, then the unit counter
+    extern __shared__ __attribute__((aligned(16))) float bfrag[];  // [y][j][i][g][n] = B[16 j + 4 i + g][16 y + n], then the bias, then the unit counter
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (said to be uniform: loop counts and load bases that depend on it stay scalar)
     const int li = lane & 15, g = lane >> 4;
@@ -119,9 +121,9 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
                 const int v = min(v0 + u * TALL_THREADS, nvec - 1);
                 const int pair = v >> 6, l = v & 63, y = pair / KJ, j = pair - y * KJ;
                 // transposed B is stored [n][k]: lane (gg, nn) reads the four i of (j, gg) for column 16 y + nn;
-                // plain B is stored [k][n]: lane (i, gg, n4) reads four neighbouring columns of row k = 16 j + 4 gg + i
+                // plain B is stored [k][n]: lane (i, gg, n4) reads four neighbouring columns of row k = 16 j + 4 i + gg
                 const long at = p.transB ? (long)(16 * y + (l & 15)) * p.ldb + 16 * j + 4 * (l >> 4)
-                                         : (long)(16 * j + 4 * ((l >> 2) & 3) + (l >> 4)) * p.ldb + 16 * y + 4 * (l & 3);
+                                         : (long)(16 * j + 4 * (l >> 4) + ((l >> 2) & 3)) * p.ldb + 16 * y + 4 * (l & 3);
                 x[u] = *reinterpret_cast<const f4t*>(p.B + at);
             }
 #pragma unroll
@@ -131,8 +133,15 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
                 const int pair = v >> 6, l = v & 63;
                 float* dst = bfrag + pair * 256;
                 if (p.transB) {
+                    // the lane holds k = 16 j + 4 q + i for q = l >> 4, i = 0..3: element i belongs to lane group i of step q.
+                    // The four are written in an order rotated by q, so that the lanes of a store fall on distinct banks.
+                    const int q = l >> 4, n = l & 15;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) dst[i * 64 + l] = x[u][i];
+                    for (int i = 0; i < 4; ++i) {
+                        const int e = (i + q) & 3;
+                        const float v = e == 0 ? x[u][0] : e == 1 ? x[u][1] : e == 2 ? x[u][2] : x[u][3];
+                        dst[q * 64 + e * 16 + n] = v;
+                    }
                 } else {
                     *reinterpret_cast<f4t*>(dst + (l >> 4) * 64 + ((l >> 2) & 3) * 16 + 4 * (l & 3)) = x[u];
                 }
@@ -145,6 +154,22 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
 
     if (!working) return;
     f4t acc[NYW];
+    // A lane (m, g) loaded A[m][16 j + 4 g + e], e = 0..3, in one vector; MFMA step q of the group needs A[m][16 j + 4 q + g]
+    // in lane group g (the assignment of k to steps and lane groups that the tiled kernels use: k = 4 s + g, s ascending).
+    // That is a 4 x 4 transpose between the vector's elements and the wavefront's four lane groups: two swaps of lane
+    // halves, then two swaps of odd with even groups, four instructions per sixteen k.
+    auto transpose_k = [](f4t& v) {
+        typedef unsigned u2t __attribute__((ext_vector_type(2)));
+        // (element by element through plain floats: a bit cast applied to a vector element reads element 0)
+        const float f0 = v[0], f1 = v[1], f2 = v[2], f3 = v[3];
+        unsigned r0 = __float_as_uint(f0), r1 = __float_as_uint(f1), r2 = __float_as_uint(f2), r3 = __float_as_uint(f3);
+        u2t t;
+        t = __builtin_amdgcn_permlane32_swap(r0, r2, false, false); r0 = t[0]; r2 = t[1];
+        t = __builtin_amdgcn_permlane32_swap(r1, r3, false, false); r1 = t[0]; r3 = t[1];
+        t = __builtin_amdgcn_permlane16_swap(r0, r1, false, false); r0 = t[0]; r1 = t[1];
+        t = __builtin_amdgcn_permlane16_swap(r2, r3, false, false); r2 = t[0]; r3 = t[1];
+        v[0] = __uint_as_float(r0); v[1] = __uint_as_float(r1); v[2] = __uint_as_float(r2); v[3] = __uint_as_float(r3);
+    };
     // One k step (j, i) at a time across all NYW accumulators, so that consecutive MFMAs never depend on each other; the
     // NYW values of B for a step are read from LDS one step ahead of the MFMAs that use them.
     auto multiply_half = [&](int unit, int c, int h) {
@@ -164,6 +189,7 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) {
             const int j = h * HALF + t / 4, i = t % 4;
+            if (i == 0) transpose_k(a[j]);
             if (t + 1 < STEPS) read_b(t + 1);
 #pragma unroll
             for (int y = 0; y < NYW; ++y) acc[y] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[t & 1][y], a[j][i], acc[y], 0, 0, 0);

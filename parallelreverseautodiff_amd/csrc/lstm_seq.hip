@@ -101,8 +101,10 @@ __device__ __forceinline__ bool wait_for_group(const unsigned* flags, int blocks
 // 1021 us with the values announcing themselves and 1099 us with device-scope stores.)
 constexpr unsigned SEQ_SENTINEL = 0xFFFFFFFFu;
 __device__ __forceinline__ bool arrived(const f4v v) {
-    return __builtin_bit_cast(unsigned, v[0]) != SEQ_SENTINEL && __builtin_bit_cast(unsigned, v[1]) != SEQ_SENTINEL &&
-           __builtin_bit_cast(unsigned, v[2]) != SEQ_SENTINEL && __builtin_bit_cast(unsigned, v[3]) != SEQ_SENTINEL;
+    // (each element through a plain float first: a bit cast applied directly to a vector element reads element 0)
+    const float a = v[0], b = v[1], c = v[2], d = v[3];
+    return __float_as_uint(a) != SEQ_SENTINEL && __float_as_uint(b) != SEQ_SENTINEL && __float_as_uint(c) != SEQ_SENTINEL &&
+           __float_as_uint(d) != SEQ_SENTINEL;
 }
 __device__ __forceinline__ float never_the_sentinel(float x) { return x != x ? __builtin_bit_cast(float, 0x7FC00000u) : x; }
 // The XCD this wavefront runs on (hardware register XCC_ID).

@@ -629,19 +629,17 @@ def test_rows_of_a_tall_product_do_not_depend_on_how_many_rows_there_are(gpu, or
     tile the sizes select (a tall product runs on 128 x 128 tiles, its first 4096 rows alone on smaller ones): the first
     4096 rows of the tall product equal the product of the first 4096 rows bit for bit - for every epilogue (bias,
     pre-activation copy, activation, the upstream activation's derivative, accumulation), both layouts of B, and a
-    ragged last tile.  From 8192 rows on, products with K a multiple of 96 run on the streaming kernel, whose MFMA steps
-    group K differently (k = 16 j + 4 g + i instead of 4 s + g): there the two agree to rounding, not to the bit."""
+    ragged last tile.  From 8192 rows on, products with K a multiple of 96 run on the streaming kernel, which loads four
+    consecutive k per lane and transposes them across the lane groups so that its MFMA steps see k = 4 s + g as well:
+    the same bits there too."""
     lib = _lib.load()
     from parallelreverseautodiff_amd.exceptions import check
     dtype = np.float32
     M, K, N = shape
     head = 4096
-    streaming = M >= 8192 and K % 96 == 0          # the full product runs on the streaming kernel, the head on tiles
 
     def same(x, y):
-        if not streaming:
-            return np.array_equal(x, y)
-        return rel_err(x, y) <= 1e-5
+        return np.array_equal(x, y)
     A = seeded.uniform(43, 1, (M, K), -1, 1, dtype)
     B = seeded.uniform(43, 2, (K, N), -1, 1, dtype)
     Bt = np.ascontiguousarray(B.T)                                  # N x K: the operand of dC . W^T
