@@ -101,6 +101,9 @@ int32_t prad_alloc_stats(int64_t* device_mallocs, int64_t* device_frees, int64_t
 int32_t prad_buf_shape(prad_buf_t b, int64_t* depth, int64_t* rows, int64_t* cols, int32_t* dtype);
 void* prad_buf_device_ptr(prad_buf_t b); /* getter: NULL for a bad handle */
 int32_t prad_buf_zero(prad_buf_t b);
+/* GradientClearer.Clear over a model's layers (src/RMAD/GradientClearer.cs:21-86): n buffers zeroed by one launch (one per
+ * 40 buffers). */
+int32_t prad_zero_multi(const prad_buf_t* bufs, int32_t n);
 /* Jagged upload: row_ptrs[i] points at row i (cols elements).  row_lengths may be NULL; when given,
  * any length != cols fails with PRAD_ERR_NOT_RECTANGULAR. For a deep buffer pass depth*rows pointers. */
 int32_t prad_buf_upload_rows(prad_buf_t b, const void* const* row_ptrs, const int64_t* row_lengths);

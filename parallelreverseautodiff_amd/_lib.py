@@ -53,6 +53,7 @@ SIGNATURES = {
     "prad_buf_shape": (_i32, [_vp, _i64p, _i64p, _i64p, _i32p]),
     "prad_buf_device_ptr": (_vp, [_vp]),
     "prad_buf_zero": (_i32, [_vp]),
+    "prad_zero_multi": (_i32, [_vp, _i32]),
     "prad_buf_upload_rows": (_i32, [_vp, _vpp, _i64p]),
     "prad_buf_download_rows": (_i32, [_vp, _vpp]),
     "prad_buf_upload": (_i32, [_vp, _vp, _i64]),

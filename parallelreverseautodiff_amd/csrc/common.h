@@ -276,6 +276,9 @@ template <typename T> hipError_t launch_add_broadcast_fwd(const T* x, const T* b
 int colsum_chunks(int64_t rows);
 template <typename T> hipError_t launch_colsum(const T* dy, T* db, int64_t rows, int64_t cols, double* workspace, hipStream_t s);
 template <typename T> hipError_t launch_fill_zero(T* p, int64_t n, hipStream_t s);
+// n regions (16-byte aligned, sizes multiples of 4 bytes) zeroed by one launch per ZERO_TABLE_MAX of them.
+constexpr int ZERO_TABLE_MAX = 40;
+hipError_t launch_fill_zero_multi(void* const* ptrs, const size_t* bytes, int n, hipStream_t s);
 
 // Descriptor of one tensor of a multi-tensor clip / Adam launch.
 template <typename T>

@@ -225,6 +225,50 @@ hipError_t launch_fill_zero(T* p, int64_t n, hipStream_t s) {
     return hipGetLastError();
 }
 
+// Several tensors zeroed by one launch (GradientClearer over a model's layers): a table of up to ZERO_TABLE_MAX regions as a
+// kernel argument, cut into chunks of 16 KB; a workgroup finds its region by walking the table.
+struct ZeroTable {
+    unsigned char* ptr[ZERO_TABLE_MAX];
+    unsigned long long bytes[ZERO_TABLE_MAX];
+    unsigned first_chunk[ZERO_TABLE_MAX + 1];
+    int n;
+};
+constexpr unsigned ZERO_CHUNK = 16384;
+__global__ void __launch_bounds__(EW_THREADS) fill_zero_multi_kernel(const ZeroTable tab) {
+    int t = 0;
+    while (t + 1 < tab.n && blockIdx.x >= tab.first_chunk[t + 1]) ++t;
+    const unsigned long long begin = (unsigned long long)(blockIdx.x - tab.first_chunk[t]) * ZERO_CHUNK;
+    const unsigned long long end = min(begin + ZERO_CHUNK, tab.bytes[t]);
+    unsigned char* base = tab.ptr[t];
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const u4 z = {0u, 0u, 0u, 0u};
+    unsigned long long at = begin + 16ull * threadIdx.x;  // (regions start 16-byte aligned, their sizes are multiples of 4 bytes)
+    for (; at + 16 <= end; at += 16ull * EW_THREADS) *reinterpret_cast<u4*>(base + at) = z;
+    if (at < end)
+        for (unsigned long long b = at; b < end; b += 4) *reinterpret_cast<unsigned*>(base + b) = 0u;
+}
+hipError_t launch_fill_zero_multi(void* const* ptrs, const size_t* bytes, int n, hipStream_t s) {
+    for (int g0 = 0; g0 < n; g0 += ZERO_TABLE_MAX) {
+        ZeroTable tab{};
+        tab.n = 0;
+        unsigned chunks = 0;
+        for (int i = g0; i < n && tab.n < ZERO_TABLE_MAX; ++i) {
+            if (bytes[i] == 0) continue;
+            if (reinterpret_cast<uintptr_t>(ptrs[i]) % 16 != 0 || bytes[i] % 4 != 0) return hipErrorInvalidValue;
+            tab.ptr[tab.n] = static_cast<unsigned char*>(ptrs[i]);
+            tab.bytes[tab.n] = bytes[i];
+            tab.first_chunk[tab.n] = chunks;
+            chunks += (unsigned)((bytes[i] + ZERO_CHUNK - 1) / ZERO_CHUNK);
+            ++tab.n;
+        }
+        if (tab.n == 0) continue;
+        tab.first_chunk[tab.n] = chunks;
+        hipLaunchKernelGGL(fill_zero_multi_kernel, dim3(chunks), dim3(EW_THREADS), 0, s, tab);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 // ---- bias broadcast: y[i][j] = x[i][j] + bias[j] -----------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(EW_THREADS) add_broadcast_kernel(const T* __restrict__ x, const T* __restrict__ bias,

@@ -75,7 +75,7 @@ int32_t prad_hostwalk_mlp(int32_t dtype, int32_t batch, int32_t nlayers, const i
             return b;
         };
         auto step = [&](int iteration) {
-            for (prad_buf_t grad : g) ok(prad_buf_zero(grad));                                   // GradientClearer.Clear
+            ok(prad_zero_multi(g.data(), (int32_t)g.size()));                                    // GradientClearer.Clear
             prad_buf_t value = x;
             for (int l = 0; l < nlayers; ++l) {                                                  // forward walk
                 Layer& L = net[(size_t)l];

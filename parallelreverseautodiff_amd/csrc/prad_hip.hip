@@ -718,6 +718,21 @@ int32_t prad_buf_zero(prad_buf_t b) {
     return PRAD_OK;
 }
 
+int32_t prad_zero_multi(const prad_buf_t* bufs, int32_t n) {
+    REQUIRE_INIT();
+    if (n < 0 || (n > 0 && bufs == nullptr)) return fail(PRAD_ERR_ARG, "bad tensor list");
+    std::vector<void*> ptrs;
+    std::vector<size_t> bytes;
+    for (int32_t i = 0; i < n; ++i) {
+        REQUIRE_BUF(bufs[i]);
+        ptrs.push_back(bufs[i]->ptr);
+        bytes.push_back((size_t)count(bufs[i]) * (bufs[i]->dtype == PRAD_F64 ? 8 : 4));
+    }
+    ENQUEUE_LOCK();
+    HIP_TRY(prad::launch_fill_zero_multi(ptrs.data(), bytes.data(), n, CUR_STREAM), PRAD_ERR_LAUNCH);
+    return PRAD_OK;
+}
+
 int32_t prad_buf_upload_rows(prad_buf_t b, const void* const* row_ptrs, const int64_t* row_lengths) {
     REQUIRE_INIT();
     REQUIRE_BUF(b);

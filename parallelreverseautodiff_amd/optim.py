@@ -146,14 +146,18 @@ class GradientClearer:
     a host-only one gets new zero rows as in the reference."""
 
     def Clear(self, layers):
+        on_device = []
         for g in _collect(layers, "Gradient"):
             for m in (g if isinstance(g, DeepMatrix) else [g]):
                 if m._dev is not None:
-                    m._dev.zero()
-                    m._device_written()
+                    on_device.append(m)
                 else:
                     for i in range(m.Rows):
                         m[i] = np.zeros(m.Cols, dtype=m.dtype)
+        if on_device:  # one launch for all of them
+            check(_lib.load().prad_zero_multi(handle_array([m._dev for m in on_device]), len(on_device)))
+            for m in on_device:
+                m._device_written()
 
 
 class GradientClipper:

@@ -233,3 +233,28 @@ def test_device_resident_state_survives_a_checkpoint(gpu, tmp_path, dtype):
     for i in range(len(shapes)):
         for element in ("Weight", "FirstMoment", "SecondMoment"):
             assert np.array_equal(a["W%d" % i, element].to_numpy(), b["W%d" % i, element].to_numpy()), (i, element)
+
+
+def test_gradient_clearer_zeroes_every_gradient_in_one_call(gpu):
+    """GradientClearer.Clear (src/RMAD/GradientClearer.cs:21-86): device-resident gradients of both element types, of odd
+    sizes (a 16-byte vector does not divide them), more of them than one launch's table holds, and a host-only one; the
+    buffers next to them keep their values."""
+    from parallelreverseautodiff_amd.optim import GradientClearer
+    shapes = [(1, 1), (3, 5), (1, 10), (7, 9), (128, 10), (255, 33), (64, 4097)] * 7   # 49 tensors: two tables
+    mats, guards = [], []
+    for i, s in enumerate(shapes):
+        dtype = np.float64 if i % 2 else np.float32
+        m = Matrix.from_numpy(seeded.normal(61, i, s, 1.0, dtype))
+        m.device()                                                       # the gradient lives on the device
+        g = Matrix.from_numpy(seeded.normal(62, i, s, 1.0, dtype))
+        g.device()
+        mats.append(m)
+        guards.append((g, g.to_numpy().copy()))
+    host_only = Matrix.from_numpy(np.ones((4, 6)))
+    GradientClearer().Clear([layer_of(mats + [host_only], mats + [host_only])])
+    for m, s in zip(mats, shapes):
+        got = m.to_numpy()
+        assert got.shape == s and not got.any()
+    assert not host_only.to_numpy().any()
+    for g, ref in guards:
+        assert np.array_equal(g.to_numpy(), ref)
