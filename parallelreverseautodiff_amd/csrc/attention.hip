@@ -148,15 +148,19 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, FR ? 3 : 2) window_attention_f
         for (int j = 0; j < NC; ++j) v[j] = j < wt ? row[j] * p.scale : -INFINITY;
         float m = v[0];
 #pragma unroll
-        for (int j = 1; j < NC; ++j) m = v[j] > m ? v[j] : m;
+        for (int j = 1; j < NC; ++j) m = fmaxf(m, v[j]);
         float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; ++j) {
             v[j] = j < wt ? att_exp(v[j] - m) : 0.f;
             sum = sum + v[j];
         }
+        // one division per row, a multiplication per element (within an ulp of the quotient): the float MFMA runs on the
+        // vector unit's multipliers, so the ten instructions of a division, forty-nine times a row, were time the
+        // products of the other wavefronts on this SIMD did not get
+        const float inv = 1.0f / sum;
 #pragma unroll
-        for (int j = 0; j < NC; ++j) row[j] = j < wt ? v[j] / sum : 0.f;
+        for (int j = 0; j < NC; ++j) row[j] = j < wt ? v[j] * inv : 0.f;
 #pragma unroll
         for (int j = NC; j < 4 * KS; ++j) row[j] = 0.f;  // (FR: the k steps of the second product reach column 51)
     }

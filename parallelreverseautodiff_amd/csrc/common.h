@@ -68,6 +68,43 @@ __device__ __forceinline__ float gelu_tanh(float u) {
 __device__ __forceinline__ float gelu_cube(float x) { return x * x * x; }
 __device__ __forceinline__ double gelu_cube(double x) { return x * x * x; }
 
+// GELU as the reference writes it, 0.5 x (1 + tanh(u)) with u = sqrt(2/pi) (x + 0.044715 x^3) (src/RMAD/GELUOperation.cs:86-92),
+// and the factor its Backward multiplies by (:94-101; as written there, not the derivative).
+__device__ __forceinline__ double gelu_value(double x) {
+    const double a = 0.5 * (1.0 + gelu_tanh(GeluConst<double>::s() * (x + (GeluConst<double>::c0() * gelu_cube(x)))));
+    return a * x;
+}
+__device__ __forceinline__ double gelu_factor(double s) {
+    const double b = gelu_tanh(GeluConst<double>::s() * (s + (GeluConst<double>::c0() * gelu_cube(s))));
+    const double omb = 1.0 - b * b;
+    const double c = omb * omb;
+    const double d = GeluConst<double>::s() * ((GeluConst<double>::c0() * 3.0 * (s * s)) + 1.0);
+    return (0.5 * s * ((c * d) + b)) + (0.5 * (1.0 + b));
+}
+// In float the same functions in as few instructions as they take (PRADLite evaluates them in double and rounds; both forms
+// are within 5e-7 of that, far inside the 1e-5 parity bar).  On this chip the float and double matrix instructions run on
+// the vector unit's multipliers, so every vector instruction of an epilogue is time the matrix cores do not get:
+// 0.5 (1 + tanh u) = 1 / (1 + e^(-2u)), e^(-2u) = 2^(x (k1 + k2 x^2)) on the hardware exponential and reciprocal - seven
+// instructions for the value, about twenty for the factor.
+__device__ __forceinline__ float gelu_exp_minus_2u(float x, float x2, float limit) {
+    const float k1 = -2.302208185195923f;   // -2 s log2(e), s = PRADLite's float sqrt(2/pi)
+    const float k2 = -0.10294323414564133f;  // k1 * 0.044715f
+    return __builtin_amdgcn_exp2f(fminf(x * __builtin_fmaf(k2, x2, k1), limit));
+}
+__device__ __forceinline__ float gelu_value(float x) {
+    const float e = gelu_exp_minus_2u(x, x * x, INFINITY);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+__device__ __forceinline__ float gelu_factor(float s) {
+    const float x2 = s * s;
+    const float e = gelu_exp_minus_2u(s, x2, 126.0f);  // (bounded, so that (1 - e) / (1 + e) stays -1 instead of inf / inf)
+    const float b = (1.0f - e) * __builtin_amdgcn_rcpf(1.0f + e);  // tanh u
+    const float omb = 1.0f - b * b;
+    const float c = omb * omb;
+    const float d = __builtin_fmaf(0.10703221708536148f, x2, 0.7978845238685608f);  // s (3 * 0.044715f x^2 + 1)
+    return __builtin_fmaf(0.5f * s, __builtin_fmaf(c, d, b), 0.5f * (1.0f + b));
+}
+
 // AmplifiedSigmoid: pow(b, -x) with b = (float)pi - 2 (PradMath.PI is a float, src/PRAD/PradMath.cs:20, and the
 // subtraction a float one), evaluated as exp(-x * ln b).
 template <typename T>
@@ -82,10 +119,7 @@ __device__ __forceinline__ T act_forward(int act, T x, T alpha) {
         case ACT_LEAKYRELU: return x > (T)0 ? x : alpha * x;
         case ACT_SIGMOID: return (T)1 / ((T)1 + dev_exp(-x));
         case ACT_TANH: return dev_tanh(x);
-        case ACT_GELU: {
-            T a = (T)0.5 * ((T)1 + gelu_tanh(GeluConst<T>::s() * (x + (GeluConst<T>::c0() * gelu_cube(x)))));
-            return a * x;
-        }
+        case ACT_GELU: return gelu_value(x);
         case ACT_AMPLIFIED_SIGMOID: return (T)1 / ((T)1 + amp_pow_neg<T>(x));
         default: return x;
     }
@@ -98,13 +132,7 @@ __device__ __forceinline__ T act_derivative(int act, T s, T alpha) {
         case ACT_LEAKYRELU: return s > (T)0 ? (T)1 : alpha;
         case ACT_SIGMOID: return s * ((T)1 - s);
         case ACT_TANH: return (T)1 - s * s;
-        case ACT_GELU: {
-            T b = gelu_tanh(GeluConst<T>::s() * (s + (GeluConst<T>::c0() * gelu_cube(s))));
-            T omb = (T)1 - b * b;
-            T c = omb * omb;
-            T d = GeluConst<T>::s() * ((GeluConst<T>::c0() * (T)3 * (s * s)) + (T)1);
-            return ((T)0.5 * s * ((c * d) + b)) + ((T)0.5 * ((T)1 + b));
-        }
+        case ACT_GELU: return gelu_factor(s);
         case ACT_AMPLIFIED_SIGMOID: {  // as written: pow(b, -x) / pow(1 + pow(b, -x), 2), no ln(b) factor
             const T e = amp_pow_neg<T>(s);
             const T q = (T)1 + e;

@@ -113,24 +113,26 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
     {
         constexpr int FILL = 9;
         static_assert(TALL_MAX_B / 16 <= (size_t)FILL * TALL_THREADS, "one round copies the largest B");
-        const int nvec = (p.N / 16) * KJ * 64;  // = K * N / 4
-        for (int v0 = tid; v0 < nvec; v0 += FILL * TALL_THREADS) {
+        const int npairs = (p.N / 16) * KJ;  // = K * N / 256
+        const int l = lane;
+        // the lane's part of a pair's addresses (the pair's part, from the wavefront's number, is scalar arithmetic: every
+        // vector instruction here is time taken from the matrix pipeline, which the float MFMA shares with the vector unit)
+        const long lane_at = p.transB ? (long)(l & 15) * p.ldb + 4 * (l >> 4) : (long)(4 * (l >> 4) + ((l >> 2) & 3)) * p.ldb + 4 * (l & 3);
+        const int lane_dst = (l >> 4) * 64 + ((l >> 2) & 3) * 16 + 4 * (l & 3);
+        for (int pair0 = wave; pair0 < npairs; pair0 += FILL * TALL_WAVES) {
             f4t x[FILL];
 #pragma unroll
             for (int u = 0; u < FILL; ++u) {
-                const int v = min(v0 + u * TALL_THREADS, nvec - 1);
-                const int pair = v >> 6, l = v & 63, y = pair / KJ, j = pair - y * KJ;
+                const int pair = min(pair0 + u * TALL_WAVES, npairs - 1), y = pair / KJ, j = pair - y * KJ;
                 // transposed B is stored [n][k]: lane (gg, nn) reads the four i of (j, gg) for column 16 y + nn;
                 // plain B is stored [k][n]: lane (i, gg, n4) reads four neighbouring columns of row k = 16 j + 4 i + gg
-                const long at = p.transB ? (long)(16 * y + (l & 15)) * p.ldb + 16 * j + 4 * (l >> 4)
-                                         : (long)(16 * j + 4 * (l >> 4) + ((l >> 2) & 3)) * p.ldb + 16 * y + 4 * (l & 3);
-                x[u] = *reinterpret_cast<const f4t*>(p.B + at);
+                const long pair_at = p.transB ? (long)(16 * y) * p.ldb + 16 * j : (long)(16 * j) * p.ldb + 16 * y;
+                x[u] = *reinterpret_cast<const f4t*>(p.B + pair_at + lane_at);
             }
 #pragma unroll
             for (int u = 0; u < FILL; ++u) {
-                const int v = v0 + u * TALL_THREADS;
-                if (v >= nvec) continue;
-                const int pair = v >> 6, l = v & 63;
+                const int pair = pair0 + u * TALL_WAVES;
+                if (pair >= npairs) continue;
                 float* dst = bfrag + pair * 256;
                 if (p.transB) {
                     // the lane holds k = 16 j + 4 q + i for q = l >> 4, i = 0..3: element i belongs to lane group i of step q.
@@ -143,7 +145,7 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
                         dst[q * 64 + e * 16 + n] = v;
                     }
                 } else {
-                    *reinterpret_cast<f4t*>(dst + (l >> 4) * 64 + ((l >> 2) & 3) * 16 + 4 * (l & 3)) = x[u];
+                    *reinterpret_cast<f4t*>(dst + lane_dst) = x[u];
                 }
             }
         }
