@@ -304,6 +304,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
 
     // (not const: they are formed again after the K loop, see there)
     int tid = threadIdx.x;
+    const int wave_scalar = __builtin_amdgcn_readfirstlane(tid >> 6);
     int lane = tid & 63, wave = tid >> 6;
     int wm = wave >> 1, wn = wave & 1;
     int li = lane & 15, g = lane >> 4;
@@ -593,11 +594,16 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     // The epilogues use the thread's coordinates again.  Kept alive across the K loop, where every register is taken,
     // they were spilled before it (five dwords per lane, 5 MiB of scratch writes per launch of the 128 x 128 kernel in
     // double); formed anew from a thread index the compiler cannot tie to the one above, they cost a few instructions.
-    {
-        int t = threadIdx.x;
-        asm volatile("" : "+v"(t));
-        tid = t; lane = tid & 63; wave = tid >> 6; wm = wave >> 1; wn = wave & 1; li = lane & 15; g = lane >> 4;
-    }
+    // (Each epilogue path forms them for itself: held from here across the other paths they were spilled again.)
+    // (The lane comes from the hardware's lane count and the wavefront's number from a scalar register: the thread index
+    // itself would have to be kept, which is a spilled register as well.)
+    auto coordinates = [&] {
+        unsigned all = ~0u;
+        asm volatile("" : "+s"(all));  // (opaque, so that the count is taken anew at every call instead of being kept)
+        const int l = (int)__builtin_amdgcn_mbcnt_hi(all, __builtin_amdgcn_mbcnt_lo(all, 0u));
+        lane = l; wave = wave_scalar; tid = 64 * wave + lane; wm = wave >> 1; wn = wave & 1; li = lane & 15; g = lane >> 4;
+    };
+    coordinates();
     if (FOLD) {
 #pragma unroll
         for (int x = 0; x < WTM; ++x)
@@ -629,6 +635,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     }
 
     if (EPI != EPI_TILE_SUM && p.split_counters != nullptr && g_.gz > 1) {
+        coordinates();
         // Several workgroups share this tile, a K range each.  Every one parks its partial tile in the workspace
         // and counts its arrival; the one that arrives last adds the partial tiles in split order (its own
         // included, read back like the others, so that the sum does not depend on who arrives last) and goes on
@@ -703,6 +710,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     }
 
     if (WT == 4 && EPI != EPI_TILE_SUM && p.shared_splits > 1 && g_.gz > 1) {
+        coordinates();
         // One of the workgroups that share a tile of an otherwise unsplit launch: its partial tile goes to the workspace
         // as a plain 128 x 128 row-major block (tile by tile, split by split); shared_reduce_kernel adds the blocks of a
         // tile in split order and applies the epilogue.
@@ -801,6 +809,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
     T* __restrict__ C = p.C + b_outer * p.strideC + b_inner * p.istrideC +
                         ((g_.gz > 1 && p.split_counters == nullptr) ? (int64_t)g_.bz * g_.gy * p.strideC : 0);
     if (EPI == EPI_ELEMENTWISE) {
+        coordinates();
         // The accumulators go through LDS, 16 rows of the wavefront's share at a time, and are read back
         // row-major: the elementwise arithmetic (which includes exp/tanh code) then sits in one runtime loop
         // instead of being inlined into 64 unrolled stores, and every global access covers whole rows.
@@ -904,6 +913,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs<T>& p, const int tilesM
         return;
     }
 
+    coordinates();
 #pragma unroll
     for (int x = 0; x < WTM; ++x) {
 #pragma unroll
