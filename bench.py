@@ -4,7 +4,7 @@ One step = MatrixMultiplyOperation forward (C = A.B) plus backward (dA = dC.B^T,
 device-resident square double matrices, N = 4096 by default: three launches of the MFMA product
 kernel, 6 N^3 floating-point operations.  The LAST line printed is one compact JSON object (the
 figures of the headline leg with its roofline and CPU baseline, under 1800 characters); the line
-before it, also written to gpurun_out/bench_detail.json, carries every other leg and the table.
+before it (also written to the file --detail-file names, if any) carries every other leg and the table.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--n N] [--dtype f64|f32] [--no-cpu]
 """
@@ -614,6 +614,7 @@ def main():
     ap.add_argument("--dtype", choices=["f64", "f32"], default="f64")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="gemm mode: skip the other-precision and MLP legs")
+    ap.add_argument("--detail-file", default=None, help="gemm mode: also write the detail line to this file")
     ap.add_argument("--mode", choices=["gemm", "bandwidth", "mlp", "mlp_ops", "matmul_sum", "lstm", "swin", "oneshot"], default="gemm",
                     help="gemm: the headline forward+backward step; bandwidth: the elementwise / clip / Adam kernels; "
                          "mlp: the feed-forward training step of configs[0]")
@@ -691,12 +692,13 @@ def main():
     line, detail = headline_lines(args, head, cpu, also, table)
     text = json.dumps({"detail": detail})
     print(text)
-    try:  # the same detail as a file, for runs whose captured output is cut short
-        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-        with open(os.path.join(ROOT, "gpurun_out", "bench_detail.json"), "w") as f:
-            f.write(text + "\n")
-    except OSError:
-        pass
+    if args.detail_file:  # the same detail as a file, for runs whose captured output is cut short
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.detail_file)), exist_ok=True)
+            with open(args.detail_file, "w") as f:
+                f.write(text + "\n")
+        except OSError:
+            pass
     sys.stdout.flush()
     print(json.dumps(line, separators=(",", ":")))
 

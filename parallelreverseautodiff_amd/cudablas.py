@@ -12,15 +12,22 @@ from .exceptions import check
 class _CudaBlas:
     def __init__(self):
         self.DeviceId = 0
+        # set once the library has said it is initialised, cleared by Dispose: lets the operations skip one library call
+        # per Forward / Backward.  (A shutdown behind this object's back is still caught: every entry point then returns
+        # the not-initialised status.)
+        self.known_ready = False
 
     @property
     def IsInitialized(self):
-        return bool(_lib.load().prad_is_initialized())
+        self.known_ready = bool(_lib.load().prad_is_initialized())
+        return self.known_ready
 
     def Initialize(self):
         check(_lib.load().prad_init(int(self.DeviceId)))
+        self.known_ready = True
 
     def Dispose(self):
+        self.known_ready = False
         check(_lib.load().prad_shutdown())
 
     def Synchronize(self):

@@ -70,15 +70,17 @@ class BackwardResultBuilder:
 
 
 def _require_initialized():
-    if not CudaBlas.Instance.IsInitialized:
+    inst = CudaBlas.Instance
+    if not inst.known_ready and not inst.IsInitialized:
         raise CudaNotInitializedException()
 
 
 def _ensure_initialized():
     # MatrixMultiplyOperation has no initialisation requirement in the reference; starting the
     # device on first use keeps that.
-    if not CudaBlas.Instance.IsInitialized:
-        CudaBlas.Instance.Initialize()
+    inst = CudaBlas.Instance
+    if not inst.known_ready and not inst.IsInitialized:
+        inst.Initialize()
 
 
 def _null():

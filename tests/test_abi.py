@@ -68,15 +68,16 @@ def test_missing_library_fails_loudly(monkeypatch):
 
 
 def test_integration_notes_declare_every_function_for_pinvoke():
-    """The C# block of INTEGRATION.md is the output of parallelreverseautodiff_amd.pinvoke and lists every function the
-    header declares, with a C# type for every parameter."""
+    """The C# block of the integration notes is the output of parallelreverseautodiff_amd.pinvoke and lists every
+    function the header declares, with a C# type for every parameter."""
     from parallelreverseautodiff_amd import pinvoke
     decls = pinvoke.declarations()
     protos = pinvoke.prototypes()
     assert len(decls) == len(protos) > 80
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    notes = os.path.join(ROOT, "INTEGRATION.md")
+    text = open(notes).read()
     for d in decls:
-        assert d in text, "INTEGRATION.md lacks: " + d
+        assert d in text, "%s lacks: %s" % (os.path.basename(notes), d)
     header_names = {p[1] for p in protos}
     from parallelreverseautodiff_amd import _lib
     assert header_names == set(_lib.SIGNATURES)
