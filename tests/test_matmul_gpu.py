@@ -728,3 +728,25 @@ def test_weight_gradient_of_a_tall_batch_in_one_pass(gpu, oracle, shape):
     assert np.max(np.abs(first[1] - (old + ref))) <= 2e-5 * np.max(np.abs(ref)), "dB accumulated"
     assert_parity(first[2], ref_db.astype(dtype), dtype, "bias gradient")
     assert np.array_equal(first[2], first[3])
+
+
+@pytest.mark.parametrize("shape", [(16, 40, 16), (33, 128, 10), (7, 5, 3)])
+def test_a_product_is_one_chain_of_fused_multiply_adds_along_k(gpu, shape):
+    """What fixes a product's bits on this hardware: the matrix instruction adds its terms as fused multiply-adds along
+    ascending k (one rounding per term), and every kernel hands it k in ascending order.  In double this is checked
+    against exact rational arithmetic rounded once per term; it is what lets kernels of different shapes (and the
+    one-workgroup classifier head, which restates the products) give identical results."""
+    from fractions import Fraction
+    M, K, N = shape
+    A = seeded.normal(77, 1, (M, K), 1.0, np.float64)
+    B = seeded.normal(77, 2, (K, N), 1.0, np.float64)
+    op = MatrixMultiplyOperation.Instantiate(None)
+    C = op.Forward(Matrix.from_numpy(A), Matrix.from_numpy(B)).to_numpy()
+    ref = np.empty((M, N))
+    for i in range(M):
+        for j in range(N):
+            acc = 0.0
+            for k in range(K):
+                acc = float(Fraction(A[i, k]) * Fraction(B[k, j]) + Fraction(acc))   # correctly rounded: one fma
+            ref[i, j] = acc
+    assert np.array_equal(C, ref)
