@@ -51,6 +51,23 @@ def test_lstm_benchmark_configuration_full_size(gpu, oracle):
           "reference arithmetic %.2e" % errs)
 
 
+def test_long_sequence_on_the_sequence_kernels_matches_the_oracle(gpu, oracle):
+    """The whole-sequence kernels evaluate the cell's sigmoids and tanhs in float on the hardware exponential (each within
+    3e-7 of the rounded double value) and the difference feeds the recurrence: 512 time steps, four times the benchmark's
+    count, on a small layer, against the oracle's node-by-node composition at the float bar."""
+    I, H, B, T = 32, 64, 16, 512
+    layer = LSTMLayer(I, H, B, T, dtype=np.float32, sequence=True)
+    layer.step(update=False)
+    zero_b = np.zeros((1, 4 * H), np.float32)
+    loss, Hout, dW, db, dX = compose.lstm_forward_backward(layer.host_W, zero_b, layer.host_X, layer.host_Y, I, H, B, T)
+    assert abs(float(layer.loss.download()[0, 0]) - loss) <= 1e-5 * abs(loss)
+    for what, got, ref in (("hidden states", layer.H_out, Hout), ("db", layer.db, db), ("dX", layer.dX, dX)):
+        err = assert_parity(got.download(), ref, np.float32, what)
+        print("LSTM 32/64/16/512 float %s: relative %.2e" % (what, err))
+    XH = np.concatenate([layer.host_X, layer.Hs.download()[:T * B]], axis=1)
+    assert_long_sum_parity(layer.dW.download(), dW, XH, layer.dG.download(), np.float32, "dW")
+
+
 def test_lstm_recorded_step_equals_eager(gpu):
     a, b = LSTMLayer(16, 32, 8, 6, dtype=np.float64), LSTMLayer(16, 32, 8, 6, dtype=np.float64)
     a.step(); b.step()
