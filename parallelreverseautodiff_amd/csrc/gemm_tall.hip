@@ -358,8 +358,9 @@ hipError_t launch_nyw(const TallArgs& k, unsigned grid, size_t lds, hipStream_t 
 
 // Tiles per unit for a product of `ny` 16-column tiles: four, three or two, whichever divides ny first.  Narrow units
 // keep the epilogue's registers few (the general one holds a second value per accumulator) and give every matrix core
-// many units, so that their shares differ by little; wider ones (six, eight, nine tiles) were measured no faster for
-// the plain store and up to 40 % slower for the general epilogue.
+// many units, so that their shares differ by little; wider ones (six, eight, nine tiles; six again with the lane-group
+// transposes in place, which a wider unit shares among more MFMAs) were measured no faster for the plain store and up to
+// 40 % slower for the general epilogue.
 int tall_unit_tiles(int64_t ny) {
     static const int forced = [] { const char* e = getenv("PRAD_GEMM_TALL_UNIT_TILES"); return e ? atoi(e) : 0; }();  // tuning aid
     for (int w : {4, 3, 2})
