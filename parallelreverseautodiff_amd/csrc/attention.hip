@@ -155,9 +155,9 @@ __global__ void __launch_bounds__(64 * ATT_WAVES, FR ? 3 : 2) window_attention_f
             v[j] = j < wt ? att_exp(v[j] - m) : 0.f;
             sum = sum + v[j];
         }
-        // one division per row, a multiplication per element (within an ulp of the quotient): the float MFMA runs on the
-        // vector unit's multipliers, so the ten instructions of a division, forty-nine times a row, were time the
-        // products of the other wavefronts on this SIMD did not get
+        // one division per row, a multiplication per element (within an ulp of the quotient): float MFMAs do not overlap
+        // with vector instructions on this chip (measured), so the ten instructions of a division, forty-nine times a
+        // row, were time the products of the other wavefronts on this SIMD did not get
         const float inv = 1.0f / sum;
 #pragma unroll
         for (int j = 0; j < NC; ++j) row[j] = j < wt ? v[j] * inv : 0.f;

@@ -116,7 +116,7 @@ __global__ void __launch_bounds__(TALL_THREADS, 1) gemm_tall_kernel(const TallAr
         const int npairs = (p.N / 16) * KJ;  // = K * N / 256
         const int l = lane;
         // the lane's part of a pair's addresses (the pair's part, from the wavefront's number, is scalar arithmetic: every
-        // vector instruction here is time taken from the matrix pipeline, which the float MFMA shares with the vector unit)
+        // vector instruction here is time the float MFMAs of other wavefronts do not get: the two do not overlap on this chip)
         const long lane_at = p.transB ? (long)(l & 15) * p.ldb + 4 * (l >> 4) : (long)(4 * (l >> 4) + ((l >> 2) & 3)) * p.ldb + 4 * (l & 3);
         const int lane_dst = (l >> 4) * 64 + ((l >> 2) & 3) * 16 + 4 * (l & 3);
         for (int pair0 = wave; pair0 < npairs; pair0 += FILL * TALL_WAVES) {

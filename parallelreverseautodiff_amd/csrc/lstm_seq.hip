@@ -101,10 +101,11 @@ __device__ __forceinline__ bool wait_for_group(const unsigned* flags, int blocks
 // 1021 us with the values announcing themselves and 1099 us with device-scope stores.)
 constexpr unsigned SEQ_SENTINEL = 0xFFFFFFFFu;
 __device__ __forceinline__ bool arrived(const f4v v) {
-    // (each element through a plain float first: a bit cast applied directly to a vector element reads element 0)
+    // (each element through a plain float first: a bit cast applied directly to a vector element reads element 0.)
+    // The sentinel is the largest unsigned value: none of the four is it exactly when their maximum is not.
     const float a = v[0], b = v[1], c = v[2], d = v[3];
-    return __float_as_uint(a) != SEQ_SENTINEL && __float_as_uint(b) != SEQ_SENTINEL && __float_as_uint(c) != SEQ_SENTINEL &&
-           __float_as_uint(d) != SEQ_SENTINEL;
+    const unsigned m = max(max(__float_as_uint(a), __float_as_uint(b)), max(__float_as_uint(c), __float_as_uint(d)));
+    return m != SEQ_SENTINEL;
 }
 __device__ __forceinline__ float never_the_sentinel(float x) { return x != x ? __builtin_bit_cast(float, 0x7FC00000u) : x; }
 // The XCD this wavefront runs on (hardware register XCC_ID).
