@@ -133,3 +133,17 @@ def test_host_entry_points_on_flat_arrays(gpu, oracle, dtype):
     assert_parity(dA, rA, dtype, "flat host dA")
     assert_parity(dB, rB, dtype, "flat host dB")
     assert lib.prad_tensor_matmul_host(code, p(A), p(B), p(C), m, k, k + 1, n, 1.0) == _lib.PRAD_ERR_SHAPE
+
+
+def test_the_layer_of_the_references_own_tape_test(gpu):
+    """The operands of the one tape-engine test that multiplies matrices (test/ParallelReverseAutoDiff.Test/PRAD/
+    PradOpTests.cs:4151-4171: a 1 x 4 input, 4 x 3 weights; the test asserts no values).  The products are small enough
+    to be written down: 0.7, 0.8, 0.9 forward; with an upstream gradient of ones the input gradient is the row sums of
+    the weights and the weight gradient repeats the input along its rows."""
+    x = Tensor([1, 4], np.array([0.1, 0.2, 0.3, 0.4]))
+    w = Tensor([4, 3], np.array([0.1, 0.2, 0.3, 0.4, 0.5, 0.6, 0.7, 0.8, 0.9, 1.0, 1.1, 1.2]))
+    y = x.MatrixMultiply(w)
+    np.testing.assert_allclose(y.to_numpy(), [[0.7, 0.8, 0.9]], rtol=1e-15, atol=0)
+    gx, gw = TensorReverse([x, w]).MatrixMultiplyReverse(Tensor([1, 3], np.ones(3)))
+    np.testing.assert_allclose(gx.to_numpy(), [[0.6, 1.5, 2.4, 3.3]], rtol=1e-15, atol=0)
+    assert np.array_equal(gw.to_numpy(), np.repeat(np.array([[0.1], [0.2], [0.3], [0.4]]), 3, axis=1))
