@@ -723,13 +723,19 @@ int32_t prad_zero_multi(const prad_buf_t* bufs, int32_t n) {
     if (n < 0 || (n > 0 && bufs == nullptr)) return fail(PRAD_ERR_ARG, "bad tensor list");
     std::vector<void*> ptrs;
     std::vector<size_t> bytes;
+    std::vector<prad_buf_t> alone;  // views that do not start on a 16-byte boundary get a launch of their own
     for (int32_t i = 0; i < n; ++i) {
         REQUIRE_BUF(bufs[i]);
+        if (reinterpret_cast<uintptr_t>(bufs[i]->ptr) % 16 != 0) { alone.push_back(bufs[i]); continue; }
         ptrs.push_back(bufs[i]->ptr);
         bytes.push_back((size_t)count(bufs[i]) * (bufs[i]->dtype == PRAD_F64 ? 8 : 4));
     }
     ENQUEUE_LOCK();
-    HIP_TRY(prad::launch_fill_zero_multi(ptrs.data(), bytes.data(), n, CUR_STREAM), PRAD_ERR_LAUNCH);
+    HIP_TRY(prad::launch_fill_zero_multi(ptrs.data(), bytes.data(), (int)ptrs.size(), CUR_STREAM), PRAD_ERR_LAUNCH);
+    for (prad_buf_t b : alone) {
+        if (b->dtype == PRAD_F64) HIP_TRY(launch_fill_zero<double>(static_cast<double*>(b->ptr), count(b), CUR_STREAM), PRAD_ERR_LAUNCH);
+        else HIP_TRY(launch_fill_zero<float>(static_cast<float*>(b->ptr), count(b), CUR_STREAM), PRAD_ERR_LAUNCH);
+    }
     return PRAD_OK;
 }
 

@@ -252,6 +252,16 @@ def test_gradient_clearer_zeroes_every_gradient_in_one_call(gpu):
         guards.append((g, g.to_numpy().copy()))
     host_only = Matrix.from_numpy(np.ones((4, 6)))
     GradientClearer().Clear([layer_of(mats + [host_only], mats + [host_only])])
+    # a view whose first element is not on a 16-byte boundary (rows 1.. of a 3-column double matrix), straight through the C ABI
+    import ctypes
+    from parallelreverseautodiff_amd import _lib
+    from parallelreverseautodiff_amd.exceptions import check
+    from parallelreverseautodiff_amd.matrix import DeviceBuffer
+    whole = DeviceBuffer.alloc(np.float64, 5, 3)
+    whole.upload(np.arange(15.0).reshape(5, 3) + 1)
+    part = whole.view_rows(1, 3)
+    check(_lib.load().prad_zero_multi((ctypes.c_void_p * 2)(part.handle.value, mats[0].device().handle.value), 2))
+    assert np.array_equal(whole.download(), np.array([[1, 2, 3], [0, 0, 0], [0, 0, 0], [0, 0, 0], [13, 14, 15]], dtype=np.float64))
     for m, s in zip(mats, shapes):
         got = m.to_numpy()
         assert got.shape == s and not got.any()
