@@ -1926,8 +1926,11 @@ int32_t prad_dense_softmax_cce(prad_buf_t A, prad_buf_t W, prad_buf_t bias, prad
                         (act_src == nullptr || (act_src->rows == B && act_src->cols == H)) &&
                         (loss == nullptr || (loss->rows == 1 && loss->cols == 1));
     ENQUEUE_LOCK();
-    const bool one_launch = shapes && (A->dtype == PRAD_F64 ? prad::classifier_head_eligible<double>(B, H, C)
-                                                            : prad::classifier_head_eligible<float>(B, H, C));
+    // (the one-launch kernel reads the cached operand of later tiles after it has stored earlier ones: an input gradient
+    // written over that operand, which the separate launches allow element by element, goes to them)
+    const bool in_place = act_src != nullptr && dA->ptr == act_src->ptr;
+    const bool one_launch = shapes && !in_place && (A->dtype == PRAD_F64 ? prad::classifier_head_eligible<double>(B, H, C)
+                                                                         : prad::classifier_head_eligible<float>(B, H, C));
     if (!one_launch) {  // the separate launches, which also word the complaint about a shape that fits none of them
         Epilogue fwd;
         fwd.bias = bias; fwd.alpha = alpha;
