@@ -969,17 +969,18 @@ __global__ void __launch_bounds__(GEMM_THREADS, 4) gemm_short_kernel(const GemmA
 
 // The two gradient products of a layer, dA = dC . B^T (both operands k-contiguous; the upstream activation's
 // backward may be its epilogue) and dB = A^T . dC (both operands mn-contiguous; the bias gradient may ride along),
-// in one launch on 32 x 32 tiles: small layers cost what their chain of dependent launches costs.  Workgroups
+// in one launch on 32 x 32 or 64 x 64 tiles (WT = 1, 2): small layers cost what their chain of dependent launches
+// costs, and the launch ramp, first slab and epilogue of one product hide behind the other's main loop.  Workgroups
 // [0, first) belong to the first product, the rest to the second.  Neither product is split or batched.
-template <typename T, bool EDGE1, int EPI1, bool EDGE2>
+template <typename T, int WT, bool EDGE1, int EPI1, bool EDGE2>
 __global__ void __launch_bounds__(GEMM_THREADS, 2) gemm_pair_kernel(const GemmArgs<T> p1, const int tilesM1, const int tilesN1,
                                                                      const GemmArgs<T> p2, const int tilesM2, const int tilesN2,
                                                                      const unsigned first) {
     // (one block of LDS serves whichever product the workgroup belongs to, so two workgroups fit on a compute unit)
-    constexpr int LDS1 = gemm_lds_elems<T, 1, true, true>(), LDS2 = gemm_lds_elems<T, 1, false, false>();
+    constexpr int LDS1 = gemm_lds_elems<T, WT, true, true>(), LDS2 = gemm_lds_elems<T, WT, false, false>();
     __shared__ __attribute__((aligned(16))) T lds[LDS1 > LDS2 ? LDS1 : LDS2];
-    if (blockIdx.x < first) gemm_tile<T, 1, true, true, EDGE1, EPI1>(p1, tilesM1, tilesN1, GridPos{blockIdx.x, 0u, 0u, 1u, 1u}, lds);
-    else gemm_tile<T, 1, false, false, EDGE2, EPI_PLAIN>(p2, tilesM2, tilesN2, GridPos{blockIdx.x - first, 0u, 0u, 1u, 1u}, lds);
+    if (blockIdx.x < first) gemm_tile<T, WT, true, true, EDGE1, EPI1>(p1, tilesM1, tilesN1, GridPos{blockIdx.x, 0u, 0u, 1u, 1u}, lds);
+    else gemm_tile<T, WT, false, false, EDGE2, EPI_PLAIN>(p2, tilesM2, tilesN2, GridPos{blockIdx.x - first, 0u, 0u, 1u, 1u}, lds);
 }
 
 // Which products go to the single-stage kernel (PRAD_GEMM_SHORT=0 switches it off: tuning aid): batches of small
@@ -1363,44 +1364,62 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
 }
 
 // Both gradient products of a layer in one launch (gemm_pair_kernel).  Taken only where each product alone would
-// run unsplit on 32 x 32 tiles, so that the results are those of the two separate launches bit for bit, and where
-// the two together still give every workgroup a compute unit of its own.  hipErrorNotSupported otherwise: the
-// caller then launches the products one after the other.
+// run unsplit on the same tile, 32 x 32 or 64 x 64, so that the results are those of the two separate launches bit
+// for bit.  Measured against the separate launches, forward and backward of square products in float / double:
+// N = 768 +21 / +15 %, 1024 +9 / +3 %, 1536 +13 / +12 %, 1792 +9 / +9 % (the tail of one product overlaps the other's
+// start; PRAD_GEMM_DUAL_MAX caps the workgroups of such a launch, PRAD_GEMM_DUAL_64=0 keeps 64 x 64 tiles out: tuning
+// aids).  hipErrorNotSupported otherwise: the caller then launches the products one after the other.
 template <typename T>
 hipError_t launch_gemm_pair(const GemmArgs<T>& first_in, const GemmArgs<T>& second_in, hipStream_t stream) {
     static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_DUAL"); return !(e && e[0] == '0'); }();  // tuning aid
+    static const bool wide = [] { const char* e = getenv("PRAD_GEMM_DUAL_64"); return !(e && e[0] == '0'); }();  // tuning aid
     if (!enabled) return hipErrorNotSupported;
     GemmArgs<T> p1 = first_in, p2 = second_in;
     auto epilogue = [](const GemmArgs<T>& a) {
         return (a.bias != nullptr || a.Z != nullptr || a.act_fwd != ACT_NONE || a.act_bwd != ACT_NONE) ? EPI_ELEMENTWISE : EPI_PLAIN;
     };
-    auto small = [](const GemmArgs<T>& a) {
-        return a.M > 0 && a.N > 0 && a.K > 0 && a.batch == 1 && a.batch_inner <= 1 && a.nseg <= 1 && a.tile_sums == nullptr &&
-               choose_tile(a.M, a.N, 1, false) == TILE_32x32 && gemm_split_factor(a.M, a.N, a.K, 1, (int)sizeof(T)) == 1 &&
-               !gemm_pairs(a.M, a.N, a.K, 1, (int)sizeof(T));
+    // (a product that launch_gemm would move to shared 128 x 128 tiles adds its partial tiles in another order)
+    auto shared_ways = [](const GemmArgs<T>& a) { int tiles = 0; return gemm_shared_tiles_plan(a.M, a.N, a.K, 1, (int)sizeof(T), &tiles); };
+    // (nor one that has a kernel of its own: the streaming kernel for tall products, the one-pass weight gradient)
+    auto special = [](const GemmArgs<T>& a) {
+        if constexpr (sizeof(T) == 4) return gemm_tall_eligible(a) || gemm_skinny_eligible(a);
+        else return false;
     };
-    if (p1.transA || !p1.transB || !p2.transA || p2.transB || !small(p1) || !small(p2)) return hipErrorNotSupported;
+    auto small = [shared_ways, special](const GemmArgs<T>& a, TileShape tile) {
+        return !special(a) && a.M > 0 && a.N > 0 && a.K > 0 && a.batch == 1 && a.batch_inner <= 1 && a.nseg <= 1 && a.tile_sums == nullptr &&
+               choose_tile(a.M, a.N, 1, false) == tile && gemm_split_factor(a.M, a.N, a.K, 1, (int)sizeof(T)) == 1 &&
+               !gemm_pairs(a.M, a.N, a.K, 1, (int)sizeof(T)) && shared_ways(a) <= 1;
+    };
+    if (p1.transA || !p1.transB || !p2.transA || p2.transB || p1.M <= 0 || p1.N <= 0) return hipErrorNotSupported;
+    const TileShape tile = choose_tile(p1.M, p1.N, 1, false);
+    if (tile == TILE_128x128 || (tile == TILE_64x64 && !wide) || !small(p1, tile) || !small(p2, tile)) return hipErrorNotSupported;
     if (epilogue(p2) != EPI_PLAIN || p1.colsum_dst != nullptr) return hipErrorNotSupported;
     for (GemmArgs<T>* p : {&p1, &p2}) { p->ksplit = 0; p->zstrideA = 0; p->zstrideB = 0; p->split_counters = nullptr; }
-    const int tilesM1 = (int)((p1.M + 31) / 32), tilesN1 = (int)((p1.N + 31) / 32);
-    const int tilesM2 = (int)((p2.M + 31) / 32), tilesN2 = (int)((p2.N + 31) / 32);
+    const int edge = tile == TILE_64x64 ? 64 : 32;
+    const int tilesM1 = (int)((p1.M + edge - 1) / edge), tilesN1 = (int)((p1.N + edge - 1) / edge);
+    const int tilesM2 = (int)((p2.M + edge - 1) / edge), tilesN2 = (int)((p2.N + edge - 1) / edge);
     const unsigned first = (unsigned)(tilesM1 * tilesN1);
     const unsigned riders = p2.colsum_dst != nullptr ? (unsigned)((p2.colsum_cols + 63) / 64) : 0u;
     const unsigned total = first + (unsigned)(tilesM2 * tilesN2) + riders;
-    static const unsigned max_total = [] { const char* e = getenv("PRAD_GEMM_DUAL_MAX"); const int x = e ? atoi(e) : 0; return (unsigned)(x > 0 ? x : 512); }();  // tuning aid
+    static const unsigned max_total = [] { const char* e = getenv("PRAD_GEMM_DUAL_MAX"); const int x = e ? atoi(e) : 0; return x > 0 ? (unsigned)x : ~0u; }();  // tuning aid
     if (total > max_total) return hipErrorNotSupported;
     const int epi1 = epilogue(p1);
-    const bool edge1 = !vector_loads_ok(p1, epi1, 32), edge2 = !vector_loads_ok(p2, EPI_PLAIN, 32);
+    const bool edge1 = !vector_loads_ok(p1, epi1, edge), edge2 = !vector_loads_ok(p2, EPI_PLAIN, edge);
     const dim3 grid(total), block(GEMM_THREADS);
-#define PRAD_LAUNCH(E1_, EPI_, E2_) \
-    hipLaunchKernelGGL((gemm_pair_kernel<T, E1_, EPI_, E2_>), grid, block, 0, stream, p1, tilesM1, tilesN1, p2, tilesM2, tilesN2, first)
-    if (edge1 || edge2) {
+#define PRAD_LAUNCH(WT_, E1_, EPI_, E2_) \
+    hipLaunchKernelGGL((gemm_pair_kernel<T, WT_, E1_, EPI_, E2_>), grid, block, 0, stream, p1, tilesM1, tilesN1, p2, tilesM2, tilesN2, first)
+    if (tile == TILE_64x64) {
+        // (misaligned operands on this tile take the separate launches)
+        if (edge1 || edge2) return hipErrorNotSupported;
+        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(2, false, EPI_PLAIN, false);
+        else PRAD_LAUNCH(2, false, EPI_ELEMENTWISE, false);
+    } else if (edge1 || edge2) {
         // misaligned operands: both products on the guarded loads
-        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(true, EPI_PLAIN, true);
-        else PRAD_LAUNCH(true, EPI_ELEMENTWISE, true);
+        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(1, true, EPI_PLAIN, true);
+        else PRAD_LAUNCH(1, true, EPI_ELEMENTWISE, true);
     } else {
-        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(false, EPI_PLAIN, false);
-        else PRAD_LAUNCH(false, EPI_ELEMENTWISE, false);
+        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(1, false, EPI_PLAIN, false);
+        else PRAD_LAUNCH(1, false, EPI_ELEMENTWISE, false);
     }
 #undef PRAD_LAUNCH
     return hipGetLastError();
