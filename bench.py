@@ -715,7 +715,8 @@ def headline_lines(args, head, cpu, also, table):
     ms_per_step = head["ms"] / steps
     tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
     peak = PEAK_TFLOPS[args.dtype]
-    # dominant kernel: the MFMA product kernel, three launches per step of 2 N^3 flop each
+    # dominant kernel: the MFMA product kernel, three products per step of 2 N^3 flop each (three launches at N = 4096;
+    # below N = 2600 both gradient products share one launch)
     launch_ms = head["ms"] / (3 * steps)
     achieved = 2.0 * n ** 3 / (launch_ms * 1e-3) / 1e12
     iso = head.get("isolated_launch_ms") or {}
@@ -726,7 +727,7 @@ def headline_lines(args, head, cpu, also, table):
         "ms_per_step": sig(ms_per_step), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "configs[1]: MatrixMultiplyOperation forward+backward, %s, M=N=K=%d, A,B~U[-1,1], dC~N(0,1), seed %d, "
-                               "device-resident, 3 launches, 6N^3 flop/step" % (args.dtype, n, 20240611)},
+                               "device-resident, 3 products, 6N^3 flop/step" % (args.dtype, n, 20240611)},
         "roofline": {"bound": "mfma", "achieved": sig(achieved), "peak": peak, "unit": "TFLOP/s", "frac": sig(achieved / peak, 4),
                      "traffic": load_traffic(n, args.dtype), "kernel": "prad::gemm_kernel<%s> NN/NT/TN" % ("double" if args.dtype == "f64" else "float"),
                      "launch_ms": sig(launch_ms), "launch_ms_isolated": sig(iso_mean),
@@ -736,7 +737,7 @@ def headline_lines(args, head, cpu, also, table):
         line["cpu_baseline"] = {"value": sig(cpu["value"]), "unit": cpu["unit"], "cores": cpu["cores"], "kind": cpu["kind"],
                                 "sample": "fp64 fwd+bwd at N=%d, 1 pass, %.1f s" % (cpu["n"], cpu["secs"])}
     detail = {"headline": {"wall_ms_per_step": head["wall_ms"] / steps, "spot_check_error": head["spot"], "errors": head["errors"],
-                           "isolated_launch_ms": iso, "flop_per_step": flops_per_step, "launches_per_step": 3},
+                           "isolated_launch_ms": iso, "flop_per_step": flops_per_step, "products_per_step": 3},
               "cpu_baseline": cpu, "also": also, "table": table}
     if head["errors"] is not None:
         line["err_vs_reference_arithmetic"] = sig(head["errors"]["against_reference_arithmetic"]["elementwise_floor_rms"], 3)

@@ -273,7 +273,7 @@ inline int64_t gemm_tiles_per_product(int64_t M, int64_t N) { return ((M + 127) 
 
 template <typename T> hipError_t launch_gemm(const GemmArgs<T>& args, hipStream_t stream);
 // first = dC . B^T (transB) and second = A^T . dC (transA, may carry the column-sum rider) in one launch;
-// hipErrorNotSupported (nothing launched) unless each alone would run unsplit on the same 32 x 32 or 64 x 64 tile.
+// hipErrorNotSupported (nothing launched) unless each alone would run unsplit on tiles of the same size.
 template <typename T> hipError_t launch_gemm_pair(const GemmArgs<T>& first, const GemmArgs<T>& second, hipStream_t stream);
 
 // One LSTM time step forward in one launch: gates = act(C + A . B) with C (rows x 4H) holding the input

@@ -969,7 +969,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 4) gemm_short_kernel(const GemmA
 
 // The two gradient products of a layer, dA = dC . B^T (both operands k-contiguous; the upstream activation's
 // backward may be its epilogue) and dB = A^T . dC (both operands mn-contiguous; the bias gradient may ride along),
-// in one launch on 32 x 32 or 64 x 64 tiles (WT = 1, 2): small layers cost what their chain of dependent launches
+// in one launch on tiles of one size (WT = 1, 2, 4): small layers cost what their chain of dependent launches
 // costs, and the launch ramp, first slab and epilogue of one product hide behind the other's main loop.  Workgroups
 // [0, first) belong to the first product, the rest to the second.  Neither product is split or batched.
 template <typename T, int WT, bool EDGE1, int EPI1, bool EDGE2>
@@ -1364,10 +1364,9 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
 }
 
 // Both gradient products of a layer in one launch (gemm_pair_kernel).  Taken only where each product alone would
-// run unsplit on the same tile, 32 x 32 or 64 x 64, so that the results are those of the two separate launches bit
-// for bit.  Measured against the separate launches, forward and backward of square products in float / double:
+// run unsplit on the same tile, so that the results are those of the two separate launches bit for bit.  Measured against the separate launches, forward and backward of square products in float / double:
 // N = 768 +21 / +15 %, 1024 +9 / +3 %, 1536 +13 / +12 %, 1792 +9 / +9 % (the tail of one product overlaps the other's
-// start; PRAD_GEMM_DUAL_MAX caps the workgroups of such a launch, PRAD_GEMM_DUAL_64=0 keeps 64 x 64 tiles out: tuning
+// start; PRAD_GEMM_DUAL_MAX caps the workgroups of such a launch, PRAD_GEMM_DUAL_64=0 keeps the 64 x 64 and 128 x 128 tiles out: tuning
 // aids).  hipErrorNotSupported otherwise: the caller then launches the products one after the other.
 template <typename T>
 hipError_t launch_gemm_pair(const GemmArgs<T>& first_in, const GemmArgs<T>& second_in, hipStream_t stream) {
@@ -1392,27 +1391,38 @@ hipError_t launch_gemm_pair(const GemmArgs<T>& first_in, const GemmArgs<T>& seco
     };
     if (p1.transA || !p1.transB || !p2.transA || p2.transB || p1.M <= 0 || p1.N <= 0) return hipErrorNotSupported;
     const TileShape tile = choose_tile(p1.M, p1.N, 1, false);
-    if (tile == TILE_128x128 || (tile == TILE_64x64 && !wide) || !small(p1, tile) || !small(p2, tile)) return hipErrorNotSupported;
+    if ((tile != TILE_32x32 && !wide) || !small(p1, tile) || !small(p2, tile)) return hipErrorNotSupported;
+    // (float products of few K slabs on 128 x 128 tiles have the half-depth kernel)
+    if (tile == TILE_128x128 && sizeof(T) == 4 && (p1.K <= 384 || p2.K <= 384)) return hipErrorNotSupported;
     if (epilogue(p2) != EPI_PLAIN || p1.colsum_dst != nullptr) return hipErrorNotSupported;
-    for (GemmArgs<T>* p : {&p1, &p2}) { p->ksplit = 0; p->zstrideA = 0; p->zstrideB = 0; p->split_counters = nullptr; }
-    const int edge = tile == TILE_64x64 ? 64 : 32;
+    for (GemmArgs<T>* p : {&p1, &p2}) { p->ksplit = 0; p->zstrideA = 0; p->zstrideB = 0; p->split_counters = nullptr; p->shared_splits = 0; p->shared_tiles = 0; }
+    const int edge = tile == TILE_128x128 ? 128 : tile == TILE_64x64 ? 64 : 32;
     const int tilesM1 = (int)((p1.M + edge - 1) / edge), tilesN1 = (int)((p1.N + edge - 1) / edge);
     const int tilesM2 = (int)((p2.M + edge - 1) / edge), tilesN2 = (int)((p2.N + edge - 1) / edge);
     const unsigned first = (unsigned)(tilesM1 * tilesN1);
     const unsigned riders = p2.colsum_dst != nullptr ? (unsigned)((p2.colsum_cols + 63) / 64) : 0u;
     const unsigned total = first + (unsigned)(tilesM2 * tilesN2) + riders;
     static const unsigned max_total = [] { const char* e = getenv("PRAD_GEMM_DUAL_MAX"); const int x = e ? atoi(e) : 0; return x > 0 ? (unsigned)x : ~0u; }();  // tuning aid
-    if (total > max_total) return hipErrorNotSupported;
+    // (on 128 x 128 tiles a product of 512 tiles or more fills both workgroup slots of every compute unit by itself:
+    // N = 2048, 256 + 256 tiles, +4 % in float and +1.5 % in double for forward and backward together; N = 2304, 324 + 324, +20 %;
+    // N = 2560, 400 + 400, +1 %; N = 3072 and 4096 level within 0.8 %, and left as the launches they were)
+    static const unsigned max_total_128 = [] { const char* e = getenv("PRAD_GEMM_DUAL_MAX_128"); const int x = e ? atoi(e) : 0; return x > 0 ? (unsigned)x : 1024u; }();  // tuning aid
+    if (total > max_total || (tile == TILE_128x128 && total > max_total_128)) return hipErrorNotSupported;
     const int epi1 = epilogue(p1);
     const bool edge1 = !vector_loads_ok(p1, epi1, edge), edge2 = !vector_loads_ok(p2, EPI_PLAIN, edge);
     const dim3 grid(total), block(GEMM_THREADS);
 #define PRAD_LAUNCH(WT_, E1_, EPI_, E2_) \
     hipLaunchKernelGGL((gemm_pair_kernel<T, WT_, E1_, EPI_, E2_>), grid, block, 0, stream, p1, tilesM1, tilesN1, p2, tilesM2, tilesN2, first)
-    if (tile == TILE_64x64) {
-        // (misaligned operands on this tile take the separate launches)
+    if (tile != TILE_32x32) {
+        // (misaligned operands on these tiles take the separate launches)
         if (edge1 || edge2) return hipErrorNotSupported;
-        if (epi1 == EPI_PLAIN) PRAD_LAUNCH(2, false, EPI_PLAIN, false);
-        else PRAD_LAUNCH(2, false, EPI_ELEMENTWISE, false);
+        if (tile == TILE_128x128) {
+            if (epi1 == EPI_PLAIN) PRAD_LAUNCH(4, false, EPI_PLAIN, false);
+            else PRAD_LAUNCH(4, false, EPI_ELEMENTWISE, false);
+        } else {
+            if (epi1 == EPI_PLAIN) PRAD_LAUNCH(2, false, EPI_PLAIN, false);
+            else PRAD_LAUNCH(2, false, EPI_ELEMENTWISE, false);
+        }
     } else if (edge1 || edge2) {
         // misaligned operands: both products on the guarded loads
         if (epi1 == EPI_PLAIN) PRAD_LAUNCH(1, true, EPI_PLAIN, true);
