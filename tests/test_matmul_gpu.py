@@ -464,11 +464,14 @@ def test_bias_gradient_riding_with_the_weight_gradient(gpu, dtype, shape):
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("accumulate", [0, 1])
 @pytest.mark.parametrize("shape", [(64, 784, 256), (64, 256, 128), (64, 128, 10), (33, 17, 129), (50, 49, 49), (1, 1, 1),
-                                   (96, 200, 72), (300, 300, 300)])
+                                   (96, 200, 72), (300, 300, 300), (1024, 1024, 1024), (1000, 1100, 1040), (1000, 1001, 1003),
+                                   (2000, 2100, 2050), (2304, 2304, 2304)])
 def test_both_gradients_in_one_launch(gpu, dtype, accumulate, shape):
-    """Small layers get dA = dC . B^T (with the activation's backward) and dB = A^T . dC (+ bias gradient) from one
-    launch; asking for one gradient at a time takes the single-product launches.  Same bits either way, for aligned
-    and misaligned operands, with and without accumulation into dB, and for a shape too large for the joint launch."""
+    """A layer gets dA = dC . B^T (with the activation's backward) and dB = A^T . dC (+ bias gradient) from one
+    launch where both products run unsplit on tiles of one size (32 x 32, 64 x 64 around a thousand rows and columns,
+    128 x 128 around two thousand); asking for one gradient at a time takes the single-product launches.  Same bits
+    either way, for aligned and misaligned operands, whole and ragged tiles, with and without accumulation into dB,
+    and for a shape too large for the joint launch."""
     from parallelreverseautodiff_amd.exceptions import check
     from parallelreverseautodiff_amd.matrix import DeviceBuffer
     lib = _lib.load()
