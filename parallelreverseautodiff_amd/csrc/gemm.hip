@@ -1081,7 +1081,7 @@ enum TileShape { TILE_128x128, TILE_64x64, TILE_32x32 };
 // on 64 x 64 tiles than on 128 x 128, N = 512 4.8x faster on 32 x 32; a 128 x 64 tile was measured at
 // N = 2048 and 4096 and was never faster than 128 x 128).  PRAD_GEMM_TILE=128x128|64x64|32x32 in the
 // environment overrides the choice (a tuning aid).
-static TileShape choose_tile(int64_t M, int64_t N, int batch, bool tile_sums, int elem_size) {
+static TileShape choose_tile(int64_t M, int64_t N, int64_t K, int batch, bool tile_sums, int elem_size) {
     if (tile_sums) return TILE_128x128;  // the tile_sums layout is defined on 128 x 128 tiles
     static const int forced = []() {
         const char* e = getenv("PRAD_GEMM_TILE");
@@ -1105,6 +1105,20 @@ static TileShape choose_tile(int64_t M, int64_t N, int batch, bool tile_sums, in
     // at 768 (144), -6 / -10 % at 640 (100); the 128 x 128 tile against the 64 x 64 one is level at N = 1920 (225 tiles)
     // and 6 to 8 % behind at 1792 (196), so its threshold stays.
     auto ok = [&](int64_t e) { return padded(e) <= 2 * least; };
+    // Between 256 and 512 tiles of 128 x 128 some compute units hold two workgroups and the others one, and the launch
+    // lasts as long as two: forward and backward at N = 2304 (324 tiles) ran at 61 % of peak in double, at N = 2560
+    // (400) at 75 %, while four times as many 64 x 64 tiles, spread more evenly, reach 79 and 83 % (float: 70 and 72 %
+    // against 74 and 78 %); at N = 2816 (484 tiles) the large tile is ahead again, 90 against 84 %.  Taking a compute
+    // unit to work through its workgroups at one rate however many it holds, a launch of t tiles lasts ceil(t / 256)
+    // rounds, and the tile with the better even-ness times its own efficiency (measured: 0.956 and 0.90 in double,
+    // 0.93 and 0.85 in float) wins.  Only for a K of a thousand or more: shallow products on some four hundred tiles
+    // have the half-depth kernel, measured on the large tile.
+    if (ok(128) && ok(64) && K >= 1024 && tiles(128) > 256 && tiles(128) < 512) {
+        auto evenness = [](int64_t t) { return (double)t / (double)((t + 255) / 256 * 256); };
+        const double large = evenness(tiles(128)) * (elem_size == 4 ? 0.93 : 0.956);
+        const double small = evenness(tiles(64)) * (elem_size == 4 ? 0.85 : 0.90);
+        return small > large ? TILE_64x64 : TILE_128x128;
+    }
     if (ok(128) && tiles(128) >= 256) return TILE_128x128;
     if (ok(64) && tiles(64) >= (elem_size == 4 ? 144 : 192)) return TILE_64x64;
     if (ok(32)) return TILE_32x32;
@@ -1152,7 +1166,7 @@ static int64_t slab_depth(TileShape t, int elem_size) {
 bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
     static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_PAIRS"); return e && e[0] == '1'; }();
     if (!enabled || gemm_split_factor(M, N, K, batch, elem_size) > 1) return false;
-    const TileShape t = choose_tile(M, N, batch, false, elem_size);
+    const TileShape t = choose_tile(M, N, K, batch, false, elem_size);
     const int64_t e = t == TILE_128x128 ? 128 : t == TILE_64x64 ? 64 : 32;
     const int64_t wgs = ((M + e - 1) / e) * ((N + e - 1) / e) * batch;
     return t != TILE_128x128 && wgs >= 128 && wgs <= GEMM_SPLIT_MAX_TILES && K >= 32 * slab_depth(t, elem_size);
@@ -1166,7 +1180,7 @@ bool gemm_pairs(int64_t M, int64_t N, int64_t K, int batch, int elem_size) {
 // Returns the ways (0: not such a product) and the number of tiles.
 static int few_tiles_long_k_plan(int64_t M, int64_t N, int64_t K, int elem_size, int* tiles_out) {
     static const bool enabled = [] { const char* e = getenv("PRAD_GEMM_FEW_TILES"); return !(e && e[0] == '0'); }();  // tuning aid
-    if (!enabled || choose_tile(M, N, 1, false, elem_size) == TILE_128x128) return 0;
+    if (!enabled || choose_tile(M, N, K, 1, false, elem_size) == TILE_128x128) return 0;
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     if (tiles * 128 * 128 * 4 > M * N * 5) return 0;  // more than a quarter of padding: the smaller tiles multiply less
     const int64_t bk = slab_depth(TILE_128x128, elem_size);
@@ -1186,7 +1200,7 @@ int gemm_shared_tiles_plan(int64_t M, int64_t N, int64_t K, int batch, int elem_
     if (!enabled || batch != 1) return 0;
     if (gemm_split_factor(M, N, K, batch, elem_size) > 1) return 0;
     if (const int ways = few_tiles_long_k_plan(M, N, K, elem_size, shared_tiles)) return ways;
-    if (choose_tile(M, N, batch, false, elem_size) != TILE_128x128) return 0;
+    if (choose_tile(M, N, K, batch, false, elem_size) != TILE_128x128) return 0;
     constexpr int64_t SLOTS = 512;  // two workgroups of the 128 x 128 kernels per compute unit
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     // (fewer tiles than slots - 256 tiles, one per compute unit - were measured with every tile shared two ways: +2 %,
@@ -1289,7 +1303,7 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         part.accumulate = 0;
         part.bias = nullptr; part.Z = nullptr; part.act_fwd = ACT_NONE; part.act_bwd = ACT_NONE; part.act_src = nullptr;
         hipError_t e;
-        switch (choose_tile(a.M, a.N, a.nseg, false, (int)sizeof(T))) {
+        switch (choose_tile(a.M, a.N, a.K, a.nseg, false, (int)sizeof(T))) {
             case TILE_128x128: e = launch_tile<T, 4>(part, EPI_PLAIN, stream); break;
             case TILE_64x64: e = launch_tile<T, 2>(part, EPI_PLAIN, stream); break;
             default: e = launch_tile<T, 1>(part, EPI_PLAIN, stream); break;
@@ -1329,7 +1343,7 @@ hipError_t launch_gemm(const GemmArgs<T>& a_in, hipStream_t stream) {
         hipLaunchKernelGGL((split_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, a, a.split_ws, splits);
         return hipGetLastError();
     }
-    TileShape tile = choose_tile(a.M, a.N, a.batch, a.tile_sums != nullptr, (int)sizeof(T));
+    TileShape tile = choose_tile(a.M, a.N, a.K, a.batch, a.tile_sums != nullptr, (int)sizeof(T));
     a.shared_tiles = 0; a.shared_splits = 0;
     int shared_tiles = 0;
     const int shared_ways = (a.tile_sums == nullptr && a.split_ws != nullptr && epi != EPI_TILE_SUM &&
@@ -1390,11 +1404,11 @@ hipError_t launch_gemm_pair(const GemmArgs<T>& first_in, const GemmArgs<T>& seco
     };
     auto small = [shared_ways, special](const GemmArgs<T>& a, TileShape tile) {
         return !special(a) && a.M > 0 && a.N > 0 && a.K > 0 && a.batch == 1 && a.batch_inner <= 1 && a.nseg <= 1 && a.tile_sums == nullptr &&
-               choose_tile(a.M, a.N, 1, false, (int)sizeof(T)) == tile && gemm_split_factor(a.M, a.N, a.K, 1, (int)sizeof(T)) == 1 &&
+               choose_tile(a.M, a.N, a.K, 1, false, (int)sizeof(T)) == tile && gemm_split_factor(a.M, a.N, a.K, 1, (int)sizeof(T)) == 1 &&
                !gemm_pairs(a.M, a.N, a.K, 1, (int)sizeof(T)) && shared_ways(a) <= 1;
     };
     if (p1.transA || !p1.transB || !p2.transA || p2.transB || p1.M <= 0 || p1.N <= 0) return hipErrorNotSupported;
-    const TileShape tile = choose_tile(p1.M, p1.N, 1, false, (int)sizeof(T));
+    const TileShape tile = choose_tile(p1.M, p1.N, p1.K, 1, false, (int)sizeof(T));
     if ((tile != TILE_32x32 && !wide) || !small(p1, tile) || !small(p2, tile)) return hipErrorNotSupported;
     // (float products of few K slabs on 128 x 128 tiles have the half-depth kernel)
     if (tile == TILE_128x128 && sizeof(T) == 4 && (p1.K <= 384 || p2.K <= 384)) return hipErrorNotSupported;
