@@ -1105,18 +1105,37 @@ static TileShape choose_tile(int64_t M, int64_t N, int64_t K, int batch, bool ti
     // at 768 (144), -6 / -10 % at 640 (100); the 128 x 128 tile against the 64 x 64 one is level at N = 1920 (225 tiles)
     // and 6 to 8 % behind at 1792 (196), so its threshold stays.
     auto ok = [&](int64_t e) { return padded(e) <= 2 * least; };
-    // Between 256 and 512 tiles of 128 x 128 some compute units hold two workgroups and the others one, and the launch
-    // lasts as long as two: forward and backward at N = 2304 (324 tiles) ran at 61 % of peak in double, at N = 2560
-    // (400) at 75 %, while four times as many 64 x 64 tiles, spread more evenly, reach 79 and 83 % (float: 70 and 72 %
-    // against 74 and 78 %); at N = 2816 (484 tiles) the large tile is ahead again, 90 against 84 %.  Taking a compute
-    // unit to work through its workgroups at one rate however many it holds, a launch of t tiles lasts ceil(t / 256)
-    // rounds, and the tile with the better even-ness times its own efficiency (measured: 0.956 and 0.90 in double,
-    // 0.93 and 0.85 in float) wins.  Only for a K of a thousand or more: shallow products on some four hundred tiles
-    // have the half-depth kernel, measured on the large tile.
-    if (ok(128) && ok(64) && K >= 1024 && tiles(128) > 256 && tiles(128) < 512) {
-        auto evenness = [](int64_t t) { return (double)t / (double)((t + 255) / 256 * 256); };
-        const double large = evenness(tiles(128)) * (elem_size == 4 ? 0.93 : 0.956);
-        const double small = evenness(tiles(64)) * (elem_size == 4 ? 0.85 : 0.90);
+    // Past 256 tiles of 128 x 128 the launch is rounds of unequal fill: 400 tiles put two workgroups on some compute
+    // units and one on the rest and last as long as 512; 784 tiles last as long as 1024.  Forward and backward at
+    // N = 2304 (324 tiles) ran at 61 % of peak in double, at 2560 (400) at 75 %, at 3584 (784) at 73 %, at 3840 (900) at
+    // 85 %, while four times as many 64 x 64 tiles, spread more evenly, reach 84, 89, 91 and 90 % (float: 70, 72, 72
+    // and 82 % against 77, 83, 87 and 86 %).  Where the large tile fills its rounds it stays ahead: N = 2816 (484
+    // tiles) 90 against 84 %, 3328 (676, the last 164 shared three ways, see gemm_shared_tiles_plan) 93 against 91 %,
+    // 4096 96.3 against 95.4 %, 5120 95 against 84 %.  The model that reproduces every one of these: a compute unit works through its
+    // workgroups at one rate however many it holds, so t tiles last ceil(t / 256) rounds (a shared last round:
+    // ceil(rest * ways / 256) / ways), and the tile with the better work / rounds times its own efficiency wins
+    // (0.956, shared 0.94, against 0.90 in double; 0.93, 0.885 against 0.87 in float: the small tile's own figure was
+    // measured between 0.84 and 0.95 from one machine and size to the next - it moves twice the bytes per flop and
+    // falls to 0.83 at N = 6144 - so it is set where the clear cases above go its way and the close ones do not).
+    // Only for a K of a thousand or more: shallow products on hundreds of tiles have the half-depth kernel,
+    // measured on the large tile.
+    if (ok(128) && ok(64) && K >= 1024 && tiles(128) > 256) {
+        const int64_t t = tiles(128), q = t / 512, rest = t % 512;
+        double rounds = (double)((t + 255) / 256);
+        bool shared = false;
+        if (t >= 512 && rest != 0 && rest <= 256 && batch == 1) {
+            const int64_t bk = elem_size == 8 ? Slab<double, 4>::BK : Slab<float, 4>::BK;
+            int64_t ways = 512 / rest < 4 ? 512 / rest : 4;
+            if (ways > K / (8 * bk)) ways = K / (8 * bk);
+            if (ways >= 2) {
+                shared = true;
+                rounds = 2.0 * (double)q + (double)((rest * ways + 255) / 256) / (double)ways;
+            }
+        }
+        const bool f32 = elem_size == 4;
+        const double large = (double)t / 256.0 / rounds * (shared ? (f32 ? 0.885 : 0.94) : (f32 ? 0.93 : 0.956));
+        const int64_t t64 = tiles(64);
+        const double small = (double)t64 / (double)((t64 + 255) / 256 * 256) * (f32 ? 0.87 : 0.90);
         return small > large ? TILE_64x64 : TILE_128x128;
     }
     if (ok(128) && tiles(128) >= 256) return TILE_128x128;
