@@ -348,10 +348,12 @@ int32_t attach_split_workspace(GemmArgs<T>& a) {
             return PRAD_OK;
         }
     }
+    // (in launch_gemm's order: split along K, else tiles shared several ways, else pairs of workgroups - a product that
+    // qualifies for the last two is launched on shared tiles and needs their room)
     const int splits = gemm_split_factor(a.M, a.N, a.K, a.batch, (int)sizeof(T));
-    const bool pairs = splits <= 1 && gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T));
     int shared_tiles = 0;
-    const int shared = (splits <= 1 && !pairs) ? gemm_shared_tiles_plan(a.M, a.N, a.K, a.batch, (int)sizeof(T), &shared_tiles) : 0;
+    const int shared = splits <= 1 ? gemm_shared_tiles_plan(a.M, a.N, a.K, a.batch, (int)sizeof(T), &shared_tiles) : 0;
+    const bool pairs = splits <= 1 && shared <= 1 && gemm_pairs(a.M, a.N, a.K, a.batch, (int)sizeof(T));
     if (splits <= 1 && !pairs && shared <= 1) return PRAD_OK;
     const size_t bytes = shared > 1 ? (size_t)shared_tiles * shared * 128 * 128 * sizeof(T)
                                   : (size_t)(pairs ? 2 : splits) * a.batch * a.M * a.N * sizeof(T);

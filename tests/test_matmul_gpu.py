@@ -681,11 +681,16 @@ def test_rows_of_a_tall_product_do_not_depend_on_how_many_rows_there_are(gpu, or
     assert same(f[0][:head], q[0])
 
 
-def test_workgroup_pairs_when_switched_on(gpu):
+@pytest.mark.parametrize("forced_tile", [None, "64x64"])
+def test_workgroup_pairs_when_switched_on(gpu, forced_tile):
     """Pairs of workgroups per tile are a tuning aid that is off by default (the library reads PRAD_GEMM_PAIRS once):
-    the test above runs again in a process of its own with the switch on."""
+    the test above runs again in a process of its own with the switch on - and once more with the tile size forced as
+    well, where a product can qualify both for pairs and for tiles shared several ways (it is launched on the shared
+    tiles, and the workspace has to be sized for those)."""
     import os, subprocess, sys
     env = dict(os.environ, PRAD_GEMM_PAIRS="1")
+    if forced_tile:
+        env["PRAD_GEMM_TILE"] = forced_tile
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(root, "tests", "test_matmul_gpu.py"), "-q", "-x", "-m", "gpu",
                         "-k", "test_products_of_few_tiles_and_long_k", "-p", "no:cacheprovider"],
